@@ -1,0 +1,139 @@
+// Shared declarations of libbitsmoe_hip: device views of packed expert matrices, the
+// bit-plane decode rule, error plumbing.  gfx950 only (wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <hip/hip_bf16.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "../../include/bitsmoe_hip.h"
+
+namespace bitsmoe {
+
+constexpr int K_SLAB = 64;    // rows per slab (at most)
+constexpr int K_STAGE = 16;   // rows per stage inside a slab
+constexpr int N_TILE = 128;   // columns per tile
+constexpr int N_MICRO = 32;   // columns per plane word
+constexpr int MICROS = N_TILE / N_MICRO;
+
+// One packed expert matrix as the kernels see it.
+struct MatView {
+    const uint32_t* payload;
+    const int32_t* rank_idx;
+    const int32_t* tile_meta;  // [num_tiles][3] = pack_off, scale_off, n_valid
+    const int32_t* slab_meta;  // [num_slabs][4] = bits, k_slab, rank_off, tile_off
+    const __half* scale;
+    const __half* s;
+    int32_t num_slabs;
+    int32_t num_tiles;
+    int32_t rank_len;
+    int32_t flags;             // bit0: regular layout
+};
+
+struct SlabTask {              // one (expert, slab) unit of the down projection
+    int32_t expert;
+    int32_t slab;
+};
+
+}  // namespace bitsmoe
+
+// The opaque handle of the C ABI.
+struct bitsmoe_matset {
+    int32_t n_experts = 0;
+    int32_t intermediate_size = 0;
+    int32_t n_tiles = 0;              // ceil(I / 128)
+    int32_t max_slabs = 0;            // largest num_slabs over experts
+    int64_t total_slabs = 0;
+    int32_t max_rank_plus1 = 0;       // 1 + largest logical rank referenced by rank_idx
+    int32_t min_rank = 0;             // smallest logical rank
+    bool regular = false;             // every matrix: 2/3/4-bit, k_slab % 16 == 0, full tiles
+    int device = -1;
+    std::vector<bitsmoe_matrix_desc> descs;
+    std::vector<std::vector<int32_t>> slab_meta_host;
+    std::vector<std::vector<int32_t>> tile_meta_host;
+    bitsmoe::MatView* d_views = nullptr;      // [n_experts]
+    bitsmoe::SlabTask* d_slab_tasks = nullptr;  // [total_slabs]
+};
+
+struct bitsmoe_profile {
+    hipEvent_t ev[BITSMOE_PROFILE_PHASES + 1];
+    bool recorded = false;
+};
+
+namespace bitsmoe {
+
+void set_error(const char* fmt, ...);
+int hip_fail(hipError_t e, const char* what);
+
+#define BITSMOE_HIP_TRY(expr)                                        \
+    do {                                                             \
+        hipError_t _e = (expr);                                      \
+        if (_e != hipSuccess) return ::bitsmoe::hip_fail(_e, #expr); \
+    } while (0)
+
+#define BITSMOE_REQUIRE(cond, ...)           \
+    do {                                     \
+        if (!(cond)) {                       \
+            ::bitsmoe::set_error(__VA_ARGS__); \
+            return BITSMOE_E_INVALID;        \
+        }                                    \
+    } while (0)
+
+__host__ __device__ inline int words_per_row(int bits) { return bits == 16 ? 16 : bits; }
+
+__host__ __device__ inline int level_offset(int bits) {
+    // stored code u = level + offset; 1-bit stores (level+1)/2
+    switch (bits) {
+        case 2: return 2;
+        case 3: return 4;
+        case 4: return 8;
+        case 6: return 32;
+        case 8: return 128;
+        default: return 0;
+    }
+}
+
+__host__ inline bool bits_supported(int b) {
+    return b == 1 || b == 2 || b == 3 || b == 4 || b == 6 || b == 8 || b == 16;
+}
+
+// Decode one element from the words of one (row, micro-tile): `w` points at the first
+// plane word of that row; returns the level (low-bit) or the stored half (16-bit) as fp32,
+// without the scale.
+__device__ inline float decode_from_row_words(const uint32_t* w, int bits, int lane) {
+    if (bits == 16) {
+        const uint32_t word = w[lane >> 1];
+        const uint16_t hb = (lane & 1) ? (uint16_t)(word >> 16) : (uint16_t)(word & 0xFFFFu);
+        return __half2float(__ushort_as_half(hb));
+    }
+    int u = 0;
+    for (int p = 0; p < bits; ++p) u |= (int)((w[p] >> lane) & 1u) << p;
+    const int q = (bits == 1) ? (2 * u - 1) : (u - level_offset(bits));
+    return (float)q;
+}
+
+template <typename T>
+__device__ inline float to_f32(T v);
+template <>
+__device__ inline float to_f32<__half>(__half v) { return __half2float(v); }
+template <>
+__device__ inline float to_f32<__hip_bfloat16>(__hip_bfloat16 v) { return __bfloat162float(v); }
+
+__device__ inline float silu_f32(float x) { return x / (1.0f + __expf(-x)); }
+
+// launchers implemented in the kernel translation units
+int launch_fill_zero(float* p, int64_t n, hipStream_t st);
+int launch_forward_generic(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                           const bitsmoe_matset* down, const void* h_gate, const void* h_up,
+                           int act_dtype, int64_t T, int Rg, int Ru, const int32_t* tok,
+                           const int32_t* off, const float* rw, int64_t A, int rank_out, int I,
+                           float* rank_accum, float* G, float* U, bitsmoe_profile* prof,
+                           hipStream_t st);
+
+}  // namespace bitsmoe

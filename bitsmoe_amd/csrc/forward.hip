@@ -1,0 +1,78 @@
+// C-ABI entry point of the routed-expert forward: argument checks, workspace carving and
+// kernel-path selection.
+#include "common.h"
+
+using namespace bitsmoe;
+
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+extern "C" size_t bitsmoe_forward_workspace_bytes(int64_t n_tokens, int64_t n_assign,
+                                                  int32_t intermediate_size, int32_t n_experts,
+                                                  int32_t rank_out) {
+    (void)n_tokens;
+    (void)n_experts;
+    (void)rank_out;
+    if (n_assign < 0 || intermediate_size < 0) return 0;
+    // two fp32 [A, I] intermediates (gate and up outputs)
+    const size_t inter = align_up((size_t)n_assign * (size_t)intermediate_size * sizeof(float), 256);
+    return 2 * inter + 256;
+}
+
+extern "C" int bitsmoe_moe_forward(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                                   const bitsmoe_matset* down, const void* h_gate, const void* h_up,
+                                   int32_t act_dtype, int64_t n_tokens, int32_t rank_gate,
+                                   int32_t rank_up, const int32_t* token_indices,
+                                   const int32_t* expert_offsets, const float* route_w,
+                                   int64_t n_assign, int32_t rank_out, int32_t intermediate_size,
+                                   int32_t act_type, int32_t path, float* rank_accum, void* workspace,
+                                   size_t workspace_bytes, bitsmoe_profile* profile, void* stream) {
+    hipStream_t st = (hipStream_t)stream;
+    BITSMOE_REQUIRE(gate && up && down, "matrix sets must not be null");
+    BITSMOE_REQUIRE(act_type == 0, "only SiLU act_type=0 is currently supported");
+    BITSMOE_REQUIRE(act_dtype == BITSMOE_DT_F16 || act_dtype == BITSMOE_DT_BF16, "act_dtype must be f16 (0) or bf16 (1)");
+    BITSMOE_REQUIRE(intermediate_size > 0, "intermediate_size must be > 0");
+    BITSMOE_REQUIRE(rank_out > 0, "rank_out must be > 0");
+    BITSMOE_REQUIRE(n_tokens >= 0 && n_assign >= 0, "negative token or assignment count");
+    BITSMOE_REQUIRE(n_tokens < ((int64_t)1 << 31) && n_assign < ((int64_t)1 << 31), "token/assignment count exceeds int32");
+    BITSMOE_REQUIRE(rank_accum != nullptr || n_tokens == 0, "rank_accum must not be null");
+    BITSMOE_REQUIRE(gate->n_experts == up->n_experts && gate->n_experts == down->n_experts,
+                    "gate/up/down sets hold different expert counts (%d, %d, %d)", gate->n_experts,
+                    up->n_experts, down->n_experts);
+    BITSMOE_REQUIRE(gate->intermediate_size == intermediate_size && up->intermediate_size == intermediate_size &&
+                        down->intermediate_size == intermediate_size,
+                    "intermediate_size %d does not match the matrix sets", intermediate_size);
+    BITSMOE_REQUIRE(path >= BITSMOE_PATH_AUTO && path <= BITSMOE_PATH_MFMA, "unknown path %d", path);
+
+    if (n_tokens == 0) return BITSMOE_OK;
+    if (n_assign == 0 || gate->n_experts == 0) {
+        if (profile) {
+            for (int i = 0; i <= BITSMOE_PROFILE_PHASES; ++i) (void)hipEventRecord(profile->ev[i], st);
+            profile->recorded = true;
+        }
+        return launch_fill_zero(rank_accum, n_tokens * (int64_t)rank_out, st);
+    }
+    BITSMOE_REQUIRE(h_gate && h_up && token_indices && expert_offsets && route_w, "null input pointer");
+    BITSMOE_REQUIRE(rank_gate > 0 && rank_up > 0, "rank_gate/rank_up must be > 0");
+    BITSMOE_REQUIRE(gate->max_rank_plus1 <= rank_gate && gate->min_rank >= 0,
+                    "gate rank_idx references rank %d but h_gate has %d columns", gate->max_rank_plus1 - 1, rank_gate);
+    BITSMOE_REQUIRE(up->max_rank_plus1 <= rank_up && up->min_rank >= 0,
+                    "up rank_idx references rank %d but h_up has %d columns", up->max_rank_plus1 - 1, rank_up);
+    const size_t need = bitsmoe_forward_workspace_bytes(n_tokens, n_assign, intermediate_size, gate->n_experts, rank_out);
+    if (workspace == nullptr || workspace_bytes < need) {
+        set_error("workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
+        return BITSMOE_E_WORKSPACE;
+    }
+    BITSMOE_REQUIRE(((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
+
+    const size_t inter = align_up((size_t)n_assign * (size_t)intermediate_size * sizeof(float), 256);
+    float* G = (float*)workspace;
+    float* U = (float*)((char*)workspace + inter);
+
+    if (path == BITSMOE_PATH_DECODE || path == BITSMOE_PATH_MFMA) {
+        set_error("path %d is not built into this library version", path);
+        return BITSMOE_E_UNSUPPORTED;
+    }
+    return launch_forward_generic(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up,
+                                  token_indices, expert_offsets, route_w, n_assign, rank_out,
+                                  intermediate_size, rank_accum, G, U, profile, st);
+}

@@ -1,0 +1,254 @@
+// Routing / permute: token-to-expert histogram, exclusive scan and STABLE scatter built
+// on wave64 ballots.  No host synchronisation; the number of kept assignments stays on
+// the device as expert_offsets[n_packed].
+#include "common.h"
+
+namespace bitsmoe {
+
+constexpr int ROUTE_THREADS = 256;
+constexpr int ROUTE_ROUNDS = 4;
+constexpr int ROUTE_CHUNK = ROUTE_THREADS * ROUTE_ROUNDS;  // flat entries per workgroup
+constexpr int ROUTE_MAX_EXPERTS = 4096;                     // histogram lives in LDS
+
+template <typename IdT>
+__device__ inline int load_local_id(const IdT* __restrict__ selected, const int32_t* __restrict__ g2l,
+                                    int n_global, int n_packed, int64_t idx, int64_t n_flat) {
+    if (idx >= n_flat) return -1;
+    const int64_t g = (int64_t)selected[idx];
+    if (g < 0 || g >= n_global) return -1;
+    const int l = g2l[g];
+    return (l >= 0 && l < n_packed) ? l : -1;
+}
+
+// Lanes of the wave holding the same non-negative id, found with one ballot per id bit.
+__device__ inline uint64_t match_same_id(int id, int id_bits) {
+    uint64_t mask = __ballot(id >= 0);
+    for (int b = 0; b < id_bits; ++b) {
+        const bool bit = (id >> b) & 1;
+        const uint64_t bal = __ballot(bit);
+        mask &= bit ? bal : ~bal;
+    }
+    return mask;
+}
+
+// Rank of each of this workgroup's entries among the earlier entries of the same expert
+// inside the workgroup's chunk (flat order), plus the chunk's histogram in `hist` (LDS).
+// Entry order inside a chunk: round-major, then thread id.
+template <typename IdT>
+__device__ inline void chunk_ranks(const IdT* __restrict__ selected, const int32_t* __restrict__ g2l,
+                                   int n_global, int n_packed, int id_bits, int64_t chunk_base,
+                                   int64_t n_flat, int* hist, int (&local)[ROUTE_ROUNDS],
+                                   int (&rank)[ROUTE_ROUNDS]) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    for (int e = tid; e < n_packed; e += ROUTE_THREADS) hist[e] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < ROUTE_ROUNDS; ++j) {
+        const int64_t idx = chunk_base + (int64_t)j * ROUTE_THREADS + tid;
+        const int id = load_local_id<IdT>(selected, g2l, n_global, n_packed, idx, n_flat);
+        const uint64_t same = match_same_id(id, id_bits);
+        const int before = __popcll(same & ((1ull << lane) - 1ull));
+        const int count = __popcll(same);
+        const bool last = (id >= 0) && (lane == 63 - __clzll((long long)same));
+        int old = 0;
+        for (int wv = 0; wv < ROUTE_THREADS / 64; ++wv) {
+            if (wave == wv && id >= 0) old = hist[id];
+            __syncthreads();
+            if (wave == wv && last) hist[id] = old + count;
+            __syncthreads();
+        }
+        local[j] = id;
+        rank[j] = old + before;
+    }
+}
+
+// Exclusive scan of data[0..n) in LDS by the whole workgroup; returns the total.
+__device__ inline int block_exclusive_scan(int* data, int n, int* wave_sums) {
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int per = (n + nthreads - 1) / nthreads;
+    const int begin = tid * per;
+    int sum = 0;
+    for (int i = 0; i < per; ++i)
+        if (begin + i < n) sum += data[begin + i];
+    int incl = sum;
+    for (int d = 1; d < 64; d <<= 1) {
+        const int v = __shfl_up(incl, d);
+        if (lane >= d) incl += v;
+    }
+    if (lane == 63) wave_sums[wave] = incl;
+    __syncthreads();
+    const int nwaves = nthreads >> 6;
+    int wave_prefix = 0, total = 0;
+    for (int wv = 0; wv < nwaves; ++wv) {
+        const int v = wave_sums[wv];
+        if (wv < wave) wave_prefix += v;
+        total += v;
+    }
+    int run = wave_prefix + incl - sum;
+    for (int i = 0; i < per; ++i) {
+        if (begin + i < n) {
+            const int v = data[begin + i];
+            data[begin + i] = run;
+            run += v;
+        }
+    }
+    __syncthreads();
+    return total;
+}
+
+// Whole routing in one workgroup for n_flat <= ROUTE_CHUNK (decode-size batches).
+template <typename IdT>
+__global__ __launch_bounds__(ROUTE_THREADS) void k_route_fused(
+    const IdT* __restrict__ selected, const float* __restrict__ weights, const int32_t* __restrict__ g2l,
+    int n_global, int64_t n_flat, int top_k, int n_packed, int id_bits,
+    int32_t* __restrict__ token_indices, int32_t* __restrict__ expert_offsets, float* __restrict__ route_flat) {
+    extern __shared__ int lds[];
+    int* hist = lds;
+    int* wave_sums = lds + n_packed;
+    int local[ROUTE_ROUNDS], rank[ROUTE_ROUNDS];
+    chunk_ranks<IdT>(selected, g2l, n_global, n_packed, id_bits, 0, n_flat, hist, local, rank);
+    const int total = block_exclusive_scan(hist, n_packed, wave_sums);
+    const int tid = threadIdx.x;
+    for (int e = tid; e < n_packed; e += ROUTE_THREADS) expert_offsets[e] = hist[e];
+    if (tid == 0) expert_offsets[n_packed] = total;
+#pragma unroll
+    for (int j = 0; j < ROUTE_ROUNDS; ++j) {
+        if (local[j] >= 0) {
+            const int64_t idx = (int64_t)j * ROUTE_THREADS + tid;
+            const int pos = hist[local[j]] + rank[j];
+            token_indices[pos] = (int32_t)(idx / top_k);
+            route_flat[pos] = weights[idx];
+        }
+    }
+}
+
+// Multi-workgroup version: (1) per-chunk ranks + histograms, (2) scan, (3) scatter.
+template <typename IdT>
+__global__ __launch_bounds__(ROUTE_THREADS) void k_route_count(
+    const IdT* __restrict__ selected, const int32_t* __restrict__ g2l, int n_global, int64_t n_flat,
+    int n_packed, int id_bits, int32_t* __restrict__ entry_rank, int32_t* __restrict__ chunk_hist) {
+    extern __shared__ int lds[];
+    int* hist = lds;
+    int local[ROUTE_ROUNDS], rank[ROUTE_ROUNDS];
+    const int64_t chunk_base = (int64_t)blockIdx.x * ROUTE_CHUNK;
+    chunk_ranks<IdT>(selected, g2l, n_global, n_packed, id_bits, chunk_base, n_flat, hist, local, rank);
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int j = 0; j < ROUTE_ROUNDS; ++j) {
+        const int64_t idx = chunk_base + (int64_t)j * ROUTE_THREADS + tid;
+        if (idx < n_flat) entry_rank[idx] = (local[j] >= 0) ? rank[j] : -1;
+    }
+    for (int e = tid; e < n_packed; e += ROUTE_THREADS) chunk_hist[(int64_t)blockIdx.x * n_packed + e] = hist[e];
+}
+
+__global__ __launch_bounds__(1024) void k_route_scan(int32_t* __restrict__ chunk_hist, int n_chunks,
+                                                      int n_packed, int32_t* __restrict__ expert_offsets) {
+    extern __shared__ int lds[];
+    int* totals = lds;
+    int* wave_sums = lds + n_packed;
+    for (int e = threadIdx.x; e < n_packed; e += blockDim.x) {
+        int run = 0;
+        for (int b = 0; b < n_chunks; ++b) {
+            const int64_t i = (int64_t)b * n_packed + e;
+            const int c = chunk_hist[i];
+            chunk_hist[i] = run;  // entries of this expert in earlier chunks
+            run += c;
+        }
+        totals[e] = run;
+    }
+    __syncthreads();
+    const int total = block_exclusive_scan(totals, n_packed, wave_sums);
+    for (int e = threadIdx.x; e < n_packed; e += blockDim.x) expert_offsets[e] = totals[e];
+    if (threadIdx.x == 0) expert_offsets[n_packed] = total;
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(ROUTE_THREADS) void k_route_scatter(
+    const IdT* __restrict__ selected, const float* __restrict__ weights, const int32_t* __restrict__ g2l,
+    int n_global, int64_t n_flat, int top_k, int n_packed, const int32_t* __restrict__ entry_rank,
+    const int32_t* __restrict__ chunk_hist, const int32_t* __restrict__ expert_offsets,
+    int32_t* __restrict__ token_indices, float* __restrict__ route_flat) {
+    const int64_t idx = (int64_t)blockIdx.x * ROUTE_THREADS + threadIdx.x;
+    if (idx >= n_flat) return;
+    const int r = entry_rank[idx];
+    if (r < 0) return;
+    const int id = load_local_id<IdT>(selected, g2l, n_global, n_packed, idx, n_flat);
+    const int64_t chunk = idx / ROUTE_CHUNK;
+    const int pos = expert_offsets[id] + chunk_hist[chunk * n_packed + id] + r;
+    token_indices[pos] = (int32_t)(idx / top_k);
+    route_flat[pos] = weights[idx];
+}
+
+template <typename IdT>
+static int route_impl(const IdT* selected, const float* weights, const int32_t* g2l, int n_global,
+                      int64_t n_flat, int top_k, int n_packed, int32_t* token_indices,
+                      int32_t* expert_offsets, float* route_flat, void* workspace, hipStream_t st) {
+    int id_bits = 0;
+    while ((1 << id_bits) < n_packed) ++id_bits;
+    const size_t lds_bytes = (size_t)(n_packed + 32) * sizeof(int);
+    if (n_flat <= ROUTE_CHUNK) {
+        hipLaunchKernelGGL(k_route_fused<IdT>, dim3(1), dim3(ROUTE_THREADS), lds_bytes, st, selected, weights,
+                           g2l, n_global, n_flat, top_k, n_packed, id_bits, token_indices, expert_offsets,
+                           route_flat);
+        BITSMOE_HIP_TRY(hipGetLastError());
+        return BITSMOE_OK;
+    }
+    const int64_t n_chunks = (n_flat + ROUTE_CHUNK - 1) / ROUTE_CHUNK;
+    int32_t* entry_rank = (int32_t*)workspace;
+    int32_t* chunk_hist = entry_rank + ((n_flat + 63) / 64) * 64;
+    hipLaunchKernelGGL(k_route_count<IdT>, dim3((unsigned)n_chunks), dim3(ROUTE_THREADS), lds_bytes, st,
+                       selected, g2l, n_global, n_flat, n_packed, id_bits, entry_rank, chunk_hist);
+    BITSMOE_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(k_route_scan, dim3(1), dim3(1024), lds_bytes, st, chunk_hist, (int)n_chunks, n_packed,
+                       expert_offsets);
+    BITSMOE_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(k_route_scatter<IdT>, dim3((unsigned)((n_flat + ROUTE_THREADS - 1) / ROUTE_THREADS)),
+                       dim3(ROUTE_THREADS), 0, st, selected, weights, g2l, n_global, n_flat, top_k, n_packed,
+                       entry_rank, chunk_hist, expert_offsets, token_indices, route_flat);
+    BITSMOE_HIP_TRY(hipGetLastError());
+    return BITSMOE_OK;
+}
+
+}  // namespace bitsmoe
+
+using namespace bitsmoe;
+
+extern "C" size_t bitsmoe_route_workspace_bytes(int64_t n_flat, int32_t n_packed) {
+    if (n_flat <= ROUTE_CHUNK || n_packed <= 0) return 256;
+    const int64_t n_chunks = (n_flat + ROUTE_CHUNK - 1) / ROUTE_CHUNK;
+    return (size_t)(((n_flat + 63) / 64) * 64 + n_chunks * (int64_t)n_packed) * sizeof(int32_t) + 256;
+}
+
+extern "C" int bitsmoe_route(const void* selected, int32_t ids_are_i64, const float* weights,
+                             const int32_t* global_to_local, int32_t n_global, int64_t n_tokens,
+                             int32_t top_k, int32_t n_packed, int32_t* token_indices,
+                             int32_t* expert_offsets, float* route_flat, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+    hipStream_t st = (hipStream_t)stream;
+    BITSMOE_REQUIRE(n_tokens >= 0 && top_k > 0, "n_tokens must be >= 0 and top_k > 0");
+    BITSMOE_REQUIRE(n_packed >= 0 && n_packed <= ROUTE_MAX_EXPERTS, "n_packed=%d outside [0,%d]", n_packed, ROUTE_MAX_EXPERTS);
+    BITSMOE_REQUIRE(n_global >= 0, "n_global must be >= 0");
+    BITSMOE_REQUIRE(expert_offsets != nullptr, "expert_offsets must not be null");
+    const int64_t n_flat = n_tokens * top_k;
+    BITSMOE_REQUIRE(n_flat < ((int64_t)1 << 31), "too many assignments");
+    if (n_packed == 0 || n_flat == 0) {
+        // all offsets are zero; one tiny fill on the stream keeps the call asynchronous
+        return launch_fill_zero((float*)expert_offsets, n_packed + 1, st);
+    }
+    BITSMOE_REQUIRE(selected && weights && global_to_local && token_indices && route_flat, "null pointer");
+    const size_t need = bitsmoe_route_workspace_bytes(n_flat, n_packed);
+    if (n_flat > ROUTE_CHUNK && (workspace == nullptr || workspace_bytes < need)) {
+        set_error("route workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
+        return BITSMOE_E_WORKSPACE;
+    }
+    if (ids_are_i64)
+        return route_impl<int64_t>((const int64_t*)selected, weights, global_to_local, n_global, n_flat, top_k,
+                                   n_packed, token_indices, expert_offsets, route_flat, workspace, st);
+    return route_impl<int32_t>((const int32_t*)selected, weights, global_to_local, n_global, n_flat, top_k,
+                               n_packed, token_indices, expert_offsets, route_flat, workspace, st);
+}

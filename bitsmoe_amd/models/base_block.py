@@ -1,0 +1,286 @@
+"""Host side of the packed routed-expert path: the sparse-MoE block base class.
+
+Method names, buffer names and call order follow the reference's
+`BitsMoE_BaseSparseMoeBlock` (bitsmoe/models/base_block.py): runtime cache of per-expert
+buffer tuples and the global->local expert map (155-243), routing tables (258-289), the
+operator call and the output projection `rank_accum @ shared_u_down.T` (368-414), dense
+"super" experts (291-307), warm-up (315-366).
+
+What differs from the reference, by design for this GPU:
+  * routing tables are built by one device kernel (stable counting sort) with no host
+    synchronisation and no boolean-mask indexing; the kept-assignment count stays on the
+    device as `expert_offsets[-1]`;
+  * the block owns its three matrix-set handles (gate, up, down) instead of relying on a
+    process-global cache keyed on raw pointers;
+  * activations may be bf16 as well as fp16.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn as nn
+
+from bitsmoe_amd.algorithms import _HAS_MLP_FORWARD_CUDA, mlp_forward_cuda
+
+_BUFFER_NAMES = ("payload", "rank_idx", "tile_meta", "slab_meta", "scale", "s")
+
+
+class BitsMoE_BaseSparseMoeBlock(nn.Module):
+    _SHARED_BASIS_BUFFER_KEYS = ("shared_vh_gate_proj", "shared_vh_up_proj", "shared_u_down")
+
+    def _init_bitsmoe_common_state(self, super_experts: Optional[List[int]] = None,
+                                   track_super_projected_weights: bool = False) -> None:
+        self.super_experts = sorted(set(int(x) for x in (super_experts or [])))
+        self._super_expert_set = set(self.super_experts)
+        self.packed_expert_mask = [False for _ in range(len(self.experts))]
+        if track_super_projected_weights:
+            self.super_projected_weights: Dict[int, Dict[str, torch.Tensor]] = {}
+        for key in self._SHARED_BASIS_BUFFER_KEYS:
+            self.register_buffer(key, torch.empty(0, dtype=torch.float16), persistent=True)
+        self._invalidate_runtime_cache()
+        self._super_expert_items: List[Tuple[int, nn.Module]] = []
+        self._packed_expert_count = 0
+        self._packed_intermediate_size = 0
+        self._packed_global_to_local: Optional[torch.Tensor] = None
+        for proj in ("gate", "up", "down"):
+            for name in _BUFFER_NAMES:
+                setattr(self, f"_{proj}_{name}_static", ())
+        self._matsets = None
+
+    # ---- configuration ------------------------------------------------------------------
+    def _runtime_device(self) -> torch.device:
+        gate = getattr(self, "gate", None)
+        weight = getattr(gate, "weight", None)
+        if isinstance(weight, torch.Tensor):
+            return weight.device
+        return next(gate.parameters()).device
+
+    def _set_buffer(self, name: str, tensor: torch.Tensor) -> None:
+        setattr(self, name, tensor.detach().to(device=self._runtime_device(), dtype=torch.float16).contiguous())
+
+    def set_shared_basis(self, gate_vh: torch.Tensor, up_vh: torch.Tensor, down_u: torch.Tensor) -> None:
+        self._set_buffer("shared_vh_gate_proj", gate_vh)
+        self._set_buffer("shared_vh_up_proj", up_vh)
+        self._set_buffer("shared_u_down", down_u)
+        self._invalidate_runtime_cache()
+
+    def set_expert(self, expert_idx: int, expert_module: nn.Module, packed: bool) -> None:
+        idx = int(expert_idx)
+        self.experts[idx] = expert_module
+        self.packed_expert_mask[idx] = bool(packed)
+        self._invalidate_runtime_cache()
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
+        # the shared bases are registered empty; size them to the checkpoint before loading
+        for key in self._SHARED_BASIS_BUFFER_KEYS:
+            tensor = state_dict.get(prefix + key)
+            if isinstance(tensor, torch.Tensor):
+                current = getattr(self, key)
+                if current.shape != tensor.shape or current.dtype != tensor.dtype:
+                    setattr(self, key, torch.empty_like(tensor))
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs)
+        self._invalidate_runtime_cache()
+
+    def set_super_expert_projected_weights(self, expert_idx: int, gate_us: torch.Tensor, up_us: torch.Tensor,
+                                           down_svh: torch.Tensor) -> None:
+        if not hasattr(self, "super_projected_weights"):
+            self.super_projected_weights = {}
+        self.super_projected_weights[int(expert_idx)] = {
+            "gate_us": gate_us.detach().to(torch.float16).contiguous(),
+            "up_us": up_us.detach().to(torch.float16).contiguous(),
+            "down_svh": down_svh.detach().to(torch.float16).contiguous(),
+        }
+
+    def _act_type(self) -> int:
+        hidden_act = str(getattr(self.config, "hidden_act", "silu")).lower()
+        if hidden_act != "silu":
+            raise RuntimeError(f"Unsupported hidden_act for packed CUDA path: {hidden_act}")
+        return 0
+
+    # ---- runtime cache --------------------------------------------------------------------
+    def _invalidate_runtime_cache(self) -> None:
+        self._runtime_cache_ready = False
+        self._runtime_cache_device: Optional[torch.device] = None
+        self._runtime_warmed = False
+        self._cached_token_count = -1
+        self._cached_flat_token_ids: Optional[torch.Tensor] = None
+        self._matsets = None
+        self._basis_cache: Dict[torch.dtype, Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = {}
+
+    def _ensure_runtime_cache(self, device: torch.device) -> None:
+        if self._runtime_cache_ready and self._runtime_cache_device == device:
+            return
+        super_items: List[Tuple[int, nn.Module]] = []
+        packed_items: List[Tuple[int, nn.Module]] = []
+        for expert_idx, layer in enumerate(self.experts):
+            if layer is None:
+                continue
+            if expert_idx in self._super_expert_set:
+                super_items.append((expert_idx, layer))
+                continue
+            if not getattr(layer, "is_bitsmoe_packed", False):
+                raise RuntimeError(
+                    f"Layer {self.layer_idx} expert {expert_idx} is active but not packed. "
+                    "BitsMoE forward expects non-super routed experts to use packed kernel."
+                )
+            packed_items.append((expert_idx, layer))
+        self._super_expert_items = super_items
+        self._packed_expert_count = len(packed_items)
+        self._packed_intermediate_size = 0
+        self._cached_token_count = -1
+        self._cached_flat_token_ids = None
+        self._matsets = None
+        g2l = torch.full((self.num_experts,), -1, dtype=torch.int32)
+        experts = [layer for _, layer in packed_items]
+        if experts:
+            self._packed_intermediate_size = int(experts[0].intermediate_size)
+            g2l[torch.tensor([idx for idx, _ in packed_items], dtype=torch.long)] = torch.arange(
+                len(experts), dtype=torch.int32)
+        self._packed_global_to_local = g2l.to(device)
+        for proj in ("gate", "up", "down"):
+            for name in _BUFFER_NAMES:
+                attr = f"{proj}_{name}_buffer" if name != "s" else f"{proj}_s_buffer"
+                setattr(self, f"_{proj}_{name}_static", tuple(getattr(e, attr) for e in experts))
+        self._runtime_cache_ready = True
+        self._runtime_cache_device = device
+        self._runtime_warmed = False
+
+    def _static_lists(self, proj: str) -> Tuple[Sequence[torch.Tensor], ...]:
+        return tuple(getattr(self, f"_{proj}_{name}_static") for name in _BUFFER_NAMES)
+
+    def _ensure_matsets(self):
+        if self._matsets is None:
+            isz = int(self._packed_intermediate_size)
+            self._matsets = tuple(
+                mlp_forward_cuda.MatrixSet(*self._static_lists(proj), intermediate_size=isz, name=f"{proj}_payload")
+                for proj in ("gate", "up", "down")
+            )
+        return self._matsets
+
+    def _shared_basis(self, dtype: torch.dtype):
+        cached = self._basis_cache.get(dtype)
+        if cached is None:
+            cached = tuple(getattr(self, k).to(dtype).contiguous() for k in self._SHARED_BASIS_BUFFER_KEYS)
+            self._basis_cache[dtype] = cached
+        return cached
+
+    def _get_flat_token_ids(self, token_count: int, device: torch.device) -> torch.Tensor:
+        if (self._cached_flat_token_ids is not None and self._cached_token_count == token_count
+                and self._cached_flat_token_ids.device == device):
+            return self._cached_flat_token_ids
+        ids = torch.arange(token_count, dtype=torch.long, device=device).repeat_interleave(self.top_k)
+        self._cached_flat_token_ids = ids
+        self._cached_token_count = token_count
+        return ids
+
+    # ---- routing / operator ---------------------------------------------------------------
+    def _build_packed_routing(self, flat_selected_experts: torch.Tensor, flat_token_ids: Optional[torch.Tensor],
+                              flat_route_weights_fp32: torch.Tensor):
+        """(token_indices int32, expert_offsets int32 [E+1], route_flat fp32) built on the
+        device; `flat_token_ids` must be the token-major arrangement the block itself makes
+        (it is implied by the flat position and therefore not read)."""
+        if self._packed_expert_count <= 0 or self._packed_global_to_local is None:
+            return None
+        if not (_HAS_MLP_FORWARD_CUDA and mlp_forward_cuda is not None):
+            raise RuntimeError("Packed routed experts require the HIP mlp_forward library; there is no fallback.")
+        sel = flat_selected_experts.reshape(-1, self.top_k)
+        w = flat_route_weights_fp32.reshape(-1, self.top_k)
+        return mlp_forward_cuda.route(sel, w, self._packed_global_to_local, self._packed_expert_count)
+
+    def _run_super_experts(self, hidden_states, final_hidden_states, flat_selected_experts, flat_token_ids,
+                           flat_route_weights_hidden) -> None:
+        for expert_idx, layer in self._super_expert_items:
+            mask = flat_selected_experts == expert_idx
+            if not bool(mask.any()):
+                continue
+            token_ids = flat_token_ids[mask]
+            out = layer(hidden_states.index_select(0, token_ids)) * flat_route_weights_hidden[mask].unsqueeze(-1)
+            final_hidden_states.index_add_(0, token_ids, out.to(hidden_states.dtype))
+
+    def prepare_runtime_fastpath(self, warmup: bool = True) -> None:
+        device = self._runtime_device()
+        self._ensure_runtime_cache(device)
+        if warmup:
+            self._warmup_runtime_once(device)
+
+    def _warmup_runtime_once(self, device: torch.device) -> None:
+        if self._runtime_warmed or device.type != "cuda":
+            return
+        if not (_HAS_MLP_FORWARD_CUDA and mlp_forward_cuda is not None):
+            return
+        if self._packed_expert_count <= 0:
+            self._runtime_warmed = True
+            return
+        if self.shared_vh_gate_proj.numel() == 0 or self.shared_vh_up_proj.numel() == 0:
+            return
+        active = min(self.top_k, self._packed_expert_count)
+        h_gate = torch.zeros((1, int(self.shared_vh_gate_proj.shape[0])), dtype=torch.float16, device=device)
+        h_up = torch.zeros((1, int(self.shared_vh_up_proj.shape[0])), dtype=torch.float16, device=device)
+        counts = torch.zeros((self._packed_expert_count,), dtype=torch.int32, device=device)
+        counts[:active] = 1
+        offsets = torch.zeros((self._packed_expert_count + 1,), dtype=torch.int32, device=device)
+        offsets[1:] = torch.cumsum(counts, dim=0)
+        with torch.no_grad():
+            self._packed_forward_cuda(
+                h_gate_proj=h_gate, h_up_proj=h_up,
+                token_indices=torch.zeros((active,), dtype=torch.int32, device=device),
+                expert_offsets_t=offsets,
+                route_flat=torch.full((active,), 1.0 / active, dtype=torch.float32, device=device),
+                token_count=1)
+        torch.cuda.synchronize(device)
+        self._runtime_warmed = True
+
+    def _packed_rank_accum(self, h_gate_proj, h_up_proj, token_indices, expert_offsets_t, route_flat) -> torch.Tensor:
+        rank_out = int(self.shared_u_down.shape[1])
+        intermediate_size = int(self._packed_intermediate_size)
+        if intermediate_size <= 0:
+            raise RuntimeError(f"Layer {self.layer_idx} has no packed experts for CUDA path.")
+        gate, up, down = self._ensure_matsets()
+        return mlp_forward_cuda.moe_forward_sets(h_gate_proj, h_up_proj, token_indices, expert_offsets_t, route_flat,
+                                                 gate, up, down, rank_out, intermediate_size, self._act_type())
+
+    def _packed_forward_cuda(self, h_gate_proj, h_up_proj, token_indices, expert_offsets_t, route_flat,
+                             token_count: int) -> torch.Tensor:
+        rank_accum = self._packed_rank_accum(h_gate_proj, h_up_proj, token_indices, expert_offsets_t, route_flat)
+        rank_out = int(self.shared_u_down.shape[1])
+        if rank_accum.shape[0] != token_count or rank_accum.shape[1] != rank_out:
+            raise RuntimeError(
+                f"Invalid rank_accum shape from kernel: got {tuple(rank_accum.shape)}, expected ({token_count}, {rank_out})")
+        u_down = self._shared_basis(h_gate_proj.dtype)[2]
+        return torch.matmul(rank_accum.to(u_down.dtype), u_down.T)
+
+    def _packed_forward_grouped(self, h_gate_proj, h_up_proj, token_indices, expert_offsets_t, route_flat,
+                                token_count: int) -> torch.Tensor:
+        if self.shared_u_down.numel() == 0:
+            raise RuntimeError(f"Layer {self.layer_idx} missing shared_u_down for packed routed experts.")
+        usable = (_HAS_MLP_FORWARD_CUDA and mlp_forward_cuda is not None and h_gate_proj.is_cuda and h_up_proj.is_cuda)
+        if not usable:
+            raise RuntimeError(
+                "Packed routed experts require CUDA mlp_forward extension; python fallback is intentionally disabled.")
+        return self._packed_forward_cuda(h_gate_proj, h_up_proj, token_indices, expert_offsets_t, route_flat, token_count)
+
+    # ---- shared forward body --------------------------------------------------------------
+    def _routed_forward(self, hidden_states: torch.Tensor, selected_experts: torch.Tensor,
+                        routing_weights_fp32: torch.Tensor) -> torch.Tensor:
+        """hidden [T,H], top-k ids [T,k], fp32 weights [T,k] -> routed-expert output [T,H]."""
+        token_count, hidden_dim = hidden_states.shape
+        if self.shared_vh_gate_proj.numel() == 0 or self.shared_vh_up_proj.numel() == 0:
+            raise RuntimeError(f"Layer {self.layer_idx} missing shared_vh basis for packed routed experts.")
+        vh_gate, vh_up, _ = self._shared_basis(hidden_states.dtype)
+        h_gate_proj = hidden_states @ vh_gate.T
+        h_up_proj = hidden_states @ vh_up.T
+        final = torch.zeros((token_count, hidden_dim), dtype=hidden_states.dtype, device=hidden_states.device)
+        flat_selected = selected_experts.reshape(-1)
+        flat_w32 = routing_weights_fp32.reshape(-1)
+        if self._super_expert_items:
+            self._run_super_experts(hidden_states, final, flat_selected,
+                                    self._get_flat_token_ids(token_count, hidden_states.device),
+                                    flat_w32.to(hidden_states.dtype))
+        routing = self._build_packed_routing(flat_selected, None, flat_w32)
+        if routing is not None:
+            token_indices, expert_offsets_t, route_flat = routing
+            packed = self._packed_forward_grouped(h_gate_proj, h_up_proj, token_indices, expert_offsets_t,
+                                                  route_flat, token_count)
+            final = final + packed.to(hidden_states.dtype)
+        return final

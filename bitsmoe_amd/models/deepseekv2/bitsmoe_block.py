@@ -1,0 +1,45 @@
+"""DeepSeek-V2 sparse block: the model's own gate module picks (ids, weights); packed routed
+experts; the always-on shared experts run on the block input
+(reference: bitsmoe/models/deepseekv2/bitsmoe_block.py:26-127)."""
+from __future__ import annotations
+
+import copy
+from typing import List, Optional
+
+import torch
+import torch.nn as nn
+
+from bitsmoe_amd.models.base_block import BitsMoE_BaseSparseMoeBlock
+
+
+class BitsMoE_DeepSeekSparseMoeBlock(BitsMoE_BaseSparseMoeBlock):
+    def __init__(self, config, layer_idx: int, source_block: Optional[nn.Module] = None,
+                 super_experts: Optional[List[int]] = None, copy_source_experts: bool = True):
+        super().__init__()
+        self.config = config
+        self.layer_idx = int(layer_idx)
+        self.top_k = int(getattr(config, "num_experts_per_tok", 0))
+        if source_block is None:
+            raise ValueError("source_block is required for BitsMoE_DeepSeekSparseMoeBlock")
+        self.gate = copy.deepcopy(source_block.gate)
+        self.experts = nn.ModuleList([None] * len(source_block.experts))
+        self.num_experts = len(self.experts)
+        if hasattr(source_block, "shared_experts"):
+            self.shared_experts = copy.deepcopy(source_block.shared_experts)
+        for attr in ("ep_size", "experts_per_rank", "ep_rank"):
+            if hasattr(source_block, attr):
+                setattr(self, attr, int(getattr(source_block, attr)))
+        self._init_bitsmoe_common_state(super_experts=super_experts, track_super_projected_weights=True)
+
+    def forward(self, hidden_states: torch.Tensor):
+        identity = hidden_states
+        orig_shape = hidden_states.shape
+        topk_idx, topk_weight, _aux = self.gate(hidden_states)
+        hidden_states = hidden_states.reshape(-1, orig_shape[-1])
+        self._ensure_runtime_cache(hidden_states.device)
+        selected = topk_idx.reshape(-1, topk_idx.shape[-1])
+        weights = topk_weight.reshape(-1, topk_weight.shape[-1]).to(torch.float32)
+        y = self._routed_forward(hidden_states, selected, weights).reshape(*orig_shape)
+        if getattr(self.config, "n_shared_experts", None) is not None and hasattr(self, "shared_experts"):
+            y = y + self.shared_experts(identity)
+        return y

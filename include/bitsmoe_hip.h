@@ -1,0 +1,167 @@
+/*
+ * bitsmoe_hip.h — C ABI of libbitsmoe_hip.so: the mixed-bit MoE routed-expert forward for
+ * AMD gfx950 (MI355X).
+ *
+ * Plain pointers and sizes only; no torch types.  Every pointer named "device" must be
+ * device memory on the GPU that is current when the call is made; `stream` is a
+ * hipStream_t passed as void* (NULL = the default stream).  All calls return 0 on success
+ * or a negative BITSMOE_E_* code; bitsmoe_last_error() returns the message of the last
+ * failure on the calling thread.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the
+ * reference tree).
+ */
+#ifndef BITSMOE_HIP_H
+#define BITSMOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BITSMOE_OK 0
+#define BITSMOE_E_INVALID (-1)   /* bad argument (shape, dtype code, null pointer, meta out of range) */
+#define BITSMOE_E_HIP (-2)       /* a HIP runtime call failed */
+#define BITSMOE_E_WORKSPACE (-3) /* workspace too small */
+#define BITSMOE_E_UNSUPPORTED (-4)
+
+/* activation dtype of h_gate / h_up */
+#define BITSMOE_DT_F16 0
+#define BITSMOE_DT_BF16 1
+
+/* kernel-path selector for bitsmoe_moe_forward (BITSMOE_PATH_AUTO in production) */
+#define BITSMOE_PATH_AUTO 0
+#define BITSMOE_PATH_GENERIC 1  /* fp32 FMA kernels that accept every legal layout */
+#define BITSMOE_PATH_DECODE 2   /* bandwidth-bound small-batch kernels (regular layouts only) */
+#define BITSMOE_PATH_MFMA 3     /* MFMA grouped-GEMM kernels (regular layouts only) */
+
+const char* bitsmoe_last_error(void);
+const char* bitsmoe_version(void);
+
+/*
+ * One packed expert matrix: the six runtime buffers of one (expert, projection).
+ * Replaces the per-expert entries of the 18 tensor lists taken by
+ * moe_packed_forward (bitsmoe/algorithms/cpp/mlp_forward_binding.cpp:53-79) and the
+ * buffer contract of bitsmoe/models/base_mlp.py:96-102.  Offsets inside tile_meta are in
+ * uint32 words (payload) and fp16 elements (scale).
+ */
+typedef struct bitsmoe_matrix_desc {
+    const void* payload;   /* device uint32 [payload_words]                                   */
+    const void* rank_idx;  /* device int32  [rank_len]: local row -> logical rank             */
+    const void* tile_meta; /* device int32  [num_tiles][3] = (pack_off, scale_off, n_valid)   */
+    const void* slab_meta; /* device int32  [num_slabs][4] = (bits, k_slab, rank_off, tile_off) */
+    const void* scale;     /* device fp16   [scale_len]                                       */
+    const void* s;         /* device fp16   [rank_len]: per-row multiplier                    */
+    int64_t payload_words;
+    int64_t scale_len;
+    int32_t rank_len;
+    int32_t num_tiles;
+    int32_t num_slabs;
+    int32_t reserved;
+} bitsmoe_matrix_desc;
+
+/*
+ * A "matrix set": the packed matrices of all E experts for one projection (gate, up or
+ * down) of one layer.  Replaces build_packed_meta_cached / PackedMeta
+ * (bitsmoe/algorithms/cpp/mlp_forward.cu:2424-2444, 2529-2697): device pointer tables,
+ * per-expert counts and the down work list.  Creation copies the slab/tile/rank_idx
+ * tables to the host once, validates every offset against the buffer sizes (so that no
+ * kernel can read out of bounds) and uploads the tables; it synchronises `stream`.
+ * The set borrows the caller's buffers: they must stay alive and unchanged until
+ * bitsmoe_matset_destroy.  Unlike the reference's cache the set is owned by the caller,
+ * not keyed on raw pointers.
+ */
+typedef struct bitsmoe_matset bitsmoe_matset;
+
+int bitsmoe_matset_create(const bitsmoe_matrix_desc* descs, int32_t n_experts,
+                          int32_t intermediate_size, void* stream, bitsmoe_matset** out);
+void bitsmoe_matset_destroy(bitsmoe_matset* set);
+/* info[0]=n_experts, [1]=intermediate_size, [2]=total slabs, [3]=max logical rank + 1,
+ * [4]=1 if every matrix is "regular" (slabs of 16-row multiples, 2/3/4-bit, full tiles) */
+int bitsmoe_matset_info(const bitsmoe_matset* set, int64_t info[8]);
+
+/*
+ * Dense dequantisation of one expert matrix to fp32 [rank_len, intermediate_size]
+ * (row-major, local row order).  Restates decode_tile_weight * scale
+ * (bitsmoe/algorithms/cpp/mlp_forward.cu:215-265, 746-749); used for bit-exact parity.
+ */
+int bitsmoe_dequant_matrix(const bitsmoe_matset* set, int32_t expert, float* out_device,
+                           void* stream);
+
+/*
+ * Routing / permute.  Replaces _get_flat_token_ids + _build_packed_routing
+ * (bitsmoe/models/base_block.py:245-289): the flat (token-major) top-k list is mapped
+ * through global_to_local (entries < 0 are dropped), counted per packed expert, scanned
+ * and scattered STABLY (ascending flat position inside every expert).  No host
+ * synchronisation; total kept assignments = expert_offsets[n_packed] on the device.
+ *   selected     device int32 or int64 [T*k]   (ids_are_i64 selects)
+ *   weights      device fp32 [T*k]
+ *   global_to_local device int32 [n_global]
+ *   token_indices device int32 [T*k] out, expert_offsets device int32 [n_packed+1] out,
+ *   route_flat   device fp32 [T*k] out         (entries past the kept count are untouched)
+ */
+size_t bitsmoe_route_workspace_bytes(int64_t n_flat, int32_t n_packed);
+int bitsmoe_route(const void* selected, int32_t ids_are_i64, const float* weights,
+                  const int32_t* global_to_local, int32_t n_global, int64_t n_tokens,
+                  int32_t top_k, int32_t n_packed, int32_t* token_indices,
+                  int32_t* expert_offsets, float* route_flat, void* workspace,
+                  size_t workspace_bytes, void* stream);
+
+/*
+ * The routed-expert forward.  Replaces moe_packed_forward
+ * (bitsmoe/algorithms/cpp/mlp_forward_binding.cpp:53-155) ->
+ * moe_packed_forward_cuda (bitsmoe/algorithms/cpp/mlp_forward.cu:2701-3074):
+ *   G = (h_gate[tok] gathered by rank_idx * s) . W_gate,  U likewise,
+ *   Z = silu(G) * U,  acc = W_down . Z,
+ *   rank_accum[tok, rank_idx_down[r]] += acc * s_down[r] * route_w[a].
+ *   h_gate device [T, rank_gate], h_up device [T, rank_up]  (fp16 or bf16, row-major)
+ *   token_indices device int32 [A], expert_offsets device int32 [E+1], route_w fp32 [A]
+ *   rank_accum device fp32 [T, rank_out] out (fully overwritten)
+ * Never allocates and never synchronises with the host: intermediates live in
+ * `workspace` (>= bitsmoe_forward_workspace_bytes).  act_type must be 0 (SiLU).
+ * n_assign == 0 or zero experts writes zeros and returns (mlp_forward.cu:2733-2737).
+ * `profile`, if not NULL, receives phase timings (see bitsmoe_profile_*).
+ */
+typedef struct bitsmoe_profile bitsmoe_profile;
+
+size_t bitsmoe_forward_workspace_bytes(int64_t n_tokens, int64_t n_assign,
+                                       int32_t intermediate_size, int32_t n_experts,
+                                       int32_t rank_out);
+int bitsmoe_moe_forward(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                        const bitsmoe_matset* down, const void* h_gate, const void* h_up,
+                        int32_t act_dtype, int64_t n_tokens, int32_t rank_gate,
+                        int32_t rank_up, const int32_t* token_indices,
+                        const int32_t* expert_offsets, const float* route_w,
+                        int64_t n_assign, int32_t rank_out, int32_t intermediate_size,
+                        int32_t act_type, int32_t path, float* rank_accum, void* workspace,
+                        size_t workspace_bytes, bitsmoe_profile* profile, void* stream);
+
+/*
+ * Phase timing with HIP events recorded on the caller's stream between the kernels of
+ * one bitsmoe_moe_forward call (no reference counterpart: the reference has no
+ * profiling hooks in the op).  After the stream has been synchronised,
+ * bitsmoe_profile_read returns milliseconds for phase i:
+ *   0 = zero-fill, 1 = gate+up kernels, 2 = down kernel(s).
+ */
+#define BITSMOE_PROFILE_PHASES 3
+int bitsmoe_profile_create(bitsmoe_profile** out);
+void bitsmoe_profile_destroy(bitsmoe_profile* p);
+int bitsmoe_profile_read(bitsmoe_profile* p, float ms[BITSMOE_PROFILE_PHASES]);
+
+/*
+ * Bit-plane pack / unpack of quantised levels.  Replaces pack_int8_{1,2,3,4,6,8}bit and
+ * unpack_int8_* (bitsmoe/quant/bitpack/bitpack_cuda_binding.cpp:36-68, kernels
+ * bitpack_cuda_kernel.cu:84-196): levels int8 [rows, cols] <-> uint32
+ * [rows, ceil(cols/32)*bits], word order [row][32-column group][plane].
+ */
+int bitsmoe_pack_bitplanes(const int8_t* levels, int64_t rows, int64_t cols, int32_t bits,
+                           uint32_t* words_out, void* stream);
+int bitsmoe_unpack_bitplanes(const uint32_t* words, int64_t rows, int64_t groups,
+                             int32_t bits, int8_t* levels_out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BITSMOE_HIP_H */
