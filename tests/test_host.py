@@ -1,0 +1,161 @@
+"""CPU-side tests: the C-ABI library loads and exports every declared symbol, the host mirror
+of the reference interface (buffer names, key schemes, argument checks, error behaviour)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+from oracle import ref_oracle as o
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    from bitsmoe_amd.algorithms import _capi
+
+    header = open(os.path.join(ROOT, "include", "bitsmoe_hip.h")).read()
+    declared = set(re.findall(r"\b(bitsmoe_[a-z_0-9]+)\s*\(", header))
+    assert declared, "no declarations found in the header"
+    lib = ctypes.CDLL(str(_capi.LIB_PATH))
+    for sym in sorted(declared):
+        assert hasattr(lib, sym), f"{sym} is declared in include/bitsmoe_hip.h but not exported"
+    assert declared == set(_capi.EXPORTED_SYMBOLS)
+    assert b"gfx950" in _capi.load().bitsmoe_version()
+
+
+def test_operator_module_names_match_reference_interface():
+    import bitsmoe_amd.algorithms as alg
+
+    for name in ("mlp_forward_cuda", "_HAS_MLP_FORWARD_CUDA", "_MLP_FORWARD_BACKEND", "get_cuda_device_name"):
+        assert hasattr(alg, name)
+    assert alg._HAS_MLP_FORWARD_CUDA and alg.mlp_forward_cuda is not None
+    import inspect
+
+    params = list(inspect.signature(alg.mlp_forward_cuda.moe_packed_forward).parameters)
+    expect = ["h_gate", "h_up", "token_indices", "expert_offsets", "route_weights"]
+    for proj in ("gate", "up", "down"):
+        expect += [f"{proj}_{n}" for n in ("payload", "rank_idx", "tile_meta", "slab_meta", "scale", "s")]
+    expect += ["rank_out", "intermediate_size", "act_type"]
+    assert params == expect
+
+
+def test_argument_checks_without_gpu():
+    from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
+
+    h = torch.zeros((2, 8), dtype=torch.float16)
+    i32 = torch.zeros((2,), dtype=torch.int32)
+    f32 = torch.zeros((2,), dtype=torch.float32)
+    off = torch.zeros((2,), dtype=torch.int32)
+    lists = [[torch.zeros(1)]] * 18
+    with pytest.raises(RuntimeError, match="h_gate must be CUDA tensor"):
+        hip.moe_packed_forward(h, h, i32, off, f32, *lists, 8, 128, 0)
+    with pytest.raises(RuntimeError, match=r"h_gate must be 2D \[tokens, rank\]"):
+        hip.moe_packed_forward(h[0], h, i32, off, f32, *lists, 8, 128, 0)
+    with pytest.raises(RuntimeError, match="h_gate/h_up token dim mismatch"):
+        hip.moe_packed_forward(h, h[:1], i32, off, f32, *lists, 8, 128, 0)
+
+
+def test_c_abi_rejects_bad_arguments_without_gpu():
+    from bitsmoe_amd.algorithms import _capi
+
+    lib = _capi.load()
+    out = ctypes.c_void_p()
+    assert lib.bitsmoe_matset_create(None, -1, 128, None, ctypes.byref(out)) == -1
+    assert b"n_experts" in lib.bitsmoe_last_error()
+    assert lib.bitsmoe_matset_create(None, 0, 0, None, ctypes.byref(out)) == -1
+    assert b"intermediate_size" in lib.bitsmoe_last_error()
+    assert lib.bitsmoe_pack_bitplanes(None, 1, 32, 5, None, None) == -1
+    assert b"Unsupported bit width: 5" in lib.bitsmoe_last_error()
+    assert lib.bitsmoe_route(None, 0, None, None, 4, 2, 0, 4, None, None, None, None, 0, None) == -1
+    assert lib.bitsmoe_forward_workspace_bytes(4, 8, 768, 128, 2048) >= 2 * 8 * 768 * 4
+    assert lib.bitsmoe_route_workspace_bytes(32768, 128) >= 32768 * 4
+
+
+def _state_dict_for(mats_by_mtype, prefix, scheme):
+    sd = {}
+    for mtype, m in mats_by_mtype.items():
+        tag = {"gate_proj": "gate", "up_proj": "up", "down_proj": "down"}[mtype]
+        field = "u" if mtype != "down_proj" else "vh"
+        t = {
+            "payload_buffer": torch.from_numpy(m["payload"].view(np.int32).copy()).view(torch.uint32),
+            "rank_idx_buffer": torch.from_numpy(m["rank_idx"]),
+            "tile_meta_buffer": torch.from_numpy(m["tile_meta"]).to(torch.int16),     # compact on disk
+            "slab_meta_buffer": torch.from_numpy(m["slab_meta"]).to(torch.int16),
+            "scale_buffer": torch.from_numpy(m["scale"]),
+            "s_buffer": torch.from_numpy(m["s"]),
+            "segments": torch.from_numpy(m["segments"]),
+            "original_indices": torch.from_numpy(m["original_indices"]),
+            "original_rank": torch.tensor(int(m["original_rank"]), dtype=torch.int32),
+            "groupsize": torch.tensor(128, dtype=torch.int16),
+        }
+        for name, v in t.items():
+            if scheme == "packer":
+                inner = f"{mtype}.{field}.{name}" if name in ("payload_buffer", "rank_idx_buffer", "tile_meta_buffer",
+                                                               "slab_meta_buffer", "scale_buffer") else f"{mtype}.{name}"
+                sd[f"{prefix}.{inner}"] = v
+            else:
+                sd[f"{prefix}.{tag}_{name}"] = v
+    return sd
+
+
+@pytest.mark.parametrize("scheme", ["packer", "module"])
+def test_expert_container_binds_both_key_schemes(scheme):
+    from types import SimpleNamespace
+
+    from bitsmoe_amd.models.qwen3moe.bitsmoe_mlp import BitsMoE_Qwen3MoeMLP
+
+    rng = np.random.default_rng(1)
+    mats = {mt: helpers.make_matrix(rng, 70, 160, [(3, (0, 40)), (2, (40, 70))]) for mt in ("gate_proj", "up_proj", "down_proj")}
+    cfg = SimpleNamespace(hidden_size=64, intermediate_size=160, hidden_act="silu")
+    mlp = BitsMoE_Qwen3MoeMLP(cfg)
+    assert not mlp.is_bitsmoe_packed and mlp.skip_expert
+    assert mlp.load_runtime_packed_from_state(_state_dict_for(mats, "quantized.layer0.expert3", scheme),
+                                              "quantized.layer0.expert3")
+    assert mlp.is_bitsmoe_packed and not mlp.skip_expert
+    assert mlp.gate_payload_buffer.dtype == torch.uint32
+    assert mlp.gate_tile_meta_buffer.dtype == torch.int32 and mlp.gate_slab_meta_buffer.dtype == torch.int32
+    assert mlp.down_scale_buffer.dtype == torch.float16 and mlp.up_s_buffer.dtype == torch.float16
+    assert mlp.runtime_meta["down_proj"]["packed_field"] == "vh"
+    assert mlp.runtime_meta["gate_proj"]["slab_meta_rows"] == [tuple(r) for r in mats["gate_proj"]["slab_meta"].tolist()]
+    # state_dict -> fresh module round trip binds the same bytes
+    sd = mlp.state_dict()
+    assert set(sd) == set(BitsMoE_Qwen3MoeMLP._runtime_buffer_leaf_keys())
+    fresh = BitsMoE_Qwen3MoeMLP(cfg)
+    fresh.load_state_dict(sd)
+    assert fresh.is_bitsmoe_packed
+    for k, v in sd.items():
+        got = getattr(fresh, k)
+        assert got.dtype == v.dtype and got.shape == v.shape
+        assert torch.equal(got.view(torch.int32) if v.dtype == torch.uint32 else got,
+                           v.view(torch.int32) if v.dtype == torch.uint32 else v)
+    with pytest.raises(NotImplementedError):
+        mlp(torch.zeros(1, 64))
+    assert not BitsMoE_Qwen3MoeMLP(cfg).load_runtime_packed_from_state({}, "missing")
+
+
+def test_block_refuses_to_run_without_gpu_path():
+    from types import SimpleNamespace
+
+    from bitsmoe_amd.models.qwen3moe.bitsmoe_block import BitsMoE_Qwen3MoeSparseMoeBlock
+
+    cfg = SimpleNamespace(hidden_size=32, intermediate_size=128, hidden_act="silu", num_experts=2,
+                          num_experts_per_tok=1, norm_topk_prob=True)
+    src = SimpleNamespace(gate=torch.nn.Linear(32, 2, bias=False), experts=[None, None])
+    block = BitsMoE_Qwen3MoeSparseMoeBlock(cfg, 0, source_block=src)
+    with pytest.raises(ValueError):
+        BitsMoE_Qwen3MoeSparseMoeBlock(cfg, 0, source_block=None)
+    h = torch.zeros((1, 32), dtype=torch.float16)
+    i32 = torch.zeros((1,), dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="missing shared_u_down"):
+        block._packed_forward_grouped(h, h, i32, torch.zeros((3,), dtype=torch.int32), torch.zeros(1), 1)
+    block.set_shared_basis(torch.eye(32), torch.eye(32), torch.eye(32))
+    assert block.shared_vh_gate_proj.dtype == torch.float16
+    with pytest.raises(RuntimeError, match="python fallback is intentionally disabled"):
+        block._packed_forward_grouped(h, h, i32, torch.zeros((3,), dtype=torch.int32), torch.zeros(1), 1)
+    cfg.hidden_act = "gelu"
+    with pytest.raises(RuntimeError, match="Unsupported hidden_act"):
+        block._act_type()
