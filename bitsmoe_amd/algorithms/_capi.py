@@ -27,6 +27,8 @@ EXPORTED_SYMBOLS = (
     "bitsmoe_matset_destroy",
     "bitsmoe_matset_info",
     "bitsmoe_dequant_matrix",
+    "bitsmoe_matset_prepare",
+    "bitsmoe_dequant_matrix_prepared",
     "bitsmoe_route_workspace_bytes",
     "bitsmoe_route",
     "bitsmoe_forward_workspace_bytes",
@@ -81,6 +83,10 @@ def load() -> ctypes.CDLL:
     lib.bitsmoe_matset_info.argtypes = [c_void_p, POINTER(c_int64)]
     lib.bitsmoe_dequant_matrix.restype = c_int32
     lib.bitsmoe_dequant_matrix.argtypes = [c_void_p, c_int32, c_void_p, c_void_p]
+    lib.bitsmoe_matset_prepare.restype = c_int32
+    lib.bitsmoe_matset_prepare.argtypes = [c_void_p, c_int32, c_void_p]
+    lib.bitsmoe_dequant_matrix_prepared.restype = c_int32
+    lib.bitsmoe_dequant_matrix_prepared.argtypes = [c_void_p, c_int32, c_void_p, c_void_p]
     lib.bitsmoe_route_workspace_bytes.restype = c_size_t
     lib.bitsmoe_route_workspace_bytes.argtypes = [c_int64, c_int32]
     lib.bitsmoe_route.restype = c_int32

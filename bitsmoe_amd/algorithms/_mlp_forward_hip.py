@@ -19,7 +19,11 @@ import torch
 
 from . import _capi
 
+import os
+
 _lib = _capi.load()
+# BITSMOE_NO_PREPARE=1 keeps every matrix set on the generic kernels (no wave-native copy)
+_AUTO_PREPARE = os.environ.get("BITSMOE_NO_PREPARE", "0") != "1"
 
 
 def _stream_ptr(device: torch.device) -> int:
@@ -79,10 +83,32 @@ class MatrixSet:
         self.total_slabs = int(info[2])
         self.max_rank_plus1 = int(info[3])
         self.regular = bool(info[4])
+        self.fast_capable = bool(int(info[7]) & 1)   # the wave-native fast kernels can take this set
+        self.role = -1                               # -1 until prepare() has re-laid the payload out
 
     @property
     def handle(self) -> ctypes.c_void_p:
         return self._handle
+
+    def prepare(self, role: int) -> bool:
+        """One-time re-layout of the payload for the fast kernels (role 0: gate/up, 1: down).
+        Returns False (and leaves the set on the generic kernels) when the layout is not regular."""
+        if self.role == role:
+            return True
+        if not self.fast_capable or self.role >= 0:
+            return False
+        with torch.cuda.device(self.device):
+            _capi.check(_lib.bitsmoe_matset_prepare(self._handle, int(role), _stream_ptr(self.device)))
+        self.role = int(role)
+        return True
+
+    def dequant_prepared(self, expert: int) -> torch.Tensor:
+        """Dense fp32 matrix decoded from the prepared (wave-native) copy."""
+        out = torch.zeros((self.rank_len(expert), self.intermediate_size), dtype=torch.float32, device=self.device)
+        with torch.cuda.device(self.device):
+            _capi.check(_lib.bitsmoe_dequant_matrix_prepared(self._handle, int(expert), out.data_ptr(),
+                                                             _stream_ptr(self.device)))
+        return out
 
     def rank_len(self, expert: int) -> int:
         return int(self._keep[1][expert].numel())
@@ -176,6 +202,12 @@ def moe_forward_sets(h_gate: torch.Tensor, h_up: torch.Tensor, token_indices: to
     n_tokens = int(h_gate.shape[0])
     n_assign = int(token_indices.numel())
     dt = _capi.DT_F16 if h_gate.dtype == torch.float16 else _capi.DT_BF16
+    if path != _capi.PATH_GENERIC and _AUTO_PREPARE and gate.role < 0 and up.role < 0 and down.role < 0:
+        # first use: lay the payloads out for the fast kernels (one-time, allocates the copy)
+        if gate.fast_capable and up.fast_capable and down.fast_capable:
+            gate.prepare(0)
+            up.prepare(0)
+            down.prepare(1)
     if out is None:
         out = torch.empty((n_tokens, int(rank_out)), dtype=torch.float32, device=dev)
     nbytes = int(_lib.bitsmoe_forward_workspace_bytes(n_tokens, n_assign, int(intermediate_size),

@@ -41,6 +41,13 @@ struct SlabTask {              // one (expert, slab) unit of the down projection
     int32_t slab;
 };
 
+bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I);
+int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                          const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru,
+                          const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out, int I,
+                          float* rank_accum, float* G, float* U, int64_t inter_floats, bitsmoe_profile* prof,
+                          hipStream_t st);
+
 }  // namespace bitsmoe
 
 // The opaque handle of the C ABI.
@@ -53,6 +60,11 @@ struct bitsmoe_matset {
     int32_t max_rank_plus1 = 0;       // 1 + largest logical rank referenced by rank_idx
     int32_t min_rank = 0;             // smallest logical rank
     bool regular = false;             // every matrix: 2/3/4-bit, k_slab % 16 == 0, full tiles
+    bool regular64 = false;           // ... and every slab has exactly 64 rows, payload 16-byte aligned
+    int role = -1;                    // -1: not prepared; 0: gate/up layout; 1: down layout
+    uint32_t* d_prepared = nullptr;   // wave-native copy of every payload (see wave_layout.h)
+    bitsmoe::MatView* d_views_prepared = nullptr;
+    std::vector<int64_t> prepared_offsets;
     int device = -1;
     std::vector<bitsmoe_matrix_desc> descs;
     std::vector<std::vector<int32_t>> slab_meta_host;

@@ -68,10 +68,19 @@ extern "C" int bitsmoe_moe_forward(const bitsmoe_matset* gate, const bitsmoe_mat
     float* G = (float*)workspace;
     float* U = (float*)((char*)workspace + inter);
 
-    if (path == BITSMOE_PATH_DECODE || path == BITSMOE_PATH_MFMA) {
+    const bool fast_ok = decode_path_supported(gate, up, down, intermediate_size);
+    if (path == BITSMOE_PATH_MFMA) {
         set_error("path %d is not built into this library version", path);
         return BITSMOE_E_UNSUPPORTED;
     }
+    if (path == BITSMOE_PATH_DECODE && !fast_ok) {
+        set_error("decode path needs matrix sets prepared with bitsmoe_matset_prepare (gate/up role 0, down role 1)");
+        return BITSMOE_E_UNSUPPORTED;
+    }
+    if (fast_ok && path != BITSMOE_PATH_GENERIC)
+        return launch_forward_decode(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up,
+                                     token_indices, expert_offsets, route_w, n_assign, rank_out, intermediate_size,
+                                     rank_accum, G, U, (int64_t)(inter / sizeof(float)), profile, st);
     return launch_forward_generic(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up,
                                   token_indices, expert_offsets, route_w, n_assign, rank_out,
                                   intermediate_size, rank_accum, G, U, profile, st);

@@ -1,0 +1,196 @@
+// One-time re-layout of a matrix set's payload into the wave64-native field layout
+// (wave_layout.h) and the dense dequantiser that reads it back (parity check of the layout).
+#include "wave_layout.h"
+
+namespace bitsmoe {
+
+// code (unsigned, before the level offset) of element (row, col) of a (slab, tile) block
+// in the reference bit-plane layout; `blk` points at the block's first word, rows = 64.
+__device__ inline uint32_t ref_code(const uint32_t* __restrict__ blk, int w, int row, int col) {
+    const int stage = row >> 4, r = row & 15, micro = col >> 5, lane = col & 31;
+    const uint32_t* words = blk + stage * (K_STAGE * MICROS * w) + micro * (K_STAGE * w) + r * w;
+    uint32_t u = 0;
+    for (int p = 0; p < w; ++p) u |= ((words[p] >> lane) & 1u) << p;
+    return u;
+}
+
+// (row, col) of contraction index x of the run owned by (nb, kg, n)
+__device__ inline void run_element(int role, int nb, int kg, int n, int x, int* row, int* col) {
+    if (role == ROLE_GATE_UP) {          // 16 rows 16*kg + x, column 16*nb + n
+        *row = 16 * kg + x;
+        *col = 16 * nb + n;
+    } else {                              // row 16*nb + n, columns 32*(x/8) + 8*kg + x%8
+        *row = 16 * nb + n;
+        *col = 32 * (x >> 3) + 8 * kg + (x & 7);
+    }
+}
+
+// grid: (slab tasks, tiles); every thread builds whole output words of one block.
+__global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src, const MatView* __restrict__ dst,
+                                                 const SlabTask* __restrict__ tasks, int role) {
+    const SlabTask task = tasks[blockIdx.x];
+    const MatView mv = src[task.expert];
+    const int si = task.slab;
+    const int w = mv.slab_meta[si * 4 + 0];
+    const int tile_off = mv.slab_meta[si * 4 + 3];
+    const int t = tile_off + blockIdx.y;
+    const int pack_off = mv.tile_meta[t * 3 + 0];
+    const uint32_t* __restrict__ in = mv.payload + pack_off;
+    uint32_t* __restrict__ out = const_cast<uint32_t*>(dst[task.expert].payload) + pack_off;
+    const int nbs = (role == ROLE_GATE_UP) ? 8 : 4;        // output blocks per lane
+    const int run = (role == ROLE_GATE_UP) ? 16 : 32;      // contraction indices per (lane, nb)
+    const int n_words = 256 * w;
+    for (int idx = threadIdx.x; idx < n_words; idx += blockDim.x) {
+        uint32_t word = 0;
+        if (w == 3 && idx >= 512) {
+            // third bit of the 3-bit codes
+            const int j = idx - 512;
+            if (role == ROLE_GATE_UP) {   // j = (kg*8 + n8)*8 + nb, shared by lanes n8 and n8 + 8
+                const int nb = j & 7, n8 = (j >> 3) & 7, kg = j >> 6;
+                for (int upper = 0; upper < 2; ++upper)
+                    for (int x = 0; x < 16; ++x) {
+                        int row, col;
+                        run_element(role, nb, kg, n8 + 8 * upper, x, &row, &col);
+                        word |= ((ref_code(in, w, row, col) >> 2) & 1u) << (pos1(x) + 8 * upper);
+                    }
+            } else {                      // j = l*4 + nb
+                const int nb = j & 3, l = j >> 2, n = l & 15, kg = l >> 4;
+                for (int x = 0; x < 32; ++x) {
+                    int row, col;
+                    run_element(role, nb, kg, n, x, &row, &col);
+                    word |= ((ref_code(in, w, row, col) >> 2) & 1u) << pos1(x);
+                }
+            }
+            out[idx] = word;
+            continue;
+        }
+        // two-bit / four-bit field words: words per (lane, nb) = run * fieldbits / 32
+        const int fb = (w == 4) ? 4 : 2;
+        const int per = run * fb / 32;                   // role0: 1 (w=2,3) or 2 (w=4); role1: 2 or 4
+        const int sub = idx % per;
+        const int nb = (idx / per) % nbs;
+        const int l = idx / (per * nbs);
+        const int n = l & 15, kg = l >> 4;
+        const int codes = 32 / fb;                       // codes per word
+        for (int i = 0; i < codes; ++i) {
+            const int x = sub * codes + i;
+            int row, col;
+            run_element(role, nb, kg, n, x, &row, &col);
+            const uint32_t u = ref_code(in, w, row, col);
+            if (fb == 4)
+                word |= (u & 15u) << pos4(i);
+            else
+                word |= (u & 3u) << pos2(i);
+        }
+        out[idx] = word;
+    }
+}
+
+// Dense fp32 dequantisation FROM THE PREPARED LAYOUT, written to mirror the decode of the
+// hot kernels (fields, not planes); output identical to k_dequant_matrix.
+__global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* payload = prepared */, int role, int I,
+                                                          float* __restrict__ out) {
+    const int si = blockIdx.x;
+    const int w = mv.slab_meta[si * 4 + 0];
+    const int rank_off = mv.slab_meta[si * 4 + 2];
+    const int t = mv.slab_meta[si * 4 + 3] + blockIdx.y;
+    const int pack_off = mv.tile_meta[t * 3 + 0];
+    const int scale_off = mv.tile_meta[t * 3 + 1];
+    const uint32_t* __restrict__ blk = mv.payload + pack_off;
+    const int nbs = (role == ROLE_GATE_UP) ? 8 : 4;
+    const int run = (role == ROLE_GATE_UP) ? 16 : 32;
+    for (int idx = threadIdx.x; idx < SLAB_ROWS * N_TILE; idx += blockDim.x) {
+        // enumerate (lane, nb, x) instead of (row, col) so the layout is read the way kernels read it
+        const int x = idx % run;
+        const int nb = (idx / run) % nbs;
+        const int l = idx / (run * nbs);
+        const int n = l & 15, kg = l >> 4;
+        int row, col;
+        run_element(role, nb, kg, n, x, &row, &col);
+        uint32_t u;
+        if (w == 4) {
+            const int per = run / 8;
+            u = (blk[(l * nbs + nb) * per + (x >> 3)] >> pos4(x & 7)) & 15u;
+        } else {
+            const int per = run / 16;
+            u = (blk[(l * nbs + nb) * per + (x >> 4)] >> pos2(x & 15)) & 3u;
+            if (w == 3) {
+                uint32_t hi;
+                int p;
+                if (role == ROLE_GATE_UP) {
+                    hi = blk[512 + hi_index0(kg, n, nb)];
+                    p = pos1(x) + 8 * (n >> 3);
+                } else {
+                    hi = blk[512 + l * 4 + nb];
+                    p = pos1(x);
+                }
+                u |= ((hi >> p) & 1u) << 2;
+            }
+        }
+        const int c = blockIdx.y * N_TILE + col;
+        if (c < I) {
+            const float q = (float)((int)u - level_offset(w));
+            out[(int64_t)(rank_off + row) * I + c] = q * __half2float(mv.scale[scale_off + row]);
+        }
+    }
+}
+
+}  // namespace bitsmoe
+
+using namespace bitsmoe;
+
+extern "C" int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* stream) {
+    BITSMOE_REQUIRE(set != nullptr, "set must not be null");
+    BITSMOE_REQUIRE(role == ROLE_GATE_UP || role == ROLE_DOWN, "role must be 0 (gate/up) or 1 (down)");
+    hipStream_t st = (hipStream_t)stream;
+    if (set->role == role) return BITSMOE_OK;
+    BITSMOE_REQUIRE(set->role < 0, "matrix set is already prepared for the other role");
+    if (!set->regular64 || set->total_slabs == 0) {
+        set_error("matrix set is not regular (every slab 64 rows of 2/3/4 bits, full 128-column tiles): "
+                  "only the generic kernels can run it");
+        return BITSMOE_E_UNSUPPORTED;
+    }
+    int64_t total_words = 0;
+    std::vector<int64_t> offs(set->n_experts);
+    for (int e = 0; e < set->n_experts; ++e) {
+        offs[e] = total_words;
+        total_words += (set->descs[e].payload_words + 63) / 64 * 64;    // keep every matrix 256-byte aligned
+    }
+    BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_prepared, (size_t)total_words * 4));
+    std::vector<MatView> views(set->n_experts);
+    BITSMOE_HIP_TRY(hipMemcpyAsync(views.data(), set->d_views, sizeof(MatView) * set->n_experts, hipMemcpyDeviceToHost, st));
+    BITSMOE_HIP_TRY(hipStreamSynchronize(st));
+    for (int e = 0; e < set->n_experts; ++e) views[e].payload = set->d_prepared + offs[e];
+    BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_views_prepared, sizeof(MatView) * set->n_experts));
+    BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_views_prepared, views.data(), sizeof(MatView) * set->n_experts, hipMemcpyHostToDevice, st));
+    hipLaunchKernelGGL(k_prepack, dim3((unsigned)set->total_slabs, set->n_tiles), dim3(256), 0, st, set->d_views,
+                       set->d_views_prepared, set->d_slab_tasks, role);
+    BITSMOE_HIP_TRY(hipGetLastError());
+    BITSMOE_HIP_TRY(hipStreamSynchronize(st));
+    set->prepared_offsets = offs;
+    set->role = role;
+    return BITSMOE_OK;
+}
+
+extern "C" int bitsmoe_dequant_matrix_prepared(const bitsmoe_matset* set, int32_t expert, float* out_device, void* stream) {
+    BITSMOE_REQUIRE(set && out_device, "null argument");
+    BITSMOE_REQUIRE(expert >= 0 && expert < set->n_experts, "expert %d out of range", expert);
+    BITSMOE_REQUIRE(set->role >= 0, "matrix set is not prepared");
+    hipStream_t st = (hipStream_t)stream;
+    const bitsmoe_matrix_desc& d = set->descs[expert];
+    MatView mv;
+    mv.payload = set->d_prepared + set->prepared_offsets[expert];
+    mv.rank_idx = (const int32_t*)d.rank_idx;
+    mv.tile_meta = (const int32_t*)d.tile_meta;
+    mv.slab_meta = (const int32_t*)d.slab_meta;
+    mv.scale = (const __half*)d.scale;
+    mv.s = (const __half*)d.s;
+    mv.num_slabs = d.num_slabs;
+    mv.num_tiles = d.num_tiles;
+    mv.rank_len = d.rank_len;
+    mv.flags = 1;
+    hipLaunchKernelGGL(k_dequant_prepared, dim3(d.num_slabs, set->n_tiles), dim3(256), 0, st, mv, set->role,
+                       set->intermediate_size, out_device);
+    BITSMOE_HIP_TRY(hipGetLastError());
+    return BITSMOE_OK;
+}

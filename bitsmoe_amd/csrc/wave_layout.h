@@ -1,0 +1,137 @@
+// The wave64-native ("prepared") payload layout and its in-register decode.
+//
+// The reference layout stores bit PLANES: one 32-bit word holds one bit of 32 neighbouring
+// columns.  That is hostile to MFMA, whose operands want, per lane, 8 consecutive
+// contraction indices of one output index.  Matrix sets are therefore re-laid out ONCE
+// (bitsmoe_matset_prepare) into blocks with the same size and the same per-(slab, tile)
+// word offsets as the reference payload, but ordered for a wave:
+//
+//   block (slab of 64 rows, tile of 128 columns), bit-width w, 256*w words.
+//   lane l = 16*kg + n of a wavefront owns, for each 16-wide block `nb` of OUTPUT indices,
+//   the codes of a run of contraction indices, stored as w-bit FIELDS (not planes):
+//
+//   role 0 (gate / up: contraction over rows, outputs are columns; nb = 0..7)
+//     output column 16*nb + n, rows 16*kg + e, e = 0..15              (16 codes)
+//   role 1 (down: contraction over columns, outputs are rows; nb = 0..3)
+//     output row 16*nb + n, columns 32*m + 8*kg + e', m = 0..3, e' = 0..7   (32 codes)
+//
+//   A run of 16 codes with index x = 0..15 sits in a word at bit 2*(x/2)... precisely:
+//     2-bit fields:  field LSB at  (x & ~1) + 16*(x & 1)
+//     4-bit fields:  8 codes per word, field LSB at 4*(x'/2) + 16*(x' & 1), x' = x % 8
+//     3-bit codes :  low two bits as 2-bit fields, bit 2 as single bits at
+//                    (y/2) + 16*(y & 1) of a separate word (y = index in a run of 32;
+//                    role 0 shares one such word between lanes n and n+8: the upper lane
+//                    uses the positions + 8)
+//   so that ONE rotate and ONE and-or turn a word into a packed pair of 16-bit floats
+//   (2^w + code) for two neighbouring contraction indices: the pair lives 16 bits apart.
+//
+// Word order inside a block (every lane reads one contiguous run):
+//   role 0   w=2: word[(l*8 + nb)]                 w=4: word[(l*8 + nb)*2 + j]
+//            w=3: low  word[(l*8 + nb)]            high word[512 + ((16*kg + n%8)... see hi_index0)]
+//   role 1   w=2: word[(l*4 + nb)*2 + h]           w=4: word[(l*4 + nb)*4 + m]
+//            w=3: low  word[(l*4 + nb)*2 + h]      high word[512 + l*4 + nb]
+//
+// Decoded operand value is (2^w + code); the true level is code - 2^(w-1), so every dot
+// product carries the constant 1.5 * 2^w times the sum of the other operand, which the
+// kernels remove with one extra MFMA against a constant operand.
+#pragma once
+
+#include <cstdint>
+
+#include "common.h"
+
+namespace bitsmoe {
+
+constexpr int ROLE_GATE_UP = 0;
+constexpr int ROLE_DOWN = 1;
+constexpr int SLAB_ROWS = 64;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+// position of the field LSB for index x (0..15) of a run of 16 two-bit fields
+__host__ __device__ inline int pos2(int x) { return (x & ~1) + 16 * (x & 1); }
+// index x' (0..7) of a run of 8 four-bit fields
+__host__ __device__ inline int pos4(int x) { return 4 * (x >> 1) + 16 * (x & 1); }
+// index y (0..31) of a run of 32 single bits (role 1) / (0..15) + 8*upper (role 0)
+__host__ __device__ inline int pos1(int y) { return (y >> 1) + 16 * (y & 1); }
+
+// role 0, 3-bit: word index (inside the 256-word high region) shared by lanes n and n+8
+__host__ __device__ inline int hi_index0(int kg, int n, int nb) { return ((kg * 8 + (n & 7)) * 8 + nb); }
+
+template <bool BF16>
+struct FloatFmt {
+    static constexpr int MANT = BF16 ? 7 : 10;
+    static constexpr int BIAS = BF16 ? 127 : 15;
+};
+
+// Per bit-width constants of the packed-pair decode.
+template <int W, bool BF16>
+struct Codec {
+    static constexpr int POS = FloatFmt<BF16>::MANT - W;                              // field LSB in each half
+    static constexpr uint32_t MAGIC = (uint32_t)((FloatFmt<BF16>::BIAS + W) << FloatFmt<BF16>::MANT) * 0x10001u;  // 2^W
+    static constexpr uint32_t FMASK_2BIT = (3u << POS) * 0x10001u;
+    static constexpr uint32_t FMASK_4BIT = (15u << POS) * 0x10001u;
+    static constexpr uint32_t FMASK_HIBIT = (1u << (POS + 2)) * 0x10001u;                  // bit 2 of a 3-bit code
+    // 1.5 * 2^W: exponent BIAS + W, top mantissa bit set
+    static constexpr uint32_t CORR =
+        (uint32_t)(((FloatFmt<BF16>::BIAS + W) << FloatFmt<BF16>::MANT) | (1 << (FloatFmt<BF16>::MANT - 1))) * 0x10001u;
+};
+
+__device__ inline uint32_t rotr32(uint32_t x, int s) { return __builtin_amdgcn_alignbit(x, x, (uint32_t)(s & 31)); }
+
+// Four packed registers (8 values = one MFMA k-step) from two-bit fields: `first` is the
+// run index of the first of the 8 codes (0 or 8).
+template <int W, bool BF16>
+__device__ inline u32x4 decode_fields2(uint32_t z, int first) {
+    using C = Codec<W, BF16>;
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = (rotr32(z, first + 2 * i - C::POS) & C::FMASK_2BIT) | C::MAGIC;
+    return r;
+}
+
+template <bool BF16>
+__device__ inline u32x4 decode_fields4(uint32_t z) {
+    using C = Codec<4, BF16>;
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = (rotr32(z, 4 * i - C::POS) & C::FMASK_4BIT) | C::MAGIC;
+    return r;
+}
+
+// 3-bit: two-bit fields from `z`, third bit from `hi`; `hi_first` = position of the bit of
+// the first of the 8 codes inside `hi` (pos1 of its run index, plus 8 for an upper lane).
+template <bool BF16>
+__device__ inline u32x4 decode_fields3(uint32_t z, int first, uint32_t hi, int hi_first) {
+    using C = Codec<3, BF16>;
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t lo = (rotr32(z, first + 2 * i - C::POS) & C::FMASK_2BIT) | C::MAGIC;
+        r[i] = (rotr32(hi, hi_first + i - (C::POS + 2)) & C::FMASK_HIBIT) | lo;
+    }
+    return r;
+}
+
+template <bool BF16>
+__device__ inline f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+    if constexpr (BF16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+// fp32 -> 16-bit operand type, round to nearest even
+template <bool BF16>
+__device__ inline uint16_t to_operand(float v) {
+    if constexpr (BF16) {
+        return __bfloat16_as_ushort(__float2bfloat16(v));
+    } else {
+        return __half_as_ushort(__float2half(v));
+    }
+}
+
+}  // namespace bitsmoe

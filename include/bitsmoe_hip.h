@@ -78,8 +78,25 @@ typedef struct bitsmoe_matset bitsmoe_matset;
 int bitsmoe_matset_create(const bitsmoe_matrix_desc* descs, int32_t n_experts,
                           int32_t intermediate_size, void* stream, bitsmoe_matset** out);
 void bitsmoe_matset_destroy(bitsmoe_matset* set);
+/*
+ * One-time re-layout of a set's payload into the wave64-native field layout the fast
+ * kernels read (same byte count as the reference payload; the caller's buffers are not
+ * modified, the library allocates the copy once and frees it in bitsmoe_matset_destroy).
+ * role 0: gate / up (contraction over rows), role 1: down (contraction over columns).
+ * Plays the part of the reference's one-time meta build
+ * (bitsmoe/algorithms/cpp/mlp_forward.cu:2529-2697).  Returns BITSMOE_E_UNSUPPORTED for
+ * sets that are not "regular" (every slab 64 rows of 2/3/4 bits, full 128-column tiles,
+ * 16-byte aligned payload): those run on the generic kernels only.  Synchronises `stream`.
+ */
+int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* stream);
+/* Dense fp32 dequantisation read back FROM THE PREPARED LAYOUT (parity check of it). */
+int bitsmoe_dequant_matrix_prepared(const bitsmoe_matset* set, int32_t expert, float* out_device,
+                                    void* stream);
+
 /* info[0]=n_experts, [1]=intermediate_size, [2]=total slabs, [3]=max logical rank + 1,
- * [4]=1 if every matrix is "regular" (slabs of 16-row multiples, 2/3/4-bit, full tiles) */
+ * [4]=1 if every matrix has slabs of 16-row multiples, 2/3/4-bit, full tiles,
+ * [5]=largest slab count, [6]=smallest logical rank, [7]=bit0: fast kernels applicable,
+ * bit1: prepared */
 int bitsmoe_matset_info(const bitsmoe_matset* set, int64_t info[8]);
 
 /*

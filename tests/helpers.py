@@ -11,8 +11,14 @@ from oracle import ref_oracle as o
 BUF_KEYS = ("payload", "rank_idx", "tile_meta", "slab_meta", "scale", "s")
 
 
-def random_segments(rng: np.random.Generator, rank: int, choices=(2, 3, 4), n_cuts: int = 3, drop: bool = False):
-    cuts = sorted(set(int(c) for c in rng.integers(1, rank, size=n_cuts))) if rank > 1 else []
+def random_segments(rng: np.random.Generator, rank: int, choices=(2, 3, 4), n_cuts: int = 3, drop: bool = False,
+                    multiple: int = 1):
+    if multiple > 1:       # cut only at multiples so that every slab is full
+        units = rank // multiple
+        cuts = sorted(set(int(c) * multiple for c in rng.integers(1, max(units, 2), size=n_cuts))) if units > 1 else []
+        cuts = [c for c in cuts if 0 < c < rank]
+    else:
+        cuts = sorted(set(int(c) for c in rng.integers(1, rank, size=n_cuts))) if rank > 1 else []
     edges = [0] + cuts + [rank]
     segs = []
     for a, b in zip(edges[:-1], edges[1:]):
@@ -32,7 +38,7 @@ def make_matrix(rng, rank: int, dim: int, segments, s_mode="rand", std=0.02) -> 
 
 
 def make_experts(seed: int, n_experts: int, rank_in: int, rank_out: int, dim: int, choices=(2, 3, 4),
-                 uniform_bits: bool = False, s_mode="rand", permute_rank: bool = False):
+                 uniform_bits: bool = False, s_mode="rand", permute_rank: bool = False, slab_multiple=None):
     """gate/up/down lists of oracle matrices.  gate/up rows index h columns [0, rank_in);
     down rows index output ranks [0, rank_out)."""
     rng = np.random.default_rng(seed)
@@ -42,7 +48,7 @@ def make_experts(seed: int, n_experts: int, rank_in: int, rank_out: int, dim: in
             if uniform_bits:
                 segs = [(int(rng.choice(choices)), (0, rank))]
             else:
-                segs = random_segments(rng, rank, choices)
+                segs = random_segments(rng, rank, choices, multiple=slab_multiple or 1)
             lst.append(make_matrix(rng, rank, dim, segs, s_mode=s_mode))
     return gate, up, down
 

@@ -82,7 +82,7 @@ def _block_reference(block, x):
              for e in range(spec.num_experts)] for p in ("gate", "up", "down")]
     x64 = x.float().cpu().numpy().astype(np.float64)
     if spec.family == "deepseekv2":
-        gw = block.gate.weight.float().cpu().numpy()
+        gw = block.gate.weight.detach().float().cpu().numpy()
         idx, w = o.router_deepseek((x64 @ gw.T.astype(np.float64)).astype(np.float32), spec.top_k)
     else:
         # the router's logits are taken from the block's own (bf16) gate so that near-ties
@@ -96,12 +96,12 @@ def _block_reference(block, x):
                         idx, w, mats[0], mats[1], mats[2], isz)
 
     def dense_mlp(mod, inp):
-        f = lambda lin: lin.weight.float().cpu().numpy().astype(np.float64)
+        f = lambda lin: lin.weight.detach().float().cpu().numpy().astype(np.float64)
         g, u = inp @ f(mod.gate_proj).T, inp @ f(mod.up_proj).T
         return (g / (1 + np.exp(-g)) * u) @ f(mod.down_proj).T
 
     if spec.family == "qwen3next":
-        gate_w = block.shared_expert_gate.weight.float().cpu().numpy().astype(np.float64)
+        gate_w = block.shared_expert_gate.weight.detach().float().cpu().numpy().astype(np.float64)
         y = y + 1.0 / (1.0 + np.exp(-(x64 @ gate_w.T))) * dense_mlp(block.shared_expert, x64)
     if spec.family == "deepseekv2" and hasattr(block, "shared_experts"):
         y = y + dense_mlp(block.shared_experts, x64)

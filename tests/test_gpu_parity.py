@@ -70,13 +70,13 @@ def test_routing_tables_bit_exact(cuda_device, tokens, top_k, n_global, n_super,
 
 
 def _forward_case(cuda_device, seed, n_experts, tokens, top_k, rank_in, rank_out, dim, dtype_name, choices,
-                  path=None, tol=1e-2, uniform_bits=False):
+                  path=None, tol=1e-2, uniform_bits=False, slab_multiple=None):
     import torch
 
     hip = _hip()
     rng = np.random.default_rng(seed)
     gate, up, down = helpers.make_experts(seed, n_experts, rank_in, rank_out, dim, choices=choices,
-                                          uniform_bits=uniform_bits)
+                                          uniform_bits=uniform_bits, slab_multiple=slab_multiple)
     dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
     h_gate = torch.from_numpy(rng.normal(size=(tokens, rank_in)).astype(np.float32)).to(dt)
     h_up = torch.from_numpy(rng.normal(size=(tokens, rank_in)).astype(np.float32)).to(dt)
@@ -178,3 +178,49 @@ def test_bitpack_words_bit_exact(cuda_device, bits, rows, cols):
     assert np.array_equal(words.cpu().view(torch.int32).numpy().view(np.uint32), ref)
     back = BitPack.unpack(words, bits, cols)
     assert np.array_equal(back.cpu().numpy(), q)
+
+
+# ------------------------------------------------------------------ wave-native fast path
+@pytest.mark.parametrize("role", [0, 1])
+@pytest.mark.parametrize("dim", [128, 768])
+def test_prepared_layout_dequant_bit_exact(cuda_device, role, dim):
+    hip = _hip()
+    rng = np.random.default_rng(dim + role)
+    rank = 192
+    mats = [helpers.make_matrix(rng, rank, dim, [(4, (0, 64)), (3, (64, 128)), (2, (128, 192))]),
+            helpers.make_matrix(rng, rank, dim, [(3, (0, 192))]),
+            helpers.make_matrix(rng, rank, dim, [(2, (0, 128)), (4, (128, 192))])]
+    ms = hip.MatrixSet(*helpers.to_device_lists(mats, cuda_device), intermediate_size=dim)
+    assert ms.fast_capable
+    assert ms.prepare(role)
+    for e, m in enumerate(mats):
+        ref = o.dequant_matrix(m, dim)
+        got = ms.dequant_prepared(e).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), f"expert {e}: prepared layout decodes differently"
+        assert np.array_equal(ms.dequant(e).cpu().numpy().view(np.uint32), ref.view(np.uint32))
+
+
+def test_irregular_sets_stay_on_generic_kernels(cuda_device):
+    hip = _hip()
+    rng = np.random.default_rng(1)
+    mats = [helpers.make_matrix(rng, 80, 128, [(2, (0, 80))])]       # 64 + 16 rows: not regular
+    ms = hip.MatrixSet(*helpers.to_device_lists(mats, cuda_device), intermediate_size=128)
+    assert not ms.fast_capable and not ms.prepare(0)
+
+
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+@pytest.mark.parametrize("shape", [
+    # experts, tokens, top_k, rank_in, rank_out, dim
+    (4, 5, 2, 128, 128, 256),
+    (8, 1, 4, 512, 256, 128),
+    (6, 40, 3, 576, 192, 384),      # some experts get more than 16 assignments -> several passes
+    (16, 64, 8, 1024, 512, 768),
+])
+def test_forward_decode_path(cuda_device, shape, dtype_name):
+    from bitsmoe_amd.algorithms import _capi
+
+    e, t, k, rin, rout, dim = shape
+    tol = 1e-2
+    err = _forward_case(cuda_device, 100 + e, e, t, k, rin, rout, dim, dtype_name, (2, 3, 4),
+                        path=_capi.PATH_DECODE, tol=tol, uniform_bits=False, slab_multiple=64)
+    print(f"decode {shape} {dtype_name}: err {err:.2e}")
