@@ -48,7 +48,8 @@ def build_library(verbose: bool = True, jobs: int = 8) -> Path:
 
     def compile_one(src: Path) -> Path:
         obj = objdir / (src.stem + ".o")
-        cmd = [hipcc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]
+        extra = os.environ.get("BITSMOE_HIPCC_EXTRA", "").split()   # e.g. -DNAME for kernel experiments
+        cmd = [hipcc, *HIPCC_FLAGS, *extra, "-c", str(src), "-o", str(obj)]
         if verbose:
             print("[bitsmoe build]", " ".join(cmd), flush=True)
         res = subprocess.run(cmd, capture_output=True, text=True)

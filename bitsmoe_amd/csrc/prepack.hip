@@ -45,8 +45,9 @@ __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src
         if (w == 3 && idx >= 512) {
             // third bit of the 3-bit codes
             const int j = idx - 512;
-            if (role == ROLE_GATE_UP) {   // j = (kg*8 + n8)*8 + nb, shared by lanes n8 and n8 + 8
-                const int nb = j & 7, n8 = (j >> 3) & 7, kg = j >> 6;
+            if (role == ROLE_GATE_UP) {   // j = hi_index0(kg, n8, nb), shared by lanes n8 and n8 + 8
+                const int q = (j >> 1) & 31;
+                const int nb = 2 * (j >> 6) + (j & 1), n8 = q & 7, kg = q >> 3;
                 for (int upper = 0; upper < 2; ++upper)
                     for (int x = 0; x < 16; ++x) {
                         int row, col;
@@ -68,8 +69,15 @@ __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src
         const int fb = (w == 4) ? 4 : 2;
         const int per = run * fb / 32;                   // role0: 1 (w=2,3) or 2 (w=4); role1: 2 or 4
         const int sub = idx % per;
-        const int nb = (idx / per) % nbs;
-        const int l = idx / (per * nbs);
+        int nb, l;
+        if (role == ROLE_GATE_UP) {      // idx / per = idx2_role0(nb, l)
+            const int i2 = idx / per;
+            nb = 2 * (i2 >> 7) + (i2 & 1);
+            l = (i2 >> 1) & 63;
+        } else {
+            nb = (idx / per) % nbs;
+            l = idx / (per * nbs);
+        }
         const int n = l & 15, kg = l >> 4;
         const int codes = 32 / fb;                       // codes per word
         for (int i = 0; i < codes; ++i) {
@@ -108,12 +116,13 @@ __global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* payload 
         int row, col;
         run_element(role, nb, kg, n, x, &row, &col);
         uint32_t u;
+        const int unit = (role == ROLE_GATE_UP) ? idx2_role0(nb, l) : (l * nbs + nb);
         if (w == 4) {
             const int per = run / 8;
-            u = (blk[(l * nbs + nb) * per + (x >> 3)] >> pos4(x & 7)) & 15u;
+            u = (blk[unit * per + (x >> 3)] >> pos4(x & 7)) & 15u;
         } else {
             const int per = run / 16;
-            u = (blk[(l * nbs + nb) * per + (x >> 4)] >> pos2(x & 15)) & 3u;
+            u = (blk[unit * per + (x >> 4)] >> pos2(x & 15)) & 3u;
             if (w == 3) {
                 uint32_t hi;
                 int p;

@@ -26,10 +26,13 @@
 //   (2^w + code) for two neighbouring contraction indices: the pair lives 16 bits apart.
 //
 // Word order inside a block (every lane reads one contiguous run):
-//   role 0   w=2: word[(l*8 + nb)]                 w=4: word[(l*8 + nb)*2 + j]
-//            w=3: low  word[(l*8 + nb)]            high word[512 + ((16*kg + n%8)... see hi_index0)]
-//   role 1   w=2: word[(l*4 + nb)*2 + h]           w=4: word[(l*4 + nb)*4 + m]
-//            w=3: low  word[(l*4 + nb)*2 + h]      high word[512 + l*4 + nb]
+//   role 0: the four wavefronts of a workgroup own the column-block PAIRS nbp = nb/2, so
+//           the words of one pair are contiguous over the 64 lanes:
+//           w=2: word[idx2(nb, l)]   idx2 = ((nb/2)*64 + l)*2 + nb%2
+//           w=4: word[idx2(nb, l)*2 + j]
+//           w=3: low word[idx2(nb, l)], high word[512 + hi_index0(kg, n, nb)]
+//   role 1: w=2: word[(l*4 + nb)*2 + h]           w=4: word[(l*4 + nb)*4 + m]
+//           w=3: low  word[(l*4 + nb)*2 + h]      high word[512 + l*4 + nb]
 //
 // Decoded operand value is (2^w + code); the true level is code - 2^(w-1), so every dot
 // product carries the constant 1.5 * 2^w times the sum of the other operand, which the
@@ -58,8 +61,12 @@ __host__ __device__ inline int pos4(int x) { return 4 * (x >> 1) + 16 * (x & 1);
 // index y (0..31) of a run of 32 single bits (role 1) / (0..15) + 8*upper (role 0)
 __host__ __device__ inline int pos1(int y) { return (y >> 1) + 16 * (y & 1); }
 
+// role 0: word index of column block nb for lane l (two-bit field words)
+__host__ __device__ inline int idx2_role0(int nb, int l) { return ((nb >> 1) * 64 + l) * 2 + (nb & 1); }
 // role 0, 3-bit: word index (inside the 256-word high region) shared by lanes n and n+8
-__host__ __device__ inline int hi_index0(int kg, int n, int nb) { return ((kg * 8 + (n & 7)) * 8 + nb); }
+__host__ __device__ inline int hi_index0(int kg, int n, int nb) {
+    return ((nb >> 1) * 32 + kg * 8 + (n & 7)) * 2 + (nb & 1);
+}
 
 template <bool BF16>
 struct FloatFmt {
@@ -82,14 +89,30 @@ struct Codec {
 
 __device__ inline uint32_t rotr32(uint32_t x, int s) { return __builtin_amdgcn_alignbit(x, x, (uint32_t)(s & 31)); }
 
+// Pointers that come out of a table in memory are generic; the hot kernels cast them to the
+// global address space so that loads become global_load / s_load instead of flat_load.
+template <class T>
+using gptr = const T __attribute__((address_space(1)))*;
+template <class T>
+__device__ inline gptr<T> as_global(const T* p) { return (gptr<T>)p; }
+typedef const u32x4 __attribute__((address_space(1)))* gptr_u32x4;
+
+// (x & mask) | magic as ONE v_and_or_b32: gfx9 VALU encodings take a single scalar/literal
+// operand, so the mask is kept in a vector register and the magic in a scalar one.
+__device__ inline uint32_t vreg(uint32_t c) {
+    asm("" : "+v"(c));
+    return c;
+}
+
 // Four packed registers (8 values = one MFMA k-step) from two-bit fields: `first` is the
 // run index of the first of the 8 codes (0 or 8).
 template <int W, bool BF16>
 __device__ inline u32x4 decode_fields2(uint32_t z, int first) {
     using C = Codec<W, BF16>;
     u32x4 r;
+    const uint32_t m = vreg(C::FMASK_2BIT);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) r[i] = (rotr32(z, first + 2 * i - C::POS) & C::FMASK_2BIT) | C::MAGIC;
+    for (int i = 0; i < 4; ++i) r[i] = (rotr32(z, first + 2 * i - C::POS) & m) | C::MAGIC;
     return r;
 }
 
@@ -97,8 +120,9 @@ template <bool BF16>
 __device__ inline u32x4 decode_fields4(uint32_t z) {
     using C = Codec<4, BF16>;
     u32x4 r;
+    const uint32_t m = vreg(C::FMASK_4BIT);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) r[i] = (rotr32(z, 4 * i - C::POS) & C::FMASK_4BIT) | C::MAGIC;
+    for (int i = 0; i < 4; ++i) r[i] = (rotr32(z, 4 * i - C::POS) & m) | C::MAGIC;
     return r;
 }
 
@@ -108,10 +132,11 @@ template <bool BF16>
 __device__ inline u32x4 decode_fields3(uint32_t z, int first, uint32_t hi, int hi_first) {
     using C = Codec<3, BF16>;
     u32x4 r;
+    const uint32_t m = vreg(C::FMASK_2BIT), mh = vreg(C::FMASK_HIBIT);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const uint32_t lo = (rotr32(z, first + 2 * i - C::POS) & C::FMASK_2BIT) | C::MAGIC;
-        r[i] = (rotr32(hi, hi_first + i - (C::POS + 2)) & C::FMASK_HIBIT) | lo;
+        const uint32_t lo = (rotr32(z, first + 2 * i - C::POS) & m) | C::MAGIC;
+        r[i] = (rotr32(hi, hi_first + i - (C::POS + 2)) & mh) | lo;
     }
     return r;
 }
