@@ -36,6 +36,24 @@ struct MatView {
     int32_t flags;             // bit0: regular layout
 };
 
+// Flattened tables of a prepared ("regular") matrix set: everything a fast kernel needs
+// to find a (slab, tile) block is addressable from the expert index alone, so the loads
+// of one workgroup's metadata do not depend on each other.
+struct FastExpert {
+    const uint32_t* payload;   // prepared (wave-native) payload of this expert
+    const __half* scale;
+    const __half* s;
+    const int32_t* rank_idx;
+    int32_t num_slabs;
+    int32_t pad[7];            // 64 bytes
+};
+struct FastSlab {              // tile t of the slab: payload word pack_off + t*256*bits, scale scale_off + t*64
+    int32_t bits;              // 0 = no such slab
+    int32_t pack_off;
+    int32_t scale_off;
+    int32_t rank_off;
+};
+
 struct SlabTask {              // one (expert, slab) unit of the down projection
     int32_t expert;
     int32_t slab;
@@ -64,6 +82,8 @@ struct bitsmoe_matset {
     int role = -1;                    // -1: not prepared; 0: gate/up layout; 1: down layout
     uint32_t* d_prepared = nullptr;   // wave-native copy of every payload (see wave_layout.h)
     bitsmoe::MatView* d_views_prepared = nullptr;
+    bitsmoe::FastExpert* d_fast_experts = nullptr;   // [n_experts]
+    bitsmoe::FastSlab* d_fast_slabs = nullptr;       // [n_experts][max_slabs]
     std::vector<int64_t> prepared_offsets;
     int device = -1;
     std::vector<bitsmoe_matrix_desc> descs;

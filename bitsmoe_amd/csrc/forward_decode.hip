@@ -10,46 +10,40 @@
 //
 // MFMA operands: A = activations (row index = assignment), B = weights (column index =
 // output column / output rank row); D[4*(lane/16)+j][lane%16].
+//
+// Both kernels are latency-engineered rather than compute-engineered: one memory round
+// trip costs 1-2 us on a loaded MI355X, so (1) all metadata a workgroup needs is
+// addressable from its block index (FastExpert / FastSlab tables: one round trip, not a
+// chain of five), (2) every workgroup walks several tiles and keeps the payload of the next
+// tile in flight while it computes the current one.
+#include <type_traits>
+#include <utility>
+
 #include "wave_layout.h"
 
 namespace bitsmoe {
 
-constexpr int GU_SLABS_PER_WG = 8;                    // slabs (64 rows each) staged per workgroup
-constexpr int GU_ROWS = GU_SLABS_PER_WG * SLAB_ROWS;  // contraction rows staged per workgroup
-constexpr int GU_STRIDE = GU_ROWS + 8;                // 16-bit elements; +8 staggers LDS banks
-constexpr int DN_SLABS_PER_WG = 4;                    // one slab per wavefront
-constexpr int MAX_A = 16;                             // assignments per MFMA pass
+constexpr int GU_SLABS = 8;                        // slabs (64 rows each) per workgroup
+constexpr int GU_STRIDE = GU_SLABS * SLAB_ROWS + 8;  // 16-bit elements; +8 staggers LDS banks
+constexpr int DN_SLABS_PER_WG = 4;                 // one slab per wavefront
+constexpr int MAX_A = 16;                          // assignments per MFMA pass
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef const u32x2 __attribute__((address_space(1)))* gptr_u32x2;
-
-// A packed matrix with every pointer in the global address space.
-struct GView {
-    gptr<uint32_t> payload;
-    gptr<int32_t> rank_idx;
-    gptr<int32_t> tile_meta;
-    gptr<int32_t> slab_meta;
-    gptr<__half> scale;
-    gptr<__half> s;
-    int num_slabs;
-};
-
-__device__ inline GView load_view(const MatView* __restrict__ views, int e) {
-    const MatView mv = views[e];
-    GView g;
-    g.payload = as_global(mv.payload);
-    g.rank_idx = as_global(mv.rank_idx);
-    g.tile_meta = as_global(mv.tile_meta);
-    g.slab_meta = as_global(mv.slab_meta);
-    g.scale = as_global(mv.scale);
-    g.s = as_global(mv.s);
-    g.num_slabs = mv.num_slabs;
-    return g;
-}
+typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 
 __device__ inline float gload_half(gptr<__half> p) {
     const uint16_t bits = *reinterpret_cast<gptr<uint16_t>>(p);
     return __half2float(__ushort_as_half(bits));
+}
+
+// raw 16-bit activation -> fp32
+template <bool BF16>
+__device__ inline float operand_to_f32(uint16_t v) {
+    if constexpr (BF16)
+        return __uint_as_float((uint32_t)v << 16);
+    else
+        return __half2float(__ushort_as_half(v));
 }
 
 template <int W, bool BF16>
@@ -59,23 +53,34 @@ __device__ inline u32x4 corr_operand() {
     return r;
 }
 
-// Keeps a value's computation inside the loop iteration it is written in (the decode of
-// the payload does not depend on the assignment chunk, and hoisting it out of the chunk
-// loop would park every decoded operand in registers).
-__device__ inline void pin(uint32_t& v) { asm volatile("" : "+v"(v)); }
+// Calls f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): an unrolled loop whose
+// index is a compile-time constant (register-array indices must be static).
+template <class F, int... Q>
+__device__ inline void static_for(F&& f, std::integer_sequence<int, Q...>) {
+    (f(std::integral_constant<int, Q>{}), ...);
+}
+
+// The index is wave-uniform at every call site; readfirstlane tells the compiler so (scalar
+// registers, scalar branches, scalar-base addressing downstream).
+__device__ inline FastSlab load_fast_slab(const FastSlab* __restrict__ tab, int idx) {
+    const i32x4 v = *reinterpret_cast<const i32x4*>(tab + idx);
+    return FastSlab{__builtin_amdgcn_readfirstlane(v[0]), __builtin_amdgcn_readfirstlane(v[1]),
+                    __builtin_amdgcn_readfirstlane(v[2]), __builtin_amdgcn_readfirstlane(v[3])};
+}
 
 // ------------------------------------------------------------------------------ gate / up
 // The words of one wavefront's column-block pair for one (slab, tile) block: 2-bit {nb0, nb1};
 // 4-bit {nb0 j0, nb0 j1, nb1 j0, nb1 j1}; 3-bit {low nb0, low nb1, high nb0, high nb1}.
-__device__ inline void load_pair_role0(gptr<uint32_t> blk, int bits, int pair, int lane, uint32_t (&w)[4]) {
+// `blk` is wave-uniform, `unit` = pair*64 + lane and `hi_unit` are 32-bit lane offsets.
+__device__ inline void load_pair_role0(gptr<uint32_t> blk, int bits, uint32_t unit, uint32_t hi_unit, uint32_t (&w)[4]) {
     if (bits == 4) {
-        const u32x4 v = *reinterpret_cast<gptr_u32x4>(blk + (pair * 64 + lane) * 4);
+        const u32x4 v = *reinterpret_cast<gptr_u32x4>(blk + unit * 4u);
         w[0] = v[0]; w[1] = v[1]; w[2] = v[2]; w[3] = v[3];
     } else {
-        const u32x2 v = *reinterpret_cast<gptr_u32x2>(blk + (pair * 64 + lane) * 2);
+        const u32x2 v = *reinterpret_cast<gptr_u32x2>(blk + unit * 2u);
         w[0] = v[0]; w[1] = v[1]; w[2] = 0; w[3] = 0;
         if (bits == 3) {
-            const u32x2 h = *reinterpret_cast<gptr_u32x2>(blk + 512 + hi_index0(lane >> 4, lane & 15, 2 * pair));
+            const u32x2 h = *reinterpret_cast<gptr_u32x2>(blk + 512u + hi_unit);
             w[2] = h[0]; w[3] = h[1];
         }
     }
@@ -106,107 +111,215 @@ __device__ inline void gateup_pair(const uint32_t (&w)[4], u32x4 a0, u32x4 a1, i
     }
 }
 
-// grid.x = E * n_tiles * n_groups, grid.y = 2 (gate, up); 256 threads = 4 wavefronts.
-// A workgroup takes one expert, one projection, one 128-column tile and up to 8 slabs
-// (512 contraction rows).  Wavefront p owns columns [32p, 32p+32) of the tile for all of the
-// workgroup's slabs, so partial sums never cross wavefronts; they go to G / U with fp32
-// atomics (the slab groups of one tile add into the same outputs).
-template <typename HT, bool BF16>
+// grid.x = E * n_groups * n_tchunks, grid.y = 2 (gate, up); 256 threads = 4 wavefronts.
+// A workgroup takes one expert, one projection, up to 8 slabs (512 contraction rows) and a
+// run of 128-column tiles [t0, t1).  Wavefront p owns columns [32p, 32p+32) of every tile,
+// so partial sums never cross wavefronts; they go to G / U with fp32 atomics (the slab
+// groups of one tile add into the same outputs).  The gather h[tok, rank_idx[k]] is done
+// once per workgroup and kept in registers; per tile only the scale changes.
+// Every wavefront walks the (tile, slab) blocks of its column pair as one sequence and
+// keeps the payload of the next three blocks in flight (four rotating register buffers).
+template <bool BF16>
 __global__ __launch_bounds__(256) void k_gateup_decode(
-    const MatView* __restrict__ gate, const MatView* __restrict__ up, const HT* __restrict__ h_gate,
-    const HT* __restrict__ h_up, int Rg, int Ru, const int32_t* __restrict__ token_indices,
-    const int32_t* __restrict__ expert_offsets, int T, int A, int I, int n_tiles, int n_groups,
-    float* __restrict__ G, float* __restrict__ U) {
+    const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
+    const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
+    const uint16_t* __restrict__ h_gate, const uint16_t* __restrict__ h_up, int Rg, int Ru,
+    const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
+    int n_tiles, int n_groups, int n_tchunks, int tiles_per_wg, float* __restrict__ G, float* __restrict__ U) {
     const int mt = blockIdx.y;
     const int bid = blockIdx.x;
-    const int grp = bid % n_groups;
-    const int tile = (bid / n_groups) % n_tiles;
-    const int e = bid / (n_groups * n_tiles);
-    const int a_begin = max(expert_offsets[e], 0);
-    const int a_end = min(expert_offsets[e + 1], A);
-    if (a_end <= a_begin) return;
-    const GView mv = load_view(mt ? up : gate, e);
-    const int s0 = grp * GU_SLABS_PER_WG;
-    const int s1 = min(s0 + GU_SLABS_PER_WG, mv.num_slabs);
-    if (s0 >= s1) return;
-    const HT* __restrict__ h = mt ? h_up : h_gate;
-    const int R = mt ? Ru : Rg;
-    float* __restrict__ out = mt ? U : G;
-
-    __shared__ __attribute__((aligned(16))) uint16_t hs[MAX_A * GU_STRIDE];
-    __shared__ int tok_sh[MAX_A];
-
+    const int tchunk = bid % n_tchunks;
+    const int grp = (bid / n_tchunks) % n_groups;
+    const int e = bid / (n_tchunks * n_groups);
     const int tid = threadIdx.x;
-    const int pair = tid >> 6, lane = tid & 63;
+    const int pair = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform
+    const int lane = tid & 63;
     const int n = lane & 15, kg = lane >> 4;
 
-    // 1. issue every payload load of this wavefront before anything else
-    uint32_t pw[GU_SLABS_PER_WG][4];
-    int bits_s[GU_SLABS_PER_WG];
+    // one round trip: assignment range, expert record, the group's slab records
+    const int a_begin = max(expert_offsets[e], 0);
+    const int a_end = min(expert_offsets[e + 1], A);
+    const FastExpert* __restrict__ fe_tab = mt ? up_fe : gate_fe;
+    const FastSlab* __restrict__ fs_tab = mt ? up_fs : gate_fs;
+    const int max_slabs = mt ? up_max_slabs : gate_max_slabs;
+    const int s0 = grp * GU_SLABS;
+    if (s0 >= max_slabs) return;
+    const FastExpert fe = fe_tab[e];
+    int sbits[GU_SLABS], spack[GU_SLABS];
 #pragma unroll
-    for (int q = 0; q < GU_SLABS_PER_WG; ++q) {
-        const int s = s0 + q;
-        bits_s[q] = 0;
-        if (s < s1) {
-            bits_s[q] = mv.slab_meta[s * 4 + 0];
-            const int t = mv.slab_meta[s * 4 + 3] + tile;
-            load_pair_role0(mv.payload + mv.tile_meta[t * 3 + 0], bits_s[q], pair, lane, pw[q]);
+    for (int q = 0; q < GU_SLABS; ++q) {
+        sbits[q] = 0;
+        spack[q] = 0;
+        if (s0 + q < max_slabs) {
+            const FastSlab fs = load_fast_slab(fs_tab, e * max_slabs + s0 + q);
+            sbits[q] = fs.bits;
+            spack[q] = fs.pack_off;
         }
     }
+    // the two slabs whose rows this wavefront converts (lane = row)
+    FastSlab mine[2];
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        mine[it] = FastSlab{0, 0, 0, 0};
+        if (s0 + pair + 4 * it < max_slabs) mine[it] = load_fast_slab(fs_tab, e * max_slabs + s0 + pair + 4 * it);
+    }
+    if (a_end <= a_begin || sbits[0] == 0) return;
+
+    gptr<uint32_t> payload = as_global(fe.payload);
+    gptr<__half> scale = as_global(fe.scale);
+    gptr<__half> svec = as_global(fe.s);
+    gptr<int32_t> rank_idx = as_global(fe.rank_idx);
+    const uint16_t* __restrict__ h = mt ? h_up : h_gate;
+    const int R = mt ? Ru : Rg;
+    float* __restrict__ out = mt ? U : G;
+    const int t0_wg = tchunk * tiles_per_wg;
+    const int t1 = min(t0_wg + tiles_per_wg, n_tiles);
+    const uint32_t unit = (uint32_t)(pair * 64 + lane);
+    const uint32_t hi_unit = (uint32_t)hi_index0(kg, n, 2 * pair);
+
+    __shared__ __attribute__((aligned(16))) uint16_t hs[MAX_A * GU_STRIDE];
 
     for (int a0 = a_begin; a0 < a_end; a0 += MAX_A) {
         const int n_a = min(MAX_A, a_end - a0);
-        __syncthreads();
-        if (tid < MAX_A) tok_sh[tid] = (tid < n_a) ? token_indices[a0 + tid] : -1;
-        __syncthreads();
-        // 2. hs'[a][k] for the rows of slabs [s0, s1), the scale of this tile folded in.
-        //    Rows a >= n_a are left as they are: MFMA rows are independent and those
-        //    output rows are never stored.
-        const int n_rows = (s1 - s0) * SLAB_ROWS;
-        for (int idx = tid; idx < n_rows; idx += 256) {
-            const int s = s0 + (idx >> 6);
-            const int row = idx & 63;
-            const int k = mv.slab_meta[s * 4 + 2] + row;
-            const int t = mv.slab_meta[s * 4 + 3] + tile;
-            const int rk = mv.rank_idx[k];
-            const float sv = gload_half(mv.s + k) * gload_half(mv.scale + mv.tile_meta[t * 3 + 1] + row);
-            const bool rk_ok = rk >= 0 && rk < R;
-            for (int a = 0; a < n_a; ++a) {
-                const int tk = tok_sh[a];
-                float v = 0.0f;
-                if (rk_ok && tk >= 0 && tk < T) v = to_f32<HT>(h[(int64_t)tk * R + rk]) * sv;
-                hs[a * GU_STRIDE + idx] = to_operand<BF16>(v);
+        // an opaque zero keeps the address arithmetic of this chunk inside the loop body
+        int chunk_zero = 0;
+        asm volatile("" : "+s"(chunk_zero));
+        const int t0 = t0_wg + chunk_zero;
+
+        uint32_t pw[GU_SLABS][4];   // slab q's block of the current tile; refilled for the next tile right after use
+        auto issue = [&](auto buf_c, int t, int q_bits, int q_pack) {
+            constexpr int B = decltype(buf_c)::value;
+            load_pair_role0(payload + (uint32_t)(q_pack + t * 256 * q_bits), q_bits, unit, hi_unit, pw[B]);
+        };
+        // prologue: every block of the first tile
+        static_for([&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            if (sbits[q] != 0) issue(qc, t0, sbits[q], spack[q]);
+        }, std::make_integer_sequence<int, GU_SLABS>{});
+        // token ids of the chunk: one vector load, broadcast later with readlane
+        const int tok_lane = (lane < n_a) ? token_indices[a0 + lane] : -1;
+
+        // rows of this lane: logical rank, per-row multiplier, scale of the first tile
+        int rk[2];
+        float srow[2], sc_cur[2], sc_nxt[2] = {0.0f, 0.0f};
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            rk[it] = -1;
+            srow[it] = 0.0f;
+            sc_cur[it] = 0.0f;
+            if (mine[it].bits != 0) {
+                const int k = mine[it].rank_off + lane;
+                const int r = rank_idx[k];
+                rk[it] = (r >= 0 && r < R) ? r : -1;
+                srow[it] = gload_half(svec + k);
+                sc_cur[it] = gload_half(scale + mine[it].scale_off + t0 * SLAB_ROWS + lane);
             }
         }
-        __syncthreads();
-        // 3. decode + MFMA over the slabs
-        f32x4 acc[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
-        f32x4 corr = {0, 0, 0, 0};
-        const uint16_t* ap = hs + n * GU_STRIDE + 16 * kg;
+        // gather the activations of the chunk's assignments for both rows (raw 16-bit, two per
+        // register).  Loads are issued in two branch-free groups of eight assignments (clamped
+        // addresses, results masked afterwards) so that their round trips overlap.
+        uint32_t hp[2][MAX_A / 2];
+        const int rkc[2] = {max(rk[0], 0), max(rk[1], 0)};
 #pragma unroll
-        for (int q = 0; q < GU_SLABS_PER_WG; ++q) {
-            if (bits_s[q] == 0) continue;
+        for (int g = 0; g < 2; ++g) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) pin(pw[q][i]);
-            const u32x4 a_lo = *reinterpret_cast<const u32x4*>(ap + q * SLAB_ROWS);
-            const u32x4 a_hi = *reinterpret_cast<const u32x4*>(ap + q * SLAB_ROWS + 8);
-            if (bits_s[q] == 2)
-                gateup_pair<2, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
-            else if (bits_s[q] == 3)
-                gateup_pair<3, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
-            else
-                gateup_pair<4, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
-        }
-        // 4. remove the constant term and add into G / U: lane holds rows a = 4*kg + j of
-        //    column 32*pair + 16*nbl + n
-#pragma unroll
-        for (int nbl = 0; nbl < 2; ++nbl) {
-            const int c = tile * N_TILE + 32 * pair + 16 * nbl + n;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int a = 4 * kg + j;
-                if (a < n_a && c < I) atomicAdd(&out[(int64_t)(a0 + a) * I + c], acc[nbl][j] - corr[j]);
+            for (int ap = 4 * g; ap < 4 * g + 4; ++ap) {
+                hp[0][ap] = 0;
+                hp[1][ap] = 0;
             }
+#if defined(EXP_NO_HS) || defined(EXP_NO_GATHER)
+            if (a0 < 0) {
+#else
+            if (8 * g < n_a) {
+#endif
+                uint32_t raw[2][8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int tk = __builtin_amdgcn_readlane(tok_lane, 8 * g + j);
+                    const int tkc = min(max(tk, 0), T - 1);
+#pragma unroll
+                    for (int it = 0; it < 2; ++it) raw[it][j] = h[(int64_t)tkc * R + rkc[it]];
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int tk = __builtin_amdgcn_readlane(tok_lane, 8 * g + j);
+                    const bool tk_ok = tk >= 0 && tk < T;
+#pragma unroll
+                    for (int it = 0; it < 2; ++it)
+                        if (!(tk_ok && rk[it] >= 0)) raw[it][j] = 0;
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    hp[0][4 * g + j] = raw[0][2 * j] | (raw[0][2 * j + 1] << 16);
+                    hp[1][4 * g + j] = raw[1][2 * j] | (raw[1][2 * j + 1] << 16);
+                }
+            }
+        }
+
+        for (int t = t0; t < t1; ++t) {
+            const bool more = t + 1 < t1;
+            if (more) {
+#pragma unroll
+                for (int it = 0; it < 2; ++it)
+                    if (mine[it].bits != 0)
+                        sc_nxt[it] = gload_half(scale + mine[it].scale_off + (t + 1) * SLAB_ROWS + lane);
+            }
+            __syncthreads();   // every wavefront is done reading hs'(t-1)
+#pragma unroll
+            for (int it = 0; it < 2; ++it) {
+                if (mine[it].bits == 0) continue;
+#if defined(EXP_NO_HS) || defined(EXP_NO_WRITE)
+                if (a0 >= 0) continue;
+#endif
+                const float sv = srow[it] * sc_cur[it];
+                uint16_t* dst = &hs[(pair + 4 * it) * SLAB_ROWS + lane];
+#pragma unroll
+                for (int ap = 0; ap < MAX_A / 2; ++ap) {
+                    if (2 * ap < n_a) {
+                        dst[(2 * ap) * GU_STRIDE] = to_operand<BF16>(operand_to_f32<BF16>((uint16_t)(hp[it][ap] & 0xFFFFu)) * sv);
+                        dst[(2 * ap + 1) * GU_STRIDE] = to_operand<BF16>(operand_to_f32<BF16>((uint16_t)(hp[it][ap] >> 16)) * sv);
+                    }
+                }
+            }
+            __syncthreads();   // hs'(t) is complete
+            f32x4 acc[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+            f32x4 corr = {0, 0, 0, 0};
+            const uint16_t* ap16 = &hs[n * GU_STRIDE + 16 * kg];
+            static_for([&](auto qc) {
+                constexpr int q = decltype(qc)::value;
+                if (sbits[q] == 0) return;
+#ifdef EXP_NO_MFMA
+                acc[0][0] += __uint_as_float(pw[q][0] ^ pw[q][1] ^ pw[q][2] ^ pw[q][3]);
+#else
+                const u32x4 a_lo = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS);
+                const u32x4 a_hi = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS + 8);
+                if (sbits[q] == 2)
+                    gateup_pair<2, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
+                else if (sbits[q] == 3)
+                    gateup_pair<3, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
+                else
+                    gateup_pair<4, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
+#endif
+                // the buffer is free again: fetch the same slab's block of the next tile
+                if (more) issue(qc, t + 1, sbits[q], spack[q]);
+            }, std::make_integer_sequence<int, GU_SLABS>{});
+            // remove the constant term and add into G / U: lane holds rows a = 4*kg + j of
+            // column 32*pair + 16*nbl + n
+#pragma unroll
+            for (int nbl = 0; nbl < 2; ++nbl) {
+                const int c = t * N_TILE + 32 * pair + 16 * nbl + n;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int a = 4 * kg + j;
+#ifdef EXP_NO_ATOMIC
+                    if (a < n_a && c < I && acc[nbl][j] == 1234.5f) out[(int64_t)(a0 + a) * I + c] = acc[nbl][j] - corr[j];
+#else
+                    if (a < n_a && c < I) atomicAdd(&out[(int64_t)(a0 + a) * I + c], acc[nbl][j] - corr[j]);
+#endif
+                }
+            }
+            sc_cur[0] = sc_nxt[0];
+            sc_cur[1] = sc_nxt[1];
         }
     }
 }
@@ -261,61 +374,81 @@ __device__ inline void down_block(const Block16& b, const u32x4 (&az)[4], const 
     }
 }
 
+// One slab against every tile: the payload of the tiles is streamed through three
+// register buffers, two tiles ahead of the one being computed.
 template <int W, bool BF16>
-__device__ inline void down_slab(const GView& mv, int si, int n_tiles, int lane, const uint16_t* __restrict__ z,
-                                 int z_stride, f32x4 (&acc)[4]) {
+__device__ inline void down_slab(gptr<uint32_t> payload, gptr<__half> scale, const FastSlab fs, int n_tiles, int lane,
+                                 const uint16_t* __restrict__ z, int z_stride, f32x4 (&acc)[4]) {
     const int n = lane & 15, kg = lane >> 4;
-    const int tile_off = mv.slab_meta[si * 4 + 3];
-    Block16 cur, nxt;
-    float sc_cur[4], sc_nxt[4];
-    auto issue = [&](int t, Block16& b, float (&sc)[4]) {
-        const int tm = (tile_off + t) * 3;
-        load_block_role1<W>(mv.payload + mv.tile_meta[tm + 0], lane, b);
-        gptr<__half> sp = mv.scale + mv.tile_meta[tm + 1] + n;
+    Block16 buf[3];
+    float sc[3][4];
+    auto issue = [&](auto b_c, int t) {
+        constexpr int B = decltype(b_c)::value;
+        load_block_role1<W>(payload + fs.pack_off + t * 256 * W, lane, buf[B]);
+        gptr<__half> sp = scale + fs.scale_off + t * SLAB_ROWS + n;
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) sc[nb] = gload_half(sp + 16 * nb);
+        for (int nb = 0; nb < 4; ++nb) sc[B][nb] = gload_half(sp + 16 * nb);
     };
-    issue(0, cur, sc_cur);
-    for (int t = 0; t < n_tiles; ++t) {
-        if (t + 1 < n_tiles) issue(t + 1, nxt, sc_nxt);
+    auto compute = [&](auto b_c, int t) {
+        constexpr int B = decltype(b_c)::value;
         u32x4 az[4];
         const uint16_t* zp = z + n * z_stride + t * N_TILE + 8 * kg;
 #pragma unroll
         for (int m = 0; m < 4; ++m) az[m] = *reinterpret_cast<const u32x4*>(zp + 32 * m);
-        down_block<W, BF16>(cur, az, sc_cur, acc);
-        cur = nxt;
-#pragma unroll
-        for (int nb = 0; nb < 4; ++nb) sc_cur[nb] = sc_nxt[nb];
+        down_block<W, BF16>(buf[B], az, sc[B], acc);
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    issue(I0{}, 0);
+    if (n_tiles > 1) issue(I1{}, 1);
+    for (int t = 0; t < n_tiles; t += 3) {
+        if (t + 2 < n_tiles) issue(I2{}, t + 2);
+        compute(I0{}, t);
+        if (t + 1 < n_tiles) {
+            if (t + 3 < n_tiles) issue(I0{}, t + 3);
+            compute(I1{}, t + 1);
+        }
+        if (t + 2 < n_tiles) {
+            if (t + 4 < n_tiles) issue(I1{}, t + 4);
+            compute(I2{}, t + 2);
+        }
     }
 }
 
 // grid.x = E * n_groups; 256 threads; dynamic LDS = 16 * (n_tiles * 128 + 8) * 2 bytes.
 template <bool BF16>
 __global__ __launch_bounds__(256) void k_down_decode(
-    const MatView* __restrict__ down, const float* __restrict__ G, const float* __restrict__ U,
-    const float* __restrict__ route_w, const int32_t* __restrict__ token_indices,
-    const int32_t* __restrict__ expert_offsets, int T, int A, int I, int n_tiles, int n_groups, int rank_out,
-    float* __restrict__ rank_accum) {
+    const FastExpert* __restrict__ down_fe, const FastSlab* __restrict__ down_fs, int max_slabs,
+    const float* __restrict__ G, const float* __restrict__ U, const float* __restrict__ route_w,
+    const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
+    int n_tiles, int n_groups, int rank_out, float* __restrict__ rank_accum) {
     const int grp = blockIdx.x % n_groups;
     const int e = blockIdx.x / n_groups;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int n = lane & 15, g4 = (lane >> 4) * 4;
+    const int si = grp * DN_SLABS_PER_WG + wave;
+
     const int a_begin = max(expert_offsets[e], 0);
     const int a_end = min(expert_offsets[e + 1], A);
-    if (a_end <= a_begin) return;
-    const GView mv = load_view(down, e);
-    if (grp * DN_SLABS_PER_WG >= mv.num_slabs) return;
+    const FastExpert fe = down_fe[e];
+    FastSlab fs = FastSlab{0, 0, 0, 0};
+    if (si < max_slabs) fs = load_fast_slab(down_fs, e * max_slabs + si);
+    if (a_end <= a_begin || grp * DN_SLABS_PER_WG >= fe.num_slabs) return;
+
+    gptr<uint32_t> payload = as_global(fe.payload);
+    gptr<__half> scale = as_global(fe.scale);
+    gptr<__half> svec = as_global(fe.s);
+    gptr<int32_t> rank_idx = as_global(fe.rank_idx);
 
     extern __shared__ __attribute__((aligned(16))) unsigned char dsmem[];
     uint16_t* z = reinterpret_cast<uint16_t*>(dsmem);
     __shared__ int tok_sh[MAX_A];
     __shared__ float rw_sh[MAX_A];
     const int z_stride = n_tiles * N_TILE + 8;
-
-    const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
-    const int n = lane & 15, g4 = (lane >> 4) * 4;
-    const int si = grp * DN_SLABS_PER_WG + wave;
-    const bool active = si < mv.num_slabs;
-    const int bits = active ? mv.slab_meta[si * 4 + 0] : 0;
+    const bool active = fs.bits != 0;
 
     for (int a0 = a_begin; a0 < a_end; a0 += MAX_A) {
         const int n_a = min(MAX_A, a_end - a0);
@@ -336,19 +469,18 @@ __global__ __launch_bounds__(256) void k_down_decode(
             f32x4 acc[4];
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) acc[nb] = f32x4{0, 0, 0, 0};
-            if (bits == 2)
-                down_slab<2, BF16>(mv, si, n_tiles, lane, z, z_stride, acc);
-            else if (bits == 3)
-                down_slab<3, BF16>(mv, si, n_tiles, lane, z, z_stride, acc);
+            if (fs.bits == 2)
+                down_slab<2, BF16>(payload, scale, fs, n_tiles, lane, z, z_stride, acc);
+            else if (fs.bits == 3)
+                down_slab<3, BF16>(payload, scale, fs, n_tiles, lane, z, z_stride, acc);
             else
-                down_slab<4, BF16>(mv, si, n_tiles, lane, z, z_stride, acc);
+                down_slab<4, BF16>(payload, scale, fs, n_tiles, lane, z, z_stride, acc);
             // combine: rows of this slab are distinct output ranks
-            const int rank_off = mv.slab_meta[si * 4 + 2];
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) {
-                const int row = rank_off + 16 * nb + n;
-                const int lr = mv.rank_idx[row];
-                const float sv = gload_half(mv.s + row);
+                const int row = fs.rank_off + 16 * nb + n;
+                const int lr = rank_idx[row];
+                const float sv = gload_half(svec + row);
                 if (lr < 0 || lr >= rank_out) continue;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -398,16 +530,25 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     }
     record(prof, 1, st);
     const int max_slabs = std::max(gate->max_slabs, up->max_slabs);
-    const int gu_groups = (max_slabs + GU_SLABS_PER_WG - 1) / GU_SLABS_PER_WG;
-    dim3 grid((unsigned)(E * n_tiles * gu_groups), 2);
+    const int gu_groups = (max_slabs + GU_SLABS - 1) / GU_SLABS;
+    // Tiles per workgroup: long runs amortise the start-up round trips, but the grid must
+    // still hold a few workgroups per CU.  At most min(E, A) experts can be active.
+    const int64_t active_max = std::min<int64_t>(E, A);
+    int tiles_per_wg = n_tiles;
+    while (tiles_per_wg > 1 && active_max * 2 * gu_groups * ((n_tiles + tiles_per_wg - 1) / tiles_per_wg) < 2048)
+        tiles_per_wg = (tiles_per_wg + 1) / 2;
+    const int n_tchunks = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
+    dim3 grid((unsigned)(E * gu_groups * n_tchunks), 2);
     if (act_dtype == BITSMOE_DT_BF16) {
-        hipLaunchKernelGGL((k_gateup_decode<__hip_bfloat16, true>), grid, dim3(256), 0, st, gate->d_views_prepared,
-                           up->d_views_prepared, (const __hip_bfloat16*)h_gate, (const __hip_bfloat16*)h_up, Rg, Ru,
-                           tok, off, (int)T, (int)A, I, n_tiles, gu_groups, G, U);
+        hipLaunchKernelGGL((k_gateup_decode<true>), grid, dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs,
+                           gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs,
+                           (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, tok, off, (int)T, (int)A, I, n_tiles,
+                           gu_groups, n_tchunks, tiles_per_wg, G, U);
     } else {
-        hipLaunchKernelGGL((k_gateup_decode<__half, false>), grid, dim3(256), 0, st, gate->d_views_prepared,
-                           up->d_views_prepared, (const __half*)h_gate, (const __half*)h_up, Rg, Ru, tok, off, (int)T,
-                           (int)A, I, n_tiles, gu_groups, G, U);
+        hipLaunchKernelGGL((k_gateup_decode<false>), grid, dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs,
+                           gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs,
+                           (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, tok, off, (int)T, (int)A, I, n_tiles,
+                           gu_groups, n_tchunks, tiles_per_wg, G, U);
     }
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 2, st);
@@ -415,12 +556,12 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2;
     if (act_dtype == BITSMOE_DT_BF16) {
         hipLaunchKernelGGL((k_down_decode<true>), dim3((unsigned)(E * dn_groups)), dim3(256), z_bytes, st,
-                           down->d_views_prepared, G, U, rw, tok, off, (int)T, (int)A, I, n_tiles, dn_groups, rank_out,
-                           rank_accum);
+                           down->d_fast_experts, down->d_fast_slabs, down->max_slabs, G, U, rw, tok, off, (int)T, (int)A,
+                           I, n_tiles, dn_groups, rank_out, rank_accum);
     } else {
         hipLaunchKernelGGL((k_down_decode<false>), dim3((unsigned)(E * dn_groups)), dim3(256), z_bytes, st,
-                           down->d_views_prepared, G, U, rw, tok, off, (int)T, (int)A, I, n_tiles, dn_groups, rank_out,
-                           rank_accum);
+                           down->d_fast_experts, down->d_fast_slabs, down->max_slabs, G, U, rw, tok, off, (int)T, (int)A,
+                           I, n_tiles, dn_groups, rank_out, rank_accum);
     }
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 3, st);

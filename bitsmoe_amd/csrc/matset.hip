@@ -212,6 +212,8 @@ extern "C" void bitsmoe_matset_destroy(bitsmoe_matset* set) {
     if (set->d_slab_tasks) (void)hipFree(set->d_slab_tasks);
     if (set->d_prepared) (void)hipFree(set->d_prepared);
     if (set->d_views_prepared) (void)hipFree(set->d_views_prepared);
+    if (set->d_fast_experts) (void)hipFree(set->d_fast_experts);
+    if (set->d_fast_slabs) (void)hipFree(set->d_fast_slabs);
     delete set;
 }
 

@@ -2,6 +2,8 @@
 // (wave_layout.h) and the dense dequantiser that reads it back (parity check of the layout).
 #include "wave_layout.h"
 
+#include <cstring>
+
 namespace bitsmoe {
 
 // code (unsigned, before the level offset) of element (row, col) of a (slab, tile) block
@@ -159,6 +161,25 @@ extern "C" int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* s
                   "only the generic kernels can run it");
         return BITSMOE_E_UNSUPPORTED;
     }
+    // the flattened tables assume the tiles of a slab follow each other in payload and scale
+    std::vector<FastSlab> fslabs((size_t)set->n_experts * set->max_slabs, FastSlab{0, 0, 0, 0});
+    for (int e = 0; e < set->n_experts; ++e) {
+        const auto& slab = set->slab_meta_host[e];
+        const auto& tile = set->tile_meta_host[e];
+        for (int si = 0; si < set->descs[e].num_slabs; ++si) {
+            const int bits = slab[si * 4 + 0], tile_off = slab[si * 4 + 3];
+            for (int t = 0; t < set->n_tiles; ++t) {
+                if (tile[(tile_off + t) * 3 + 0] != tile[tile_off * 3 + 0] + t * 256 * bits ||
+                    tile[(tile_off + t) * 3 + 1] != tile[tile_off * 3 + 1] + t * SLAB_ROWS) {
+                    set_error("expert %d slab %d: tiles are not contiguous in payload/scale; only the generic "
+                              "kernels can run this set", e, si);
+                    return BITSMOE_E_UNSUPPORTED;
+                }
+            }
+            fslabs[(size_t)e * set->max_slabs + si] =
+                FastSlab{bits, tile[tile_off * 3 + 0], tile[tile_off * 3 + 1], slab[si * 4 + 2]};
+        }
+    }
     int64_t total_words = 0;
     std::vector<int64_t> offs(set->n_experts);
     for (int e = 0; e < set->n_experts; ++e) {
@@ -172,6 +193,20 @@ extern "C" int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* s
     for (int e = 0; e < set->n_experts; ++e) views[e].payload = set->d_prepared + offs[e];
     BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_views_prepared, sizeof(MatView) * set->n_experts));
     BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_views_prepared, views.data(), sizeof(MatView) * set->n_experts, hipMemcpyHostToDevice, st));
+    std::vector<FastExpert> fexp(set->n_experts);
+    for (int e = 0; e < set->n_experts; ++e) {
+        FastExpert& f = fexp[e];
+        memset(&f, 0, sizeof(f));
+        f.payload = set->d_prepared + offs[e];
+        f.scale = (const __half*)set->descs[e].scale;
+        f.s = (const __half*)set->descs[e].s;
+        f.rank_idx = (const int32_t*)set->descs[e].rank_idx;
+        f.num_slabs = set->descs[e].num_slabs;
+    }
+    BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_fast_experts, sizeof(FastExpert) * fexp.size()));
+    BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_fast_experts, fexp.data(), sizeof(FastExpert) * fexp.size(), hipMemcpyHostToDevice, st));
+    BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_fast_slabs, sizeof(FastSlab) * fslabs.size()));
+    BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_fast_slabs, fslabs.data(), sizeof(FastSlab) * fslabs.size(), hipMemcpyHostToDevice, st));
     hipLaunchKernelGGL(k_prepack, dim3((unsigned)set->total_slabs, set->n_tiles), dim3(256), 0, st, set->d_views,
                        set->d_views_prepared, set->d_slab_tasks, role);
     BITSMOE_HIP_TRY(hipGetLastError());

@@ -152,10 +152,11 @@ __device__ inline f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
 // fp32 -> 16-bit operand type, round to nearest even
 template <bool BF16>
 __device__ inline uint16_t to_operand(float v) {
+    // native conversions (v_cvt_pk_bf16_f32 / v_cvt_f16_f32), round to nearest even
     if constexpr (BF16) {
-        return __bfloat16_as_ushort(__float2bfloat16(v));
+        return __builtin_bit_cast(uint16_t, (__bf16)v);
     } else {
-        return __half_as_ushort(__float2half(v));
+        return __builtin_bit_cast(uint16_t, (_Float16)v);
     }
 }
 

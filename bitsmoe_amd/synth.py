@@ -60,9 +60,11 @@ def draw_bits(spec: LayerSpec, seed: int) -> List[int]:
 
 
 def orthonormal(n: int, seed: int, device) -> torch.Tensor:
-    g = torch.Generator(device=device).manual_seed(seed)
-    q, _ = torch.linalg.qr(torch.randn((n, n), generator=g, device=device, dtype=torch.float32))
-    return q.to(torch.float16)
+    # factorised on the host: the device QR goes through the vendor solver library, which is
+    # not needed anywhere else and does not run under the profiler
+    g = torch.Generator().manual_seed(seed)
+    q, _ = torch.linalg.qr(torch.randn((n, n), generator=g, dtype=torch.float32))
+    return q.to(torch.float16).to(device)
 
 
 def pack_uniform_experts(weights: torch.Tensor, bits: int) -> Dict[str, object]:
