@@ -179,6 +179,19 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
 
     __shared__ __attribute__((aligned(16))) uint16_t hs[MAX_A * GU_STRIDE];
 
+    // A group whose eight slabs share one bit-width and follow each other in the payload
+    // (the usual case) runs a body compiled for that width: no per-slab branches, affine
+    // block addresses.  WG == 0 is the general body with run-time widths.
+    bool uniform8 = true;
+#pragma unroll
+    for (int q = 1; q < GU_SLABS; ++q)
+        uniform8 = uniform8 && sbits[q] == sbits[0] && spack[q] == spack[0] + q * n_tiles * 256 * sbits[0];
+
+    auto body = [&](auto wg_c) {
+    constexpr int WG = decltype(wg_c)::value;
+    const int slab_words = n_tiles * 256 * WG;       // payload words from one slab to the next (WG != 0)
+    auto q_bits = [&](int q) { return WG != 0 ? WG : sbits[q]; };
+    auto q_pack = [&](int q) { return WG != 0 ? spack[0] + q * slab_words : spack[q]; };
     for (int a0 = a_begin; a0 < a_end; a0 += MAX_A) {
         const int n_a = min(MAX_A, a_end - a0);
         // an opaque zero keeps the address arithmetic of this chunk inside the loop body
@@ -194,7 +207,7 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
         // prologue: every block of the first tile
         static_for([&](auto qc) {
             constexpr int q = decltype(qc)::value;
-            if (sbits[q] != 0) issue(qc, t0, sbits[q], spack[q]);
+            if (q_bits(q) != 0) issue(qc, t0, q_bits(q), q_pack(q));
         }, std::make_integer_sequence<int, GU_SLABS>{});
         // token ids of the chunk: one vector load, broadcast later with readlane
         const int tok_lane = (lane < n_a) ? token_indices[a0 + lane] : -1;
@@ -287,21 +300,22 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
             const uint16_t* ap16 = &hs[n * GU_STRIDE + 16 * kg];
             static_for([&](auto qc) {
                 constexpr int q = decltype(qc)::value;
-                if (sbits[q] == 0) return;
+                const int bq = q_bits(q);
+                if (bq == 0) return;
 #ifdef EXP_NO_MFMA
                 acc[0][0] += __uint_as_float(pw[q][0] ^ pw[q][1] ^ pw[q][2] ^ pw[q][3]);
 #else
                 const u32x4 a_lo = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS);
                 const u32x4 a_hi = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS + 8);
-                if (sbits[q] == 2)
+                if (bq == 2)
                     gateup_pair<2, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
-                else if (sbits[q] == 3)
+                else if (bq == 3)
                     gateup_pair<3, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
                 else
                     gateup_pair<4, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
 #endif
                 // the buffer is free again: fetch the same slab's block of the next tile
-                if (more) issue(qc, t + 1, sbits[q], spack[q]);
+                if (more) issue(qc, t + 1, bq, q_pack(q));
             }, std::make_integer_sequence<int, GU_SLABS>{});
             // remove the constant term and add into G / U: lane holds rows a = 4*kg + j of
             // column 32*pair + 16*nbl + n
@@ -322,6 +336,16 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
             sc_cur[1] = sc_nxt[1];
         }
     }
+    };   // body
+
+    if (uniform8 && sbits[0] == 2)
+        body(std::integral_constant<int, 2>{});
+    else if (uniform8 && sbits[0] == 3)
+        body(std::integral_constant<int, 3>{});
+    else if (uniform8 && sbits[0] == 4)
+        body(std::integral_constant<int, 4>{});
+    else
+        body(std::integral_constant<int, 0>{});
 }
 
 // ----------------------------------------------------------------------------------- down
@@ -374,47 +398,147 @@ __device__ inline void down_block(const Block16& b, const u32x4 (&az)[4], const 
     }
 }
 
-// One slab against every tile: the payload of the tiles is streamed through three
-// register buffers, two tiles ahead of the one being computed.
+#ifdef EXP_TIMING
+__device__ unsigned long long g_dbg[16];
+#define TS(i) do { if (tid == 0) ts[i] = wall_clock64(); } while (0)
+#else
+#define TS(i) do {} while (0)
+#endif
+
+// Everything one wavefront of the down kernel does after the metadata has arrived, compiled
+// per bit-width of the wavefront's slab (W == 0: no slab, the wavefront only helps to build z).
+// The payload of the first two tiles is requested BEFORE z is built, so that the weights
+// are in flight while G and U are read and SiLU is evaluated; afterwards the tiles stream
+// through three register buffers, two tiles ahead of the one being computed.
 template <int W, bool BF16>
-__device__ inline void down_slab(gptr<uint32_t> payload, gptr<__half> scale, const FastSlab fs, int n_tiles, int lane,
-                                 const uint16_t* __restrict__ z, int z_stride, f32x4 (&acc)[4]) {
-    const int n = lane & 15, kg = lane >> 4;
-    Block16 buf[3];
-    float sc[3][4];
-    auto issue = [&](auto b_c, int t) {
-        constexpr int B = decltype(b_c)::value;
-        load_block_role1<W>(payload + fs.pack_off + t * 256 * W, lane, buf[B]);
-        gptr<__half> sp = scale + fs.scale_off + t * SLAB_ROWS + n;
-#pragma unroll
-        for (int nb = 0; nb < 4; ++nb) sc[B][nb] = gload_half(sp + 16 * nb);
-    };
-    auto compute = [&](auto b_c, int t) {
-        constexpr int B = decltype(b_c)::value;
-        u32x4 az[4];
-        const uint16_t* zp = z + n * z_stride + t * N_TILE + 8 * kg;
-#pragma unroll
-        for (int m = 0; m < 4; ++m) az[m] = *reinterpret_cast<const u32x4*>(zp + 32 * m);
-        down_block<W, BF16>(buf[B], az, sc[B], acc);
-    };
+__device__ inline void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gptr<__half> svec, gptr<int32_t> rank_idx,
+                                 const FastSlab fs, const float* __restrict__ G, const float* __restrict__ U,
+                                 const float* __restrict__ route_w, const int32_t* __restrict__ token_indices,
+                                 int a_begin, int a_end, int T, int I, int n_tiles, int rank_out,
+                                 float* __restrict__ rank_accum, uint16_t* __restrict__ z, int z_stride, int tid, int lane) {
+    const int n = lane & 15, kg = lane >> 4, g4 = kg * 4;
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>;
-    issue(I0{}, 0);
-    if (n_tiles > 1) issue(I1{}, 1);
-    for (int t = 0; t < n_tiles; t += 3) {
-        if (t + 2 < n_tiles) issue(I2{}, t + 2);
-        compute(I0{}, t);
-        if (t + 1 < n_tiles) {
-            if (t + 3 < n_tiles) issue(I0{}, t + 3);
-            compute(I1{}, t + 1);
+    constexpr int WL = W == 0 ? 2 : W;
+    for (int a0 = a_begin; a0 < a_end; a0 += MAX_A) {
+        const int n_a = min(MAX_A, a_end - a0);
+        int chunk_zero = 0;
+        asm volatile("" : "+s"(chunk_zero));   // keeps this chunk's address arithmetic inside the loop
+#ifdef EXP_TIMING
+        unsigned long long ts[6];
+#endif
+        TS(0);
+        Block16 buf[3];
+        float sc[3][4];
+        f32x4 acc[4];
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) acc[nb] = f32x4{0, 0, 0, 0};
+        auto issue = [&](auto b_c, int t) {
+            constexpr int B = decltype(b_c)::value;
+            load_block_role1<WL>(payload + (uint32_t)(fs.pack_off + (t + chunk_zero) * 256 * WL), lane, buf[B]);
+            gptr<__half> sp = scale + (uint32_t)(fs.scale_off + t * SLAB_ROWS + n);
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) sc[B][nb] = gload_half(sp + 16 * nb);
+        };
+        auto compute = [&](auto b_c, int t) {
+            constexpr int B = decltype(b_c)::value;
+            u32x4 az[4];
+            const uint16_t* zp = z + n * z_stride + t * N_TILE + 8 * kg;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) az[m] = *reinterpret_cast<const u32x4*>(zp + 32 * m);
+            down_block<WL, BF16>(buf[B], az, sc[B], acc);
+        };
+        int lr[4];
+        float sv[4];
+        if constexpr (W != 0) {
+            issue(I0{}, 0);
+            if (n_tiles > 1) issue(I1{}, 1);
+            // logical rank and multiplier of this lane's four output rows (needed by the epilogue)
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) {
+                const int row = fs.rank_off + 16 * nb + n;
+                lr[nb] = rank_idx[row];
+                sv[nb] = gload_half(svec + row);
+            }
         }
-        if (t + 2 < n_tiles) {
-            if (t + 4 < n_tiles) issue(I1{}, t + 4);
-            compute(I2{}, t + 2);
+        // token ids and routing weights of the chunk (lane a holds assignment a)
+        const int tok_lane = (lane < n_a) ? token_indices[a0 + lane] : -1;
+        const float rw_lane = (lane < n_a) ? route_w[a0 + lane] : 0.0f;
+        __syncthreads();   // the previous chunk is done with z
+        TS(1);
+        // z[a][c] = silu(G) * U as 16-bit operands for the rows a < n_a (other rows feed
+        // output rows that are never stored).  Each thread owns four neighbouring columns
+        // and walks the assignments four at a time, all eight vector loads issued together.
+        for (int c = tid * 4; c < I; c += 1024) {
+            for (int ab = 0; ab < n_a; ab += 4) {
+                f32x4 gv[4], uv[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int a = min(ab + j, n_a - 1);
+                    const int64_t gi = (int64_t)(a0 + a) * I + c;
+                    gv[j] = *reinterpret_cast<const f32x4*>(G + gi);
+                    uv[j] = *reinterpret_cast<const f32x4*>(U + gi);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (ab + j < n_a) {
+                        u32x2 packed;
+                        packed[0] = (uint32_t)to_operand<BF16>(silu_f32(gv[j][0]) * uv[j][0]) |
+                                    ((uint32_t)to_operand<BF16>(silu_f32(gv[j][1]) * uv[j][1]) << 16);
+                        packed[1] = (uint32_t)to_operand<BF16>(silu_f32(gv[j][2]) * uv[j][2]) |
+                                    ((uint32_t)to_operand<BF16>(silu_f32(gv[j][3]) * uv[j][3]) << 16);
+                        *reinterpret_cast<u32x2*>(z + (ab + j) * z_stride + c) = packed;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        TS(2);
+        if constexpr (W != 0) {
+            for (int t = 0; t < n_tiles; t += 3) {
+                if (t + 2 < n_tiles) issue(I2{}, t + 2);
+                compute(I0{}, t);
+                if (t + 1 < n_tiles) {
+                    if (t + 3 < n_tiles) issue(I0{}, t + 3);
+                    compute(I1{}, t + 1);
+                }
+                if (t + 2 < n_tiles) {
+                    if (t + 4 < n_tiles) issue(I1{}, t + 4);
+                    compute(I2{}, t + 2);
+                }
+            }
+            TS(3);
+            // combine: rows of this slab are distinct output ranks; lane holds assignments 4*kg + j
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int a = g4 + j;
+                    const int tk = __shfl(tok_lane, a);
+                    const float rw = __shfl(rw_lane, a);
+                    if (lr[nb] >= 0 && lr[nb] < rank_out && a < n_a && tk >= 0 && tk < T)
+                        atomicAdd(&rank_accum[(int64_t)tk * rank_out + lr[nb]], acc[nb][j] * sv[nb] * rw);
+                }
+            }
+            TS(4);
+#ifdef EXP_TIMING
+            if (tid == 0) {
+                for (int i = 0; i < 4; ++i) atomicAdd(&g_dbg[i], ts[i + 1] - ts[i]);
+                atomicAdd(&g_dbg[7], 1ull);
+            }
+#endif
         }
     }
 }
+#ifdef EXP_TIMING
+extern "C" int bitsmoe_debug_timing(unsigned long long* out, int reset) {
+    unsigned long long zero[16] = {0};
+    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(g_dbg), sizeof(zero)) != hipSuccess) return -1;
+    if (reset && hipMemcpyToSymbol(HIP_SYMBOL(g_dbg), zero, sizeof(zero)) != hipSuccess) return -1;
+    return 0;
+}
+#endif
 
 // grid.x = E * n_groups; 256 threads; dynamic LDS = 16 * (n_tiles * 128 + 8) * 2 bytes.
 template <bool BF16>
@@ -428,7 +552,6 @@ __global__ __launch_bounds__(256) void k_down_decode(
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
-    const int n = lane & 15, g4 = (lane >> 4) * 4;
     const int si = grp * DN_SLABS_PER_WG + wave;
 
     const int a_begin = max(expert_offsets[e], 0);
@@ -445,53 +568,22 @@ __global__ __launch_bounds__(256) void k_down_decode(
 
     extern __shared__ __attribute__((aligned(16))) unsigned char dsmem[];
     uint16_t* z = reinterpret_cast<uint16_t*>(dsmem);
-    __shared__ int tok_sh[MAX_A];
-    __shared__ float rw_sh[MAX_A];
     const int z_stride = n_tiles * N_TILE + 8;
-    const bool active = fs.bits != 0;
 
-    for (int a0 = a_begin; a0 < a_end; a0 += MAX_A) {
-        const int n_a = min(MAX_A, a_end - a0);
-        __syncthreads();
-        if (tid < MAX_A) {
-            tok_sh[tid] = (tid < n_a) ? token_indices[a0 + tid] : -1;
-            rw_sh[tid] = (tid < n_a) ? route_w[a0 + tid] : 0.0f;
-        }
-        // z[a][c] = silu(G) * U as 16-bit operands for the rows a < n_a (other rows feed
-        // output rows that are never stored)
-        for (int idx = tid; idx < n_a * I; idx += 256) {
-            const int a = idx / I, c = idx - a * I;
-            const int64_t gi = (int64_t)(a0 + a) * I + c;
-            z[a * z_stride + c] = to_operand<BF16>(silu_f32(G[gi]) * U[gi]);
-        }
-        __syncthreads();
-        if (active) {
-            f32x4 acc[4];
-#pragma unroll
-            for (int nb = 0; nb < 4; ++nb) acc[nb] = f32x4{0, 0, 0, 0};
-            if (fs.bits == 2)
-                down_slab<2, BF16>(payload, scale, fs, n_tiles, lane, z, z_stride, acc);
-            else if (fs.bits == 3)
-                down_slab<3, BF16>(payload, scale, fs, n_tiles, lane, z, z_stride, acc);
-            else
-                down_slab<4, BF16>(payload, scale, fs, n_tiles, lane, z, z_stride, acc);
-            // combine: rows of this slab are distinct output ranks
-#pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
-                const int row = fs.rank_off + 16 * nb + n;
-                const int lr = rank_idx[row];
-                const float sv = gload_half(svec + row);
-                if (lr < 0 || lr >= rank_out) continue;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int a = g4 + j;
-                    const int tk = tok_sh[a];
-                    if (a < n_a && tk >= 0 && tk < T)
-                        atomicAdd(&rank_accum[(int64_t)tk * rank_out + lr], acc[nb][j] * sv * rw_sh[a]);
-                }
-            }
-        }
-    }
+    // the four wavefronts may run four different instantiations; every one of them executes
+    // the same two workgroup barriers per assignment chunk
+    if (fs.bits == 2)
+        down_wave<2, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, n_tiles,
+                           rank_out, rank_accum, z, z_stride, tid, lane);
+    else if (fs.bits == 3)
+        down_wave<3, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, n_tiles,
+                           rank_out, rank_accum, z, z_stride, tid, lane);
+    else if (fs.bits == 4)
+        down_wave<4, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, n_tiles,
+                           rank_out, rank_accum, z, z_stride, tid, lane);
+    else
+        down_wave<0, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, n_tiles,
+                           rank_out, rank_accum, z, z_stride, tid, lane);
 }
 
 __global__ void k_fill_zero2(float* __restrict__ p1, int64_t n1, float* __restrict__ p2, int64_t n2) {
