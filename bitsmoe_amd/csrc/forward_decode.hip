@@ -240,11 +240,7 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
                 hp[0][ap] = 0;
                 hp[1][ap] = 0;
             }
-#if defined(EXP_NO_HS) || defined(EXP_NO_GATHER)
-            if (a0 < 0) {
-#else
             if (8 * g < n_a) {
-#endif
                 uint32_t raw[2][8];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
@@ -281,9 +277,6 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
 #pragma unroll
             for (int it = 0; it < 2; ++it) {
                 if (mine[it].bits == 0) continue;
-#if defined(EXP_NO_HS) || defined(EXP_NO_WRITE)
-                if (a0 >= 0) continue;
-#endif
                 const float sv = srow[it] * sc_cur[it];
                 uint16_t* dst = &hs[(pair + 4 * it) * SLAB_ROWS + lane];
 #pragma unroll
@@ -302,9 +295,6 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
                 constexpr int q = decltype(qc)::value;
                 const int bq = q_bits(q);
                 if (bq == 0) return;
-#ifdef EXP_NO_MFMA
-                acc[0][0] += __uint_as_float(pw[q][0] ^ pw[q][1] ^ pw[q][2] ^ pw[q][3]);
-#else
                 const u32x4 a_lo = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS);
                 const u32x4 a_hi = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS + 8);
                 if (bq == 2)
@@ -313,7 +303,6 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
                     gateup_pair<3, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
                 else
                     gateup_pair<4, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
-#endif
                 // the buffer is free again: fetch the same slab's block of the next tile
                 if (more) issue(qc, t + 1, bq, q_pack(q));
             }, std::make_integer_sequence<int, GU_SLABS>{});
@@ -325,11 +314,7 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int a = 4 * kg + j;
-#ifdef EXP_NO_ATOMIC
-                    if (a < n_a && c < I && acc[nbl][j] == 1234.5f) out[(int64_t)(a0 + a) * I + c] = acc[nbl][j] - corr[j];
-#else
                     if (a < n_a && c < I) atomicAdd(&out[(int64_t)(a0 + a) * I + c], acc[nbl][j] - corr[j]);
-#endif
                 }
             }
             sc_cur[0] = sc_nxt[0];
@@ -398,13 +383,6 @@ __device__ inline void down_block(const Block16& b, const u32x4 (&az)[4], const 
     }
 }
 
-#ifdef EXP_TIMING
-__device__ unsigned long long g_dbg[16];
-#define TS(i) do { if (tid == 0) ts[i] = wall_clock64(); } while (0)
-#else
-#define TS(i) do {} while (0)
-#endif
-
 // Everything one wavefront of the down kernel does after the metadata has arrived, compiled
 // per bit-width of the wavefront's slab (W == 0: no slab, the wavefront only helps to build z).
 // The payload of the first two tiles is requested BEFORE z is built, so that the weights
@@ -425,10 +403,6 @@ __device__ inline void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gpt
         const int n_a = min(MAX_A, a_end - a0);
         int chunk_zero = 0;
         asm volatile("" : "+s"(chunk_zero));   // keeps this chunk's address arithmetic inside the loop
-#ifdef EXP_TIMING
-        unsigned long long ts[6];
-#endif
-        TS(0);
         Block16 buf[3];
         float sc[3][4];
         f32x4 acc[4];
@@ -466,7 +440,6 @@ __device__ inline void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gpt
         const int tok_lane = (lane < n_a) ? token_indices[a0 + lane] : -1;
         const float rw_lane = (lane < n_a) ? route_w[a0 + lane] : 0.0f;
         __syncthreads();   // the previous chunk is done with z
-        TS(1);
         // z[a][c] = silu(G) * U as 16-bit operands for the rows a < n_a (other rows feed
         // output rows that are never stored).  Each thread owns four neighbouring columns
         // and walks the assignments four at a time, all eight vector loads issued together.
@@ -494,7 +467,6 @@ __device__ inline void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gpt
             }
         }
         __syncthreads();
-        TS(2);
         if constexpr (W != 0) {
             for (int t = 0; t < n_tiles; t += 3) {
                 if (t + 2 < n_tiles) issue(I2{}, t + 2);
@@ -508,7 +480,6 @@ __device__ inline void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gpt
                     compute(I2{}, t + 2);
                 }
             }
-            TS(3);
             // combine: rows of this slab are distinct output ranks; lane holds assignments 4*kg + j
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) {
@@ -521,24 +492,9 @@ __device__ inline void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gpt
                         atomicAdd(&rank_accum[(int64_t)tk * rank_out + lr[nb]], acc[nb][j] * sv[nb] * rw);
                 }
             }
-            TS(4);
-#ifdef EXP_TIMING
-            if (tid == 0) {
-                for (int i = 0; i < 4; ++i) atomicAdd(&g_dbg[i], ts[i + 1] - ts[i]);
-                atomicAdd(&g_dbg[7], 1ull);
-            }
-#endif
         }
     }
 }
-#ifdef EXP_TIMING
-extern "C" int bitsmoe_debug_timing(unsigned long long* out, int reset) {
-    unsigned long long zero[16] = {0};
-    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(g_dbg), sizeof(zero)) != hipSuccess) return -1;
-    if (reset && hipMemcpyToSymbol(HIP_SYMBOL(g_dbg), zero, sizeof(zero)) != hipSuccess) return -1;
-    return 0;
-}
-#endif
 
 // grid.x = E * n_groups; 256 threads; dynamic LDS = 16 * (n_tiles * 128 + 8) * 2 bytes.
 template <bool BF16>
