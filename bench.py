@@ -126,6 +126,12 @@ def run_workload(block, spec, tokens, steps, warmup, seed=42):
     return res, inputs
 
 
+# HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE,
+# each scaled by what it reads for a 256 MiB copy); collected offline with rocprofv3 --pmc on
+# this same script (profiles/c2-t64_hbm_traffic_counters.txt), None where not collected.
+HBM_TRAFFIC_BYTES = {"c2-t64": int((57351.2 * 2.0 + 12288.0) * 1024)}
+
+
 def roofline_of(res, inputs, bound):
     work = inputs["work"]
     if bound == "hbm":
@@ -190,6 +196,9 @@ def main() -> int:
     ap.add_argument("--workload", default="c2-t64", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extras", action="store_true", help="measure the primary workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="also run 5 plain fp32 copies (torch.mul(src, 1, out=dst)) of this many MiB: the known-size "
+                         "kernel that hardware byte counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures ONE GPU (one process, no collectives); run with --gpus 1", file=sys.stderr)
@@ -213,6 +222,14 @@ def main() -> int:
 
     res, inputs = run_workload(block, SPECS[spec_key], tokens, args.steps, args.warmup)
     roof = roofline_of(res, inputs, bound)
+    if args.copy_probe_mib > 0:
+        n = args.copy_probe_mib * (1 << 20) // 4
+        src = torch.ones(n, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     cpu, parity = (None, None)
     if not args.no_cpu:
         cpu, parity = cpu_baseline(block, inputs, tokens)
