@@ -80,6 +80,7 @@ struct bitsmoe_matset {
     bool regular = false;             // every matrix: 2/3/4-bit, k_slab % 16 == 0, full tiles
     bool regular64 = false;           // ... and every slab has exactly 64 rows, payload 16-byte aligned
     int role = -1;                    // -1: not prepared; 0: gate/up layout; 1: down layout
+    bool all_uniform8 = false;        // role 0: every aligned group of 8 slabs has one width and is contiguous
     uint32_t* d_prepared = nullptr;   // wave-native copy of every payload (see wave_layout.h)
     bitsmoe::MatView* d_views_prepared = nullptr;
     bitsmoe::FastExpert* d_fast_experts = nullptr;   // [n_experts]

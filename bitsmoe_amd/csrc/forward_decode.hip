@@ -23,7 +23,6 @@
 
 namespace bitsmoe {
 
-constexpr int GU_SLABS = 8;                        // slabs (64 rows each) per workgroup
 constexpr int GU_STRIDE = GU_SLABS * SLAB_ROWS + 8;  // 16-bit elements; +8 staggers LDS banks
 constexpr int DN_SLABS_PER_WG = 4;                 // one slab per wavefront
 constexpr int MAX_A = 16;                          // assignments per MFMA pass
@@ -119,7 +118,10 @@ __device__ inline void gateup_pair(const uint32_t (&w)[4], u32x4 a0, u32x4 a1, i
 // once per workgroup and kept in registers; per tile only the scale changes.
 // Every wavefront walks the (tile, slab) blocks of its column pair as one sequence and
 // keeps the payload of the next three blocks in flight (four rotating register buffers).
-template <bool BF16>
+// GENERAL == false: only the width-specialised bodies (groups of eight equal-width slabs that
+// follow each other in the payload); GENERAL == true: only the groups those skip.  Two kernels
+// instead of one keep the register budget of the common case free of the general body.
+template <bool BF16, bool GENERAL>
 __global__ __launch_bounds__(256) void k_gateup_decode(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
     const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
@@ -323,14 +325,18 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
     }
     };   // body
 
-    if (uniform8 && sbits[0] == 2)
-        body(std::integral_constant<int, 2>{});
-    else if (uniform8 && sbits[0] == 3)
-        body(std::integral_constant<int, 3>{});
-    else if (uniform8 && sbits[0] == 4)
-        body(std::integral_constant<int, 4>{});
-    else
-        body(std::integral_constant<int, 0>{});
+    const bool fast = uniform8 && sbits[0] >= 2 && sbits[0] <= 4;
+    if constexpr (GENERAL) {
+        if (!fast) body(std::integral_constant<int, 0>{});
+    } else {
+        if (!fast) return;
+        if (sbits[0] == 2)
+            body(std::integral_constant<int, 2>{});
+        else if (sbits[0] == 3)
+            body(std::integral_constant<int, 3>{});
+        else
+            body(std::integral_constant<int, 4>{});
+    }
 }
 
 // ----------------------------------------------------------------------------------- down
@@ -587,16 +593,19 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         tiles_per_wg = (tiles_per_wg + 1) / 2;
     const int n_tchunks = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
     dim3 grid((unsigned)(E * gu_groups * n_tchunks), 2);
+    auto launch_gateup = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs, gate->max_slabs,
+                           up->d_fast_experts, up->d_fast_slabs, up->max_slabs, (const uint16_t*)h_gate,
+                           (const uint16_t*)h_up, Rg, Ru, tok, off, (int)T, (int)A, I, n_tiles, gu_groups, n_tchunks,
+                           tiles_per_wg, G, U);
+    };
+    const bool need_general = !(gate->all_uniform8 && up->all_uniform8);
     if (act_dtype == BITSMOE_DT_BF16) {
-        hipLaunchKernelGGL((k_gateup_decode<true>), grid, dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs,
-                           gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs,
-                           (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, tok, off, (int)T, (int)A, I, n_tiles,
-                           gu_groups, n_tchunks, tiles_per_wg, G, U);
+        launch_gateup(k_gateup_decode<true, false>);
+        if (need_general) launch_gateup(k_gateup_decode<true, true>);
     } else {
-        hipLaunchKernelGGL((k_gateup_decode<false>), grid, dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs,
-                           gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs,
-                           (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, tok, off, (int)T, (int)A, I, n_tiles,
-                           gu_groups, n_tchunks, tiles_per_wg, G, U);
+        launch_gateup(k_gateup_decode<false, false>);
+        if (need_general) launch_gateup(k_gateup_decode<false, true>);
     }
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 2, st);

@@ -180,6 +180,21 @@ extern "C" int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* s
                 FastSlab{bits, tile[tile_off * 3 + 0], tile[tile_off * 3 + 1], slab[si * 4 + 2]};
         }
     }
+    // does every aligned group of GU_SLABS slabs have one width and follow each other in the payload?
+    // (the same test the gate/up kernel applies per workgroup)
+    bool all_uniform = set->max_slabs % GU_SLABS == 0;
+    for (int e = 0; e < set->n_experts && all_uniform; ++e) {
+        if (set->descs[e].num_slabs != set->max_slabs) all_uniform = false;
+        for (int s0 = 0; s0 < set->descs[e].num_slabs && all_uniform; s0 += GU_SLABS) {
+            const FastSlab& first = fslabs[(size_t)e * set->max_slabs + s0];
+            for (int q = 1; q < GU_SLABS; ++q) {
+                const FastSlab& f = fslabs[(size_t)e * set->max_slabs + s0 + q];
+                if (f.bits != first.bits || f.pack_off != first.pack_off + q * set->n_tiles * 256 * first.bits)
+                    all_uniform = false;
+            }
+        }
+    }
+    set->all_uniform8 = all_uniform;
     int64_t total_words = 0;
     std::vector<int64_t> offs(set->n_experts);
     for (int e = 0; e < set->n_experts; ++e) {

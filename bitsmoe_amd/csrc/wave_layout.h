@@ -48,6 +48,7 @@ namespace bitsmoe {
 constexpr int ROLE_GATE_UP = 0;
 constexpr int ROLE_DOWN = 1;
 constexpr int SLAB_ROWS = 64;
+constexpr int GU_SLABS = 8;   // slabs (64 rows each) one gate/up workgroup contracts over
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
