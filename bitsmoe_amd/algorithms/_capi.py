@@ -32,6 +32,7 @@ EXPORTED_SYMBOLS = (
     "bitsmoe_route_workspace_bytes",
     "bitsmoe_route",
     "bitsmoe_forward_workspace_bytes",
+    "bitsmoe_forward_workspace_bytes_sets",
     "bitsmoe_moe_forward",
     "bitsmoe_profile_create",
     "bitsmoe_profile_destroy",
@@ -96,6 +97,8 @@ def load() -> ctypes.CDLL:
     ]
     lib.bitsmoe_forward_workspace_bytes.restype = c_size_t
     lib.bitsmoe_forward_workspace_bytes.argtypes = [c_int64, c_int64, c_int32, c_int32, c_int32]
+    lib.bitsmoe_forward_workspace_bytes_sets.restype = c_size_t
+    lib.bitsmoe_forward_workspace_bytes_sets.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32]
     lib.bitsmoe_moe_forward.restype = c_int32
     lib.bitsmoe_moe_forward.argtypes = [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32,

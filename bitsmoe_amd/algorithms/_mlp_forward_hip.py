@@ -210,8 +210,8 @@ def moe_forward_sets(h_gate: torch.Tensor, h_up: torch.Tensor, token_indices: to
             down.prepare(1)
     if out is None:
         out = torch.empty((n_tokens, int(rank_out)), dtype=torch.float32, device=dev)
-    nbytes = int(_lib.bitsmoe_forward_workspace_bytes(n_tokens, n_assign, int(intermediate_size),
-                                                      gate.n_experts, int(rank_out)))
+    nbytes = int(_lib.bitsmoe_forward_workspace_bytes_sets(gate.handle, up.handle, down.handle, n_tokens,
+                                                           n_assign, int(path)))
     ws = _workspace(dev, nbytes)
     with torch.cuda.device(dev):
         _capi.check(_lib.bitsmoe_moe_forward(

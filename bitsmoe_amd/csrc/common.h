@@ -66,6 +66,13 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
                           float* rank_accum, float* G, float* U, int64_t inter_floats, bitsmoe_profile* prof,
                           hipStream_t st);
 
+bool mfma_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I);
+size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, int64_t A, int I);
+int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                        const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru,
+                        const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out, int I,
+                        float* rank_accum, void* workspace, bitsmoe_profile* prof, hipStream_t st);
+
 }  // namespace bitsmoe
 
 // The opaque handle of the C ABI.
@@ -80,6 +87,7 @@ struct bitsmoe_matset {
     bool regular = false;             // every matrix: 2/3/4-bit, k_slab % 16 == 0, full tiles
     bool regular64 = false;           // ... and every slab has exactly 64 rows, payload 16-byte aligned
     int role = -1;                    // -1: not prepared; 0: gate/up layout; 1: down layout
+    bool vector_aligned = false;      // scale / s / rank_idx of every expert start on 16-byte boundaries
     bool all_uniform8 = false;        // role 0: every aligned group of 8 slabs has one width and is contiguous
     uint32_t* d_prepared = nullptr;   // wave-native copy of every payload (see wave_layout.h)
     bitsmoe::MatView* d_views_prepared = nullptr;

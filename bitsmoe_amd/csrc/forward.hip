@@ -18,6 +18,39 @@ extern "C" size_t bitsmoe_forward_workspace_bytes(int64_t n_tokens, int64_t n_as
     return 2 * inter + 256;
 }
 
+// The path bitsmoe_moe_forward takes for these sets, sizes and `path` request
+// (BITSMOE_PATH_*), or a negative error code.
+static int resolve_path(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                        int64_t n_assign, int32_t intermediate_size, int32_t path) {
+    const bool decode_ok = decode_path_supported(gate, up, down, intermediate_size);
+    const bool mfma_ok = mfma_path_supported(gate, up, down, intermediate_size);
+    if (path == BITSMOE_PATH_MFMA && !mfma_ok) {
+        set_error("MFMA path needs matrix sets prepared with bitsmoe_matset_prepare (gate/up role 0, down role 1), "
+                  "intermediate_size a multiple of 128 and 16-byte aligned scale / s / rank_idx buffers");
+        return BITSMOE_E_UNSUPPORTED;
+    }
+    if (path == BITSMOE_PATH_DECODE && !decode_ok) {
+        set_error("decode path needs matrix sets prepared with bitsmoe_matset_prepare (gate/up role 0, down role 1)");
+        return BITSMOE_E_UNSUPPORTED;
+    }
+    if (path != BITSMOE_PATH_AUTO) return path;
+    // grouped GEMM once the experts see enough assignments on average to fill 128-row tiles
+    if (mfma_ok && n_assign >= (int64_t)48 * gate->n_experts) return BITSMOE_PATH_MFMA;
+    if (decode_ok) return BITSMOE_PATH_DECODE;
+    if (mfma_ok && n_assign >= (int64_t)16 * gate->n_experts) return BITSMOE_PATH_MFMA;
+    return BITSMOE_PATH_GENERIC;
+}
+
+extern "C" size_t bitsmoe_forward_workspace_bytes_sets(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                                                       const bitsmoe_matset* down, int64_t n_tokens,
+                                                       int64_t n_assign, int32_t path) {
+    if (!gate || !up || !down || n_assign < 0) return 0;
+    const int I = gate->intermediate_size;
+    const int chosen = resolve_path(gate, up, down, n_assign, I, path);
+    if (chosen == BITSMOE_PATH_MFMA) return mfma_workspace_bytes(gate, up, n_assign, I);
+    return bitsmoe_forward_workspace_bytes(n_tokens, n_assign, I, gate->n_experts, 0);
+}
+
 extern "C" int bitsmoe_moe_forward(const bitsmoe_matset* gate, const bitsmoe_matset* up,
                                    const bitsmoe_matset* down, const void* h_gate, const void* h_up,
                                    int32_t act_dtype, int64_t n_tokens, int32_t rank_gate,
@@ -57,27 +90,23 @@ extern "C" int bitsmoe_moe_forward(const bitsmoe_matset* gate, const bitsmoe_mat
                     "gate rank_idx references rank %d but h_gate has %d columns", gate->max_rank_plus1 - 1, rank_gate);
     BITSMOE_REQUIRE(up->max_rank_plus1 <= rank_up && up->min_rank >= 0,
                     "up rank_idx references rank %d but h_up has %d columns", up->max_rank_plus1 - 1, rank_up);
-    const size_t need = bitsmoe_forward_workspace_bytes(n_tokens, n_assign, intermediate_size, gate->n_experts, rank_out);
+    const int chosen = resolve_path(gate, up, down, n_assign, intermediate_size, path);
+    if (chosen < 0) return chosen;
+    const size_t need = bitsmoe_forward_workspace_bytes_sets(gate, up, down, n_tokens, n_assign, chosen);
     if (workspace == nullptr || workspace_bytes < need) {
         set_error("workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
         return BITSMOE_E_WORKSPACE;
     }
     BITSMOE_REQUIRE(((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
 
+    if (chosen == BITSMOE_PATH_MFMA)
+        return launch_forward_mfma(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, token_indices,
+                                   expert_offsets, route_w, n_assign, rank_out, intermediate_size, rank_accum, workspace,
+                                   profile, st);
     const size_t inter = align_up((size_t)n_assign * (size_t)intermediate_size * sizeof(float), 256);
     float* G = (float*)workspace;
     float* U = (float*)((char*)workspace + inter);
-
-    const bool fast_ok = decode_path_supported(gate, up, down, intermediate_size);
-    if (path == BITSMOE_PATH_MFMA) {
-        set_error("path %d is not built into this library version", path);
-        return BITSMOE_E_UNSUPPORTED;
-    }
-    if (path == BITSMOE_PATH_DECODE && !fast_ok) {
-        set_error("decode path needs matrix sets prepared with bitsmoe_matset_prepare (gate/up role 0, down role 1)");
-        return BITSMOE_E_UNSUPPORTED;
-    }
-    if (fast_ok && path != BITSMOE_PATH_GENERIC)
+    if (chosen == BITSMOE_PATH_DECODE)
         return launch_forward_decode(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up,
                                      token_indices, expert_offsets, route_w, n_assign, rank_out, intermediate_size,
                                      rank_accum, G, U, (int64_t)(inter / sizeof(float)), profile, st);

@@ -19,22 +19,13 @@
 #include <type_traits>
 #include <utility>
 
-#include "wave_layout.h"
+#include "fast_helpers.h"
 
 namespace bitsmoe {
 
 constexpr int GU_STRIDE = GU_SLABS * SLAB_ROWS + 8;  // 16-bit elements; +8 staggers LDS banks
 constexpr int DN_SLABS_PER_WG = 4;                 // one slab per wavefront
 constexpr int MAX_A = 16;                          // assignments per MFMA pass
-
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef const u32x2 __attribute__((address_space(1)))* gptr_u32x2;
-typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
-
-__device__ inline float gload_half(gptr<__half> p) {
-    const uint16_t bits = *reinterpret_cast<gptr<uint16_t>>(p);
-    return __half2float(__ushort_as_half(bits));
-}
 
 // raw 16-bit activation -> fp32
 template <bool BF16>
@@ -52,39 +43,7 @@ __device__ inline u32x4 corr_operand() {
     return r;
 }
 
-// Calls f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): an unrolled loop whose
-// index is a compile-time constant (register-array indices must be static).
-template <class F, int... Q>
-__device__ inline void static_for(F&& f, std::integer_sequence<int, Q...>) {
-    (f(std::integral_constant<int, Q>{}), ...);
-}
-
-// The index is wave-uniform at every call site; readfirstlane tells the compiler so (scalar
-// registers, scalar branches, scalar-base addressing downstream).
-__device__ inline FastSlab load_fast_slab(const FastSlab* __restrict__ tab, int idx) {
-    const i32x4 v = *reinterpret_cast<const i32x4*>(tab + idx);
-    return FastSlab{__builtin_amdgcn_readfirstlane(v[0]), __builtin_amdgcn_readfirstlane(v[1]),
-                    __builtin_amdgcn_readfirstlane(v[2]), __builtin_amdgcn_readfirstlane(v[3])};
-}
-
 // ------------------------------------------------------------------------------ gate / up
-// The words of one wavefront's column-block pair for one (slab, tile) block: 2-bit {nb0, nb1};
-// 4-bit {nb0 j0, nb0 j1, nb1 j0, nb1 j1}; 3-bit {low nb0, low nb1, high nb0, high nb1}.
-// `blk` is wave-uniform, `unit` = pair*64 + lane and `hi_unit` are 32-bit lane offsets.
-__device__ inline void load_pair_role0(gptr<uint32_t> blk, int bits, uint32_t unit, uint32_t hi_unit, uint32_t (&w)[4]) {
-    if (bits == 4) {
-        const u32x4 v = *reinterpret_cast<gptr_u32x4>(blk + unit * 4u);
-        w[0] = v[0]; w[1] = v[1]; w[2] = v[2]; w[3] = v[3];
-    } else {
-        const u32x2 v = *reinterpret_cast<gptr_u32x2>(blk + unit * 2u);
-        w[0] = v[0]; w[1] = v[1]; w[2] = 0; w[3] = 0;
-        if (bits == 3) {
-            const u32x2 h = *reinterpret_cast<gptr_u32x2>(blk + 512u + hi_unit);
-            w[2] = h[0]; w[3] = h[1];
-        }
-    }
-}
-
 // One (slab, tile) block restricted to one column-block pair: 2 column blocks x 2 k-steps,
 // plus the two MFMAs that accumulate the constant term.
 template <int W, bool BF16>
@@ -340,30 +299,6 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
 }
 
 // ----------------------------------------------------------------------------------- down
-struct Block16 {   // up to 16 payload words of one lane for one (slab, tile) block
-    uint32_t w[16];
-};
-
-// role 1 loads: 2-bit 8 words [nb][h], 4-bit 16 words [nb][m], 3-bit 8 low words + 4 high words [nb]
-template <int W>
-__device__ inline void load_block_role1(gptr<uint32_t> blk, int lane, Block16& b) {
-    gptr_u32x4 p = reinterpret_cast<gptr_u32x4>(blk + (W == 4 ? lane * 16 : lane * 8));
-    u32x4 v0 = p[0], v1 = p[1], v2 = {0, 0, 0, 0}, v3 = {0, 0, 0, 0};
-    if constexpr (W == 4) {
-        v2 = p[2];
-        v3 = p[3];
-    } else if constexpr (W == 3) {
-        v2 = *reinterpret_cast<gptr_u32x4>(blk + 512 + lane * 4);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        b.w[i] = v0[i];
-        b.w[4 + i] = v1[i];
-        b.w[8 + i] = v2[i];
-        b.w[12 + i] = v3[i];
-    }
-}
-
 // One (slab, tile) block of a down matrix: 4 row blocks x 4 k-steps (micro-tiles).
 template <int W, bool BF16>
 __device__ inline void down_block(const Block16& b, const u32x4 (&az)[4], const float (&sc)[4], f32x4 (&acc)[4]) {

@@ -1,0 +1,597 @@
+// Prefill-sized kernels of the routed-expert forward: every expert sees tens to hundreds of
+// assignments, so the work is a grouped GEMM and the weights are decoded once per 128-row
+// tile of assignments instead of once per 16.
+//
+//   k_build_mtiles   expert_offsets -> list of (expert, first assignment, rows <= 128) tiles
+//   k_pregather      Hs[a, k] = f16( h[tok_a, rank_idx[k]] * s[k] )  for gate and up, rows in
+//                    expert-sorted assignment order, columns in the expert's local row order
+//   k_gateup_mfma    z[a, c] = f16( silu(G) * U ),  G = Hs_gate . W_gate,  U = Hs_up . W_up
+//   k_down_mfma      rank_accum[tok_a, rank_idx[r]] += route_w[a] * s[r] * sum_c W_down[r, c] z[a, c]
+//
+// Both GEMM kernels use a 128 x 128 workgroup tile (four wavefronts, 64 x 64 each) and
+// 16x16x32 f16 MFMA.  The activation operand is staged through LDS in 128 x 64 pieces (double
+// buffered, one barrier per piece); the weight operand never touches LDS: every lane loads
+// its words of the prepared payload (wave_layout.h), expands them to packed f16 pairs
+// (2^w + code) with a rotate and an and-or, and one packed FMA per pair turns that into
+// (code - 2^(w-1)) * scale -- the same "weight rounded to half" operand the reference's
+// tensor-core path builds (bitsmoe/algorithms/cpp/mlp_forward.cu:691-751, 1554-1694).
+// Operands are f16 for f16 and bf16 inputs alike (f16 keeps more mantissa than bf16).
+#include "fast_helpers.h"
+
+namespace bitsmoe {
+
+constexpr int PF_M = 128;        // assignments per workgroup tile
+constexpr int PF_LDS_ROW = 72;   // 16-bit elements per LDS row: 64 + 8 (bank stagger, keeps 16-byte alignment)
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+struct MTile {
+    int32_t expert;   // -1: unused slot
+    int32_t a_begin;
+    int32_t rows;
+    int32_t pad;
+};
+
+__device__ inline uint32_t pk_fma_f16(uint32_t a, uint32_t b, uint32_t c) {
+    const h2 r = __builtin_elementwise_fma(__builtin_bit_cast(h2, a), __builtin_bit_cast(h2, b), __builtin_bit_cast(h2, c));
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ inline uint32_t pk_add_f16(uint32_t a, uint32_t b) {
+    const h2 r = __builtin_bit_cast(h2, a) + __builtin_bit_cast(h2, b);
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ inline uint32_t pk_mul_f16(uint32_t a, uint32_t b) {
+    const h2 r = __builtin_bit_cast(h2, a) * __builtin_bit_cast(h2, b);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+// -(1.5 * 2^W) as a packed f16 pair: times the scale it is the constant that turns
+// (2^W + code) * scale into (code - 2^(W-1)) * scale.
+template <int W>
+__device__ inline uint32_t neg_offset_pair() {
+    return Codec<W, false>::CORR | 0x80008000u;
+}
+
+// ------------------------------------------------------------------------------ schedule
+__global__ __launch_bounds__(256) void k_build_mtiles(const int32_t* __restrict__ expert_offsets, int E, int A,
+                                                      int max_tiles, MTile* __restrict__ tiles,
+                                                      int32_t* __restrict__ n_tiles_out) {
+    __shared__ int scan[256];
+    __shared__ int base_s;
+    const int tid = threadIdx.x;
+    if (tid == 0) base_s = 0;
+    __syncthreads();
+    for (int e0 = 0; e0 < E; e0 += 256) {
+        const int e = e0 + tid;
+        int begin = 0, cnt = 0;
+        if (e < E) {
+            begin = min(max(expert_offsets[e], 0), A);
+            const int end = min(max(expert_offsets[e + 1], 0), A);
+            cnt = max(end - begin, 0);
+        }
+        const int nt = (cnt + PF_M - 1) / PF_M;
+        scan[tid] = nt;
+        __syncthreads();
+        for (int d = 1; d < 256; d <<= 1) {
+            const int v = tid >= d ? scan[tid - d] : 0;
+            __syncthreads();
+            scan[tid] += v;
+            __syncthreads();
+        }
+        const int excl = scan[tid] - nt + base_s;
+        for (int j = 0; j < nt; ++j)
+            if (excl + j < max_tiles) tiles[excl + j] = MTile{e, begin + j * PF_M, min(PF_M, cnt - j * PF_M), 0};
+        __syncthreads();
+        if (tid == 255) base_s += scan[255];
+        __syncthreads();
+    }
+    const int total = min(base_s, max_tiles);
+    for (int i = total + tid; i < max_tiles; i += 256) tiles[i] = MTile{-1, 0, 0, 0};
+    if (tid == 0) *n_tiles_out = total;
+}
+
+// ------------------------------------------------------------------------------- gather
+template <bool BF16>
+__device__ inline float raw_to_f32(uint32_t v) {
+    if constexpr (BF16)
+        return __uint_as_float(v << 16);
+    else
+        return __half2float(__ushort_as_half((uint16_t)v));
+}
+
+// grid (ceil(A / 4), 2): one wavefront per (assignment, projection).
+template <bool BF16>
+__global__ __launch_bounds__(256) void k_pregather(const FastExpert* __restrict__ gate_fe,
+                                                   const FastExpert* __restrict__ up_fe,
+                                                   const uint16_t* __restrict__ h_gate,
+                                                   const uint16_t* __restrict__ h_up, int Rg, int Ru,
+                                                   const int32_t* __restrict__ token_indices,
+                                                   const int32_t* __restrict__ expert_offsets, int E, int T, int A,
+                                                   uint16_t* __restrict__ Hs_g, uint16_t* __restrict__ Hs_u, int ldg,
+                                                   int ldu) {
+    const int lane = threadIdx.x & 63;
+    const int a = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int mt = blockIdx.y;
+    if (a >= A) return;
+    // the expert of assignment a = number of experts whose range ends at or before a
+    int cnt = 0;
+    for (int j = lane; j < E; j += 64) cnt += (expert_offsets[j + 1] <= a) ? 1 : 0;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) cnt += __shfl_xor(cnt, d);
+    const int e = __builtin_amdgcn_readfirstlane(cnt);
+    if (e >= E) return;   // past the last kept assignment
+    const FastExpert fe = (mt ? up_fe : gate_fe)[e];
+    const uint16_t* __restrict__ h = mt ? h_up : h_gate;
+    const int R = mt ? Ru : Rg;
+    const int ld = mt ? ldu : ldg;
+    uint16_t* __restrict__ out = (mt ? Hs_u : Hs_g) + (int64_t)a * ld;
+    const int tok = token_indices[a];
+    const bool tok_ok = tok >= 0 && tok < T;
+    const int64_t hrow = (int64_t)(tok_ok ? tok : 0) * R;
+    const int K = min(fe.num_slabs * SLAB_ROWS, ld);
+    gptr<int32_t> rank_idx = as_global(fe.rank_idx);
+    gptr<__half> svec = as_global(fe.s);
+    for (int k0 = lane * 8; k0 < K; k0 += 512) {
+        const i32x4 r0 = *reinterpret_cast<const i32x4 __attribute__((address_space(1)))*>(rank_idx + k0);
+        const i32x4 r1 = *reinterpret_cast<const i32x4 __attribute__((address_space(1)))*>(rank_idx + k0 + 4);
+        const u32x4 sv = *reinterpret_cast<gptr_u32x4>(svec + k0);
+        uint32_t raw[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int r = i < 4 ? r0[i] : r1[i - 4];
+            raw[i] = h[hrow + min(max(r, 0), R - 1)];
+        }
+        u32x4 packed;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int r = i < 4 ? r0[i] : r1[i - 4];
+            const uint32_t sw = sv[i >> 1];
+            const float sf = __half2float(__ushort_as_half((uint16_t)((i & 1) ? (sw >> 16) : (sw & 0xFFFFu))));
+            const float v = (tok_ok && r >= 0 && r < R) ? raw_to_f32<BF16>(raw[i]) * sf : 0.0f;
+            const uint32_t hb = __builtin_bit_cast(uint16_t, (_Float16)v);
+            if (i & 1)
+                packed[i >> 1] |= hb << 16;
+            else
+                packed[i >> 1] = hb;
+        }
+        *reinterpret_cast<u32x4*>(out + k0) = packed;
+    }
+}
+
+// --------------------------------------------------------------------------- shared GEMM parts
+// Workgroup id -> logical work index such that consecutive logical indices (which share the
+// activation tile) run on the same XCD: hardware places workgroup b on XCD b % 8.
+__device__ inline int xcd_logical(int bid, int n_real) {
+    const int per = (n_real + 7) >> 3;
+    const int slot = bid >> 3;
+    if (slot >= per) return -1;
+    const int logical = (bid & 7) * per + slot;
+    return logical < n_real ? logical : -1;
+}
+
+// 128 x 64 16-bit activation piece: thread i owns rows i/8 + 32*j (j = 0..3), elements 8*(i%8)..+7
+struct APiece {
+    u32x4 v[4];
+};
+__device__ inline void load_piece(const uint16_t* __restrict__ src, int64_t ld, int a_begin, int rows, int col0, int tid,
+                                  APiece& p) {
+    const int r0 = tid >> 3, kc = (tid & 7) * 8;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int row = min(r0 + 32 * j, rows - 1);   // rows past the tile's end repeat the last one; never stored
+        p.v[j] = *reinterpret_cast<const u32x4*>(src + (int64_t)(a_begin + row) * ld + col0 + kc);
+    }
+}
+__device__ inline void store_piece(uint16_t* __restrict__ stage, int tid, const APiece& p) {
+    const int r0 = tid >> 3, kc = (tid & 7) * 8;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(stage + (r0 + 32 * j) * PF_LDS_ROW + kc) = p.v[j];
+}
+
+__device__ inline void zero_acc(f32x4 (&acc)[4][4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
+}
+
+// ------------------------------------------------------------------------------ gate / up
+// Everything one thread fetches from global memory for one slab of one projection.
+struct GuFetch {
+    APiece a;          // this thread's part of the 128 x 64 activation piece
+    u32x4 sc;          // scale pairs of contraction rows 8*(tid%8) .. +7 of the slab (tile t)
+    uint32_t bw[2][4]; // payload words of the wavefront's two column-block pairs
+};
+
+// One slab (64 contraction rows, `bits` wide) of one projection for a wavefront's 64 x 64 tile;
+// the weight operand is the raw (2^bits + code), the scale already sits in the activations.
+__device__ inline void gateup_slab_mfma(int bits, const uint16_t* __restrict__ stage, const uint32_t (&bw)[2][4], int wm,
+                                        int lane, f32x4 (&acc)[4][4]) {
+    const int n = lane & 15, kg = lane >> 4;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        u32x4 a[4];
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+            a[mb] = *reinterpret_cast<const u32x4*>(stage + (64 * wm + 16 * mb + n) * PF_LDS_ROW + 16 * kg + 8 * ks);
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) {
+            const uint32_t(&w)[4] = bw[nb >> 1];
+            const int nbl = nb & 1;
+            // the width switch wraps the decode of one operand only, so that the accumulators do not
+            // flow through alternative paths (which multiplies the register demand)
+            u32x4 b;
+            if (bits == 2)
+                b = decode_fields2<2, false>(w[nbl], 8 * ks);
+            else if (bits == 4)
+                b = decode_fields4<false>(w[2 * nbl + ks]);
+            else
+                b = decode_fields3<false>(w[nbl], 8 * ks, w[2 + nbl], 8 * (n >> 3) + 4 * ks);
+#pragma unroll
+            for (int mb = 0; mb < 4; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
+        }
+    }
+}
+
+// grid.x = 8 * ceil(max_mtiles * n_tiles / 8); workgroup = (assignment tile, 128-column tile),
+// gate then up for the same output tile, then z = silu(G) * U.
+//
+// Per slab the staging threads multiply their part of the activation piece by the slab's
+// per-row scale of this tile (packed f16), write it to LDS and keep a running sum of what they
+// wrote, weighted with 1.5 * 2^W: sum_k A'[a,k] * (2^W + code) - 1.5 * 2^W * sum_k A'[a,k] is the
+// dot product with the true levels code - 2^(W-1).  Loads run two slabs ahead of the MFMAs in
+// two alternating register sets.
+__global__ __launch_bounds__(256, 2) void k_gateup_mfma(
+    const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
+    const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
+    const uint16_t* __restrict__ Hs_g, const uint16_t* __restrict__ Hs_u, int ldg, int ldu,
+    const MTile* __restrict__ mtiles, const int32_t* __restrict__ n_mtiles, int I, int n_tiles,
+    uint16_t* __restrict__ z) {
+    __shared__ __attribute__((aligned(16))) uint16_t lds[2][PF_M * PF_LDS_ROW];
+    __shared__ float rowsum[2][PF_M];
+    const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles) * n_tiles);
+    if (logical < 0) return;
+    const int mt_i = logical / n_tiles, t = logical - mt_i * n_tiles;
+    const i32x4 tv = *reinterpret_cast<const i32x4*>(mtiles + mt_i);
+    const int e = __builtin_amdgcn_readfirstlane(tv[0]);
+    const int a_begin = __builtin_amdgcn_readfirstlane(tv[1]);
+    const int rows = __builtin_amdgcn_readfirstlane(tv[2]);
+    if (e < 0 || rows <= 0) return;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int n = lane & 15, kg = lane >> 4;
+    const bool active = 64 * wm < rows;   // a wavefront whose 64 rows are all past the end only helps to stage
+
+    f32x4 accg[4][4], accu[4][4];
+    zero_acc(accg);
+    zero_acc(accu);
+
+    auto run = [&](const FastExpert* __restrict__ fe_tab, const FastSlab* __restrict__ fs_tab, int max_slabs,
+                   const uint16_t* __restrict__ Hs, int ld, int proj, f32x4(&acc)[4][4]) {
+        const FastExpert fe = fe_tab[e];
+        const int nslabs = __builtin_amdgcn_readfirstlane(min(fe.num_slabs, max_slabs));
+        gptr<uint32_t> payload = as_global(fe.payload);
+        gptr<__half> scale = as_global(fe.scale);
+        const FastSlab* __restrict__ fs_row = fs_tab + (int64_t)e * max_slabs;
+        GuFetch f[2];
+        FastSlab fs[3];          // records of slabs s, s+1, s+2 (rotating)
+        float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        auto slab_rec = [&](int s) { return s < nslabs ? load_fast_slab(fs_row, s) : FastSlab{0, 0, 0, 0}; };
+        auto issue = [&](GuFetch& dst, const FastSlab& r, int s) {
+            load_piece(Hs, ld, a_begin, rows, s * SLAB_ROWS, tid, dst.a);
+            dst.sc = *reinterpret_cast<gptr_u32x4>(scale + (uint32_t)(r.scale_off + t * SLAB_ROWS + (tid & 7) * 8));
+            gptr<uint32_t> blk = payload + (uint32_t)(r.pack_off + t * 256 * r.bits);
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int pair = 2 * wn + p;
+                load_pair_role0(blk, r.bits, (uint32_t)(pair * 64 + lane), (uint32_t)hi_index0(kg, n, 2 * pair), dst.bw[p]);
+            }
+        };
+        // scale the fetched piece, add its weighted row sums, write it to an LDS stage
+        auto stage_piece = [&](GuFetch& src, int bits, uint16_t* __restrict__ stage) {
+            const uint32_t cw = bits == 2 ? Codec<2, false>::CORR : bits == 3 ? Codec<3, false>::CORR : Codec<4, false>::CORR;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t scaled = pk_mul_f16(src.a.v[j][i], src.sc[i]);
+                    src.a.v[j][i] = scaled;
+                    sum[j] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, scaled), __builtin_bit_cast(h2, cw), sum[j], false);
+                }
+            }
+            store_piece(stage, tid, src.a);
+        };
+        auto compute = [&](int bits, const uint16_t* __restrict__ stage, const uint32_t(&bw)[2][4]) {
+            if (active && bits != 0) gateup_slab_mfma(bits, stage, bw, wm, lane, acc);
+        };
+        if (nslabs > 0) {
+            fs[0] = slab_rec(0);
+            fs[1] = slab_rec(1);
+            fs[2] = slab_rec(2);
+            issue(f[0], fs[0], 0);
+            if (nslabs > 1) issue(f[1], fs[1], 1);
+            stage_piece(f[0], fs[0].bits, lds[0]);
+            __syncthreads();
+            // one step: slab s is in LDS stage s % 2 and its words in set X; slab s + 1 is in flight in set Y
+            auto step = [&](int s, GuFetch& X, GuFetch& Y) {
+                uint32_t bw[2][4];
+#pragma unroll
+                for (int p = 0; p < 2; ++p)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) bw[p][i] = X.bw[p][i];
+                const int bits = fs[0].bits;
+                fs[0] = fs[1];
+                fs[1] = fs[2];
+                fs[2] = slab_rec(s + 3);
+                if (s + 2 < nslabs) issue(X, fs[1], s + 2);
+                compute(bits, lds[s & 1], bw);
+                if (s + 1 < nslabs) stage_piece(Y, fs[0].bits, lds[(s + 1) & 1]);
+                __syncthreads();
+            };
+            for (int s = 0; s < nslabs; s += 2) {
+                step(s, f[0], f[1]);
+                if (s + 1 < nslabs) step(s + 1, f[1], f[0]);
+            }
+        }
+        // row sums: the eight threads that share a row hold its eight 8-column parts
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float v = sum[j];
+            v += __shfl_xor(v, 1);
+            v += __shfl_xor(v, 2);
+            v += __shfl_xor(v, 4);
+            if ((tid & 7) == 0) rowsum[proj][(tid >> 3) + 32 * j] = v;
+        }
+    };
+    run(gate_fe, gate_fs, gate_max_slabs, Hs_g, ldg, 0, accg);
+    run(up_fe, up_fs, up_max_slabs, Hs_u, ldu, 1, accu);
+    __syncthreads();
+
+    if (!active) return;
+    // lane holds rows 64*wm + 16*mb + 4*kg + j, column 128*t + 64*wn + 16*nb + n
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = 64 * wm + 16 * mb + 4 * kg + j;
+            if (row >= rows) continue;
+            const float cg = rowsum[0][row], cu = rowsum[1][row];
+            uint16_t* zr = z + (int64_t)(a_begin + row) * I + N_TILE * t + 64 * wn + n;
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) {
+                const float v = silu_f32(accg[mb][nb][j] - cg) * (accu[mb][nb][j] - cu);
+                zr[16 * nb] = __builtin_bit_cast(uint16_t, (_Float16)v);
+            }
+        }
+}
+
+// ----------------------------------------------------------------------------------- down
+// Half a tile (64 columns = micro-tiles 2*HH, 2*HH+1) of one (slab, tile) block for a
+// wavefront's 64 assignments x 64 output rows.  scp: this lane's row scale (both
+// halves of a pair) and its offset constant, per 16-row block.
+template <int W, int HH>
+__device__ inline void down_half_mfma(const uint16_t* __restrict__ stage, const Block16& blk, const uint32_t (&scp)[4],
+                                      int wm, int lane, f32x4 (&acc)[4][4]) {
+    const int n = lane & 15, kg = lane >> 4;
+#pragma unroll
+    for (int km = 0; km < 2; ++km) {
+        const int m = 2 * HH + km;
+        u32x4 a[4];
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+            a[mb] = *reinterpret_cast<const u32x4*>(stage + (64 * wm + 16 * mb + n) * PF_LDS_ROW + 32 * km + 8 * kg);
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) {
+            u32x4 b;
+            if constexpr (W == 2)
+                b = decode_fields2<2, false>(blk.w[nb * 2 + HH], 8 * km);
+            else if constexpr (W == 4)
+                b = decode_fields4<false>(blk.w[nb * 4 + m]);
+            else
+                b = decode_fields3<false>(blk.w[nb * 2 + HH], 8 * km, blk.w[8 + nb], 4 * m);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) b[i] = pk_mul_f16(pk_add_f16(b[i], neg_offset_pair<W>()), scp[nb]);
+#pragma unroll
+            for (int mb = 0; mb < 4; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
+        }
+    }
+}
+
+template <int W>
+__device__ inline void down_tile_loop(gptr<uint32_t> payload, gptr<__half> scale, const FastSlab fs,
+                                      const uint16_t* __restrict__ z, int I, int n_tiles, int a_begin, int rows,
+                                      uint16_t (*lds)[PF_M * PF_LDS_ROW], int tid, int lane, int wm, bool active,
+                                      f32x4 (&acc)[4][4]) {
+    const int n = lane & 15;
+    constexpr int WL = W == 0 ? 2 : W;
+    APiece piece;
+    Block16 blk, blk_n;
+    uint32_t scp[4], scp_n[4];
+    auto issue_b = [&](int t, Block16& b, uint32_t(&s4)[4]) {
+        if constexpr (W != 0) {
+            load_block_role1<WL>(payload + (uint32_t)(fs.pack_off + t * 256 * WL), lane, b);
+            gptr<uint16_t> sp = reinterpret_cast<gptr<uint16_t>>(scale + (uint32_t)(fs.scale_off + t * SLAB_ROWS + n));
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) s4[nb] = (uint32_t)sp[16 * nb] * 0x10001u;
+        }
+    };
+    load_piece(z, I, a_begin, rows, 0, tid, piece);
+    issue_b(0, blk, scp);
+    store_piece(lds[0], tid, piece);
+    __syncthreads();
+    for (int t = 0; t < n_tiles; ++t) {
+        const bool more = t + 1 < n_tiles;
+        // first half: columns 128*t .. +63 are in lds[0]; fetch the second half meanwhile
+        load_piece(z, I, a_begin, rows, N_TILE * t + 64, tid, piece);
+        if (more) issue_b(t + 1, blk_n, scp_n);
+        if constexpr (W != 0) {
+            if (active) down_half_mfma<WL, 0>(lds[0], blk, scp, wm, lane, acc);
+        }
+        store_piece(lds[1], tid, piece);
+        __syncthreads();
+        if (more) load_piece(z, I, a_begin, rows, N_TILE * (t + 1), tid, piece);
+        if constexpr (W != 0) {
+            if (active) down_half_mfma<WL, 1>(lds[1], blk, scp, wm, lane, acc);
+        }
+        if (more) store_piece(lds[0], tid, piece);
+        __syncthreads();
+        if (more) {
+            if constexpr (W != 0) {
+                blk = blk_n;
+#pragma unroll
+                for (int nb = 0; nb < 4; ++nb) scp[nb] = scp_n[nb];
+            }
+        }
+    }
+}
+
+// grid.x = 8 * ceil(max_mtiles * n_pairs / 8); workgroup = (assignment tile, pair of slabs):
+// wavefront (wm, wn) = assignments 64*wm..+63 x the 64 output rows of slab 2*pair + wn.
+__global__ __launch_bounds__(256) void k_down_mfma(const FastExpert* __restrict__ down_fe,
+                                                   const FastSlab* __restrict__ down_fs, int max_slabs,
+                                                   const uint16_t* __restrict__ z, const MTile* __restrict__ mtiles,
+                                                   const int32_t* __restrict__ n_mtiles,
+                                                   const int32_t* __restrict__ token_indices,
+                                                   const float* __restrict__ route_w, int T, int I, int n_tiles,
+                                                   int n_pairs, int rank_out, float* __restrict__ rank_accum) {
+    __shared__ __attribute__((aligned(16))) uint16_t lds[2][PF_M * PF_LDS_ROW];
+    const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles) * n_pairs);
+    if (logical < 0) return;
+    const int mt_i = logical / n_pairs, sp = logical - mt_i * n_pairs;
+    const i32x4 tv = *reinterpret_cast<const i32x4*>(mtiles + mt_i);
+    const int e = __builtin_amdgcn_readfirstlane(tv[0]);
+    const int a_begin = __builtin_amdgcn_readfirstlane(tv[1]);
+    const int rows = __builtin_amdgcn_readfirstlane(tv[2]);
+    if (e < 0 || rows <= 0) return;
+    const FastExpert fe = down_fe[e];
+    const int nslabs = __builtin_amdgcn_readfirstlane(min(fe.num_slabs, max_slabs));
+    if (2 * sp >= nslabs) return;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int n = lane & 15, kg = lane >> 4;
+    const int si = 2 * sp + wn;
+    FastSlab fs = FastSlab{0, 0, 0, 0};
+    if (si < nslabs) fs = load_fast_slab(down_fs + (int64_t)e * max_slabs, si);
+    const bool active = 64 * wm < rows;
+    gptr<uint32_t> payload = as_global(fe.payload);
+    gptr<__half> scale = as_global(fe.scale);
+
+    f32x4 acc[4][4];
+    zero_acc(acc);
+    // the four wavefronts may run different instantiations; all execute the same barriers
+    if (fs.bits == 2)
+        down_tile_loop<2>(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, wm, active, acc);
+    else if (fs.bits == 3)
+        down_tile_loop<3>(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, wm, active, acc);
+    else if (fs.bits == 4)
+        down_tile_loop<4>(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, wm, active, acc);
+    else
+        down_tile_loop<0>(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, wm, active, acc);
+    if (!active || fs.bits == 0) return;
+
+    // combine: lane holds assignments 64*wm + 16*mb + 4*kg + j, output rows 16*nb + n of the slab
+    gptr<int32_t> rank_idx = as_global(fe.rank_idx);
+    gptr<__half> svec = as_global(fe.s);
+    int lr[4];
+    float sv[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+        const int row = fs.rank_off + 16 * nb + n;
+        lr[nb] = rank_idx[row];
+        sv[nb] = gload_half(svec + row);
+    }
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int a = 64 * wm + 16 * mb + 4 * kg + j;
+            if (a >= rows) continue;
+            const int tk = token_indices[a_begin + a];
+            const float rw = route_w[a_begin + a];
+            if (tk < 0 || tk >= T) continue;
+            float* dst = rank_accum + (int64_t)tk * rank_out;
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb)
+                if (lr[nb] >= 0 && lr[nb] < rank_out) atomicAdd(dst + lr[nb], acc[mb][nb][j] * sv[nb] * rw);
+        }
+}
+
+// ---------------------------------------------------------------------------------- host
+static inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+static inline void record(bitsmoe_profile* p, int i, hipStream_t st) {
+    if (p) (void)hipEventRecord(p->ev[i], st);
+}
+
+bool mfma_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I) {
+    return gate->role == ROLE_GATE_UP && up->role == ROLE_GATE_UP && down->role == ROLE_DOWN && I % N_TILE == 0 &&
+           gate->vector_aligned && up->vector_aligned && down->vector_aligned;
+}
+
+size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, int64_t A, int I) {
+    const int64_t max_mtiles = A / PF_M + gate->n_experts;
+    return align256((size_t)max_mtiles * sizeof(MTile)) + 256 + align256((size_t)A * gate->max_slabs * SLAB_ROWS * 2) +
+           align256((size_t)A * up->max_slabs * SLAB_ROWS * 2) + align256((size_t)A * I * 2);
+}
+
+int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                        const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru,
+                        const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out, int I,
+                        float* rank_accum, void* workspace, bitsmoe_profile* prof, hipStream_t st) {
+    const int E = gate->n_experts;
+    const int n_tiles = gate->n_tiles;
+    const int ldg = gate->max_slabs * SLAB_ROWS, ldu = up->max_slabs * SLAB_ROWS;
+    const int64_t max_mtiles = A / PF_M + E;
+    char* ws = (char*)workspace;
+    MTile* mtiles = (MTile*)ws;
+    ws += align256((size_t)max_mtiles * sizeof(MTile));
+    int32_t* n_mtiles = (int32_t*)ws;
+    ws += 256;
+    uint16_t* Hs_g = (uint16_t*)ws;
+    ws += align256((size_t)A * ldg * 2);
+    uint16_t* Hs_u = (uint16_t*)ws;
+    ws += align256((size_t)A * ldu * 2);
+    uint16_t* z = (uint16_t*)ws;
+
+    record(prof, 0, st);
+    BITSMOE_REQUIRE(launch_fill_zero(rank_accum, T * (int64_t)rank_out, st) == BITSMOE_OK, "zero fill failed");
+    hipLaunchKernelGGL(k_build_mtiles, dim3(1), dim3(256), 0, st, off, E, (int)A, (int)max_mtiles, mtiles, n_mtiles);
+    BITSMOE_HIP_TRY(hipGetLastError());
+    {
+        dim3 grid((unsigned)((A + 3) / 4), 2);
+        if (act_dtype == BITSMOE_DT_BF16)
+            hipLaunchKernelGGL((k_pregather<true>), grid, dim3(256), 0, st, gate->d_fast_experts, up->d_fast_experts,
+                               (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, tok, off, E, (int)T, (int)A, Hs_g,
+                               Hs_u, ldg, ldu);
+        else
+            hipLaunchKernelGGL((k_pregather<false>), grid, dim3(256), 0, st, gate->d_fast_experts, up->d_fast_experts,
+                               (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, tok, off, E, (int)T, (int)A, Hs_g,
+                               Hs_u, ldg, ldu);
+        BITSMOE_HIP_TRY(hipGetLastError());
+    }
+    record(prof, 1, st);
+    {
+        const int64_t wgs = (max_mtiles * n_tiles + 7) / 8 * 8;
+        hipLaunchKernelGGL(k_gateup_mfma, dim3((unsigned)wgs), dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs,
+                           gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs, Hs_g, Hs_u, ldg, ldu,
+                           mtiles, n_mtiles, I, n_tiles, z);
+        BITSMOE_HIP_TRY(hipGetLastError());
+    }
+    record(prof, 2, st);
+    {
+        const int n_pairs = (down->max_slabs + 1) / 2;
+        const int64_t wgs = (max_mtiles * n_pairs + 7) / 8 * 8;
+        hipLaunchKernelGGL(k_down_mfma, dim3((unsigned)wgs), dim3(256), 0, st, down->d_fast_experts, down->d_fast_slabs,
+                           down->max_slabs, z, mtiles, n_mtiles, tok, rw, (int)T, I, n_tiles, n_pairs, rank_out,
+                           rank_accum);
+        BITSMOE_HIP_TRY(hipGetLastError());
+    }
+    record(prof, 3, st);
+    if (prof) prof->recorded = true;
+    return BITSMOE_OK;
+}
+
+}  // namespace bitsmoe

@@ -195,6 +195,12 @@ extern "C" int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* s
         }
     }
     set->all_uniform8 = all_uniform;
+    bool aligned = true;
+    for (int e = 0; e < set->n_experts; ++e) {
+        const bitsmoe_matrix_desc& d = set->descs[e];
+        if ((((uintptr_t)d.scale) | ((uintptr_t)d.s) | ((uintptr_t)d.rank_idx)) & 15) aligned = false;
+    }
+    set->vector_aligned = aligned;
     int64_t total_words = 0;
     std::vector<int64_t> offs(set->n_experts);
     for (int e = 0; e < set->n_experts; ++e) {

@@ -137,7 +137,7 @@ int bitsmoe_route(const void* selected, int32_t ids_are_i64, const float* weight
  *   token_indices device int32 [A], expert_offsets device int32 [E+1], route_w fp32 [A]
  *   rank_accum device fp32 [T, rank_out] out (fully overwritten)
  * Never allocates and never synchronises with the host: intermediates live in
- * `workspace` (>= bitsmoe_forward_workspace_bytes).  act_type must be 0 (SiLU).
+ * `workspace` (>= bitsmoe_forward_workspace_bytes_sets for the same sets, count and path).  act_type must be 0 (SiLU).
  * n_assign == 0 or zero experts writes zeros and returns (mlp_forward.cu:2733-2737).
  * `profile`, if not NULL, receives phase timings (see bitsmoe_profile_*).
  */
@@ -146,6 +146,17 @@ typedef struct bitsmoe_profile bitsmoe_profile;
 size_t bitsmoe_forward_workspace_bytes(int64_t n_tokens, int64_t n_assign,
                                        int32_t intermediate_size, int32_t n_experts,
                                        int32_t rank_out);
+/*
+ * Workspace size for the kernel path that bitsmoe_moe_forward takes with these sets, this
+ * assignment count and this `path` request (BITSMOE_PATH_AUTO chooses by size: the grouped
+ * GEMM path stages activations as f16 [n_assign, rows of a matrix] and needs more than the
+ * two fp32 [n_assign, intermediate] buffers of the other paths).  Takes the place of the
+ * reference's per-call torch allocations (bitsmoe/algorithms/cpp/mlp_forward.cu:2837-2847,
+ * 2999-3001).  bitsmoe_forward_workspace_bytes is the size of the generic and decode paths.
+ */
+size_t bitsmoe_forward_workspace_bytes_sets(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                                            const bitsmoe_matset* down, int64_t n_tokens,
+                                            int64_t n_assign, int32_t path);
 int bitsmoe_moe_forward(const bitsmoe_matset* gate, const bitsmoe_matset* up,
                         const bitsmoe_matset* down, const void* h_gate, const void* h_up,
                         int32_t act_dtype, int64_t n_tokens, int32_t rank_gate,

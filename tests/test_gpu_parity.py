@@ -224,3 +224,35 @@ def test_forward_decode_path(cuda_device, shape, dtype_name):
     err = _forward_case(cuda_device, 100 + e, e, t, k, rin, rout, dim, dtype_name, (2, 3, 4),
                         path=_capi.PATH_DECODE, tol=tol, uniform_bits=False, slab_multiple=64)
     print(f"decode {shape} {dtype_name}: err {err:.2e}")
+
+
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+@pytest.mark.parametrize("shape", [
+    # experts, tokens, top_k, rank_in, rank_out, dim
+    (4, 300, 2, 256, 128, 256),     # ~150 assignments per expert: two row tiles, ragged tails
+    (3, 200, 2, 192, 192, 128),     # odd slab count in the down matrices: a slab pair with one slab
+    (8, 20, 2, 128, 64, 384),       # a handful of rows per expert: half-empty tiles
+    (2, 700, 1, 320, 256, 512),     # several full 128-row tiles per expert
+])
+def test_forward_mfma_path(cuda_device, shape, dtype_name):
+    from bitsmoe_amd.algorithms import _capi
+
+    e, t, k, rin, rout, dim = shape
+    err = _forward_case(cuda_device, 200 + e, e, t, k, rin, rout, dim, dtype_name, (2, 3, 4),
+                        path=_capi.PATH_MFMA, tol=1e-2, uniform_bits=False, slab_multiple=64)
+    print(f"mfma {shape} {dtype_name}: err {err:.2e}")
+    assert err < 3e-3      # f16 operands: well inside the 1e-2 bar
+
+
+def test_forward_mfma_path_needs_prepared_sets(cuda_device):
+    import torch
+
+    from bitsmoe_amd.algorithms import _capi
+
+    hip = _hip()
+    gate, up, down = helpers.make_experts(5, 2, 80, 80, 128, choices=(2,), uniform_bits=True)   # 64 + 16 rows
+    sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=128) for m in (gate, up, down)]
+    z = lambda *s, dt=torch.float16: torch.zeros(s, dtype=dt, device=cuda_device)
+    with pytest.raises(RuntimeError, match="MFMA path needs"):
+        hip.moe_forward_sets(z(4, 80), z(4, 80), z(4, dt=torch.int32), z(3, dt=torch.int32), z(4, dt=torch.float32),
+                             sets[0], sets[1], sets[2], 80, 128, 0, path=_capi.PATH_MFMA)
