@@ -45,7 +45,9 @@ struct FastExpert {
     const __half* s;
     const int32_t* rank_idx;
     int32_t num_slabs;
-    int32_t pad[7];            // 64 bytes
+    int32_t pad0;
+    const __half* scale_s;     // gate/up sets: scale[tile][row] * s[row], same offsets as `scale`
+    int32_t pad[4];            // 64 bytes
 };
 struct FastSlab {              // tile t of the slab: payload word pack_off + t*256*bits, scale scale_off + t*64
     int32_t bits;              // 0 = no such slab
@@ -67,7 +69,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
                           hipStream_t st);
 
 bool mfma_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I);
-size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, int64_t A, int I);
+size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, int64_t T, int64_t A, int I);
 int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
                         const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru,
                         const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out, int I,
@@ -87,6 +89,9 @@ struct bitsmoe_matset {
     bool regular = false;             // every matrix: 2/3/4-bit, k_slab % 16 == 0, full tiles
     bool regular64 = false;           // ... and every slab has exactly 64 rows, payload 16-byte aligned
     int role = -1;                    // -1: not prepared; 0: gate/up layout; 1: down layout
+    bool rank_chunked8 = false;       // slab i holds local rows 64*i.., and every aligned run of 8 local rows
+                                      // maps to 8 consecutive logical ranks starting at a multiple of 8
+    __half* d_scale_s = nullptr;      // gate/up sets: scale folded with the per-row multiplier s
     bool vector_aligned = false;      // scale / s / rank_idx of every expert start on 16-byte boundaries
     bool all_uniform8 = false;        // role 0: every aligned group of 8 slabs has one width and is contiguous
     uint32_t* d_prepared = nullptr;   // wave-native copy of every payload (see wave_layout.h)

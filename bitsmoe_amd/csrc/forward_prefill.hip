@@ -16,6 +16,8 @@
 // (code - 2^(w-1)) * scale -- the same "weight rounded to half" operand the reference's
 // tensor-core path builds (bitsmoe/algorithms/cpp/mlp_forward.cu:691-751, 1554-1694).
 // Operands are f16 for f16 and bf16 inputs alike (f16 keeps more mantissa than bf16).
+#include <algorithm>
+
 #include "fast_helpers.h"
 
 namespace bitsmoe {
@@ -158,6 +160,26 @@ __global__ __launch_bounds__(256) void k_pregather(const FastExpert* __restrict_
     }
 }
 
+// bf16 activations [T, R] -> f16 [T, ld] (columns < ld <= R); grid-stride over 8-element groups.
+__global__ __launch_bounds__(256) void k_bf16_to_f16(const uint16_t* __restrict__ src, int64_t T, int R, int ld,
+                                                     uint16_t* __restrict__ dst) {
+    const int per_row = ld >> 3;
+    const int64_t total = T * per_row;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t row = i / per_row;
+        const int c = (int)(i - row * per_row) * 8;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(src + row * R + c);
+        u32x4 o;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t lo = __builtin_bit_cast(uint16_t, (_Float16)__uint_as_float(v[k] << 16));
+            const uint32_t hi = __builtin_bit_cast(uint16_t, (_Float16)__uint_as_float(v[k] & 0xFFFF0000u));
+            o[k] = lo | (hi << 16);
+        }
+        *reinterpret_cast<u32x4*>(dst + row * ld + c) = o;
+    }
+}
+
 // --------------------------------------------------------------------------- shared GEMM parts
 // Workgroup id -> logical work index such that consecutive logical indices (which share the
 // activation tile) run on the same XCD: hardware places workgroup b on XCD b % 8.
@@ -241,10 +263,17 @@ __device__ inline void gateup_slab_mfma(int bits, const uint16_t* __restrict__ s
 // wrote, weighted with 1.5 * 2^W: sum_k A'[a,k] * (2^W + code) - 1.5 * 2^W * sum_k A'[a,k] is the
 // dot product with the true levels code - 2^(W-1).  Loads run two slabs ahead of the MFMAs in
 // two alternating register sets.
+//
+// DIRECT: the activation rows are read straight from the f16 activations [T, ld] through the
+// token index (possible when every aligned run of 8 local rows is 8 consecutive logical ranks);
+// the per-row multiplier s is then taken from the folded scale table.  Otherwise Hs_* are the
+// pre-gathered rows [A, ld].
+template <bool DIRECT>
 __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
     const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
     const uint16_t* __restrict__ Hs_g, const uint16_t* __restrict__ Hs_u, int ldg, int ldu,
+    const int32_t* __restrict__ token_indices, int T,
     const MTile* __restrict__ mtiles, const int32_t* __restrict__ n_mtiles, int I, int n_tiles,
     uint16_t* __restrict__ z) {
     __shared__ __attribute__((aligned(16))) uint16_t lds[2][PF_M * PF_LDS_ROW];
@@ -264,6 +293,17 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     const int n = lane & 15, kg = lane >> 4;
     const bool active = 64 * wm < rows;   // a wavefront whose 64 rows are all past the end only helps to stage
 
+    // DIRECT: the activation row of each of this thread's four staging rows (invalid tokens read
+    // row 0: their outputs are dropped by the combine)
+    uint32_t rowbase[4] = {0, 0, 0, 0};   // element offsets (the launcher checks T * ld < 2^31)
+    if constexpr (DIRECT) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int tk = token_indices[a_begin + min((tid >> 3) + 32 * j, rows - 1)];
+            rowbase[j] = (uint32_t)((tk >= 0 && tk < T) ? tk : 0);
+        }
+    }
+
     f32x4 accg[4][4], accu[4][4];
     zero_acc(accg);
     zero_acc(accu);
@@ -273,14 +313,23 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
         const FastExpert fe = fe_tab[e];
         const int nslabs = __builtin_amdgcn_readfirstlane(min(fe.num_slabs, max_slabs));
         gptr<uint32_t> payload = as_global(fe.payload);
-        gptr<__half> scale = as_global(fe.scale);
+        gptr<__half> scale = as_global(DIRECT ? fe.scale_s : fe.scale);
+        gptr<int32_t> rank_idx = as_global(fe.rank_idx);
         const FastSlab* __restrict__ fs_row = fs_tab + (int64_t)e * max_slabs;
         GuFetch f[2];
         FastSlab fs[3];          // records of slabs s, s+1, s+2 (rotating)
+        int rb[3] = {0, 0, 0};   // DIRECT: logical rank of this thread's first column in those slabs
         float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         auto slab_rec = [&](int s) { return s < nslabs ? load_fast_slab(fs_row, s) : FastSlab{0, 0, 0, 0}; };
-        auto issue = [&](GuFetch& dst, const FastSlab& r, int s) {
-            load_piece(Hs, ld, a_begin, rows, s * SLAB_ROWS, tid, dst.a);
+        auto rank_base = [&](int s) { return (DIRECT && s < nslabs) ? rank_idx[s * SLAB_ROWS + (tid & 7) * 8] : 0; };
+        auto issue = [&](GuFetch& dst, const FastSlab& r, int rbase, int s) {
+            if constexpr (DIRECT) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    dst.a.v[j] = *reinterpret_cast<const u32x4*>(Hs + (rowbase[j] * (uint32_t)ld + (uint32_t)rbase));
+            } else {
+                load_piece(Hs, ld, a_begin, rows, s * SLAB_ROWS, tid, dst.a);
+            }
             dst.sc = *reinterpret_cast<gptr_u32x4>(scale + (uint32_t)(r.scale_off + t * SLAB_ROWS + (tid & 7) * 8));
             gptr<uint32_t> blk = payload + (uint32_t)(r.pack_off + t * 256 * r.bits);
 #pragma unroll
@@ -310,8 +359,11 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
             fs[0] = slab_rec(0);
             fs[1] = slab_rec(1);
             fs[2] = slab_rec(2);
-            issue(f[0], fs[0], 0);
-            if (nslabs > 1) issue(f[1], fs[1], 1);
+            rb[0] = rank_base(0);
+            rb[1] = rank_base(1);
+            rb[2] = rank_base(2);
+            issue(f[0], fs[0], rb[0], 0);
+            if (nslabs > 1) issue(f[1], fs[1], rb[1], 1);
             stage_piece(f[0], fs[0].bits, lds[0]);
             __syncthreads();
             // one step: slab s is in LDS stage s % 2 and its words in set X; slab s + 1 is in flight in set Y
@@ -325,7 +377,10 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
                 fs[0] = fs[1];
                 fs[1] = fs[2];
                 fs[2] = slab_rec(s + 3);
-                if (s + 2 < nslabs) issue(X, fs[1], s + 2);
+                rb[0] = rb[1];
+                rb[1] = rb[2];
+                rb[2] = rank_base(s + 3);
+                if (s + 2 < nslabs) issue(X, fs[1], rb[1], s + 2);
                 compute(bits, lds[s & 1], bw);
                 if (s + 1 < nslabs) stage_piece(Y, fs[0].bits, lds[(s + 1) & 1]);
                 __syncthreads();
@@ -368,77 +423,92 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
 }
 
 // ----------------------------------------------------------------------------------- down
+constexpr int DN_SLABS_MFMA = 4;   // slabs (64 output rows each) per workgroup: one per wavefront
+
 // Half a tile (64 columns = micro-tiles 2*HH, 2*HH+1) of one (slab, tile) block for a
-// wavefront's 64 assignments x 64 output rows.  scp: this lane's row scale (both
-// halves of a pair) and its offset constant, per 16-row block.
-template <int W, int HH>
-__device__ inline void down_half_mfma(const uint16_t* __restrict__ stage, const Block16& blk, const uint32_t (&scp)[4],
-                                      int wm, int lane, f32x4 (&acc)[4][4]) {
+// wavefront's 128 assignments x 64 output rows.  scp: this lane's row scale in both halves of a
+// pair, per 16-row block.  The weight operand is (code - 2^(W-1)) * scale rounded once to f16,
+// the operand the reference builds (bitsmoe/algorithms/cpp/mlp_forward.cu:1554-1694).
+template <int HH>
+__device__ inline void down_half_mfma(int bits, const uint16_t* __restrict__ stage, const Block16& blk,
+                                      const uint32_t (&scp)[4], int lane, f32x4 (&acc)[8][4]) {
     const int n = lane & 15, kg = lane >> 4;
 #pragma unroll
     for (int km = 0; km < 2; ++km) {
         const int m = 2 * HH + km;
-        u32x4 a[4];
+        u32x4 a[8];
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
-            a[mb] = *reinterpret_cast<const u32x4*>(stage + (64 * wm + 16 * mb + n) * PF_LDS_ROW + 32 * km + 8 * kg);
+        for (int mb = 0; mb < 8; ++mb)
+            a[mb] = *reinterpret_cast<const u32x4*>(stage + (16 * mb + n) * PF_LDS_ROW + 32 * km + 8 * kg);
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
+            // the width switch wraps one operand only: accumulators that flow through alternative
+            // paths multiply the register demand
             u32x4 b;
-            if constexpr (W == 2)
+            uint32_t off;
+            if (bits == 2) {
                 b = decode_fields2<2, false>(blk.w[nb * 2 + HH], 8 * km);
-            else if constexpr (W == 4)
+                off = neg_offset_pair<2>();
+            } else if (bits == 4) {
                 b = decode_fields4<false>(blk.w[nb * 4 + m]);
-            else
+                off = neg_offset_pair<4>();
+            } else {
                 b = decode_fields3<false>(blk.w[nb * 2 + HH], 8 * km, blk.w[8 + nb], 4 * m);
+                off = neg_offset_pair<3>();
+            }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) b[i] = pk_mul_f16(pk_add_f16(b[i], neg_offset_pair<W>()), scp[nb]);
+            for (int i = 0; i < 4; ++i) b[i] = pk_mul_f16(pk_add_f16(b[i], off), scp[nb]);
 #pragma unroll
-            for (int mb = 0; mb < 4; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
+            for (int mb = 0; mb < 8; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
         }
     }
 }
 
-template <int W>
+// The column loop of one wavefront (fs.bits == 0: no slab, the wavefront only helps to stage).
+// Pieces of z (128 assignments x 64 columns) run two ahead of the MFMAs in two alternating
+// register sets, the payload block of the next tile one tile ahead.
 __device__ inline void down_tile_loop(gptr<uint32_t> payload, gptr<__half> scale, const FastSlab fs,
                                       const uint16_t* __restrict__ z, int I, int n_tiles, int a_begin, int rows,
-                                      uint16_t (*lds)[PF_M * PF_LDS_ROW], int tid, int lane, int wm, bool active,
-                                      f32x4 (&acc)[4][4]) {
+                                      uint16_t (*lds)[PF_M * PF_LDS_ROW], int tid, int lane, f32x4 (&acc)[8][4]) {
     const int n = lane & 15;
-    constexpr int WL = W == 0 ? 2 : W;
-    APiece piece;
+    const int W = fs.bits;
+    APiece p0, p1;
     Block16 blk, blk_n;
     uint32_t scp[4], scp_n[4];
     auto issue_b = [&](int t, Block16& b, uint32_t(&s4)[4]) {
-        if constexpr (W != 0) {
-            load_block_role1<WL>(payload + (uint32_t)(fs.pack_off + t * 256 * WL), lane, b);
+        if (W != 0) {
+            gptr<uint32_t> src = payload + (uint32_t)(fs.pack_off + t * 256 * W);
+            if (W == 2)
+                load_block_role1<2>(src, lane, b);
+            else if (W == 3)
+                load_block_role1<3>(src, lane, b);
+            else
+                load_block_role1<4>(src, lane, b);
             gptr<uint16_t> sp = reinterpret_cast<gptr<uint16_t>>(scale + (uint32_t)(fs.scale_off + t * SLAB_ROWS + n));
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) s4[nb] = (uint32_t)sp[16 * nb] * 0x10001u;
         }
     };
-    load_piece(z, I, a_begin, rows, 0, tid, piece);
+    const int n_halves = 2 * n_tiles;
+    load_piece(z, I, a_begin, rows, 0, tid, p0);
+    load_piece(z, I, a_begin, rows, 64, tid, p1);
     issue_b(0, blk, scp);
-    store_piece(lds[0], tid, piece);
+    store_piece(lds[0], tid, p0);
     __syncthreads();
     for (int t = 0; t < n_tiles; ++t) {
-        const bool more = t + 1 < n_tiles;
-        // first half: columns 128*t .. +63 are in lds[0]; fetch the second half meanwhile
-        load_piece(z, I, a_begin, rows, N_TILE * t + 64, tid, piece);
-        if (more) issue_b(t + 1, blk_n, scp_n);
-        if constexpr (W != 0) {
-            if (active) down_half_mfma<WL, 0>(lds[0], blk, scp, wm, lane, acc);
-        }
-        store_piece(lds[1], tid, piece);
+        const int h = 2 * t;
+        // first half of tile t is in lds[0], the second in flight in p1
+        if (h + 2 < n_halves) load_piece(z, I, a_begin, rows, 64 * (h + 2), tid, p0);
+        if (t + 1 < n_tiles) issue_b(t + 1, blk_n, scp_n);
+        if (W != 0) down_half_mfma<0>(W, lds[0], blk, scp, lane, acc);
+        store_piece(lds[1], tid, p1);
         __syncthreads();
-        if (more) load_piece(z, I, a_begin, rows, N_TILE * (t + 1), tid, piece);
-        if constexpr (W != 0) {
-            if (active) down_half_mfma<WL, 1>(lds[1], blk, scp, wm, lane, acc);
-        }
-        if (more) store_piece(lds[0], tid, piece);
+        if (h + 3 < n_halves) load_piece(z, I, a_begin, rows, 64 * (h + 3), tid, p1);
+        if (W != 0) down_half_mfma<1>(W, lds[1], blk, scp, lane, acc);
+        if (h + 2 < n_halves) store_piece(lds[0], tid, p0);
         __syncthreads();
-        if (more) {
-            if constexpr (W != 0) {
+        {
+            if (W != 0 && t + 1 < n_tiles) {
                 blk = blk_n;
 #pragma unroll
                 for (int nb = 0; nb < 4; ++nb) scp[nb] = scp_n[nb];
@@ -447,19 +517,21 @@ __device__ inline void down_tile_loop(gptr<uint32_t> payload, gptr<__half> scale
     }
 }
 
-// grid.x = 8 * ceil(max_mtiles * n_pairs / 8); workgroup = (assignment tile, pair of slabs):
-// wavefront (wm, wn) = assignments 64*wm..+63 x the 64 output rows of slab 2*pair + wn.
-__global__ __launch_bounds__(256) void k_down_mfma(const FastExpert* __restrict__ down_fe,
-                                                   const FastSlab* __restrict__ down_fs, int max_slabs,
-                                                   const uint16_t* __restrict__ z, const MTile* __restrict__ mtiles,
-                                                   const int32_t* __restrict__ n_mtiles,
-                                                   const int32_t* __restrict__ token_indices,
-                                                   const float* __restrict__ route_w, int T, int I, int n_tiles,
-                                                   int n_pairs, int rank_out, float* __restrict__ rank_accum) {
+// grid.x = 8 * ceil(max_mtiles * n_groups / 8); workgroup = (assignment tile, group of four
+// slabs): wavefront w = all 128 assignments x the 64 output rows of slab 4*group + w.
+__global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restrict__ down_fe,
+                                                      const FastSlab* __restrict__ down_fs, int max_slabs,
+                                                      const uint16_t* __restrict__ z, const MTile* __restrict__ mtiles,
+                                                      const int32_t* __restrict__ n_mtiles,
+                                                      const int32_t* __restrict__ token_indices,
+                                                      const float* __restrict__ route_w, int T, int I, int n_tiles,
+                                                      int n_groups, int rank_out, float* __restrict__ rank_accum) {
     __shared__ __attribute__((aligned(16))) uint16_t lds[2][PF_M * PF_LDS_ROW];
-    const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles) * n_pairs);
+    __shared__ int32_t tok_s[PF_M];
+    __shared__ float rw_s[PF_M];
+    const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles) * n_groups);
     if (logical < 0) return;
-    const int mt_i = logical / n_pairs, sp = logical - mt_i * n_pairs;
+    const int mt_i = logical / n_groups, grp = logical - mt_i * n_groups;
     const i32x4 tv = *reinterpret_cast<const i32x4*>(mtiles + mt_i);
     const int e = __builtin_amdgcn_readfirstlane(tv[0]);
     const int a_begin = __builtin_amdgcn_readfirstlane(tv[1]);
@@ -467,33 +539,33 @@ __global__ __launch_bounds__(256) void k_down_mfma(const FastExpert* __restrict_
     if (e < 0 || rows <= 0) return;
     const FastExpert fe = down_fe[e];
     const int nslabs = __builtin_amdgcn_readfirstlane(min(fe.num_slabs, max_slabs));
-    if (2 * sp >= nslabs) return;
+    if (DN_SLABS_MFMA * grp >= nslabs) return;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
     const int n = lane & 15, kg = lane >> 4;
-    const int si = 2 * sp + wn;
+    const int si = DN_SLABS_MFMA * grp + wave;
     FastSlab fs = FastSlab{0, 0, 0, 0};
     if (si < nslabs) fs = load_fast_slab(down_fs + (int64_t)e * max_slabs, si);
-    const bool active = 64 * wm < rows;
     gptr<uint32_t> payload = as_global(fe.payload);
     gptr<__half> scale = as_global(fe.scale);
+    if (tid < PF_M) {
+        const bool ok = tid < rows;
+        const int tk = ok ? token_indices[a_begin + tid] : -1;
+        tok_s[tid] = (tk >= 0 && tk < T) ? tk : -1;
+        rw_s[tid] = ok ? route_w[a_begin + tid] : 0.0f;
+    }
 
-    f32x4 acc[4][4];
-    zero_acc(acc);
-    // the four wavefronts may run different instantiations; all execute the same barriers
-    if (fs.bits == 2)
-        down_tile_loop<2>(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, wm, active, acc);
-    else if (fs.bits == 3)
-        down_tile_loop<3>(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, wm, active, acc);
-    else if (fs.bits == 4)
-        down_tile_loop<4>(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, wm, active, acc);
-    else
-        down_tile_loop<0>(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, wm, active, acc);
-    if (!active || fs.bits == 0) return;
+    f32x4 acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
+    // wavefronts without a slab skip the MFMAs; all execute the same barriers
+    down_tile_loop(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, acc);
+    if (fs.bits == 0) return;   // (the loops end with a barrier, so tok_s / rw_s are complete)
 
-    // combine: lane holds assignments 64*wm + 16*mb + 4*kg + j, output rows 16*nb + n of the slab
+    // combine: lane holds assignments 16*mb + 4*kg + j, output rows 16*nb + n of the slab
     gptr<int32_t> rank_idx = as_global(fe.rank_idx);
     gptr<__half> svec = as_global(fe.s);
     int lr[4];
@@ -501,23 +573,25 @@ __global__ __launch_bounds__(256) void k_down_mfma(const FastExpert* __restrict_
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) {
         const int row = fs.rank_off + 16 * nb + n;
-        lr[nb] = rank_idx[row];
+        const int r = rank_idx[row];
+        lr[nb] = (r >= 0 && r < rank_out) ? r : -1;
         sv[nb] = gload_half(svec + row);
     }
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
+    for (int mb = 0; mb < 8; ++mb) {
+        if (16 * mb >= rows) break;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int a = 64 * wm + 16 * mb + 4 * kg + j;
-            if (a >= rows) continue;
-            const int tk = token_indices[a_begin + a];
-            const float rw = route_w[a_begin + a];
-            if (tk < 0 || tk >= T) continue;
+            const int a = 16 * mb + 4 * kg + j;
+            const int tk = tok_s[a];
+            const float rw = rw_s[a];
+            if (tk < 0) continue;
             float* dst = rank_accum + (int64_t)tk * rank_out;
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb)
-                if (lr[nb] >= 0 && lr[nb] < rank_out) atomicAdd(dst + lr[nb], acc[mb][nb][j] * sv[nb] * rw);
+                if (lr[nb] >= 0) atomicAdd(dst + lr[nb], acc[mb][nb][j] * sv[nb] * rw);
         }
+    }
 }
 
 // ---------------------------------------------------------------------------------- host
@@ -531,10 +605,20 @@ bool mfma_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, c
            gate->vector_aligned && up->vector_aligned && down->vector_aligned;
 }
 
-size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, int64_t A, int I) {
+// Can the gate/up kernel read activation rows through the token index (no pre-gather)?
+static bool direct_ok(const bitsmoe_matset* gate, const bitsmoe_matset* up) {
+    return gate->rank_chunked8 && up->rank_chunked8 && gate->d_scale_s && up->d_scale_s;
+}
+static inline int direct_ld(const bitsmoe_matset* set) { return (set->max_rank_plus1 + 7) / 8 * 8; }
+
+size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, int64_t T, int64_t A, int I) {
     const int64_t max_mtiles = A / PF_M + gate->n_experts;
-    return align256((size_t)max_mtiles * sizeof(MTile)) + 256 + align256((size_t)A * gate->max_slabs * SLAB_ROWS * 2) +
-           align256((size_t)A * up->max_slabs * SLAB_ROWS * 2) + align256((size_t)A * I * 2);
+    const size_t direct = align256((size_t)T * direct_ld(gate) * 2) + align256((size_t)T * direct_ld(up) * 2);
+    const size_t gathered = align256((size_t)A * gate->max_slabs * SLAB_ROWS * 2) + align256((size_t)A * up->max_slabs * SLAB_ROWS * 2);
+    // the direct form falls back to the gathered one when the activation pointers or row
+    // lengths do not allow 16-byte loads, which is only known at the call
+    return align256((size_t)max_mtiles * sizeof(MTile)) + 256 + std::max(direct_ok(gate, up) ? direct : 0, gathered) +
+           align256((size_t)A * I * 2);
 }
 
 int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
@@ -543,46 +627,63 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
                         float* rank_accum, void* workspace, bitsmoe_profile* prof, hipStream_t st) {
     const int E = gate->n_experts;
     const int n_tiles = gate->n_tiles;
-    const int ldg = gate->max_slabs * SLAB_ROWS, ldu = up->max_slabs * SLAB_ROWS;
     const int64_t max_mtiles = A / PF_M + E;
+    const bool direct = direct_ok(gate, up) && Rg % 8 == 0 && Ru % 8 == 0 && (((uintptr_t)h_gate | (uintptr_t)h_up) & 15) == 0 &&
+                        T * (int64_t)std::max(Rg, Ru) < ((int64_t)1 << 31);
+    const int ldg = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(gate) : Rg) : gate->max_slabs * SLAB_ROWS;
+    const int ldu = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(up) : Ru) : up->max_slabs * SLAB_ROWS;
     char* ws = (char*)workspace;
     MTile* mtiles = (MTile*)ws;
     ws += align256((size_t)max_mtiles * sizeof(MTile));
     int32_t* n_mtiles = (int32_t*)ws;
     ws += 256;
-    uint16_t* Hs_g = (uint16_t*)ws;
-    ws += align256((size_t)A * ldg * 2);
-    uint16_t* Hs_u = (uint16_t*)ws;
-    ws += align256((size_t)A * ldu * 2);
+    const uint16_t* Hs_g = (const uint16_t*)ws;
+    ws += direct ? align256((size_t)T * direct_ld(gate) * 2) : align256((size_t)A * ldg * 2);
+    const uint16_t* Hs_u = (const uint16_t*)ws;
+    ws = (char*)workspace + mfma_workspace_bytes(gate, up, T, A, I) - align256((size_t)A * I * 2);
     uint16_t* z = (uint16_t*)ws;
 
     record(prof, 0, st);
     BITSMOE_REQUIRE(launch_fill_zero(rank_accum, T * (int64_t)rank_out, st) == BITSMOE_OK, "zero fill failed");
     hipLaunchKernelGGL(k_build_mtiles, dim3(1), dim3(256), 0, st, off, E, (int)A, (int)max_mtiles, mtiles, n_mtiles);
     BITSMOE_HIP_TRY(hipGetLastError());
-    {
+    if (direct) {
+        if (act_dtype == BITSMOE_DT_BF16) {
+            hipLaunchKernelGGL(k_bf16_to_f16, dim3(1024), dim3(256), 0, st, (const uint16_t*)h_gate, T, Rg, ldg, (uint16_t*)Hs_g);
+            hipLaunchKernelGGL(k_bf16_to_f16, dim3(1024), dim3(256), 0, st, (const uint16_t*)h_up, T, Ru, ldu, (uint16_t*)Hs_u);
+            BITSMOE_HIP_TRY(hipGetLastError());
+        } else {
+            Hs_g = (const uint16_t*)h_gate;
+            Hs_u = (const uint16_t*)h_up;
+        }
+    } else {
         dim3 grid((unsigned)((A + 3) / 4), 2);
         if (act_dtype == BITSMOE_DT_BF16)
             hipLaunchKernelGGL((k_pregather<true>), grid, dim3(256), 0, st, gate->d_fast_experts, up->d_fast_experts,
-                               (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, tok, off, E, (int)T, (int)A, Hs_g,
-                               Hs_u, ldg, ldu);
+                               (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, tok, off, E, (int)T, (int)A,
+                               (uint16_t*)Hs_g, (uint16_t*)Hs_u, ldg, ldu);
         else
             hipLaunchKernelGGL((k_pregather<false>), grid, dim3(256), 0, st, gate->d_fast_experts, up->d_fast_experts,
-                               (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, tok, off, E, (int)T, (int)A, Hs_g,
-                               Hs_u, ldg, ldu);
+                               (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, tok, off, E, (int)T, (int)A,
+                               (uint16_t*)Hs_g, (uint16_t*)Hs_u, ldg, ldu);
         BITSMOE_HIP_TRY(hipGetLastError());
     }
     record(prof, 1, st);
     {
         const int64_t wgs = (max_mtiles * n_tiles + 7) / 8 * 8;
-        hipLaunchKernelGGL(k_gateup_mfma, dim3((unsigned)wgs), dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs,
-                           gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs, Hs_g, Hs_u, ldg, ldu,
-                           mtiles, n_mtiles, I, n_tiles, z);
+        if (direct)
+            hipLaunchKernelGGL(k_gateup_mfma<true>, dim3((unsigned)wgs), dim3(256), 0, st, gate->d_fast_experts,
+                               gate->d_fast_slabs, gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs,
+                               Hs_g, Hs_u, ldg, ldu, tok, (int)T, mtiles, n_mtiles, I, n_tiles, z);
+        else
+            hipLaunchKernelGGL(k_gateup_mfma<false>, dim3((unsigned)wgs), dim3(256), 0, st, gate->d_fast_experts,
+                               gate->d_fast_slabs, gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs,
+                               Hs_g, Hs_u, ldg, ldu, tok, (int)T, mtiles, n_mtiles, I, n_tiles, z);
         BITSMOE_HIP_TRY(hipGetLastError());
     }
     record(prof, 2, st);
     {
-        const int n_pairs = (down->max_slabs + 1) / 2;
+        const int n_pairs = (down->max_slabs + DN_SLABS_MFMA - 1) / DN_SLABS_MFMA;
         const int64_t wgs = (max_mtiles * n_pairs + 7) / 8 * 8;
         hipLaunchKernelGGL(k_down_mfma, dim3((unsigned)wgs), dim3(256), 0, st, down->d_fast_experts, down->d_fast_slabs,
                            down->max_slabs, z, mtiles, n_mtiles, tok, rw, (int)T, I, n_tiles, n_pairs, rank_out,

@@ -145,6 +145,7 @@ extern "C" int bitsmoe_matset_create(const bitsmoe_matrix_desc* descs, int32_t n
     std::vector<SlabTask> tasks;
     std::vector<int32_t> rk;
     int max_rank = -1, min_rank = 0x7fffffff;
+    bool chunked8 = n_experts > 0;
     for (int e = 0; e < n_experts; ++e) {
         const bitsmoe_matrix_desc& d = descs[e];
         BITSMOE_REQUIRE(d.num_slabs >= 0 && d.num_tiles >= 0 && d.rank_len >= 0 && d.payload_words >= 0 && d.scale_len >= 0,
@@ -174,6 +175,14 @@ extern "C" int bitsmoe_matset_create(const bitsmoe_matrix_desc* descs, int32_t n
             max_rank = std::max(max_rank, v);
             min_rank = std::min(min_rank, v);
         }
+        for (int si = 0; si < d.num_slabs && chunked8; ++si)
+            if (slab[si * 4 + 2] != si * K_SLAB) chunked8 = false;
+        if (d.rank_len % 8 != 0) chunked8 = false;
+        for (size_t k0 = 0; k0 + 8 <= rk.size() && chunked8; k0 += 8) {
+            if (rk[k0] < 0 || rk[k0] % 8 != 0) chunked8 = false;
+            for (int i = 1; i < 8; ++i)
+                if (rk[k0 + i] != rk[k0] + i) chunked8 = false;
+        }
         MatView& mv = views[e];
         mv.payload = (const uint32_t*)d.payload;
         mv.rank_idx = (const int32_t*)d.rank_idx;
@@ -188,6 +197,7 @@ extern "C" int bitsmoe_matset_create(const bitsmoe_matrix_desc* descs, int32_t n
         set->max_slabs = std::max(set->max_slabs, d.num_slabs);
         for (int s = 0; s < d.num_slabs; ++s) tasks.push_back(SlabTask{e, s});
     }
+    set->rank_chunked8 = chunked8;
     set->total_slabs = (int64_t)tasks.size();
     set->max_rank_plus1 = max_rank + 1;
     set->min_rank = (min_rank == 0x7fffffff) ? 0 : min_rank;
@@ -211,6 +221,7 @@ extern "C" void bitsmoe_matset_destroy(bitsmoe_matset* set) {
     if (set->d_views) (void)hipFree(set->d_views);
     if (set->d_slab_tasks) (void)hipFree(set->d_slab_tasks);
     if (set->d_prepared) (void)hipFree(set->d_prepared);
+    if (set->d_scale_s) (void)hipFree(set->d_scale_s);
     if (set->d_views_prepared) (void)hipFree(set->d_views_prepared);
     if (set->d_fast_experts) (void)hipFree(set->d_fast_experts);
     if (set->d_fast_slabs) (void)hipFree(set->d_fast_slabs);

@@ -2,6 +2,7 @@
 // (wave_layout.h) and the dense dequantiser that reads it back (parity check of the layout).
 #include "wave_layout.h"
 
+#include <algorithm>
 #include <cstring>
 
 namespace bitsmoe {
@@ -146,6 +147,21 @@ __global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* payload 
     }
 }
 
+// scale_s[scale_off(slab, tile) + row] = scale[...] * s[rank_off(slab) + row], rounded once to fp16.
+// grid (slab tasks, tiles), 64 threads.
+__global__ __launch_bounds__(64) void k_fold_scale_s(const MatView* __restrict__ views, const SlabTask* __restrict__ tasks,
+                                                     const int64_t* __restrict__ out_offsets, __half* __restrict__ out) {
+    const SlabTask task = tasks[blockIdx.x];
+    const MatView mv = views[task.expert];
+    const int si = task.slab;
+    const int rank_off = mv.slab_meta[si * 4 + 2];
+    const int t = mv.slab_meta[si * 4 + 3] + blockIdx.y;
+    const int scale_off = mv.tile_meta[t * 3 + 1];
+    const int row = threadIdx.x;
+    const float v = __half2float(mv.scale[scale_off + row]) * __half2float(mv.s[rank_off + row]);
+    out[out_offsets[task.expert] + scale_off + row] = __float2half(v);
+}
+
 }  // namespace bitsmoe
 
 using namespace bitsmoe;
@@ -214,10 +230,31 @@ extern "C" int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* s
     for (int e = 0; e < set->n_experts; ++e) views[e].payload = set->d_prepared + offs[e];
     BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_views_prepared, sizeof(MatView) * set->n_experts));
     BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_views_prepared, views.data(), sizeof(MatView) * set->n_experts, hipMemcpyHostToDevice, st));
+    // gate/up sets also get a copy of the scales folded with the per-row multiplier
+    std::vector<int64_t> sc_offs(set->n_experts, 0);
+    if (role == ROLE_GATE_UP) {
+        int64_t total_scale = 0;
+        for (int e = 0; e < set->n_experts; ++e) {
+            sc_offs[e] = total_scale;
+            total_scale += (set->descs[e].scale_len + 127) / 128 * 128;    // keep every expert 256-byte aligned
+        }
+        int64_t* d_offs = nullptr;
+        BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_scale_s, (size_t)std::max<int64_t>(total_scale, 1) * 2));
+        BITSMOE_HIP_TRY(hipMalloc((void**)&d_offs, sizeof(int64_t) * set->n_experts));
+        BITSMOE_HIP_TRY(hipMemcpyAsync(d_offs, sc_offs.data(), sizeof(int64_t) * set->n_experts, hipMemcpyHostToDevice, st));
+        hipLaunchKernelGGL(k_fold_scale_s, dim3((unsigned)set->total_slabs, set->n_tiles), dim3(64), 0, st, set->d_views,
+                           set->d_slab_tasks, d_offs, set->d_scale_s);
+        const hipError_t launch_err = hipGetLastError();
+        const hipError_t sync_err = hipStreamSynchronize(st);
+        (void)hipFree(d_offs);
+        BITSMOE_HIP_TRY(launch_err);
+        BITSMOE_HIP_TRY(sync_err);
+    }
     std::vector<FastExpert> fexp(set->n_experts);
     for (int e = 0; e < set->n_experts; ++e) {
         FastExpert& f = fexp[e];
         memset(&f, 0, sizeof(f));
+        f.scale_s = set->d_scale_s ? set->d_scale_s + sc_offs[e] : nullptr;
         f.payload = set->d_prepared + offs[e];
         f.scale = (const __half*)set->descs[e].scale;
         f.s = (const __half*)set->descs[e].s;

@@ -70,13 +70,16 @@ def test_routing_tables_bit_exact(cuda_device, tokens, top_k, n_global, n_super,
 
 
 def _forward_case(cuda_device, seed, n_experts, tokens, top_k, rank_in, rank_out, dim, dtype_name, choices,
-                  path=None, tol=1e-2, uniform_bits=False, slab_multiple=None):
+                  path=None, tol=1e-2, uniform_bits=False, slab_multiple=None, scramble_ranks=False):
     import torch
 
     hip = _hip()
     rng = np.random.default_rng(seed)
     gate, up, down = helpers.make_experts(seed, n_experts, rank_in, rank_out, dim, choices=choices,
                                           uniform_bits=uniform_bits, slab_multiple=slab_multiple)
+    if scramble_ranks:       # rows of gate / up read arbitrary columns of h instead of runs of eight
+        for m in gate + up:
+            m["rank_idx"] = rng.permutation(rank_in).astype(np.int32)[m["rank_idx"]]
     dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
     h_gate = torch.from_numpy(rng.normal(size=(tokens, rank_in)).astype(np.float32)).to(dt)
     h_up = torch.from_numpy(rng.normal(size=(tokens, rank_in)).astype(np.float32)).to(dt)
@@ -242,6 +245,16 @@ def test_forward_mfma_path(cuda_device, shape, dtype_name):
                         path=_capi.PATH_MFMA, tol=1e-2, uniform_bits=False, slab_multiple=64)
     print(f"mfma {shape} {dtype_name}: err {err:.2e}")
     assert err < 3e-3      # f16 operands: well inside the 1e-2 bar
+
+
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+def test_forward_mfma_path_scattered_ranks(cuda_device, dtype_name):
+    """rank_idx without runs of eight consecutive ranks: the activations are gathered first."""
+    from bitsmoe_amd.algorithms import _capi
+
+    err = _forward_case(cuda_device, 311, 3, 260, 2, 192, 128, 256, dtype_name, (2, 3, 4),
+                        path=_capi.PATH_MFMA, tol=1e-2, slab_multiple=64, scramble_ranks=True)
+    assert err < 3e-3
 
 
 def test_forward_mfma_path_needs_prepared_sets(cuda_device):
