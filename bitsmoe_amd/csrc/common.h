@@ -45,7 +45,7 @@ struct FastExpert {
     const __half* s;
     const int32_t* rank_idx;
     int32_t num_slabs;
-    int32_t pad0;
+    int32_t uniform_bits;      // the bit-width every slab of this expert shares, or 0
     const __half* scale_s;     // gate/up sets: scale[tile][row] * s[row], same offsets as `scale`
     int32_t pad[4];            // 64 bytes
 };

@@ -218,15 +218,19 @@ __device__ inline void zero_acc(f32x4 (&acc)[4][4]) {
 }
 
 // ------------------------------------------------------------------------------ gate / up
-// Everything one thread fetches from global memory for one slab of one projection.
+constexpr int GU_SETS = 4;   // register sets of fetched slabs: loads run GU_SETS - 1 slabs ahead of the MFMAs
+
+// Everything one thread fetches from global memory for one slab.
 struct GuFetch {
     APiece a;          // this thread's part of the 128 x 64 activation piece
     u32x4 sc;          // scale pairs of contraction rows 8*(tid%8) .. +7 of the slab (tile t)
     uint32_t bw[2][4]; // payload words of the wavefront's two column-block pairs
 };
 
-// One slab (64 contraction rows, `bits` wide) of one projection for a wavefront's 64 x 64 tile;
-// the weight operand is the raw (2^bits + code), the scale already sits in the activations.
+// One slab (64 contraction rows, `bits` wide) for a wavefront's 64 x 64 tile; the weight
+// operand is the raw (2^bits + code), the scale already sits in the activations.
+// WU != 0: the width is a compile-time constant (experts whose slabs all share it).
+template <int WU>
 __device__ inline void gateup_slab_mfma(int bits, const uint16_t* __restrict__ stage, const uint32_t (&bw)[2][4], int wm,
                                         int lane, f32x4 (&acc)[4][4]) {
     const int n = lane & 15, kg = lane >> 4;
@@ -240,12 +244,12 @@ __device__ inline void gateup_slab_mfma(int bits, const uint16_t* __restrict__ s
         for (int nb = 0; nb < 4; ++nb) {
             const uint32_t(&w)[4] = bw[nb >> 1];
             const int nbl = nb & 1;
-            // the width switch wraps the decode of one operand only, so that the accumulators do not
-            // flow through alternative paths (which multiplies the register demand)
+            // WU == 0: the width switch wraps the decode of one operand only, so that the accumulators
+            // do not flow through alternative paths (which multiplies the register demand)
             u32x4 b;
-            if (bits == 2)
+            if (WU == 2 || (WU == 0 && bits == 2))
                 b = decode_fields2<2, false>(w[nbl], 8 * ks);
-            else if (bits == 4)
+            else if (WU == 4 || (WU == 0 && bits == 4))
                 b = decode_fields4<false>(w[2 * nbl + ks]);
             else
                 b = decode_fields3<false>(w[nbl], 8 * ks, w[2 + nbl], 8 * (n >> 3) + 4 * ks);
@@ -255,37 +259,26 @@ __device__ inline void gateup_slab_mfma(int bits, const uint16_t* __restrict__ s
     }
 }
 
-// grid.x = 8 * ceil(max_mtiles * n_tiles / 8); workgroup = (assignment tile, 128-column tile),
-// gate then up for the same output tile, then z = silu(G) * U.
+// One workgroup = (assignment tile, projection, 128-column tile): out[a, c] = f16 of
+// sum_k A[a, k] * level[k, c] * scale[tile(c), k] over all slabs of the expert's matrix.
 //
 // Per slab the staging threads multiply their part of the activation piece by the slab's
 // per-row scale of this tile (packed f16), write it to LDS and keep a running sum of what they
 // wrote, weighted with 1.5 * 2^W: sum_k A'[a,k] * (2^W + code) - 1.5 * 2^W * sum_k A'[a,k] is the
-// dot product with the true levels code - 2^(W-1).  Loads run two slabs ahead of the MFMAs in
-// two alternating register sets.
+// dot product with the true levels code - 2^(W-1).  Global loads run GU_SETS - 1 slabs ahead of
+// the MFMAs in rotating register sets (one memory round trip is several times longer than the
+// MFMAs of one slab).
 //
 // DIRECT: the activation rows are read straight from the f16 activations [T, ld] through the
 // token index (possible when every aligned run of 8 local rows is 8 consecutive logical ranks);
-// the per-row multiplier s is then taken from the folded scale table.  Otherwise Hs_* are the
-// pre-gathered rows [A, ld].
-template <bool DIRECT>
-__global__ __launch_bounds__(256, 2) void k_gateup_mfma(
-    const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
-    const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
-    const uint16_t* __restrict__ Hs_g, const uint16_t* __restrict__ Hs_u, int ldg, int ldu,
-    const int32_t* __restrict__ token_indices, int T,
-    const MTile* __restrict__ mtiles, const int32_t* __restrict__ n_mtiles, int I, int n_tiles,
-    uint16_t* __restrict__ z) {
-    __shared__ __attribute__((aligned(16))) uint16_t lds[2][PF_M * PF_LDS_ROW];
-    __shared__ float rowsum[2][PF_M];
-    const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles) * n_tiles);
-    if (logical < 0) return;
-    const int mt_i = logical / n_tiles, t = logical - mt_i * n_tiles;
-    const i32x4 tv = *reinterpret_cast<const i32x4*>(mtiles + mt_i);
-    const int e = __builtin_amdgcn_readfirstlane(tv[0]);
-    const int a_begin = __builtin_amdgcn_readfirstlane(tv[1]);
-    const int rows = __builtin_amdgcn_readfirstlane(tv[2]);
-    if (e < 0 || rows <= 0) return;
+// the per-row multiplier s is then taken from the folded scale table.  Otherwise Hs is the
+// pre-gathered [A, ld].  WU: the bit-width shared by every slab of the matrix, or 0 (mixed).
+template <bool DIRECT, int WU>
+__device__ inline void gateup_tile_body(const FastExpert fe, const FastSlab* __restrict__ fs_row, int nslabs,
+                                        const uint16_t* __restrict__ Hs, int ld,
+                                        const int32_t* __restrict__ token_indices, int T, int I,
+                                        uint16_t* __restrict__ out, int a_begin, int rows, int t,
+                                        uint16_t (*lds)[PF_M * PF_LDS_ROW], float* __restrict__ rowsum) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -300,110 +293,103 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int tk = token_indices[a_begin + min((tid >> 3) + 32 * j, rows - 1)];
-            rowbase[j] = (uint32_t)((tk >= 0 && tk < T) ? tk : 0);
+            rowbase[j] = (uint32_t)((tk >= 0 && tk < T) ? tk : 0) * (uint32_t)ld;
         }
     }
 
-    f32x4 accg[4][4], accu[4][4];
-    zero_acc(accg);
-    zero_acc(accu);
-
-    auto run = [&](const FastExpert* __restrict__ fe_tab, const FastSlab* __restrict__ fs_tab, int max_slabs,
-                   const uint16_t* __restrict__ Hs, int ld, int proj, f32x4(&acc)[4][4]) {
-        const FastExpert fe = fe_tab[e];
-        const int nslabs = __builtin_amdgcn_readfirstlane(min(fe.num_slabs, max_slabs));
-        gptr<uint32_t> payload = as_global(fe.payload);
-        gptr<__half> scale = as_global(DIRECT ? fe.scale_s : fe.scale);
-        gptr<int32_t> rank_idx = as_global(fe.rank_idx);
-        const FastSlab* __restrict__ fs_row = fs_tab + (int64_t)e * max_slabs;
-        GuFetch f[2];
-        FastSlab fs[3];          // records of slabs s, s+1, s+2 (rotating)
-        int rb[3] = {0, 0, 0};   // DIRECT: logical rank of this thread's first column in those slabs
-        float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        auto slab_rec = [&](int s) { return s < nslabs ? load_fast_slab(fs_row, s) : FastSlab{0, 0, 0, 0}; };
-        auto rank_base = [&](int s) { return (DIRECT && s < nslabs) ? rank_idx[s * SLAB_ROWS + (tid & 7) * 8] : 0; };
-        auto issue = [&](GuFetch& dst, const FastSlab& r, int rbase, int s) {
-            if constexpr (DIRECT) {
+    f32x4 acc[4][4];
+    zero_acc(acc);
+    gptr<uint32_t> payload = as_global(fe.payload);
+    gptr<__half> scale = as_global(DIRECT ? fe.scale_s : fe.scale);
+    gptr<int32_t> rank_idx = as_global(fe.rank_idx);
+    GuFetch f[GU_SETS];
+    int bits_of[GU_SETS];      // width of the slab held by each set
+    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto slab_rec = [&](int s) { return s < nslabs ? load_fast_slab(fs_row, s) : FastSlab{0, 0, 0, 0}; };
+    auto rank_base = [&](int s) { return (DIRECT && s < nslabs) ? rank_idx[s * SLAB_ROWS + (tid & 7) * 8] : 0; };
+    auto issue = [&](GuFetch& dst, const FastSlab& r, int rbase, int s) {
+        const int wb = WU != 0 ? WU : r.bits;
+        if constexpr (DIRECT) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    dst.a.v[j] = *reinterpret_cast<const u32x4*>(Hs + (rowbase[j] * (uint32_t)ld + (uint32_t)rbase));
-            } else {
-                load_piece(Hs, ld, a_begin, rows, s * SLAB_ROWS, tid, dst.a);
-            }
-            dst.sc = *reinterpret_cast<gptr_u32x4>(scale + (uint32_t)(r.scale_off + t * SLAB_ROWS + (tid & 7) * 8));
-            gptr<uint32_t> blk = payload + (uint32_t)(r.pack_off + t * 256 * r.bits);
-#pragma unroll
-            for (int p = 0; p < 2; ++p) {
-                const int pair = 2 * wn + p;
-                load_pair_role0(blk, r.bits, (uint32_t)(pair * 64 + lane), (uint32_t)hi_index0(kg, n, 2 * pair), dst.bw[p]);
-            }
-        };
-        // scale the fetched piece, add its weighted row sums, write it to an LDS stage
-        auto stage_piece = [&](GuFetch& src, int bits, uint16_t* __restrict__ stage) {
-            const uint32_t cw = bits == 2 ? Codec<2, false>::CORR : bits == 3 ? Codec<3, false>::CORR : Codec<4, false>::CORR;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const uint32_t scaled = pk_mul_f16(src.a.v[j][i], src.sc[i]);
-                    src.a.v[j][i] = scaled;
-                    sum[j] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, scaled), __builtin_bit_cast(h2, cw), sum[j], false);
-                }
-            }
-            store_piece(stage, tid, src.a);
-        };
-        auto compute = [&](int bits, const uint16_t* __restrict__ stage, const uint32_t(&bw)[2][4]) {
-            if (active && bits != 0) gateup_slab_mfma(bits, stage, bw, wm, lane, acc);
-        };
-        if (nslabs > 0) {
-            fs[0] = slab_rec(0);
-            fs[1] = slab_rec(1);
-            fs[2] = slab_rec(2);
-            rb[0] = rank_base(0);
-            rb[1] = rank_base(1);
-            rb[2] = rank_base(2);
-            issue(f[0], fs[0], rb[0], 0);
-            if (nslabs > 1) issue(f[1], fs[1], rb[1], 1);
-            stage_piece(f[0], fs[0].bits, lds[0]);
-            __syncthreads();
-            // one step: slab s is in LDS stage s % 2 and its words in set X; slab s + 1 is in flight in set Y
-            auto step = [&](int s, GuFetch& X, GuFetch& Y) {
-                uint32_t bw[2][4];
-#pragma unroll
-                for (int p = 0; p < 2; ++p)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) bw[p][i] = X.bw[p][i];
-                const int bits = fs[0].bits;
-                fs[0] = fs[1];
-                fs[1] = fs[2];
-                fs[2] = slab_rec(s + 3);
-                rb[0] = rb[1];
-                rb[1] = rb[2];
-                rb[2] = rank_base(s + 3);
-                if (s + 2 < nslabs) issue(X, fs[1], rb[1], s + 2);
-                compute(bits, lds[s & 1], bw);
-                if (s + 1 < nslabs) stage_piece(Y, fs[0].bits, lds[(s + 1) & 1]);
-                __syncthreads();
-            };
-            for (int s = 0; s < nslabs; s += 2) {
-                step(s, f[0], f[1]);
-                if (s + 1 < nslabs) step(s + 1, f[1], f[0]);
-            }
+            for (int j = 0; j < 4; ++j)
+                dst.a.v[j] = *reinterpret_cast<const u32x4*>(Hs + (rowbase[j] + (uint32_t)rbase));
+        } else {
+            load_piece(Hs, ld, a_begin, rows, s * SLAB_ROWS, tid, dst.a);
         }
-        // row sums: the eight threads that share a row hold its eight 8-column parts
+        dst.sc = *reinterpret_cast<gptr_u32x4>(scale + (uint32_t)(r.scale_off + t * SLAB_ROWS + (tid & 7) * 8));
+        gptr<uint32_t> blk = payload + (uint32_t)(r.pack_off + t * 256 * wb);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            float v = sum[j];
-            v += __shfl_xor(v, 1);
-            v += __shfl_xor(v, 2);
-            v += __shfl_xor(v, 4);
-            if ((tid & 7) == 0) rowsum[proj][(tid >> 3) + 32 * j] = v;
+        for (int p = 0; p < 2; ++p) {
+            const int pair = 2 * wn + p;
+            load_pair_role0(blk, wb, (uint32_t)(pair * 64 + lane), (uint32_t)hi_index0(kg, n, 2 * pair), dst.bw[p]);
         }
     };
-    run(gate_fe, gate_fs, gate_max_slabs, Hs_g, ldg, 0, accg);
-    run(up_fe, up_fs, up_max_slabs, Hs_u, ldu, 1, accu);
+    // scale the fetched piece, add its weighted row sums, write it to an LDS stage
+    auto stage_piece = [&](GuFetch& src, int bits, uint16_t* __restrict__ stage) {
+        const int wb = WU != 0 ? WU : bits;
+        const uint32_t cw = wb == 2 ? Codec<2, false>::CORR : wb == 3 ? Codec<3, false>::CORR : Codec<4, false>::CORR;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t scaled = pk_mul_f16(src.a.v[j][i], src.sc[i]);
+                src.a.v[j][i] = scaled;
+                sum[j] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, scaled), __builtin_bit_cast(h2, cw), sum[j], false);
+            }
+        }
+        store_piece(stage, tid, src.a);
+    };
+    if (nslabs > 0) {
+        // prologue: slabs 0 .. GU_SETS-2 go into sets 0 .. GU_SETS-2; slab 0 is staged
+        FastSlab pending = slab_rec(0);
+        int pending_rb = rank_base(0);
+        static_for([&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            if (q < nslabs) {
+                const FastSlab rec = pending;
+                const int rb = pending_rb;
+                pending = slab_rec(q + 1);
+                pending_rb = rank_base(q + 1);
+                bits_of[q] = rec.bits;
+                issue(f[q], rec, rb, q);
+            }
+        }, std::make_integer_sequence<int, GU_SETS - 1>{});
+        stage_piece(f[0], bits_of[0], lds[0]);
+        __syncthreads();
+        // step s (set q = s % GU_SETS): slab s is in LDS stage s % 2, its words in set q; the slab
+        // s + GU_SETS - 1 is requested into the set that slab s - 1 just left; slab s + 1 is staged.
+        for (int s0 = 0; s0 < nslabs; s0 += GU_SETS) {
+            static_for([&](auto qc) {
+                constexpr int q = decltype(qc)::value;
+                constexpr int q_issue = (q + GU_SETS - 1) % GU_SETS;
+                constexpr int q_next = (q + 1) % GU_SETS;
+                const int s = s0 + q;
+                if (s < nslabs) {
+                    if (s + GU_SETS - 1 < nslabs) {
+                        const FastSlab rec = pending;
+                        const int rb = pending_rb;
+                        pending = slab_rec(s + GU_SETS);
+                        pending_rb = rank_base(s + GU_SETS);
+                        bits_of[q_issue] = rec.bits;
+                        issue(f[q_issue], rec, rb, s + GU_SETS - 1);
+                    }
+                    if (active && bits_of[q] != 0) gateup_slab_mfma<WU>(bits_of[q], lds[s & 1], f[q].bw, wm, lane, acc);
+                    if (s + 1 < nslabs) stage_piece(f[q_next], bits_of[q_next], lds[(s + 1) & 1]);
+                    __syncthreads();
+                }
+            }, std::make_integer_sequence<int, GU_SETS>{});
+        }
+    }
+    // row sums: the eight threads that share a row hold its eight 8-column parts
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float v = sum[j];
+        v += __shfl_xor(v, 1);
+        v += __shfl_xor(v, 2);
+        v += __shfl_xor(v, 4);
+        if ((tid & 7) == 0) rowsum[(tid >> 3) + 32 * j] = v;
+    }
     __syncthreads();
-
     if (!active) return;
     // lane holds rows 64*wm + 16*mb + 4*kg + j, column 128*t + 64*wn + 16*nb + n
 #pragma unroll
@@ -412,14 +398,74 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
         for (int j = 0; j < 4; ++j) {
             const int row = 64 * wm + 16 * mb + 4 * kg + j;
             if (row >= rows) continue;
-            const float cg = rowsum[0][row], cu = rowsum[1][row];
-            uint16_t* zr = z + (int64_t)(a_begin + row) * I + N_TILE * t + 64 * wn + n;
+            const float c = rowsum[row];
+            uint16_t* dst = out + (int64_t)(a_begin + row) * I + N_TILE * t + 64 * wn + n;
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
-                const float v = silu_f32(accg[mb][nb][j] - cg) * (accu[mb][nb][j] - cu);
-                zr[16 * nb] = __builtin_bit_cast(uint16_t, (_Float16)v);
-            }
+            for (int nb = 0; nb < 4; ++nb) dst[16 * nb] = __builtin_bit_cast(uint16_t, (_Float16)(acc[mb][nb][j] - c));
         }
+}
+
+// grid.x = 8 * ceil(max_mtiles * 2 * n_tiles / 8); G and U are f16 [A, I].
+template <bool DIRECT>
+__global__ __launch_bounds__(256, 2) void k_gateup_mfma(
+    const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
+    const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
+    const uint16_t* __restrict__ Hs_g, const uint16_t* __restrict__ Hs_u, int ldg, int ldu,
+    const int32_t* __restrict__ token_indices, int T,
+    const MTile* __restrict__ mtiles, const int32_t* __restrict__ n_mtiles, int I, int n_tiles,
+    uint16_t* __restrict__ G, uint16_t* __restrict__ U) {
+    __shared__ __attribute__((aligned(16))) uint16_t lds[2][PF_M * PF_LDS_ROW];
+    __shared__ float rowsum[PF_M];
+    const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles) * 2 * n_tiles);
+    if (logical < 0) return;
+    // the column tiles of one (assignment tile, projection) are neighbours: they share the activations
+    const int t = logical % n_tiles;
+    const int proj = (logical / n_tiles) & 1;
+    const int mt_i = logical / (2 * n_tiles);
+    const i32x4 tv = *reinterpret_cast<const i32x4*>(mtiles + mt_i);
+    const int e = __builtin_amdgcn_readfirstlane(tv[0]);
+    const int a_begin = __builtin_amdgcn_readfirstlane(tv[1]);
+    const int rows = __builtin_amdgcn_readfirstlane(tv[2]);
+    if (e < 0 || rows <= 0) return;
+    const FastExpert fe = (proj ? up_fe : gate_fe)[e];
+    const int max_slabs = proj ? up_max_slabs : gate_max_slabs;
+    const FastSlab* __restrict__ fs_row = (proj ? up_fs : gate_fs) + (int64_t)e * max_slabs;
+    const int nslabs = __builtin_amdgcn_readfirstlane(min(fe.num_slabs, max_slabs));
+    const uint16_t* __restrict__ Hs = proj ? Hs_u : Hs_g;
+    const int ld = proj ? ldu : ldg;
+    uint16_t* __restrict__ out = proj ? U : G;
+    const int w = __builtin_amdgcn_readfirstlane(fe.uniform_bits);
+#define BITSMOE_GU_BODY(W) \
+    gateup_tile_body<DIRECT, W>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, out, a_begin, rows, t, lds, rowsum)
+    if (w == 2)
+        BITSMOE_GU_BODY(2);
+    else if (w == 3)
+        BITSMOE_GU_BODY(3);
+    else if (w == 4)
+        BITSMOE_GU_BODY(4);
+    else
+        BITSMOE_GU_BODY(0);
+#undef BITSMOE_GU_BODY
+}
+
+// z = f16( silu(G) * U ), written over G; 8 elements per thread and iteration.
+__global__ __launch_bounds__(256) void k_silu_mul_f16(uint16_t* __restrict__ G, const uint16_t* __restrict__ U, int64_t n8) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += (int64_t)gridDim.x * blockDim.x) {
+        const u32x4 g = *reinterpret_cast<const u32x4*>(G + i * 8);
+        const u32x4 u = *reinterpret_cast<const u32x4*>(U + i * 8);
+        u32x4 o;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float g0 = __half2float(__ushort_as_half((uint16_t)(g[k] & 0xFFFFu)));
+            const float g1 = __half2float(__ushort_as_half((uint16_t)(g[k] >> 16)));
+            const float u0 = __half2float(__ushort_as_half((uint16_t)(u[k] & 0xFFFFu)));
+            const float u1 = __half2float(__ushort_as_half((uint16_t)(u[k] >> 16)));
+            const uint32_t lo = __builtin_bit_cast(uint16_t, (_Float16)(silu_f32(g0) * u0));
+            const uint32_t hi = __builtin_bit_cast(uint16_t, (_Float16)(silu_f32(g1) * u1));
+            o[k] = lo | (hi << 16);
+        }
+        *reinterpret_cast<u32x4*>(G + i * 8) = o;
+    }
 }
 
 // ----------------------------------------------------------------------------------- down
@@ -618,7 +664,7 @@ size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up
     // the direct form falls back to the gathered one when the activation pointers or row
     // lengths do not allow 16-byte loads, which is only known at the call
     return align256((size_t)max_mtiles * sizeof(MTile)) + 256 + std::max(direct_ok(gate, up) ? direct : 0, gathered) +
-           align256((size_t)A * I * 2);
+           2 * align256((size_t)A * I * 2);
 }
 
 int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
@@ -640,8 +686,9 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     const uint16_t* Hs_g = (const uint16_t*)ws;
     ws += direct ? align256((size_t)T * direct_ld(gate) * 2) : align256((size_t)A * ldg * 2);
     const uint16_t* Hs_u = (const uint16_t*)ws;
-    ws = (char*)workspace + mfma_workspace_bytes(gate, up, T, A, I) - align256((size_t)A * I * 2);
-    uint16_t* z = (uint16_t*)ws;
+    ws = (char*)workspace + mfma_workspace_bytes(gate, up, T, A, I) - 2 * align256((size_t)A * I * 2);
+    uint16_t* z = (uint16_t*)ws;     // gate output, then silu(gate) * up in place
+    uint16_t* Ubuf = (uint16_t*)(ws + align256((size_t)A * I * 2));
 
     record(prof, 0, st);
     BITSMOE_REQUIRE(launch_fill_zero(rank_accum, T * (int64_t)rank_out, st) == BITSMOE_OK, "zero fill failed");
@@ -670,15 +717,19 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     }
     record(prof, 1, st);
     {
-        const int64_t wgs = (max_mtiles * n_tiles + 7) / 8 * 8;
+        const int64_t wgs = (max_mtiles * 2 * n_tiles + 7) / 8 * 8;
         if (direct)
             hipLaunchKernelGGL(k_gateup_mfma<true>, dim3((unsigned)wgs), dim3(256), 0, st, gate->d_fast_experts,
                                gate->d_fast_slabs, gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs,
-                               Hs_g, Hs_u, ldg, ldu, tok, (int)T, mtiles, n_mtiles, I, n_tiles, z);
+                               Hs_g, Hs_u, ldg, ldu, tok, (int)T, mtiles, n_mtiles, I, n_tiles, z, Ubuf);
         else
             hipLaunchKernelGGL(k_gateup_mfma<false>, dim3((unsigned)wgs), dim3(256), 0, st, gate->d_fast_experts,
                                gate->d_fast_slabs, gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs,
-                               Hs_g, Hs_u, ldg, ldu, tok, (int)T, mtiles, n_mtiles, I, n_tiles, z);
+                               Hs_g, Hs_u, ldg, ldu, tok, (int)T, mtiles, n_mtiles, I, n_tiles, z, Ubuf);
+        BITSMOE_HIP_TRY(hipGetLastError());
+        const int64_t n8 = A * (int64_t)I / 8;
+        hipLaunchKernelGGL(k_silu_mul_f16, dim3((unsigned)std::min<int64_t>((n8 + 255) / 256, 4096)), dim3(256), 0, st, z,
+                           Ubuf, n8);
         BITSMOE_HIP_TRY(hipGetLastError());
     }
     record(prof, 2, st);

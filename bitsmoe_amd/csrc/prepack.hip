@@ -260,6 +260,9 @@ extern "C" int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* s
         f.s = (const __half*)set->descs[e].s;
         f.rank_idx = (const int32_t*)set->descs[e].rank_idx;
         f.num_slabs = set->descs[e].num_slabs;
+        f.uniform_bits = f.num_slabs > 0 ? set->slab_meta_host[e][0] : 0;
+        for (int si = 1; si < f.num_slabs; ++si)
+            if (set->slab_meta_host[e][si * 4] != f.uniform_bits) f.uniform_bits = 0;
     }
     BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_fast_experts, sizeof(FastExpert) * fexp.size()));
     BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_fast_experts, fexp.data(), sizeof(FastExpert) * fexp.size(), hipMemcpyHostToDevice, st));
