@@ -218,7 +218,7 @@ __device__ inline void zero_acc(f32x4 (&acc)[4][4]) {
 }
 
 // ------------------------------------------------------------------------------ gate / up
-constexpr int GU_SETS = 4;   // register sets of fetched slabs: loads run GU_SETS - 1 slabs ahead of the MFMAs
+constexpr int GU_SETS = 3;   // register sets of fetched slabs: loads run GU_SETS - 1 slabs ahead of the MFMAs
 
 // Everything one thread fetches from global memory for one slab.
 struct GuFetch {
@@ -230,16 +230,26 @@ struct GuFetch {
 // One slab (64 contraction rows, `bits` wide) for a wavefront's 64 x 64 tile; the weight
 // operand is the raw (2^bits + code), the scale already sits in the activations.
 // WU != 0: the width is a compile-time constant (experts whose slabs all share it).
-template <int WU>
-__device__ inline void gateup_slab_mfma(int bits, const uint16_t* __restrict__ stage, const uint32_t (&bw)[2][4], int wm,
-                                        int lane, f32x4 (&acc)[4][4]) {
+// The activation operands of one slab for a wavefront: [ks][mb], read from an LDS stage.
+struct GuOperands {
+    u32x4 a[2][4];
+};
+__device__ inline void read_operands(const uint16_t* __restrict__ stage, int wm, int lane, GuOperands& o) {
     const int n = lane & 15, kg = lane >> 4;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-        u32x4 a[4];
+    for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb)
-            a[mb] = *reinterpret_cast<const u32x4*>(stage + (64 * wm + 16 * mb + n) * PF_LDS_ROW + 16 * kg + 8 * ks);
+            o.a[ks][mb] = *reinterpret_cast<const u32x4*>(stage + (64 * wm + 16 * mb + n) * PF_LDS_ROW + 16 * kg + 8 * ks);
+}
+
+template <int WU>
+__device__ inline void gateup_slab_mfma(int bits, const GuOperands& ops, const uint32_t (&bw)[2][4], int lane,
+                                        f32x4 (&acc)[4][4]) {
+    const int n = lane & 15;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        const u32x4(&a)[4] = ops.a[ks];
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
             const uint32_t(&w)[4] = bw[nb >> 1];
@@ -373,8 +383,14 @@ __device__ inline void gateup_tile_body(const FastExpert fe, const FastSlab* __r
                         bits_of[q_issue] = rec.bits;
                         issue(f[q_issue], rec, rb, s + GU_SETS - 1);
                     }
-                    if (active && bits_of[q] != 0) gateup_slab_mfma<WU>(bits_of[q], lds[s & 1], f[q].bw, wm, lane, acc);
+                    // the operand reads are requested first, so that their LDS round trip passes while
+                    // the next piece is scaled and written; the MFMAs then separate that write from
+                    // the barrier
+                    GuOperands ops;
+                    const bool mul = active && bits_of[q] != 0;
+                    if (mul) read_operands(lds[s & 1], wm, lane, ops);
                     if (s + 1 < nslabs) stage_piece(f[q_next], bits_of[q_next], lds[(s + 1) & 1]);
+                    if (mul) gateup_slab_mfma<WU>(bits_of[q], ops, f[q].bw, lane, acc);
                     __syncthreads();
                 }
             }, std::make_integer_sequence<int, GU_SETS>{});
