@@ -69,7 +69,7 @@ def algorithmic_work(block, counts, tokens, n_assign):
             "flops": flops, "flops_gateup": fl_gateup, "flops_down": flops - fl_gateup, "active_experts": len(active)}
 
 
-def run_workload(block, spec, tokens, steps, warmup, seed=42):
+def run_workload(block, spec, tokens, steps, warmup, seed=42, use_graph=True):
     import torch
 
     from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
@@ -97,12 +97,52 @@ def run_workload(block, spec, tokens, steps, warmup, seed=42):
     for _ in range(max(warmup, 1)):
         tok, off, rw, out = step()
     torch.cuda.synchronize(dev)
-    profiles = [hip.Profile() for _ in range(steps)]
+    # (1) eager launches, no instrumentation: what a caller of the operator sees per call
     t0 = time.perf_counter()
+    for i in range(steps):
+        step()
+    torch.cuda.synchronize(dev)
+    eager = time.perf_counter() - t0
+    # (2) the same steps with HIP events between the kernels (per-kernel durations for the roofline)
+    profiles = [hip.Profile() for _ in range(steps)]
     for i in range(steps):
         step(profiles[i])
     torch.cuda.synchronize(dev)
-    elapsed = time.perf_counter() - t0
+    # (3) the step captured once into a HIP graph and replayed: the operator never allocates or
+    # synchronises, so a serving loop can drop the per-launch host cost this way
+    elapsed, launch, graph_ms = eager, "eager", None
+    if use_graph:
+        try:
+            graph = torch.cuda.CUDAGraph()
+            side = torch.cuda.Stream(device=dev)
+            side.wait_stream(torch.cuda.current_stream(dev))
+            with torch.cuda.stream(side):
+                step()
+            torch.cuda.current_stream(dev).wait_stream(side)
+            torch.cuda.synchronize(dev)
+            with torch.cuda.graph(graph):
+                g_tok, g_off, g_rw, g_out = step()
+            # every replay must reproduce the eager result (fp32 atomics: summation order may differ)
+            for _ in range(3):
+                graph.replay()
+                torch.cuda.synchronize(dev)
+                ref_out = step()[3]
+                torch.cuda.synchronize(dev)
+                if not torch.allclose(g_out, ref_out, rtol=1e-4, atol=1e-5 * float(ref_out.abs().max())):
+                    raise RuntimeError("graph replay differs from the eager result")
+            for _ in range(max(warmup, 1)):
+                graph.replay()
+            torch.cuda.synchronize(dev)
+            t0 = time.perf_counter()
+            for i in range(steps):
+                graph.replay()
+            torch.cuda.synchronize(dev)
+            replay = time.perf_counter() - t0
+            if replay < eager:       # large steps hide the launch cost anyway and replay has its own
+                elapsed, launch = replay, "hipgraph"
+            graph_ms = replay / steps * 1e3
+        except Exception as exc:   # noqa: BLE001 - the eager figure stands
+            print(f"bench.py: graph replay unavailable ({exc}); reporting eager launches", file=sys.stderr)
     phases = [p.read() for p in profiles]
     ms_fill = sum(p[0] for p in phases) / steps
     ms_gateup = sum(p[1] for p in phases) / steps
@@ -111,6 +151,7 @@ def run_workload(block, spec, tokens, steps, warmup, seed=42):
     work = algorithmic_work(block, counts, tokens, int(tok.numel()))
     res = {
         "tokens": tokens, "ms_per_step": elapsed / steps * 1e3, "tokens_per_s": tokens * steps / elapsed,
+        "launch": launch, "eager_ms_per_step": eager / steps * 1e3, "hipgraph_ms_per_step": graph_ms,
         "kernel_ms": {"zero_fill": ms_fill, "gate_up": ms_gateup, "down": ms_down},
         "active_experts": work["active_experts"], "algorithmic_bytes": work["bytes_total"],
         "algorithmic_flops": work["flops"],
@@ -196,6 +237,7 @@ def main() -> int:
     ap.add_argument("--workload", default="c2-t64", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extras", action="store_true", help="measure the primary workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches only (no HIP graph replay)")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run 5 plain fp32 copies (torch.mul(src, 1, out=dst)) of this many MiB: the known-size "
                          "kernel that hardware byte counters are scaled by")
@@ -220,7 +262,7 @@ def main() -> int:
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
 
-    res, inputs = run_workload(block, SPECS[spec_key], tokens, args.steps, args.warmup)
+    res, inputs = run_workload(block, SPECS[spec_key], tokens, args.steps, args.warmup, use_graph=not args.no_graph)
     roof = roofline_of(res, inputs, bound)
     if args.copy_probe_mib > 0:
         n = args.copy_probe_mib * (1 << 20) // 4
@@ -239,7 +281,8 @@ def main() -> int:
             if name == args.workload:
                 continue
             # c2 and c3 are the same layer (same seed, shape and bit draw); only routing differs
-            r, inp = run_workload(block, SPECS[skey], toks, max(5, args.steps // 2), max(2, args.warmup // 2))
+            r, inp = run_workload(block, SPECS[skey], toks, max(5, args.steps // 2), max(2, args.warmup // 2),
+                                  use_graph=not args.no_graph)
             r["roofline"] = roofline_of(r, inp, bnd)
             extras[name] = r
     bits = block.expert_bits
@@ -250,7 +293,9 @@ def main() -> int:
         "config": {"workload": f"{args.workload}: {WORKLOAD_DESC[spec_key]}, {tokens} tokens, operator scope "
                                "(routing kernel + gate/up + SiLU*mul + down + combine), inputs resident in HBM",
                    "tokens": tokens, "mean_bits": sum(bits) / len(bits), "active_experts": res["active_experts"],
-                   "device": get_cuda_device_name(), "layer_build_s": round(build_s, 2)},
+                   "device": get_cuda_device_name(), "layer_build_s": round(build_s, 2),
+                   "launch": res["launch"]},
+        "eager_ms_per_step": res["eager_ms_per_step"], "hipgraph_ms_per_step": res["hipgraph_ms_per_step"],
         "kernel_ms": res["kernel_ms"], "algorithmic_bytes": res["algorithmic_bytes"],
         "algorithmic_flops": res["algorithmic_flops"],
         "roofline": roof, "cpu_baseline": cpu, "parity": parity, "extras": extras,

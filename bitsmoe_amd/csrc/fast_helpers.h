@@ -36,7 +36,7 @@ __device__ inline FastSlab load_fast_slab(const FastSlab* __restrict__ tab, int 
 // The words of one wavefront's column-block pair for one (slab, tile) block: 2-bit {nb0, nb1};
 // 4-bit {nb0 j0, nb0 j1, nb1 j0, nb1 j1}; 3-bit {low nb0, low nb1, high nb0, high nb1}.
 // `blk` is wave-uniform, `unit` = pair*64 + lane and `hi_unit` are 32-bit lane offsets.
-__device__ inline void load_pair_role0(gptr<uint32_t> blk, int bits, uint32_t unit, uint32_t hi_unit, uint32_t (&w)[4]) {
+__device__ __forceinline__ void load_pair_role0(gptr<uint32_t> blk, int bits, uint32_t unit, uint32_t hi_unit, uint32_t (&w)[4]) {
     if (bits == 4) {
         const u32x4 v = *reinterpret_cast<gptr_u32x4>(blk + unit * 4u);
         w[0] = v[0]; w[1] = v[1]; w[2] = v[2]; w[3] = v[3];
@@ -56,7 +56,7 @@ struct Block16 {   // up to 16 payload words of one lane for one (slab, tile) bl
 
 // role 1 loads: 2-bit 8 words [nb][h], 4-bit 16 words [nb][m], 3-bit 8 low words + 4 high words [nb]
 template <int W>
-__device__ inline void load_block_role1(gptr<uint32_t> blk, int lane, Block16& b) {
+__device__ __forceinline__ void load_block_role1(gptr<uint32_t> blk, int lane, Block16& b) {
     gptr_u32x4 p = reinterpret_cast<gptr_u32x4>(blk + (W == 4 ? lane * 16 : lane * 8));
     u32x4 v0 = p[0], v1 = p[1], v2 = {0, 0, 0, 0}, v3 = {0, 0, 0, 0};
     if constexpr (W == 4) {

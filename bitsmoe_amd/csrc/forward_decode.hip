@@ -43,11 +43,33 @@ __device__ inline u32x4 corr_operand() {
     return r;
 }
 
+// With few assignments most experts are idle; launching a workgroup per (expert, ...) then
+// costs more than the work.  The kernels can instead be launched over `slots` and let every
+// workgroup find the slot-th ACTIVE expert (non-empty assignment range) itself: one
+// wave-parallel pass over expert_offsets.  Returns -1 when fewer experts are active.
+__device__ inline int nth_active_expert(const int32_t* __restrict__ expert_offsets, int E, int A, int slot, int lane) {
+    int found = -1;
+    for (int e0 = 0; e0 < E && found < 0; e0 += 64) {
+        const int e = e0 + lane;
+        bool active = false;
+        if (e < E) active = min(expert_offsets[e + 1], A) > max(expert_offsets[e], 0);
+        const uint64_t mask = __ballot(active);
+        const int count = __popcll(mask);
+        if (slot < count) {
+            const int rank = __popcll(mask & ((1ull << lane) - 1ull));
+            const uint64_t hit = __ballot(active && rank == slot);
+            found = e0 + (int)__builtin_ctzll(hit);
+        }
+        slot -= count;
+    }
+    return __builtin_amdgcn_readfirstlane(found);
+}
+
 // ------------------------------------------------------------------------------ gate / up
 // One (slab, tile) block restricted to one column-block pair: 2 column blocks x 2 k-steps,
 // plus the two MFMAs that accumulate the constant term.
 template <int W, bool BF16>
-__device__ inline void gateup_pair(const uint32_t (&w)[4], u32x4 a0, u32x4 a1, int upper, f32x4 (&acc)[2], f32x4& corr) {
+__device__ __forceinline__ void gateup_pair(const uint32_t (&w)[4], u32x4 a0, u32x4 a1, int upper, f32x4 (&acc)[2], f32x4& corr) {
     const u32x4 bc = corr_operand<W, BF16>();
     corr = mfma16<BF16>(a0, bc, corr);
     corr = mfma16<BF16>(a1, bc, corr);
@@ -80,19 +102,24 @@ __device__ inline void gateup_pair(const uint32_t (&w)[4], u32x4 a0, u32x4 a1, i
 // GENERAL == false: only the width-specialised bodies (groups of eight equal-width slabs that
 // follow each other in the payload); GENERAL == true: only the groups those skip.  Two kernels
 // instead of one keep the register budget of the common case free of the general body.
-template <bool BF16, bool GENERAL>
+// COMPACT: the expert coordinate of the grid counts active experts (see nth_active_expert).
+template <bool BF16, bool GENERAL, bool COMPACT>
 __global__ __launch_bounds__(256) void k_gateup_decode(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
     const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
     const uint16_t* __restrict__ h_gate, const uint16_t* __restrict__ h_up, int Rg, int Ru,
     const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
-    int n_tiles, int n_groups, int n_tchunks, int tiles_per_wg, float* __restrict__ G, float* __restrict__ U) {
+    int E, int n_tiles, int n_groups, int n_tchunks, int tiles_per_wg, float* __restrict__ G, float* __restrict__ U) {
     const int mt = blockIdx.y;
     const int bid = blockIdx.x;
     const int tchunk = bid % n_tchunks;
     const int grp = (bid / n_tchunks) % n_groups;
-    const int e = bid / (n_tchunks * n_groups);
     const int tid = threadIdx.x;
+    int e = bid / (n_tchunks * n_groups);
+    if constexpr (COMPACT) {
+        e = nth_active_expert(expert_offsets, E, A, e, tid & 63);
+        if (e < 0) return;
+    }
     const int pair = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform
     const int lane = tid & 63;
     const int n = lane & 15, kg = lane >> 4;
@@ -301,7 +328,7 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
 // ----------------------------------------------------------------------------------- down
 // One (slab, tile) block of a down matrix: 4 row blocks x 4 k-steps (micro-tiles).
 template <int W, bool BF16>
-__device__ inline void down_block(const Block16& b, const u32x4 (&az)[4], const float (&sc)[4], f32x4 (&acc)[4]) {
+__device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4], const float (&sc)[4], f32x4 (&acc)[4]) {
     const u32x4 bc = corr_operand<W, BF16>();
     f32x4 corr = {0, 0, 0, 0};
 #pragma unroll
@@ -330,10 +357,10 @@ __device__ inline void down_block(const Block16& b, const u32x4 (&az)[4], const 
 // are in flight while G and U are read and SiLU is evaluated; afterwards the tiles stream
 // through three register buffers, two tiles ahead of the one being computed.
 template <int W, bool BF16>
-__device__ inline void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gptr<__half> svec, gptr<int32_t> rank_idx,
+__device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gptr<__half> svec, gptr<int32_t> rank_idx,
                                  const FastSlab fs, const float* __restrict__ G, const float* __restrict__ U,
                                  const float* __restrict__ route_w, const int32_t* __restrict__ token_indices,
-                                 int a_begin, int a_end, int T, int I, int n_tiles, int rank_out,
+                                 int a_begin, int a_end, int T, int I, int tb, int nt, int rank_out,
                                  float* __restrict__ rank_accum, uint16_t* __restrict__ z, int z_stride, int tid, int lane) {
     const int n = lane & 15, kg = lane >> 4, g4 = kg * 4;
     using I0 = std::integral_constant<int, 0>;
@@ -349,17 +376,19 @@ __device__ inline void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gpt
         f32x4 acc[4];
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) acc[nb] = f32x4{0, 0, 0, 0};
-        auto issue = [&](auto b_c, int t) {
+        // the workgroup's tiles are tb .. tb + nt - 1; `i` counts from 0
+        auto issue = [&](auto b_c, int i) {
             constexpr int B = decltype(b_c)::value;
+            const int t = tb + i;
             load_block_role1<WL>(payload + (uint32_t)(fs.pack_off + (t + chunk_zero) * 256 * WL), lane, buf[B]);
             gptr<__half> sp = scale + (uint32_t)(fs.scale_off + t * SLAB_ROWS + n);
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) sc[B][nb] = gload_half(sp + 16 * nb);
         };
-        auto compute = [&](auto b_c, int t) {
+        auto compute = [&](auto b_c, int i) {
             constexpr int B = decltype(b_c)::value;
             u32x4 az[4];
-            const uint16_t* zp = z + n * z_stride + t * N_TILE + 8 * kg;
+            const uint16_t* zp = z + n * z_stride + (tb + i) * N_TILE + 8 * kg;
 #pragma unroll
             for (int m = 0; m < 4; ++m) az[m] = *reinterpret_cast<const u32x4*>(zp + 32 * m);
             down_block<WL, BF16>(buf[B], az, sc[B], acc);
@@ -368,7 +397,7 @@ __device__ inline void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gpt
         float sv[4];
         if constexpr (W != 0) {
             issue(I0{}, 0);
-            if (n_tiles > 1) issue(I1{}, 1);
+            if (nt > 1) issue(I1{}, 1);
             // logical rank and multiplier of this lane's four output rows (needed by the epilogue)
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) {
@@ -384,7 +413,7 @@ __device__ inline void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gpt
         // z[a][c] = silu(G) * U as 16-bit operands for the rows a < n_a (other rows feed
         // output rows that are never stored).  Each thread owns four neighbouring columns
         // and walks the assignments four at a time, all eight vector loads issued together.
-        for (int c = tid * 4; c < I; c += 1024) {
+        for (int c = tb * N_TILE + tid * 4; c < min((tb + nt) * N_TILE, I); c += 1024) {
             for (int ab = 0; ab < n_a; ab += 4) {
                 f32x4 gv[4], uv[4];
 #pragma unroll
@@ -409,16 +438,16 @@ __device__ inline void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gpt
         }
         __syncthreads();
         if constexpr (W != 0) {
-            for (int t = 0; t < n_tiles; t += 3) {
-                if (t + 2 < n_tiles) issue(I2{}, t + 2);
-                compute(I0{}, t);
-                if (t + 1 < n_tiles) {
-                    if (t + 3 < n_tiles) issue(I0{}, t + 3);
-                    compute(I1{}, t + 1);
+            for (int i = 0; i < nt; i += 3) {
+                if (i + 2 < nt) issue(I2{}, i + 2);
+                compute(I0{}, i);
+                if (i + 1 < nt) {
+                    if (i + 3 < nt) issue(I0{}, i + 3);
+                    compute(I1{}, i + 1);
                 }
-                if (t + 2 < n_tiles) {
-                    if (t + 4 < n_tiles) issue(I1{}, t + 4);
-                    compute(I2{}, t + 2);
+                if (i + 2 < nt) {
+                    if (i + 4 < nt) issue(I1{}, i + 4);
+                    compute(I2{}, i + 2);
                 }
             }
             // combine: rows of this slab are distinct output ranks; lane holds assignments 4*kg + j
@@ -437,16 +466,23 @@ __device__ inline void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gpt
     }
 }
 
-// grid.x = E * n_groups; 256 threads; dynamic LDS = 16 * (n_tiles * 128 + 8) * 2 bytes.
-template <bool BF16>
+// grid.x = E * n_groups * n_tchunks; 256 threads; dynamic LDS = 16 * (n_tiles * 128 + 8) * 2 bytes.
+// A workgroup takes four slabs of one expert and a run of tiles; with few active experts the
+// tiles are split over several workgroups (their partial sums meet in the atomics of the combine).
+template <bool BF16, bool COMPACT>
 __global__ __launch_bounds__(256) void k_down_decode(
     const FastExpert* __restrict__ down_fe, const FastSlab* __restrict__ down_fs, int max_slabs,
     const float* __restrict__ G, const float* __restrict__ U, const float* __restrict__ route_w,
     const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
-    int n_tiles, int n_groups, int rank_out, float* __restrict__ rank_accum) {
-    const int grp = blockIdx.x % n_groups;
-    const int e = blockIdx.x / n_groups;
+    int E, int n_tiles, int n_groups, int n_tchunks, int tiles_per_wg, int rank_out, float* __restrict__ rank_accum) {
+    const int tchunk = blockIdx.x % n_tchunks;
+    const int grp = (blockIdx.x / n_tchunks) % n_groups;
+    const int e_slot = blockIdx.x / (n_tchunks * n_groups);
     const int tid = threadIdx.x;
+    const int e = COMPACT ? nth_active_expert(expert_offsets, E, A, e_slot, tid & 63) : e_slot;
+    if (COMPACT && e < 0) return;
+    const int tb = tchunk * tiles_per_wg;
+    const int nt = min(tiles_per_wg, n_tiles - tb);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int si = grp * DN_SLABS_PER_WG + wave;
@@ -470,16 +506,16 @@ __global__ __launch_bounds__(256) void k_down_decode(
     // the four wavefronts may run four different instantiations; every one of them executes
     // the same two workgroup barriers per assignment chunk
     if (fs.bits == 2)
-        down_wave<2, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, n_tiles,
+        down_wave<2, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, tid, lane);
     else if (fs.bits == 3)
-        down_wave<3, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, n_tiles,
+        down_wave<3, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, tid, lane);
     else if (fs.bits == 4)
-        down_wave<4, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, n_tiles,
+        down_wave<4, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, tid, lane);
     else
-        down_wave<0, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, n_tiles,
+        down_wave<0, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, tid, lane);
 }
 
@@ -523,38 +559,56 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     // Tiles per workgroup: long runs amortise the start-up round trips, but the grid must
     // still hold a few workgroups per CU.  At most min(E, A) experts can be active.
     const int64_t active_max = std::min<int64_t>(E, A);
+    // few assignments: launch over the experts that can be active at most, not over all of them
+    const bool compact = active_max * 2 <= E;
+    const int e_dim = compact ? (int)active_max : E;
     int tiles_per_wg = n_tiles;
     while (tiles_per_wg > 1 && active_max * 2 * gu_groups * ((n_tiles + tiles_per_wg - 1) / tiles_per_wg) < 2048)
         tiles_per_wg = (tiles_per_wg + 1) / 2;
     const int n_tchunks = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
-    dim3 grid((unsigned)(E * gu_groups * n_tchunks), 2);
+    dim3 grid((unsigned)(e_dim * gu_groups * n_tchunks), 2);
     auto launch_gateup = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs, gate->max_slabs,
                            up->d_fast_experts, up->d_fast_slabs, up->max_slabs, (const uint16_t*)h_gate,
-                           (const uint16_t*)h_up, Rg, Ru, tok, off, (int)T, (int)A, I, n_tiles, gu_groups, n_tchunks,
+                           (const uint16_t*)h_up, Rg, Ru, tok, off, (int)T, (int)A, I, E, n_tiles, gu_groups, n_tchunks,
                            tiles_per_wg, G, U);
     };
     const bool need_general = !(gate->all_uniform8 && up->all_uniform8);
-    if (act_dtype == BITSMOE_DT_BF16) {
-        launch_gateup(k_gateup_decode<true, false>);
-        if (need_general) launch_gateup(k_gateup_decode<true, true>);
+    const bool bf16 = act_dtype == BITSMOE_DT_BF16;
+    if (bf16 && compact) {
+        launch_gateup(k_gateup_decode<true, false, true>);
+        if (need_general) launch_gateup(k_gateup_decode<true, true, true>);
+    } else if (bf16) {
+        launch_gateup(k_gateup_decode<true, false, false>);
+        if (need_general) launch_gateup(k_gateup_decode<true, true, false>);
+    } else if (compact) {
+        launch_gateup(k_gateup_decode<false, false, true>);
+        if (need_general) launch_gateup(k_gateup_decode<false, true, true>);
     } else {
-        launch_gateup(k_gateup_decode<false, false>);
-        if (need_general) launch_gateup(k_gateup_decode<false, true>);
+        launch_gateup(k_gateup_decode<false, false, false>);
+        if (need_general) launch_gateup(k_gateup_decode<false, true, false>);
     }
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 2, st);
     const int dn_groups = (down->max_slabs + DN_SLABS_PER_WG - 1) / DN_SLABS_PER_WG;
     const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2;
-    if (act_dtype == BITSMOE_DT_BF16) {
-        hipLaunchKernelGGL((k_down_decode<true>), dim3((unsigned)(E * dn_groups)), dim3(256), z_bytes, st,
-                           down->d_fast_experts, down->d_fast_slabs, down->max_slabs, G, U, rw, tok, off, (int)T, (int)A,
-                           I, n_tiles, dn_groups, rank_out, rank_accum);
-    } else {
-        hipLaunchKernelGGL((k_down_decode<false>), dim3((unsigned)(E * dn_groups)), dim3(256), z_bytes, st,
-                           down->d_fast_experts, down->d_fast_slabs, down->max_slabs, G, U, rw, tok, off, (int)T, (int)A,
-                           I, n_tiles, dn_groups, rank_out, rank_accum);
-    }
+    int dn_tiles_per_wg = n_tiles;
+    while (dn_tiles_per_wg > 1 && active_max * dn_groups * ((n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg) < 384)
+        dn_tiles_per_wg = (dn_tiles_per_wg + 1) / 2;
+    const int dn_tchunks = (n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg;
+    auto launch_down = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)(e_dim * dn_groups * dn_tchunks)), dim3(256), z_bytes, st,
+                           down->d_fast_experts, down->d_fast_slabs, down->max_slabs, G, U, rw, tok, off, (int)T, (int)A, I,
+                           E, n_tiles, dn_groups, dn_tchunks, dn_tiles_per_wg, rank_out, rank_accum);
+    };
+    if (bf16 && compact)
+        launch_down(k_down_decode<true, true>);
+    else if (bf16)
+        launch_down(k_down_decode<true, false>);
+    else if (compact)
+        launch_down(k_down_decode<false, true>);
+    else
+        launch_down(k_down_decode<false, false>);
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 3, st);
     if (prof) prof->recorded = true;

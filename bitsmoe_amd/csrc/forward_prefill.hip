@@ -195,7 +195,7 @@ __device__ inline int xcd_logical(int bid, int n_real) {
 struct APiece {
     u32x4 v[4];
 };
-__device__ inline void load_piece(const uint16_t* __restrict__ src, int64_t ld, int a_begin, int rows, int col0, int tid,
+__device__ __forceinline__ void load_piece(const uint16_t* __restrict__ src, int64_t ld, int a_begin, int rows, int col0, int tid,
                                   APiece& p) {
     const int r0 = tid >> 3, kc = (tid & 7) * 8;
 #pragma unroll
@@ -204,13 +204,13 @@ __device__ inline void load_piece(const uint16_t* __restrict__ src, int64_t ld, 
         p.v[j] = *reinterpret_cast<const u32x4*>(src + (int64_t)(a_begin + row) * ld + col0 + kc);
     }
 }
-__device__ inline void store_piece(uint16_t* __restrict__ stage, int tid, const APiece& p) {
+__device__ __forceinline__ void store_piece(uint16_t* __restrict__ stage, int tid, const APiece& p) {
     const int r0 = tid >> 3, kc = (tid & 7) * 8;
 #pragma unroll
     for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(stage + (r0 + 32 * j) * PF_LDS_ROW + kc) = p.v[j];
 }
 
-__device__ inline void zero_acc(f32x4 (&acc)[4][4]) {
+__device__ __forceinline__ void zero_acc(f32x4 (&acc)[4][4]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -234,7 +234,7 @@ struct GuFetch {
 struct GuOperands {
     u32x4 a[2][4];
 };
-__device__ inline void read_operands(const uint16_t* __restrict__ stage, int wm, int lane, GuOperands& o) {
+__device__ __forceinline__ void read_operands(const uint16_t* __restrict__ stage, int wm, int lane, GuOperands& o) {
     const int n = lane & 15, kg = lane >> 4;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
@@ -244,7 +244,7 @@ __device__ inline void read_operands(const uint16_t* __restrict__ stage, int wm,
 }
 
 template <int WU>
-__device__ inline void gateup_slab_mfma(int bits, const GuOperands& ops, const uint32_t (&bw)[2][4], int lane,
+__device__ __forceinline__ void gateup_slab_mfma(int bits, const GuOperands& ops, const uint32_t (&bw)[2][4], int lane,
                                         f32x4 (&acc)[4][4]) {
     const int n = lane & 15;
 #pragma unroll
@@ -284,7 +284,7 @@ __device__ inline void gateup_slab_mfma(int bits, const GuOperands& ops, const u
 // the per-row multiplier s is then taken from the folded scale table.  Otherwise Hs is the
 // pre-gathered [A, ld].  WU: the bit-width shared by every slab of the matrix, or 0 (mixed).
 template <bool DIRECT, int WU>
-__device__ inline void gateup_tile_body(const FastExpert fe, const FastSlab* __restrict__ fs_row, int nslabs,
+__device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const FastSlab* __restrict__ fs_row, int nslabs,
                                         const uint16_t* __restrict__ Hs, int ld,
                                         const int32_t* __restrict__ token_indices, int T, int I,
                                         uint16_t* __restrict__ out, int a_begin, int rows, int t,
@@ -492,7 +492,7 @@ constexpr int DN_SLABS_MFMA = 4;   // slabs (64 output rows each) per workgroup:
 // pair, per 16-row block.  The weight operand is (code - 2^(W-1)) * scale rounded once to f16,
 // the operand the reference builds (bitsmoe/algorithms/cpp/mlp_forward.cu:1554-1694).
 template <int HH>
-__device__ inline void down_half_mfma(int bits, const uint16_t* __restrict__ stage, const Block16& blk,
+__device__ __forceinline__ void down_half_mfma(int bits, const uint16_t* __restrict__ stage, const Block16& blk,
                                       const uint32_t (&scp)[4], int lane, f32x4 (&acc)[8][4]) {
     const int n = lane & 15, kg = lane >> 4;
 #pragma unroll
@@ -529,7 +529,7 @@ __device__ inline void down_half_mfma(int bits, const uint16_t* __restrict__ sta
 // The column loop of one wavefront (fs.bits == 0: no slab, the wavefront only helps to stage).
 // Pieces of z (128 assignments x 64 columns) run two ahead of the MFMAs in two alternating
 // register sets, the payload block of the next tile one tile ahead.
-__device__ inline void down_tile_loop(gptr<uint32_t> payload, gptr<__half> scale, const FastSlab fs,
+__device__ __forceinline__ void down_tile_loop(gptr<uint32_t> payload, gptr<__half> scale, const FastSlab fs,
                                       const uint16_t* __restrict__ z, int I, int n_tiles, int a_begin, int rows,
                                       uint16_t (*lds)[PF_M * PF_LDS_ROW], int tid, int lane, f32x4 (&acc)[8][4]) {
     const int n = lane & 15;
