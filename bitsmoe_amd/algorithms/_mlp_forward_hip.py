@@ -158,11 +158,21 @@ class Profile:
 # matrix-set cache for the list-based reference signature
 # ----------------------------------------------------------------------------------------
 _SET_CACHE: List[Tuple[tuple, MatrixSet]] = []
+_SET_BY_ADDRESS = {}
 _SET_CACHE_LIMIT = 4096
 
 
 def clear_matset_cache() -> None:
     _SET_CACHE.clear()
+    _SET_BY_ADDRESS.clear()
+
+
+def _address_key(lists: tuple, intermediate_size: int) -> tuple:
+    """Addresses and sizes of the six buffers of the first and the last expert: what identifies a
+    set when the sequences arrive as fresh list objects (calls through the dispatcher)."""
+    n = len(lists[0])
+    ends = (0, n - 1) if n > 1 else (0,)
+    return (n, int(intermediate_size)) + tuple((seq[i].data_ptr(), seq[i].numel()) for i in ends for seq in lists)
 
 
 def _lookup_set(lists: tuple, intermediate_size: int, name: str) -> MatrixSet:
@@ -171,11 +181,20 @@ def _lookup_set(lists: tuple, intermediate_size: int, name: str) -> MatrixSet:
     for key, ms in _SET_CACHE:
         if all(a is b for a, b in zip(key, lists)) and ms.intermediate_size == intermediate_size:
             return ms
+    akey = _address_key(lists, intermediate_size) if len(lists[0]) else None
+    ms = _SET_BY_ADDRESS.get(akey) if akey is not None else None
+    if ms is not None:
+        return ms
     ms = MatrixSet(*lists, intermediate_size=intermediate_size, name=name)
     if len(_SET_CACHE) >= _SET_CACHE_LIMIT:
-        _SET_CACHE.pop(0)
-    # the cache holds the sequences themselves, so their ids cannot be recycled
+        dropped = _SET_CACHE.pop(0)[1]
+        for k in [k for k, v in _SET_BY_ADDRESS.items() if v is dropped]:
+            del _SET_BY_ADDRESS[k]
+    # the cache holds the sequences themselves, so neither their ids nor the buffer addresses
+    # can be recycled while the entry lives
     _SET_CACHE.append((lists, ms))
+    if akey is not None:
+        _SET_BY_ADDRESS[akey] = ms
     return ms
 
 
@@ -329,3 +348,31 @@ def unpack_bitplanes(words: torch.Tensor, bits: int) -> torch.Tensor:
         _capi.check(_lib.bitsmoe_unpack_bitplanes(words.data_ptr(), rows, groups, int(bits), out.data_ptr(),
                                                   _stream_ptr(words.device)))
     return out
+
+
+# ----------------------------------------------------------------------------------------
+# PyTorch operator registration: torch.ops.bitsmoe.moe_packed_forward / torch.ops.bitsmoe.route
+# ----------------------------------------------------------------------------------------
+_MATRIX_ARGS = ", ".join(f"Tensor[] {m}_{b}" for m in ("gate", "up", "down")
+                         for b in ("payload", "rank_idx", "tile_meta", "slab_meta", "scale", "s"))
+_OPS = torch.library.Library("bitsmoe", "DEF")
+_OPS.define("moe_packed_forward(Tensor h_gate, Tensor h_up, Tensor token_indices, Tensor expert_offsets, "
+            f"Tensor route_weights, {_MATRIX_ARGS}, int rank_out, int intermediate_size, int act_type) -> Tensor")
+_OPS.define("route(Tensor selected_experts, Tensor route_weights, Tensor global_to_local, int n_packed) "
+            "-> (Tensor, Tensor, Tensor)")
+# only an accelerator implementation exists: on other devices the dispatcher raises
+_OPS.impl("moe_packed_forward", moe_packed_forward, "CUDA")
+_OPS.impl("route", route, "CUDA")
+
+
+@torch.library.register_fake("bitsmoe::moe_packed_forward")
+def _moe_packed_forward_fake(h_gate, h_up, token_indices, expert_offsets, route_weights, *rest):
+    return h_gate.new_empty((h_gate.shape[0], int(rest[-3])), dtype=torch.float32)
+
+
+@torch.library.register_fake("bitsmoe::route")
+def _route_fake(selected_experts, route_weights, global_to_local, n_packed):
+    n_flat = selected_experts.numel()
+    return (selected_experts.new_empty((n_flat,), dtype=torch.int32),
+            selected_experts.new_empty((int(n_packed) + 1,), dtype=torch.int32),
+            route_weights.new_empty((n_flat,), dtype=torch.float32))

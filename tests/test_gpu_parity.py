@@ -269,3 +269,31 @@ def test_forward_mfma_path_needs_prepared_sets(cuda_device):
     with pytest.raises(RuntimeError, match="MFMA path needs"):
         hip.moe_forward_sets(z(4, 80), z(4, 80), z(4, dt=torch.int32), z(3, dt=torch.int32), z(4, dt=torch.float32),
                              sets[0], sets[1], sets[2], 80, 128, 0, path=_capi.PATH_MFMA)
+
+
+def test_dispatcher_operator_equals_direct_call(cuda_device):
+    """torch.ops.bitsmoe.moe_packed_forward (fresh list objects on every call) and the module-level
+    function give the same result and share one matrix set."""
+    import torch
+
+    hip = _hip()
+    rng = np.random.default_rng(12)
+    gate, up, down = helpers.make_experts(12, 4, 128, 64, 256, choices=(2, 3, 4), slab_multiple=64)
+    lists = [helpers.to_device_lists(m, cuda_device) for m in (gate, up, down)]
+    flat = [seq for six in lists for seq in six]
+    h_gate = torch.from_numpy(rng.normal(size=(9, 128)).astype(np.float32)).to(torch.bfloat16).to(cuda_device)
+    h_up = torch.from_numpy(rng.normal(size=(9, 128)).astype(np.float32)).to(torch.bfloat16).to(cuda_device)
+    idx, w = o.router_qwen(rng.normal(size=(9, 4)).astype(np.float32), 2)
+    tok, off, rw = hip.route(torch.from_numpy(idx).to(cuda_device), torch.from_numpy(w).to(cuda_device),
+                             torch.arange(4, dtype=torch.int32, device=cuda_device), 4)
+    tok2, off2, rw2 = torch.ops.bitsmoe.route(torch.from_numpy(idx).to(cuda_device), torch.from_numpy(w).to(cuda_device),
+                                              torch.arange(4, dtype=torch.int32, device=cuda_device), 4)
+    assert torch.equal(off, off2) and torch.equal(tok[: int(off[-1])], tok2[: int(off[-1])])
+    hip.clear_matset_cache()
+    direct = hip.moe_packed_forward(h_gate, h_up, tok, off, rw, *flat, 64, 256, 0)
+    n_sets = len(hip._SET_CACHE)
+    via_op = torch.ops.bitsmoe.moe_packed_forward(h_gate, h_up, tok, off, rw, *flat, 64, 256, 0)
+    again = torch.ops.bitsmoe.moe_packed_forward(h_gate, h_up, tok, off, rw, *flat, 64, 256, 0)
+    assert len(hip._SET_CACHE) == n_sets == 3            # found by buffer address, not rebuilt
+    scale = float(direct.abs().max())
+    assert float((via_op - direct).abs().max()) <= 1e-5 * scale and float((again - direct).abs().max()) <= 1e-5 * scale

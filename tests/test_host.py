@@ -159,3 +159,21 @@ def test_block_refuses_to_run_without_gpu_path():
     cfg.hidden_act = "gelu"
     with pytest.raises(RuntimeError, match="Unsupported hidden_act"):
         block._act_type()
+
+
+def test_operators_are_registered_with_the_dispatcher():
+    """torch.ops.bitsmoe.* exist with the reference's argument list and have no CPU kernel."""
+    import torch
+
+    from bitsmoe_amd.algorithms import _HAS_MLP_FORWARD_CUDA
+
+    if not _HAS_MLP_FORWARD_CUDA:
+        pytest.skip("libbitsmoe_hip.so not built")
+    schema = torch.ops.bitsmoe.moe_packed_forward.default._schema
+    names = [a.name for a in schema.arguments]
+    assert names[:5] == ["h_gate", "h_up", "token_indices", "expert_offsets", "route_weights"]
+    assert names[5:11] == ["gate_payload", "gate_rank_idx", "gate_tile_meta", "gate_slab_meta", "gate_scale", "gate_s"]
+    assert names[-3:] == ["rank_out", "intermediate_size", "act_type"] and len(names) == 26
+    with pytest.raises(NotImplementedError):
+        torch.ops.bitsmoe.route(torch.zeros((2, 2), dtype=torch.int64), torch.zeros((2, 2)),
+                                torch.zeros((4,), dtype=torch.int32), 4)
