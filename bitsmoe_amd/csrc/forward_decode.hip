@@ -111,6 +111,7 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
     const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
     int E, int n_tiles, int n_groups, int n_tchunks, int tiles_per_wg, float* __restrict__ G, float* __restrict__ U) {
     const int mt = blockIdx.y;
+    // (consecutive workgroups land on different XCDs: that spreads experts of different cost)
     const int bid = blockIdx.x;
     const int tchunk = bid % n_tchunks;
     const int grp = (bid / n_tchunks) % n_groups;
@@ -474,10 +475,17 @@ __global__ __launch_bounds__(256) void k_down_decode(
     const FastExpert* __restrict__ down_fe, const FastSlab* __restrict__ down_fs, int max_slabs,
     const float* __restrict__ G, const float* __restrict__ U, const float* __restrict__ route_w,
     const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
-    int E, int n_tiles, int n_groups, int n_tchunks, int tiles_per_wg, int rank_out, float* __restrict__ rank_accum) {
-    const int tchunk = blockIdx.x % n_tchunks;
-    const int grp = (blockIdx.x / n_tchunks) % n_groups;
-    const int e_slot = blockIdx.x / (n_tchunks * n_groups);
+    int E, int n_tiles, int n_groups, int n_tchunks, int tiles_per_wg, int n_work, int rank_out,
+    float* __restrict__ rank_accum) {
+    // Workgroup b runs on XCD b % 8, and every XCD has its own L2: the workgroups of one expert
+    // (which all read that expert's G / U rows) are given ids of one residue class, so that they
+    // share one L2.  The grid is a multiple of 8; ids past the work exit.
+    const int per_xcd = gridDim.x >> 3;
+    const int bid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (bid >= n_work) return;
+    const int tchunk = bid % n_tchunks;
+    const int grp = (bid / n_tchunks) % n_groups;
+    const int e_slot = bid / (n_tchunks * n_groups);
     const int tid = threadIdx.x;
     const int e = COMPACT ? nth_active_expert(expert_offsets, E, A, e_slot, tid & 63) : e_slot;
     if (COMPACT && e < 0) return;
@@ -597,9 +605,10 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         dn_tiles_per_wg = (dn_tiles_per_wg + 1) / 2;
     const int dn_tchunks = (n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg;
     auto launch_down = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, dim3((unsigned)(e_dim * dn_groups * dn_tchunks)), dim3(256), z_bytes, st,
-                           down->d_fast_experts, down->d_fast_slabs, down->max_slabs, G, U, rw, tok, off, (int)T, (int)A, I,
-                           E, n_tiles, dn_groups, dn_tchunks, dn_tiles_per_wg, rank_out, rank_accum);
+        const int n_work = e_dim * dn_groups * dn_tchunks;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)((n_work + 7) / 8 * 8)), dim3(256), z_bytes, st, down->d_fast_experts,
+                           down->d_fast_slabs, down->max_slabs, G, U, rw, tok, off, (int)T, (int)A, I, E, n_tiles,
+                           dn_groups, dn_tchunks, dn_tiles_per_wg, n_work, rank_out, rank_accum);
     };
     if (bf16 && compact)
         launch_down(k_down_decode<true, true>);
