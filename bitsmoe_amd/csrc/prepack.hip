@@ -166,12 +166,28 @@ __global__ __launch_bounds__(64) void k_fold_scale_s(const MatView* __restrict__
 
 using namespace bitsmoe;
 
+static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st);
+
 extern "C" int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* stream) {
     BITSMOE_REQUIRE(set != nullptr, "set must not be null");
     BITSMOE_REQUIRE(role == ROLE_GATE_UP || role == ROLE_DOWN, "role must be 0 (gate/up) or 1 (down)");
-    hipStream_t st = (hipStream_t)stream;
     if (set->role == role) return BITSMOE_OK;
     BITSMOE_REQUIRE(set->role < 0, "matrix set is already prepared for the other role");
+    const int rc = prepare_impl(set, role, (hipStream_t)stream);
+    if (rc != BITSMOE_OK) {
+        // nothing of a failed attempt stays behind: the set remains usable by the generic kernels
+        void** owned[] = {(void**)&set->d_prepared, (void**)&set->d_views_prepared, (void**)&set->d_fast_experts,
+                          (void**)&set->d_fast_slabs, (void**)&set->d_scale_s};
+        for (void** p : owned) {
+            if (*p) (void)hipFree(*p);
+            *p = nullptr;
+        }
+        set->role = -1;
+    }
+    return rc;
+}
+
+static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
     if (!set->regular64 || set->total_slabs == 0) {
         set_error("matrix set is not regular (every slab 64 rows of 2/3/4 bits, full 128-column tiles): "
                   "only the generic kernels can run it");

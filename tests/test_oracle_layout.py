@@ -150,3 +150,48 @@ def test_dropped_and_reordered_segments():
         o.pack_matrix(np.zeros((10, 128), np.float32), np.ones(10), [(2, (0, 6)), (3, (5, 10))])
     with pytest.raises(ValueError):
         o.pack_matrix(np.zeros((10, 100), np.float32), np.ones(10), [(2, (0, 10))])
+
+
+# ---- committed vectors worked out bit by bit by tests/golden/make_layout_vectors.py (a scalar
+# ---- script that shares no code with the oracle)
+def _golden_cases():
+    import json
+    import os
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "layout_vectors.json")
+    with open(path) as f:
+        return json.load(f)
+
+
+def _golden_matrix(case):
+    """The committed buffers as an oracle matrix dict (rank_idx = identity, s = 1)."""
+    k = case["rank_len"]
+    return {"payload": np.array(case["payload"], dtype=np.uint32), "rank_idx": np.arange(k, dtype=np.int32),
+            "tile_meta": np.array(case["tile_meta"], dtype=np.int32).reshape(-1, 3),
+            "slab_meta": np.array(case["slab_meta"], dtype=np.int32).reshape(-1, 4),
+            "scale": np.array(case["scale"], dtype=np.float16), "s": np.ones(k, dtype=np.float16)}
+
+
+@pytest.mark.parametrize("name", ["two_slabs_4_and_2_bit", "three_bit_ragged", "every_low_width"])
+def test_golden_vectors_decode_and_repack(name):
+    case = _golden_cases()[name]
+    m = _golden_matrix(case)
+    dense = np.array(case["dense"], dtype=np.float32)
+    # decode: committed words -> committed values, exactly
+    got = o.dequant_matrix(m, case["dim"])
+    assert np.array_equal(got, dense)
+    for r, c in [(0, 0), (case["rank_len"] - 1, case["dim"] - 1), (case["rank_len"] // 2, case["dim"] // 3)]:
+        assert o.decode_element(m, r, c)[0] == dense[r, c]
+    # pack: the oracle packer, fed the committed levels and scales slab by slab, writes the same words
+    for (bits, k_slab, rank_off, tile_off), nxt in zip(m["slab_meta"], list(m["slab_meta"][1:]) + [None]):
+        tile_end = int(nxt[3]) if nxt is not None else len(m["tile_meta"])
+        for t in range(tile_off, tile_end):
+            pack_off, scale_off, n_valid = (int(v) for v in m["tile_meta"][t])
+            c0 = 128 * (t - tile_off)
+            sc = m["scale"][scale_off:scale_off + k_slab].astype(np.float32)
+            q = np.zeros((k_slab, 128), dtype=np.int8)            # padding columns: level 0
+            q[:, :n_valid] = np.rint(dense[rank_off:rank_off + k_slab, c0:c0 + n_valid] / sc[:, None]).astype(np.int8)
+            rows = o.pack_bitplanes(q, int(bits)).reshape(1, int(k_slab), 4, int(bits))      # [tile, row, micro, plane]
+            words = o._runtime_order(rows, int(k_slab)).reshape(-1)
+            n = int(k_slab) * 4 * int(bits)
+            assert np.array_equal(words, m["payload"][pack_off:pack_off + n]), (name, t)
