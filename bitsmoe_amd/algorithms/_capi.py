@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "bitsmoe_dequant_matrix_prepared",
     "bitsmoe_route_workspace_bytes",
     "bitsmoe_route",
+    "bitsmoe_router_softmax_topk",
     "bitsmoe_forward_workspace_bytes",
     "bitsmoe_forward_workspace_bytes_sets",
     "bitsmoe_moe_forward",
@@ -95,6 +96,9 @@ def load() -> ctypes.CDLL:
         c_void_p, c_int32, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32,
         c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p,
     ]
+    lib.bitsmoe_router_softmax_topk.restype = c_int32
+    lib.bitsmoe_router_softmax_topk.argtypes = [c_void_p, c_int32, c_int64, c_int32, c_int32, c_int32, c_int32,
+                                                c_void_p, c_int32, c_void_p, c_void_p]
     lib.bitsmoe_forward_workspace_bytes.restype = c_size_t
     lib.bitsmoe_forward_workspace_bytes.argtypes = [c_int64, c_int64, c_int32, c_int32, c_int32]
     lib.bitsmoe_forward_workspace_bytes_sets.restype = c_size_t

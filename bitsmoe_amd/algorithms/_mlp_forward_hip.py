@@ -350,6 +350,28 @@ def unpack_bitplanes(words: torch.Tensor, bits: int) -> torch.Tensor:
     return out
 
 
+def router_softmax_topk(router_logits: torch.Tensor, top_k: int, renormalize: bool = True,
+                        round_dtype: Optional[torch.dtype] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """softmax (fp32) -> top-k -> optional renormalisation -> optional round trip through
+    `round_dtype`, in one kernel.  Returns (selected int64 [T, k], weights fp32 [T, k])."""
+    _check(router_logits.dim() == 2, "router_logits must be [tokens, experts]")
+    _check(router_logits.is_cuda, "router_logits must be CUDA tensor")
+    _check(router_logits.dtype in (torch.float16, torch.bfloat16, torch.float32), "router_logits must be a float tensor")
+    _check(round_dtype in (None, torch.float16, torch.bfloat16), "round_dtype must be None, float16 or bfloat16")
+    dev = router_logits.device
+    logits = router_logits.contiguous()
+    t, e = int(logits.shape[0]), int(logits.shape[1])
+    selected = torch.empty((t, int(top_k)), dtype=torch.int64, device=dev)
+    weights = torch.empty((t, int(top_k)), dtype=torch.float32, device=dev)
+    codes = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}
+    with torch.cuda.device(dev):
+        _capi.check(_lib.bitsmoe_router_softmax_topk(
+            logits.data_ptr(), codes[logits.dtype], t, e, int(top_k), 1 if renormalize else 0,
+            -1 if round_dtype is None else codes[round_dtype], selected.data_ptr(), 1, weights.data_ptr(),
+            _stream_ptr(dev)))
+    return selected, weights
+
+
 # ----------------------------------------------------------------------------------------
 # PyTorch operator registration: torch.ops.bitsmoe.moe_packed_forward / torch.ops.bitsmoe.route
 # ----------------------------------------------------------------------------------------
@@ -360,9 +382,12 @@ _OPS.define("moe_packed_forward(Tensor h_gate, Tensor h_up, Tensor token_indices
             f"Tensor route_weights, {_MATRIX_ARGS}, int rank_out, int intermediate_size, int act_type) -> Tensor")
 _OPS.define("route(Tensor selected_experts, Tensor route_weights, Tensor global_to_local, int n_packed) "
             "-> (Tensor, Tensor, Tensor)")
+_OPS.define("router_softmax_topk(Tensor router_logits, int top_k, bool renormalize=True, ScalarType? round_dtype=None) "
+            "-> (Tensor, Tensor)")
 # only an accelerator implementation exists: on other devices the dispatcher raises
 _OPS.impl("moe_packed_forward", moe_packed_forward, "CUDA")
 _OPS.impl("route", route, "CUDA")
+_OPS.impl("router_softmax_topk", router_softmax_topk, "CUDA")
 
 
 @torch.library.register_fake("bitsmoe::moe_packed_forward")
@@ -376,3 +401,10 @@ def _route_fake(selected_experts, route_weights, global_to_local, n_packed):
     return (selected_experts.new_empty((n_flat,), dtype=torch.int32),
             selected_experts.new_empty((int(n_packed) + 1,), dtype=torch.int32),
             route_weights.new_empty((n_flat,), dtype=torch.float32))
+
+
+@torch.library.register_fake("bitsmoe::router_softmax_topk")
+def _router_fake(router_logits, top_k, renormalize=True, round_dtype=None):
+    t = router_logits.shape[0]
+    return (router_logits.new_empty((t, int(top_k)), dtype=torch.int64),
+            router_logits.new_empty((t, int(top_k)), dtype=torch.float32))

@@ -9,6 +9,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from bitsmoe_amd.algorithms import _HAS_MLP_FORWARD_CUDA, mlp_forward_cuda
 from bitsmoe_amd.models.base_block import BitsMoE_BaseSparseMoeBlock
 
 
@@ -31,6 +32,11 @@ class BitsMoE_Qwen3MoeSparseMoeBlock(BitsMoE_BaseSparseMoeBlock):
         """softmax in fp32 -> top-k -> renormalise; the weights take a round trip through the
         activation dtype, as in the reference (bitsmoe_block.py:47-51, 67-68)."""
         router_logits = self.gate(hidden_states)
+        if router_logits.is_cuda and _HAS_MLP_FORWARD_CUDA and router_logits.shape[1] <= 1024 and self.top_k <= 64:
+            # one kernel instead of softmax / topk / sum / div / two casts
+            selected, weights = mlp_forward_cuda.router_softmax_topk(router_logits, self.top_k, self.norm_topk_prob,
+                                                                     round_dtype=hidden_states.dtype)
+            return router_logits, selected, weights
         weights = F.softmax(router_logits, dim=1, dtype=torch.float)
         weights, selected = torch.topk(weights, self.top_k, dim=-1)
         if self.norm_topk_prob:

@@ -127,6 +127,20 @@ int bitsmoe_route(const void* selected, int32_t ids_are_i64, const float* weight
                   size_t workspace_bytes, void* stream);
 
 /*
+ * Router front end in one kernel.  Replaces the framework-op chain of the reference's Qwen
+ * blocks (bitsmoe/models/qwen3moe/bitsmoe_block.py:45-51,
+ * bitsmoe/models/qwen3next/bitsmoe_block.py:92-98): softmax of the logits in fp32, top-k
+ * (descending; ties go to the lower expert index), optional division by the sum of the k
+ * probabilities, optional round trip of the weights through fp16 / bf16 (round_dtype -1 / 0 / 1).
+ *   logits   device [T, n_experts], logits_dtype 0 fp16 / 1 bf16 / 2 fp32
+ *   selected device int32 or int64 [T, top_k] out, weights device fp32 [T, top_k] out
+ */
+int bitsmoe_router_softmax_topk(const void* logits, int32_t logits_dtype, int64_t n_tokens,
+                                int32_t n_experts, int32_t top_k, int32_t renormalize,
+                                int32_t round_dtype, void* selected, int32_t ids_are_i64,
+                                float* weights, void* stream);
+
+/*
  * The routed-expert forward.  Replaces moe_packed_forward
  * (bitsmoe/algorithms/cpp/mlp_forward_binding.cpp:53-155) ->
  * moe_packed_forward_cuda (bitsmoe/algorithms/cpp/mlp_forward.cu:2701-3074):

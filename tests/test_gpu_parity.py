@@ -317,3 +317,28 @@ def test_golden_vectors_dequant_on_device(cuda_device, name):
     ms = hip.MatrixSet(*helpers.to_device_lists([m], cuda_device), intermediate_size=case["dim"])
     got = ms.dequant(0).cpu().numpy()
     assert np.array_equal(got, np.array(case["dense"], dtype=np.float32))
+
+
+@pytest.mark.parametrize("tokens,n_experts,top_k,renorm", [
+    (1, 128, 8, True), (64, 128, 8, True), (256, 512, 10, True), (16, 64, 6, False), (5, 8, 1, True), (37, 1000, 3, True)])
+@pytest.mark.parametrize("logit_dtype", ["f32", "bf16"])
+def test_router_kernel_matches_oracle(cuda_device, tokens, n_experts, top_k, renorm, logit_dtype):
+    """softmax / top-k / renormalise in one kernel: the picked experts are exactly the oracle's (in
+    descending order), the weights agree to fp32 rounding; with the round trip through bf16
+    they agree to one bf16 step."""
+    import torch
+
+    hip = _hip()
+    rng = np.random.default_rng(tokens * 7 + n_experts)
+    logits = rng.normal(size=(tokens, n_experts)).astype(np.float32) * 2.0
+    t = torch.from_numpy(logits)
+    if logit_dtype == "bf16":
+        t = t.to(torch.bfloat16)
+        logits = t.float().numpy()
+    idx_ref, w_ref = o.router_qwen(logits, top_k, renorm)
+    sel, w = hip.router_softmax_topk(t.to(cuda_device), top_k, renorm)
+    assert sel.dtype == torch.int64 and np.array_equal(sel.cpu().numpy(), idx_ref)
+    assert np.allclose(w.cpu().numpy(), w_ref, rtol=2e-6, atol=1e-9)
+    sel2, w2 = hip.router_softmax_topk(t.to(cuda_device), top_k, renorm, round_dtype=torch.bfloat16)
+    assert torch.equal(sel2, sel)
+    assert np.allclose(w2.cpu().numpy(), helpers.bf16_round(w_ref), rtol=2 ** -7, atol=0)
