@@ -565,13 +565,13 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     const int max_slabs = std::max(gate->max_slabs, up->max_slabs);
     const int gu_groups = (max_slabs + GU_SLABS - 1) / GU_SLABS;
     // Tiles per workgroup: long runs amortise the start-up round trips, but the grid must
-    // still hold a few workgroups per CU.  At most min(E, A) experts can be active.
+    // still hold a few workgroups per CU (two rounds of three per CU measured best).  At most min(E, A) experts can be active.
     const int64_t active_max = std::min<int64_t>(E, A);
     // few assignments: launch over the experts that can be active at most, not over all of them
     const bool compact = active_max * 2 <= E;
     const int e_dim = compact ? (int)active_max : E;
     int tiles_per_wg = n_tiles;
-    while (tiles_per_wg > 1 && active_max * 2 * gu_groups * ((n_tiles + tiles_per_wg - 1) / tiles_per_wg) < 2048)
+    while (tiles_per_wg > 1 && active_max * 2 * gu_groups * ((n_tiles + tiles_per_wg - 1) / tiles_per_wg) < 1536)
         tiles_per_wg = (tiles_per_wg + 1) / 2;
     const int n_tchunks = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
     dim3 grid((unsigned)(e_dim * gu_groups * n_tchunks), 2);
