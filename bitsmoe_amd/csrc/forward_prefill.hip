@@ -218,38 +218,29 @@ __device__ __forceinline__ void zero_acc(f32x4 (&acc)[4][4]) {
 }
 
 // ------------------------------------------------------------------------------ gate / up
-constexpr int GU_SETS = 3;   // register sets of fetched slabs: loads run GU_SETS - 1 slabs ahead of the MFMAs
+constexpr int GU_STAGE = PF_M * PF_LDS_ROW;   // 16-bit elements of one scaled 128 x 64 activation piece in LDS
+constexpr size_t GU_LDS_BYTES = (size_t)2 * 2 * GU_STAGE * 2 + 2 * PF_M * sizeof(float);
 
 // Everything one thread fetches from global memory for one slab.
 struct GuFetch {
     APiece a;          // this thread's part of the 128 x 64 activation piece
-    u32x4 sc;          // scale pairs of contraction rows 8*(tid%8) .. +7 of the slab (tile t)
-    uint32_t bw[2][4]; // payload words of the wavefront's two column-block pairs
+    u32x4 sc[2];       // scale pairs of contraction rows 8*(tid%8) .. +7 of the slab, for the two column tiles
+    uint32_t bw[2][4]; // payload words of the wavefront's two column-block pairs (its own tile)
 };
 
-// One slab (64 contraction rows, `bits` wide) for a wavefront's 64 x 64 tile; the weight
+// One slab (64 contraction rows, `bits` wide) for a wavefront's 128 x 64 tile; the weight
 // operand is the raw (2^bits + code), the scale already sits in the activations.
 // WU != 0: the width is a compile-time constant (experts whose slabs all share it).
-// The activation operands of one slab for a wavefront: [ks][mb], read from an LDS stage.
-struct GuOperands {
-    u32x4 a[2][4];
-};
-__device__ __forceinline__ void read_operands(const uint16_t* __restrict__ stage, int wm, int lane, GuOperands& o) {
+template <int WU>
+__device__ __forceinline__ void gateup_slab_mfma(int bits, const uint16_t* __restrict__ stage,
+                                                 const uint32_t (&bw)[2][4], int lane, f32x4 (&acc)[8][4]) {
     const int n = lane & 15, kg = lane >> 4;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
-            o.a[ks][mb] = *reinterpret_cast<const u32x4*>(stage + (64 * wm + 16 * mb + n) * PF_LDS_ROW + 16 * kg + 8 * ks);
-}
-
-template <int WU>
-__device__ __forceinline__ void gateup_slab_mfma(int bits, const GuOperands& ops, const uint32_t (&bw)[2][4], int lane,
-                                        f32x4 (&acc)[4][4]) {
-    const int n = lane & 15;
-#pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-        const u32x4(&a)[4] = ops.a[ks];
+        u32x4 a[8];
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb)
+            a[mb] = *reinterpret_cast<const u32x4*>(stage + (16 * mb + n) * PF_LDS_ROW + 16 * kg + 8 * ks);
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
             const uint32_t(&w)[4] = bw[nb >> 1];
@@ -264,20 +255,21 @@ __device__ __forceinline__ void gateup_slab_mfma(int bits, const GuOperands& ops
             else
                 b = decode_fields3<false>(w[nbl], 8 * ks, w[2 + nbl], 8 * (n >> 3) + 4 * ks);
 #pragma unroll
-            for (int mb = 0; mb < 4; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
+            for (int mb = 0; mb < 8; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
         }
     }
 }
 
-// One workgroup = (assignment tile, projection, 128-column tile): out[a, c] = f16 of
-// sum_k A[a, k] * level[k, c] * scale[tile(c), k] over all slabs of the expert's matrix.
+// One workgroup = (assignment tile, projection, PAIR of 128-column tiles):
+// out[a, c] = f16 of sum_k A[a, k] * level[k, c] * scale[tile(c), k] over all slabs of the matrix.
+// Wavefront (tl, wn) owns all 128 assignments and columns 64*wn .. +63 of tile t0 + tl: a decoded
+// weight operand feeds eight MFMAs.
 //
-// Per slab the staging threads multiply their part of the activation piece by the slab's
-// per-row scale of this tile (packed f16), write it to LDS and keep a running sum of what they
-// wrote, weighted with 1.5 * 2^W: sum_k A'[a,k] * (2^W + code) - 1.5 * 2^W * sum_k A'[a,k] is the
-// dot product with the true levels code - 2^(W-1).  Global loads run GU_SETS - 1 slabs ahead of
-// the MFMAs in rotating register sets (one memory round trip is several times longer than the
-// MFMAs of one slab).
+// The activation piece of a slab (128 x 64) is fetched once for both tiles.  The staging
+// threads multiply it by the slab's per-row scale of each tile (packed f16), write the two scaled
+// pieces to LDS and keep running sums of what they wrote, weighted with 1.5 * 2^W:
+// sum_k A'[a,k] * (2^W + code) - 1.5 * 2^W * sum_k A'[a,k] is the dot product with the true levels
+// code - 2^(W-1).  The loads of slab s + 2 are issued before slab s is multiplied.
 //
 // DIRECT: the activation rows are read straight from the f16 activations [T, ld] through the
 // token index (possible when every aligned run of 8 local rows is 8 consecutive logical ranks);
@@ -285,48 +277,58 @@ __device__ __forceinline__ void gateup_slab_mfma(int bits, const GuOperands& ops
 // pre-gathered [A, ld].  WU: the bit-width shared by every slab of the matrix, or 0 (mixed).
 template <bool DIRECT, int WU>
 __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const FastSlab* __restrict__ fs_row, int nslabs,
-                                        const uint16_t* __restrict__ Hs, int ld,
-                                        const int32_t* __restrict__ token_indices, int T, int I,
-                                        uint16_t* __restrict__ out, int a_begin, int rows, int t,
-                                        uint16_t (*lds)[PF_M * PF_LDS_ROW], float* __restrict__ rowsum) {
+                                                 const uint16_t* __restrict__ Hs, int ld,
+                                                 const int32_t* __restrict__ token_indices, int T, int I, int n_tiles,
+                                                 uint16_t* __restrict__ out, int a_begin, int rows, int t0,
+                                                 uint16_t* __restrict__ lds, float* __restrict__ rowsum) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int tl = wave >> 1, wn = wave & 1;
     const int n = lane & 15, kg = lane >> 4;
-    const bool active = 64 * wm < rows;   // a wavefront whose 64 rows are all past the end only helps to stage
+    const bool two_tiles = t0 + 1 < n_tiles;
+    const bool active = tl == 0 || two_tiles;        // a wavefront without a tile only helps to stage
+    const int t = active ? t0 + tl : t0;             // (it re-reads tile t0: in bounds)
 
-    // DIRECT: the activation row of each of this thread's four staging rows (invalid tokens read
-    // row 0: their outputs are dropped by the combine)
-    uint32_t rowbase[4] = {0, 0, 0, 0};   // element offsets (the launcher checks T * ld < 2^31)
-    if constexpr (DIRECT) {
+    // this thread's four staging rows; DIRECT: their activation rows (invalid tokens read row 0:
+    // the combine drops their outputs).  Element offsets: the launcher checks that they fit 32 bits.
+    const int r0 = tid >> 3, kc = (tid & 7) * 8;
+    uint32_t rowbase[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int tk = token_indices[a_begin + min((tid >> 3) + 32 * j, rows - 1)];
+    for (int j = 0; j < 4; ++j) {
+        const int a = a_begin + min(r0 + 32 * j, rows - 1);
+        if constexpr (DIRECT) {
+            const int tk = token_indices[a];
             rowbase[j] = (uint32_t)((tk >= 0 && tk < T) ? tk : 0) * (uint32_t)ld;
+        } else {
+            rowbase[j] = (uint32_t)a * (uint32_t)ld + (uint32_t)kc;
         }
     }
 
-    f32x4 acc[4][4];
-    zero_acc(acc);
+    f32x4 acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
     gptr<uint32_t> payload = as_global(fe.payload);
     gptr<__half> scale = as_global(DIRECT ? fe.scale_s : fe.scale);
     gptr<int32_t> rank_idx = as_global(fe.rank_idx);
-    GuFetch f[GU_SETS];
-    int bits_of[GU_SETS];      // width of the slab held by each set
-    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    GuFetch f[1];              // the one slab in flight
+    float sum[2][4];           // [tile][row]
+#pragma unroll
+    for (int x = 0; x < 2; ++x)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sum[x][j] = 0.0f;
     auto slab_rec = [&](int s) { return s < nslabs ? load_fast_slab(fs_row, s) : FastSlab{0, 0, 0, 0}; };
-    auto rank_base = [&](int s) { return (DIRECT && s < nslabs) ? rank_idx[s * SLAB_ROWS + (tid & 7) * 8] : 0; };
+    auto rank_base = [&](int s) { return (DIRECT && s < nslabs) ? rank_idx[s * SLAB_ROWS + kc] : 0; };
     auto issue = [&](GuFetch& dst, const FastSlab& r, int rbase, int s) {
         const int wb = WU != 0 ? WU : r.bits;
-        if constexpr (DIRECT) {
+        const uint32_t col = DIRECT ? (uint32_t)rbase : (uint32_t)(s * SLAB_ROWS);
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                dst.a.v[j] = *reinterpret_cast<const u32x4*>(Hs + (rowbase[j] + (uint32_t)rbase));
-        } else {
-            load_piece(Hs, ld, a_begin, rows, s * SLAB_ROWS, tid, dst.a);
-        }
-        dst.sc = *reinterpret_cast<gptr_u32x4>(scale + (uint32_t)(r.scale_off + t * SLAB_ROWS + (tid & 7) * 8));
+        for (int j = 0; j < 4; ++j) dst.a.v[j] = *reinterpret_cast<const u32x4*>(Hs + (rowbase[j] + col));
+        gptr<__half> sp = scale + (uint32_t)(r.scale_off + t0 * SLAB_ROWS + kc);
+        dst.sc[0] = *reinterpret_cast<gptr_u32x4>(sp);
+        dst.sc[1] = *reinterpret_cast<gptr_u32x4>(sp + (two_tiles ? SLAB_ROWS : 0));
         gptr<uint32_t> blk = payload + (uint32_t)(r.pack_off + t * 256 * wb);
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
@@ -334,94 +336,108 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
             load_pair_role0(blk, wb, (uint32_t)(pair * 64 + lane), (uint32_t)hi_index0(kg, n, 2 * pair), dst.bw[p]);
         }
     };
-    // scale the fetched piece, add its weighted row sums, write it to an LDS stage
-    auto stage_piece = [&](GuFetch& src, int bits, uint16_t* __restrict__ stage) {
+    // scale the fetched piece for both tiles, add the weighted row sums, write the two pieces to LDS
+    auto stage_piece = [&](const GuFetch& src, int bits, uint16_t* __restrict__ stage) {
         const int wb = WU != 0 ? WU : bits;
         const uint32_t cw = wb == 2 ? Codec<2, false>::CORR : wb == 3 ? Codec<3, false>::CORR : Codec<4, false>::CORR;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int x = 0; x < 2; ++x) {
+            if (x == 1 && !two_tiles) break;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint32_t scaled = pk_mul_f16(src.a.v[j][i], src.sc[i]);
-                src.a.v[j][i] = scaled;
-                sum[j] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, scaled), __builtin_bit_cast(h2, cw), sum[j], false);
+            for (int j = 0; j < 4; ++j) {
+                u32x4 v;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t raw = src.a.v[j][i];
+                    const uint32_t scaled = pk_mul_f16(raw, src.sc[x][i]);
+                    v[i] = scaled;
+                    sum[x][j] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, scaled), __builtin_bit_cast(h2, cw), sum[x][j], false);
+                }
+                *reinterpret_cast<u32x4*>(stage + x * GU_STAGE + (r0 + 32 * j) * PF_LDS_ROW + kc) = v;
             }
         }
-        store_piece(stage, tid, src.a);
     };
     if (nslabs > 0) {
-        // prologue: slabs 0 .. GU_SETS-2 go into sets 0 .. GU_SETS-2; slab 0 is staged
-        FastSlab pending = slab_rec(0);
-        int pending_rb = rank_base(0);
-        static_for([&](auto qc) {
-            constexpr int q = decltype(qc)::value;
-            if (q < nslabs) {
-                const FastSlab rec = pending;
-                const int rb = pending_rb;
-                pending = slab_rec(q + 1);
-                pending_rb = rank_base(q + 1);
-                bits_of[q] = rec.bits;
-                issue(f[q], rec, rb, q);
-            }
-        }, std::make_integer_sequence<int, GU_SETS - 1>{});
-        stage_piece(f[0], bits_of[0], lds[0]);
+        // prologue: slab 0 is fetched and staged, slab 1 requested
+        GuFetch& F = f[0];
+        uint32_t bw[2][4];       // payload words of the slab being multiplied
+        FastSlab rec = slab_rec(0);
+        FastSlab pending = slab_rec(1);
+        int pending_rb = rank_base(1);
+        int bits = rec.bits;
+        issue(F, rec, rank_base(0), 0);
+        stage_piece(F, bits, lds);
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) bw[p][i] = F.bw[p][i];
+        int bits_next = pending.bits;
+        if (nslabs > 1) {
+            issue(F, pending, pending_rb, 1);
+            pending = slab_rec(2);
+            pending_rb = rank_base(2);
+        }
         __syncthreads();
-        // step s (set q = s % GU_SETS): slab s is in LDS stage s % 2, its words in set q; the slab
-        // s + GU_SETS - 1 is requested into the set that slab s - 1 just left; slab s + 1 is staged.
-        for (int s0 = 0; s0 < nslabs; s0 += GU_SETS) {
-            static_for([&](auto qc) {
-                constexpr int q = decltype(qc)::value;
-                constexpr int q_issue = (q + GU_SETS - 1) % GU_SETS;
-                constexpr int q_next = (q + 1) % GU_SETS;
-                const int s = s0 + q;
-                if (s < nslabs) {
-                    if (s + GU_SETS - 1 < nslabs) {
-                        const FastSlab rec = pending;
-                        const int rb = pending_rb;
-                        pending = slab_rec(s + GU_SETS);
-                        pending_rb = rank_base(s + GU_SETS);
-                        bits_of[q_issue] = rec.bits;
-                        issue(f[q_issue], rec, rb, s + GU_SETS - 1);
-                    }
-                    // the operand reads are requested first, so that their LDS round trip passes while
-                    // the next piece is scaled and written; the MFMAs then separate that write from
-                    // the barrier
-                    GuOperands ops;
-                    const bool mul = active && bits_of[q] != 0;
-                    if (mul) read_operands(lds[s & 1], wm, lane, ops);
-                    if (s + 1 < nslabs) stage_piece(f[q_next], bits_of[q_next], lds[(s + 1) & 1]);
-                    if (mul) gateup_slab_mfma<WU>(bits_of[q], ops, f[q].bw, lane, acc);
-                    __syncthreads();
+        // step s: slab s is in LDS stage s % 2 with its words in `bw`; slab s + 1 (in flight in F) is
+        // staged, slab s + 2 requested, then slab s is multiplied
+        for (int s = 0; s < nslabs; ++s) {
+            uint32_t bw_next[2][4];
+            const int bits_after = pending.bits;
+            if (s + 1 < nslabs) {
+                stage_piece(F, bits_next, lds + ((s + 1) & 1) * 2 * GU_STAGE);
+#pragma unroll
+                for (int p = 0; p < 2; ++p)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) bw_next[p][i] = F.bw[p][i];
+                if (s + 2 < nslabs) {
+                    issue(F, pending, pending_rb, s + 2);
+                    pending = slab_rec(s + 3);
+                    pending_rb = rank_base(s + 3);
                 }
-            }, std::make_integer_sequence<int, GU_SETS>{});
+            }
+            if (active && bits != 0) gateup_slab_mfma<WU>(bits, lds + ((s & 1) * 2 + tl) * GU_STAGE, bw, lane, acc);
+            __syncthreads();
+            if (s + 1 < nslabs) {
+#pragma unroll
+                for (int p = 0; p < 2; ++p)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) bw[p][i] = bw_next[p][i];
+                bits = bits_next;
+                bits_next = bits_after;
+            }
         }
     }
     // row sums: the eight threads that share a row hold its eight 8-column parts
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        float v = sum[j];
-        v += __shfl_xor(v, 1);
-        v += __shfl_xor(v, 2);
-        v += __shfl_xor(v, 4);
-        if ((tid & 7) == 0) rowsum[(tid >> 3) + 32 * j] = v;
-    }
-    __syncthreads();
-    if (!active) return;
-    // lane holds rows 64*wm + 16*mb + 4*kg + j, column 128*t + 64*wn + 16*nb + n
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
+    for (int x = 0; x < 2; ++x)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int row = 64 * wm + 16 * mb + 4 * kg + j;
+            float v = sum[x][j];
+            v += __shfl_xor(v, 1);
+            v += __shfl_xor(v, 2);
+            v += __shfl_xor(v, 4);
+            if ((tid & 7) == 0) rowsum[x * PF_M + r0 + 32 * j] = v;
+        }
+    __syncthreads();
+    if (!active) return;
+    // lane holds rows 16*mb + 4*kg + j, column 128*t + 64*wn + 16*nb + n
+#pragma unroll
+    for (int mb = 0; mb < 8; ++mb) {
+        if (16 * mb >= rows) break;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = 16 * mb + 4 * kg + j;
             if (row >= rows) continue;
-            const float c = rowsum[row];
+            const float c = rowsum[tl * PF_M + row];
             uint16_t* dst = out + (int64_t)(a_begin + row) * I + N_TILE * t + 64 * wn + n;
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) dst[16 * nb] = __builtin_bit_cast(uint16_t, (_Float16)(acc[mb][nb][j] - c));
         }
+    }
 }
 
-// grid.x = 8 * ceil(max_mtiles * 2 * n_tiles / 8); G and U are f16 [A, I].
+// grid.x = 8 * ceil(max_mtiles * 2 * ceil(n_tiles / 2) / 8), 256 threads, GU_LDS_BYTES of dynamic
+// LDS; G and U are f16 [A, I].
 template <bool DIRECT>
 __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
@@ -430,14 +446,16 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     const int32_t* __restrict__ token_indices, int T,
     const MTile* __restrict__ mtiles, const int32_t* __restrict__ n_mtiles, int I, int n_tiles,
     uint16_t* __restrict__ G, uint16_t* __restrict__ U) {
-    __shared__ __attribute__((aligned(16))) uint16_t lds[2][PF_M * PF_LDS_ROW];
-    __shared__ float rowsum[PF_M];
-    const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles) * 2 * n_tiles);
+    extern __shared__ __attribute__((aligned(16))) unsigned char gu_smem[];
+    uint16_t* lds = reinterpret_cast<uint16_t*>(gu_smem);
+    float* rowsum = reinterpret_cast<float*>(gu_smem + (size_t)2 * 2 * GU_STAGE * 2);
+    const int n_tp = (n_tiles + 1) >> 1;
+    const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles) * 2 * n_tp);
     if (logical < 0) return;
-    // the column tiles of one (assignment tile, projection) are neighbours: they share the activations
-    const int t = logical % n_tiles;
-    const int proj = (logical / n_tiles) & 1;
-    const int mt_i = logical / (2 * n_tiles);
+    // the tile pairs of one (assignment tile, projection) are neighbours: they share the activations
+    const int tp = logical % n_tp;
+    const int proj = (logical / n_tp) & 1;
+    const int mt_i = logical / (2 * n_tp);
     const i32x4 tv = *reinterpret_cast<const i32x4*>(mtiles + mt_i);
     const int e = __builtin_amdgcn_readfirstlane(tv[0]);
     const int a_begin = __builtin_amdgcn_readfirstlane(tv[1]);
@@ -451,8 +469,9 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     const int ld = proj ? ldu : ldg;
     uint16_t* __restrict__ out = proj ? U : G;
     const int w = __builtin_amdgcn_readfirstlane(fe.uniform_bits);
-#define BITSMOE_GU_BODY(W) \
-    gateup_tile_body<DIRECT, W>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, out, a_begin, rows, t, lds, rowsum)
+#define BITSMOE_GU_BODY(W)                                                                                            \
+    gateup_tile_body<DIRECT, W>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out, a_begin, rows, 2 * tp, \
+                                lds, rowsum)
     if (w == 2)
         BITSMOE_GU_BODY(2);
     else if (w == 3)
@@ -733,16 +752,20 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     }
     record(prof, 1, st);
     {
-        const int64_t wgs = (max_mtiles * 2 * n_tiles + 7) / 8 * 8;
-        if (direct)
-            hipLaunchKernelGGL(k_gateup_mfma<true>, dim3((unsigned)wgs), dim3(256), 0, st, gate->d_fast_experts,
+        const int n_tp = (n_tiles + 1) / 2;
+        const int64_t wgs = (max_mtiles * 2 * n_tp + 7) / 8 * 8;
+        auto launch = [&](auto kernel) -> hipError_t {
+            // more than 64 KB of LDS per workgroup has to be asked for explicitly (a property of
+            // the kernel, not a stream operation)
+            hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)GU_LDS_BYTES);
+            if (err != hipSuccess) return err;
+            hipLaunchKernelGGL(kernel, dim3((unsigned)wgs), dim3(256), GU_LDS_BYTES, st, gate->d_fast_experts,
                                gate->d_fast_slabs, gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs,
                                Hs_g, Hs_u, ldg, ldu, tok, (int)T, mtiles, n_mtiles, I, n_tiles, z, Ubuf);
-        else
-            hipLaunchKernelGGL(k_gateup_mfma<false>, dim3((unsigned)wgs), dim3(256), 0, st, gate->d_fast_experts,
-                               gate->d_fast_slabs, gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs,
-                               Hs_g, Hs_u, ldg, ldu, tok, (int)T, mtiles, n_mtiles, I, n_tiles, z, Ubuf);
-        BITSMOE_HIP_TRY(hipGetLastError());
+            return hipGetLastError();
+        };
+        BITSMOE_HIP_TRY(direct ? launch(k_gateup_mfma<true>) : launch(k_gateup_mfma<false>));
         const int64_t n8 = A * (int64_t)I / 8;
         hipLaunchKernelGGL(k_silu_mul_f16, dim3((unsigned)std::min<int64_t>((n8 + 255) / 256, 4096)), dim3(256), 0, st, z,
                            Ubuf, n8);
