@@ -69,7 +69,8 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
                           hipStream_t st);
 
 bool mfma_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I);
-size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, int64_t T, int64_t A, int I);
+size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int64_t T,
+                            int64_t A, int I);
 int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
                         const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru,
                         const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out, int I,
@@ -91,6 +92,7 @@ struct bitsmoe_matset {
     int role = -1;                    // -1: not prepared; 0: gate/up layout; 1: down layout
     bool rank_chunked8 = false;       // slab i holds local rows 64*i.., and every aligned run of 8 local rows
                                       // maps to 8 consecutive logical ranks starting at a multiple of 8
+    bool rank_identity = false;       // rank_idx[k] == k in every expert
     __half* d_scale_s = nullptr;      // gate/up sets: scale folded with the per-row multiplier s
     bool vector_aligned = false;      // scale / s / rank_idx of every expert start on 16-byte boundaries
     bool all_uniform8 = false;        // role 0: every aligned group of 8 slabs has one width and is contiguous

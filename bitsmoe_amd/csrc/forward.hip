@@ -47,7 +47,7 @@ extern "C" size_t bitsmoe_forward_workspace_bytes_sets(const bitsmoe_matset* gat
     if (!gate || !up || !down || n_assign < 0) return 0;
     const int I = gate->intermediate_size;
     const int chosen = resolve_path(gate, up, down, n_assign, I, path);
-    if (chosen == BITSMOE_PATH_MFMA) return mfma_workspace_bytes(gate, up, n_tokens, n_assign, I);
+    if (chosen == BITSMOE_PATH_MFMA) return mfma_workspace_bytes(gate, up, down, n_tokens, n_assign, I);
     return bitsmoe_forward_workspace_bytes(n_tokens, n_assign, I, gate->n_experts, 0);
 }
 

@@ -2,19 +2,26 @@
 // assignments, so the work is a grouped GEMM and the weights are decoded once per 128-row
 // tile of assignments instead of once per 16.
 //
-//   k_build_mtiles   expert_offsets -> list of (expert, first assignment, rows <= 128) tiles
-//   k_pregather      Hs[a, k] = f16( h[tok_a, rank_idx[k]] * s[k] )  for gate and up, rows in
-//                    expert-sorted assignment order, columns in the expert's local row order
-//   k_gateup_mfma    z[a, c] = f16( silu(G) * U ),  G = Hs_gate . W_gate,  U = Hs_up . W_up
-//   k_down_mfma      rank_accum[tok_a, rank_idx[r]] += route_w[a] * s[r] * sum_c W_down[r, c] z[a, c]
+//   k_token_count    slot of every assignment within its token (for the per-token lists)
+//   k_build_mtiles   expert_offsets -> list of (expert, first assignment, rows <= 128) tiles;
+//                    token_start = exclusive scan of the per-token assignment counts
+//   k_bf16_to_f16 /  activations as f16, read through the token index by the GEMM kernel, or
+//   k_pregather      Hs[a, k] = f16( h[tok_a, rank_idx[k]] * s[k] ) in expert-sorted assignment order
+//   k_gateup_mfma    G = Hs_gate . W_gate, U = Hs_up . W_up as f16;  k_silu_mul_f16: z = silu(G) * U
+//   k_down_mfma      y[a, r] = sum_c W_down[r, c] z[a, c] as f16, and the per-token lists
+//   k_combine_tokens rank_accum[t, rank_idx[r]] = sum over the assignments of t of route_w * s[r] * y
 //
-// Both GEMM kernels use a 128 x 128 workgroup tile (four wavefronts, 64 x 64 each) and
-// 16x16x32 f16 MFMA.  The activation operand is staged through LDS in 128 x 64 pieces (double
+// Both GEMM kernels use 16x16x32 f16 MFMA with four wavefronts of 128 rows x 64 columns per
+// workgroup.  The activation operand is staged through LDS in 128 x 64 pieces (double
 // buffered, one barrier per piece); the weight operand never touches LDS: every lane loads
-// its words of the prepared payload (wave_layout.h), expands them to packed f16 pairs
-// (2^w + code) with a rotate and an and-or, and one packed FMA per pair turns that into
-// (code - 2^(w-1)) * scale -- the same "weight rounded to half" operand the reference's
-// tensor-core path builds (bitsmoe/algorithms/cpp/mlp_forward.cu:691-751, 1554-1694).
+// its words of the prepared payload (wave_layout.h) and expands them to packed f16 pairs
+// (2^w + code) with a rotate and an and-or.  Gate/up multiply the activation rows by
+// scale * s while staging them and subtract 1.5 * 2^w * (weighted row sum) at the end; down
+// turns the pair into (code - 2^(w-1)) * scale with a packed add and a packed multiply --
+// the same "weight rounded to half" operand the reference's tensor-core path builds
+// (bitsmoe/algorithms/cpp/mlp_forward.cu:691-751, 1554-1694).  The top-k combine is a gather
+// per token instead of the reference's fp32 atomics (mlp_forward.cu:2036-2066): its result
+// does not depend on the order in which workgroups finish.
 // Operands are f16 for f16 and bf16 inputs alike (f16 keeps more mantissa than bf16).
 #include <algorithm>
 
@@ -55,9 +62,28 @@ __device__ inline uint32_t neg_offset_pair() {
 }
 
 // ------------------------------------------------------------------------------ schedule
+// slot[a] = how many assignments of the same token were counted before a (any order);
+// token_count must be zero on entry.  Assignments outside [offsets[0], offsets[E]) belong to
+// no expert and are not counted.
+__global__ __launch_bounds__(256) void k_token_count(const int32_t* __restrict__ token_indices,
+                                                     const int32_t* __restrict__ expert_offsets, int E, int A, int T,
+                                                     int32_t* __restrict__ token_count, int32_t* __restrict__ slot) {
+    const int a = blockIdx.x * 256 + threadIdx.x;
+    if (a >= A) return;
+    const int lo = min(max(expert_offsets[0], 0), A), hi = min(max(expert_offsets[E], 0), A);
+    const int t = token_indices[a];
+    int sl = -1;
+    if (a >= lo && a < hi && t >= 0 && t < T) sl = atomicAdd(token_count + t, 1);
+    slot[a] = sl;
+}
+
+// One workgroup: the list of (expert, first assignment, rows <= 128) tiles from
+// expert_offsets, then token_start = exclusive scan of token_count (T + 1 entries).
 __global__ __launch_bounds__(256) void k_build_mtiles(const int32_t* __restrict__ expert_offsets, int E, int A,
                                                       int max_tiles, MTile* __restrict__ tiles,
-                                                      int32_t* __restrict__ n_tiles_out) {
+                                                      int32_t* __restrict__ n_tiles_out,
+                                                      const int32_t* __restrict__ token_count, int T,
+                                                      int32_t* __restrict__ token_start) {
     __shared__ int scan[256];
     __shared__ int base_s;
     const int tid = threadIdx.x;
@@ -90,6 +116,28 @@ __global__ __launch_bounds__(256) void k_build_mtiles(const int32_t* __restrict_
     const int total = min(base_s, max_tiles);
     for (int i = total + tid; i < max_tiles; i += 256) tiles[i] = MTile{-1, 0, 0, 0};
     if (tid == 0) *n_tiles_out = total;
+
+    if (token_count == nullptr) return;
+    // every thread scans one contiguous run of tokens
+    const int per = (T + 255) / 256;
+    const int t0 = min(tid * per, T), t1 = min(t0 + per, T);
+    int local = 0;
+    for (int t = t0; t < t1; ++t) local += token_count[t];
+    __syncthreads();
+    scan[tid] = local;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {
+        const int v = tid >= d ? scan[tid - d] : 0;
+        __syncthreads();
+        scan[tid] += v;
+        __syncthreads();
+    }
+    int run = scan[tid] - local;
+    for (int t = t0; t < t1; ++t) {
+        token_start[t] = run;
+        run += token_count[t];
+    }
+    if (tid == 255) token_start[T] = scan[255];
 }
 
 // ------------------------------------------------------------------------------- gather
@@ -600,16 +648,19 @@ __device__ __forceinline__ void down_tile_loop(gptr<uint32_t> payload, gptr<__ha
 
 // grid.x = 8 * ceil(max_mtiles * n_groups / 8); workgroup = (assignment tile, group of four
 // slabs): wavefront w = all 128 assignments x the 64 output rows of slab 4*group + w.
+// Output: y[a, r] = sum_c W_down[r, c] z[a, c] as f16, r in the expert's own row order
+// (row `A` of y takes the stores of a tile's unused rows), and the per-token assignment lists
+// token_list[token_start[tok_a] + slot[a]] = (a, expert) that k_combine_tokens walks.
 __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restrict__ down_fe,
                                                       const FastSlab* __restrict__ down_fs, int max_slabs,
                                                       const uint16_t* __restrict__ z, const MTile* __restrict__ mtiles,
                                                       const int32_t* __restrict__ n_mtiles,
                                                       const int32_t* __restrict__ token_indices,
-                                                      const float* __restrict__ route_w, int T, int I, int n_tiles,
-                                                      int n_groups, int rank_out, float* __restrict__ rank_accum) {
+                                                      const int32_t* __restrict__ slot,
+                                                      const int32_t* __restrict__ token_start,
+                                                      int2* __restrict__ token_list, int A, int I, int n_tiles,
+                                                      int n_groups, _Float16* __restrict__ y, int ldy) {
     __shared__ __attribute__((aligned(16))) uint16_t lds[2][PF_M * PF_LDS_ROW];
-    __shared__ int32_t tok_s[PF_M];
-    __shared__ float rw_s[PF_M];
     const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles) * n_groups);
     if (logical < 0) return;
     const int mt_i = logical / n_groups, grp = logical - mt_i * n_groups;
@@ -618,10 +669,15 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
     const int a_begin = __builtin_amdgcn_readfirstlane(tv[1]);
     const int rows = __builtin_amdgcn_readfirstlane(tv[2]);
     if (e < 0 || rows <= 0) return;
+    const int tid = threadIdx.x;
+    if (grp == 0 && tid < rows) {
+        const int a = a_begin + tid;
+        const int sl = slot[a];
+        if (sl >= 0) token_list[token_start[token_indices[a]] + sl] = int2{a, e};
+    }
     const FastExpert fe = down_fe[e];
     const int nslabs = __builtin_amdgcn_readfirstlane(min(fe.num_slabs, max_slabs));
     if (DN_SLABS_MFMA * grp >= nslabs) return;
-    const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, kg = lane >> 4;
@@ -630,12 +686,6 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
     if (si < nslabs) fs = load_fast_slab(down_fs + (int64_t)e * max_slabs, si);
     gptr<uint32_t> payload = as_global(fe.payload);
     gptr<__half> scale = as_global(fe.scale);
-    if (tid < PF_M) {
-        const bool ok = tid < rows;
-        const int tk = ok ? token_indices[a_begin + tid] : -1;
-        tok_s[tid] = (tk >= 0 && tk < T) ? tk : -1;
-        rw_s[tid] = ok ? route_w[a_begin + tid] : 0.0f;
-    }
 
     f32x4 acc[8][4];
 #pragma unroll
@@ -644,33 +694,121 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
         for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
     // wavefronts without a slab skip the MFMAs; all execute the same barriers
     down_tile_loop(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, acc);
-    if (fs.bits == 0) return;   // (the loops end with a barrier, so tok_s / rw_s are complete)
+    if (fs.bits == 0) return;
 
-    // combine: lane holds assignments 16*mb + 4*kg + j, output rows 16*nb + n of the slab
-    gptr<int32_t> rank_idx = as_global(fe.rank_idx);
-    gptr<__half> svec = as_global(fe.s);
-    int lr[4];
-    float sv[4];
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
-        const int row = fs.rank_off + 16 * nb + n;
-        const int r = rank_idx[row];
-        lr[nb] = (r >= 0 && r < rank_out) ? r : -1;
-        sv[nb] = gload_half(svec + row);
-    }
+    // lane holds assignments 16*mb + 4*kg + j, output rows 16*nb + n of the slab
+    _Float16* ycol = y + fs.rank_off + n;
 #pragma unroll
     for (int mb = 0; mb < 8; ++mb) {
         if (16 * mb >= rows) break;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int a = 16 * mb + 4 * kg + j;
-            const int tk = tok_s[a];
-            const float rw = rw_s[a];
-            if (tk < 0) continue;
-            float* dst = rank_accum + (int64_t)tk * rank_out;
+            const int r = 16 * mb + 4 * kg + j;
+            _Float16* dst = ycol + (int64_t)(r < rows ? a_begin + r : A) * ldy;
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb)
-                if (lr[nb] >= 0) atomicAdd(dst + lr[nb], acc[mb][nb][j] * sv[nb] * rw);
+            for (int nb = 0; nb < 4; ++nb) dst[16 * nb] = (_Float16)acc[mb][nb][j];
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------- combine
+constexpr int CB_COLS = 4096;    // output columns one pass of the general form accumulates in LDS
+constexpr int CB_SORT = 256;     // list entries ordered at a time
+
+// rank_accum[t, rank_idx_e[r]] = sum over the assignments (a, e) of token t, in ascending a,
+// of route_w[a] * s_e[r] * y[a, r].  One workgroup per token; it writes every column of its
+// row, so rank_accum needs no zero fill.  IDENTITY: rank_idx_e[r] == r in every expert, and a
+// thread keeps its eight columns in registers; otherwise the row is accumulated in LDS, one
+// assignment after the other.
+template <bool IDENTITY>
+__global__ __launch_bounds__(256) void k_combine_tokens(const FastExpert* __restrict__ down_fe, int max_slabs,
+                                                        const _Float16* __restrict__ y, int ldy,
+                                                        const int32_t* __restrict__ token_start,
+                                                        const int2* __restrict__ token_list,
+                                                        const float* __restrict__ route_w, int rank_out,
+                                                        float* __restrict__ rank_accum) {
+    __shared__ __attribute__((aligned(16))) float out_s[IDENTITY ? 4 : CB_COLS];
+    __shared__ int2 raw_s[CB_SORT];
+    __shared__ const _Float16* y_s[CB_SORT];
+    __shared__ const __half* s_s[CB_SORT];
+    __shared__ const int32_t* idx_s[CB_SORT];
+    __shared__ int nrow_s[CB_SORT];
+    __shared__ float rw_s[CB_SORT];
+    const int t = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int begin = token_start[t], count = token_start[t + 1] - begin;
+    float* out_row = rank_accum + (int64_t)t * rank_out;
+    constexpr int STEP = IDENTITY ? 256 * 8 : CB_COLS;
+    for (int c0 = 0; c0 < rank_out; c0 += STEP) {
+        const int cols = min(STEP, rank_out - c0);
+        float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (!IDENTITY)
+            for (int i = tid; i < cols; i += 256) out_s[i] = 0.0f;
+        for (int l0 = 0; l0 < count; l0 += CB_SORT) {
+            const int nl = min(CB_SORT, count - l0);
+            __syncthreads();
+            if (tid < nl) raw_s[tid] = token_list[begin + l0 + tid];
+            __syncthreads();
+            if (tid < nl) {      // the lists were filled in arbitrary order: sort by assignment
+                const int2 mine = raw_s[tid];
+                int pos = 0;
+                for (int i = 0; i < nl; ++i) pos += raw_s[i].x < mine.x;
+                const FastExpert fe = down_fe[mine.y];
+                y_s[pos] = y + (int64_t)mine.x * ldy;
+                s_s[pos] = fe.s;
+                idx_s[pos] = fe.rank_idx;
+                nrow_s[pos] = min(fe.num_slabs, max_slabs) * SLAB_ROWS;
+                rw_s[pos] = route_w[mine.x];
+            }
+            __syncthreads();
+            if (IDENTITY) {
+                const int r0 = c0 + tid * 8;
+                for (int i = 0; i < nl; ++i) {
+                    if (r0 >= nrow_s[i]) continue;
+                    const u32x4 yv = *reinterpret_cast<const u32x4*>(y_s[i] + r0);
+                    const u32x4 sv = *reinterpret_cast<gptr<u32x4>>(as_global(s_s[i]) + r0);
+                    const float rw = rw_s[i];
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        const uint32_t yw = yv[k >> 1], sw = sv[k >> 1];
+                        const h2 yp = __builtin_bit_cast(h2, yw);
+                        const h2 sp = __builtin_bit_cast(h2, sw);
+                        acc[k] += (float)yp[k & 1] * (float)sp[k & 1] * rw;
+                    }
+                }
+            } else {
+                for (int i = 0; i < nl; ++i) {
+                    const int nrow = nrow_s[i];
+                    const float rw = rw_s[i];
+                    gptr<int32_t> rank_idx = as_global(idx_s[i]);
+                    gptr<__half> svec = as_global(s_s[i]);
+                    const _Float16* yrow = y_s[i];
+                    for (int r0 = tid * 8; r0 < nrow; r0 += 256 * 8) {
+                        const u32x4 yv = *reinterpret_cast<const u32x4*>(yrow + r0);
+                        const u32x4 sv = *reinterpret_cast<gptr<u32x4>>(svec + r0);
+                        const i32x4 ia = *reinterpret_cast<gptr<i32x4>>(rank_idx + r0);
+                        const i32x4 ib = *reinterpret_cast<gptr<i32x4>>(rank_idx + r0 + 4);
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) {
+                            const uint32_t yw = yv[k >> 1], sw = sv[k >> 1];
+                            const h2 yp = __builtin_bit_cast(h2, yw);
+                            const h2 sp = __builtin_bit_cast(h2, sw);
+                            const int col = (k < 4 ? ia[k & 3] : ib[k & 3]) - c0;
+                            if (col >= 0 && col < cols) atomicAdd(out_s + col, (float)yp[k & 1] * (float)sp[k & 1] * rw);
+                        }
+                    }
+                    __syncthreads();    // entries are added one after the other: the sum has one order
+                }
+            }
+        }
+        if (IDENTITY) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (tid * 8 + k < cols) out_row[c0 + tid * 8 + k] = acc[k];
+        } else {
+            __syncthreads();
+            for (int i = tid; i < cols; i += 256) out_row[c0 + i] = out_s[i];
+            __syncthreads();
         }
     }
 }
@@ -692,14 +830,37 @@ static bool direct_ok(const bitsmoe_matset* gate, const bitsmoe_matset* up) {
 }
 static inline int direct_ld(const bitsmoe_matset* set) { return (set->max_rank_plus1 + 7) / 8 * 8; }
 
-size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, int64_t T, int64_t A, int I) {
+// Carving of the workspace, shared by the size query and the launcher.
+struct MfmaWorkspace {
+    size_t mtiles, n_mtiles, token_count, token_start, slot, token_list, acts, z, u, y, total;
+};
+static MfmaWorkspace mfma_workspace(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                                    int64_t T, int64_t A, int I) {
     const int64_t max_mtiles = A / PF_M + gate->n_experts;
     const size_t direct = align256((size_t)T * direct_ld(gate) * 2) + align256((size_t)T * direct_ld(up) * 2);
     const size_t gathered = align256((size_t)A * gate->max_slabs * SLAB_ROWS * 2) + align256((size_t)A * up->max_slabs * SLAB_ROWS * 2);
+    MfmaWorkspace w;
+    size_t at = 0;
+    auto take = [&](size_t bytes) { const size_t here = at; at += align256(bytes); return here; };
+    w.mtiles = take((size_t)max_mtiles * sizeof(MTile));
+    w.n_mtiles = take(256);
+    w.token_count = take((size_t)(T + 1) * 4);
+    w.token_start = take((size_t)(T + 1) * 4);
+    w.slot = take((size_t)A * 4);
+    w.token_list = take((size_t)A * 8);
     // the direct form falls back to the gathered one when the activation pointers or row
     // lengths do not allow 16-byte loads, which is only known at the call
-    return align256((size_t)max_mtiles * sizeof(MTile)) + 256 + std::max(direct_ok(gate, up) ? direct : 0, gathered) +
-           2 * align256((size_t)A * I * 2);
+    w.acts = take(std::max(direct_ok(gate, up) ? direct : 0, gathered));
+    w.z = take((size_t)A * I * 2);
+    w.u = take((size_t)A * I * 2);
+    w.y = take((size_t)(A + 1) * down->max_slabs * SLAB_ROWS * 2);
+    w.total = at;
+    return w;
+}
+
+size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int64_t T,
+                            int64_t A, int I) {
+    return mfma_workspace(gate, up, down, T, A, I).total;
 }
 
 int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
@@ -713,21 +874,27 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
                         T * (int64_t)std::max(Rg, Ru) < ((int64_t)1 << 31);
     const int ldg = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(gate) : Rg) : gate->max_slabs * SLAB_ROWS;
     const int ldu = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(up) : Ru) : up->max_slabs * SLAB_ROWS;
+    const MfmaWorkspace w = mfma_workspace(gate, up, down, T, A, I);
     char* ws = (char*)workspace;
-    MTile* mtiles = (MTile*)ws;
-    ws += align256((size_t)max_mtiles * sizeof(MTile));
-    int32_t* n_mtiles = (int32_t*)ws;
-    ws += 256;
-    const uint16_t* Hs_g = (const uint16_t*)ws;
-    ws += direct ? align256((size_t)T * direct_ld(gate) * 2) : align256((size_t)A * ldg * 2);
-    const uint16_t* Hs_u = (const uint16_t*)ws;
-    ws = (char*)workspace + mfma_workspace_bytes(gate, up, T, A, I) - 2 * align256((size_t)A * I * 2);
-    uint16_t* z = (uint16_t*)ws;     // gate output, then silu(gate) * up in place
-    uint16_t* Ubuf = (uint16_t*)(ws + align256((size_t)A * I * 2));
+    MTile* mtiles = (MTile*)(ws + w.mtiles);
+    int32_t* n_mtiles = (int32_t*)(ws + w.n_mtiles);
+    int32_t* token_count = (int32_t*)(ws + w.token_count);
+    int32_t* token_start = (int32_t*)(ws + w.token_start);
+    int32_t* slot = (int32_t*)(ws + w.slot);
+    int2* token_list = (int2*)(ws + w.token_list);
+    const uint16_t* Hs_g = (const uint16_t*)(ws + w.acts);
+    const uint16_t* Hs_u = (const uint16_t*)(ws + w.acts + (direct ? align256((size_t)T * direct_ld(gate) * 2) : align256((size_t)A * ldg * 2)));
+    uint16_t* z = (uint16_t*)(ws + w.z);     // gate output, then silu(gate) * up in place
+    uint16_t* Ubuf = (uint16_t*)(ws + w.u);
+    _Float16* y = (_Float16*)(ws + w.y);
+    const int ldy = down->max_slabs * SLAB_ROWS;
 
     record(prof, 0, st);
-    BITSMOE_REQUIRE(launch_fill_zero(rank_accum, T * (int64_t)rank_out, st) == BITSMOE_OK, "zero fill failed");
-    hipLaunchKernelGGL(k_build_mtiles, dim3(1), dim3(256), 0, st, off, E, (int)A, (int)max_mtiles, mtiles, n_mtiles);
+    BITSMOE_REQUIRE(launch_fill_zero((float*)token_count, T + 1, st) == BITSMOE_OK, "zero fill failed");
+    hipLaunchKernelGGL(k_token_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, st, tok, off, E, (int)A, (int)T,
+                       token_count, slot);
+    hipLaunchKernelGGL(k_build_mtiles, dim3(1), dim3(256), 0, st, off, E, (int)A, (int)max_mtiles, mtiles, n_mtiles,
+                       token_count, (int)T, token_start);
     BITSMOE_HIP_TRY(hipGetLastError());
     if (direct) {
         if (act_dtype == BITSMOE_DT_BF16) {
@@ -776,8 +943,14 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
         const int n_pairs = (down->max_slabs + DN_SLABS_MFMA - 1) / DN_SLABS_MFMA;
         const int64_t wgs = (max_mtiles * n_pairs + 7) / 8 * 8;
         hipLaunchKernelGGL(k_down_mfma, dim3((unsigned)wgs), dim3(256), 0, st, down->d_fast_experts, down->d_fast_slabs,
-                           down->max_slabs, z, mtiles, n_mtiles, tok, rw, (int)T, I, n_tiles, n_pairs, rank_out,
-                           rank_accum);
+                           down->max_slabs, z, mtiles, n_mtiles, tok, slot, token_start, token_list, (int)A, I, n_tiles,
+                           n_pairs, y, ldy);
+        if (down->rank_identity)
+            hipLaunchKernelGGL(k_combine_tokens<true>, dim3((unsigned)T), dim3(256), 0, st, down->d_fast_experts,
+                               down->max_slabs, y, ldy, token_start, token_list, rw, rank_out, rank_accum);
+        else
+            hipLaunchKernelGGL(k_combine_tokens<false>, dim3((unsigned)T), dim3(256), 0, st, down->d_fast_experts,
+                               down->max_slabs, y, ldy, token_start, token_list, rw, rank_out, rank_accum);
         BITSMOE_HIP_TRY(hipGetLastError());
     }
     record(prof, 3, st);

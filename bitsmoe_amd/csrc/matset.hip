@@ -145,7 +145,7 @@ extern "C" int bitsmoe_matset_create(const bitsmoe_matrix_desc* descs, int32_t n
     std::vector<SlabTask> tasks;
     std::vector<int32_t> rk;
     int max_rank = -1, min_rank = 0x7fffffff;
-    bool chunked8 = n_experts > 0;
+    bool chunked8 = n_experts > 0, identity = n_experts > 0;
     for (int e = 0; e < n_experts; ++e) {
         const bitsmoe_matrix_desc& d = descs[e];
         BITSMOE_REQUIRE(d.num_slabs >= 0 && d.num_tiles >= 0 && d.rank_len >= 0 && d.payload_words >= 0 && d.scale_len >= 0,
@@ -175,6 +175,7 @@ extern "C" int bitsmoe_matset_create(const bitsmoe_matrix_desc* descs, int32_t n
             max_rank = std::max(max_rank, v);
             min_rank = std::min(min_rank, v);
         }
+        for (size_t k = 0; k < rk.size() && identity; ++k) identity = rk[k] == (int32_t)k;
         for (int si = 0; si < d.num_slabs && chunked8; ++si)
             if (slab[si * 4 + 2] != si * K_SLAB) chunked8 = false;
         if (d.rank_len % 8 != 0) chunked8 = false;
@@ -198,6 +199,7 @@ extern "C" int bitsmoe_matset_create(const bitsmoe_matrix_desc* descs, int32_t n
         for (int s = 0; s < d.num_slabs; ++s) tasks.push_back(SlabTask{e, s});
     }
     set->rank_chunked8 = chunked8;
+    set->rank_identity = identity;
     set->total_slabs = (int64_t)tasks.size();
     set->max_rank_plus1 = max_rank + 1;
     set->min_rank = (min_rank == 0x7fffffff) ? 0 : min_rank;
