@@ -257,6 +257,71 @@ def test_forward_mfma_path_scattered_ranks(cuda_device, dtype_name):
     assert err < 3e-3
 
 
+def _scramble_down_ranks(rng, down, rank_out):
+    """Down rows write permuted output ranks; two rows share a rank and two rows are dropped
+    (rank_idx outside [0, rank_out) is skipped, bitsmoe/algorithms/cpp/mlp_forward.cu:1782)."""
+    for m in down:
+        idx = rng.permutation(rank_out).astype(np.int32)[m["rank_idx"]]
+        idx[5] = idx[9]
+        idx[11] = -1
+        idx[17] = rank_out + 3
+        m["rank_idx"] = idx
+
+
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+def test_forward_mfma_path_scattered_output_ranks(cuda_device, dtype_name):
+    """The combine in its general form: arbitrary, repeated and dropped output ranks."""
+    import torch
+
+    from bitsmoe_amd.algorithms import _capi
+
+    hip = _hip()
+    rng = np.random.default_rng(77)
+    e, t, k, rin, rout, dim = 3, 260, 2, 128, 192, 256
+    gate, up, down = helpers.make_experts(77, e, rin, rout, dim, slab_multiple=64)
+    _scramble_down_ranks(rng, down, rout)
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    h_gate = torch.from_numpy(rng.normal(size=(t, rin)).astype(np.float32)).to(dt)
+    h_up = torch.from_numpy(rng.normal(size=(t, rin)).astype(np.float32)).to(dt)
+    idx, w = o.router_qwen(rng.normal(size=(t, e)).astype(np.float32), k)
+    tok, off, rw = o.build_routing(idx, w, np.arange(e, dtype=np.int32), e)
+    ref = o.moe_forward(h_gate.float().numpy(), h_up.float().numpy(), tok, off, rw, gate, up, down, rout, dim)
+    sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=dim) for m in (gate, up, down)]
+    outs = [hip.moe_forward_sets(h_gate.to(cuda_device), h_up.to(cuda_device), torch.from_numpy(tok).to(cuda_device),
+                                 torch.from_numpy(off).to(cuda_device), torch.from_numpy(rw).to(cuda_device),
+                                 sets[0], sets[1], sets[2], rout, dim, 0, path=_capi.PATH_MFMA).cpu().numpy()
+            for _ in range(2)]
+    assert helpers.norm_err(outs[0], ref) < 3e-3
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))     # one summation order
+
+
+@pytest.mark.parametrize("scramble", [False, True])
+def test_forward_mfma_path_token_with_many_assignments(cuda_device, scramble):
+    """A token may appear any number of times in the assignment list (here 310 times, more
+    than the combine orders in one go), and out of token order inside an expert."""
+    import torch
+
+    from bitsmoe_amd.algorithms import _capi
+
+    hip = _hip()
+    rng = np.random.default_rng(78)
+    e, t, rin, rout, dim = 2, 3, 128, 128, 128
+    gate, up, down = helpers.make_experts(78, e, rin, rout, dim, slab_multiple=64)
+    if scramble:
+        _scramble_down_ranks(rng, down, rout)
+    h_gate = torch.from_numpy(rng.normal(size=(t, rin)).astype(np.float32)).to(torch.float16)
+    h_up = torch.from_numpy(rng.normal(size=(t, rin)).astype(np.float32)).to(torch.float16)
+    tok = np.array([0] * 150 + [1] * 5 + [0] * 150 + [0] * 10 + [2] * 4, dtype=np.int32)
+    off = np.array([0, 305, 319], dtype=np.int32)
+    rw = rng.uniform(0.0, 0.05, size=tok.size).astype(np.float32)
+    ref = o.moe_forward(h_gate.float().numpy(), h_up.float().numpy(), tok, off, rw, gate, up, down, rout, dim)
+    sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=dim) for m in (gate, up, down)]
+    out = hip.moe_forward_sets(h_gate.to(cuda_device), h_up.to(cuda_device), torch.from_numpy(tok).to(cuda_device),
+                               torch.from_numpy(off).to(cuda_device), torch.from_numpy(rw).to(cuda_device),
+                               sets[0], sets[1], sets[2], rout, dim, 0, path=_capi.PATH_MFMA).cpu().numpy()
+    assert helpers.norm_err(out, ref) < 3e-3
+
+
 def test_forward_mfma_path_needs_prepared_sets(cuda_device):
     import torch
 
