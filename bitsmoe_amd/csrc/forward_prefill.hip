@@ -118,11 +118,20 @@ __global__ __launch_bounds__(256) void k_build_mtiles(const int32_t* __restrict_
     if (tid == 0) *n_tiles_out = total;
 
     if (token_count == nullptr) return;
-    // every thread scans one contiguous run of tokens
-    const int per = (T + 255) / 256;
+    // every thread scans one contiguous run of tokens (a multiple of four: 16-byte loads)
+    const int per = ((T + 255) / 256 + 3) / 4 * 4;
     const int t0 = min(tid * per, T), t1 = min(t0 + per, T);
+    const bool whole = t1 - t0 == per;
     int local = 0;
-    for (int t = t0; t < t1; ++t) local += token_count[t];
+    if (whole) {
+#pragma unroll 4
+        for (int t = t0; t < t1; t += 4) {
+            const i32x4 v = *reinterpret_cast<const i32x4*>(token_count + t);
+            local += v[0] + v[1] + v[2] + v[3];
+        }
+    } else {
+        for (int t = t0; t < t1; ++t) local += token_count[t];
+    }
     __syncthreads();
     scan[tid] = local;
     __syncthreads();
@@ -133,9 +142,23 @@ __global__ __launch_bounds__(256) void k_build_mtiles(const int32_t* __restrict_
         __syncthreads();
     }
     int run = scan[tid] - local;
-    for (int t = t0; t < t1; ++t) {
-        token_start[t] = run;
-        run += token_count[t];
+    if (whole) {
+#pragma unroll 4
+        for (int t = t0; t < t1; t += 4) {
+            const i32x4 v = *reinterpret_cast<const i32x4*>(token_count + t);
+            i32x4 o;
+            o[0] = run;
+            o[1] = o[0] + v[0];
+            o[2] = o[1] + v[1];
+            o[3] = o[2] + v[2];
+            run = o[3] + v[3];
+            *reinterpret_cast<i32x4*>(token_start + t) = o;
+        }
+    } else {
+        for (int t = t0; t < t1; ++t) {
+            token_start[t] = run;
+            run += token_count[t];
+        }
     }
     if (tid == 255) token_start[T] = scan[255];
 }
@@ -208,9 +231,15 @@ __global__ __launch_bounds__(256) void k_pregather(const FastExpert* __restrict_
     }
 }
 
-// bf16 activations [T, R] -> f16 [T, ld] (columns < ld <= R); grid-stride over 8-element groups.
-__global__ __launch_bounds__(256) void k_bf16_to_f16(const uint16_t* __restrict__ src, int64_t T, int R, int ld,
-                                                     uint16_t* __restrict__ dst) {
+// bf16 activations [T, R] -> f16 [T, ld] (columns < ld <= R); blockIdx.y = 0: gate, 1: up;
+// grid-stride over 8-element groups.
+__global__ __launch_bounds__(256) void k_bf16_to_f16(const uint16_t* __restrict__ src_g, const uint16_t* __restrict__ src_u,
+                                                     int64_t T, int Rg, int Ru, int ldg, int ldu,
+                                                     uint16_t* __restrict__ dst_g, uint16_t* __restrict__ dst_u) {
+    const bool is_up = blockIdx.y != 0;
+    const uint16_t* src = is_up ? src_u : src_g;
+    uint16_t* dst = is_up ? dst_u : dst_g;
+    const int R = is_up ? Ru : Rg, ld = is_up ? ldu : ldg;
     const int per_row = ld >> 3;
     const int64_t total = T * per_row;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
@@ -898,8 +927,10 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     BITSMOE_HIP_TRY(hipGetLastError());
     if (direct) {
         if (act_dtype == BITSMOE_DT_BF16) {
-            hipLaunchKernelGGL(k_bf16_to_f16, dim3(1024), dim3(256), 0, st, (const uint16_t*)h_gate, T, Rg, ldg, (uint16_t*)Hs_g);
-            hipLaunchKernelGGL(k_bf16_to_f16, dim3(1024), dim3(256), 0, st, (const uint16_t*)h_up, T, Ru, ldu, (uint16_t*)Hs_u);
+            const int64_t groups = T * (std::max(ldg, ldu) / 8);
+            hipLaunchKernelGGL(k_bf16_to_f16, dim3((unsigned)std::min<int64_t>((groups + 255) / 256, 2048), 2), dim3(256), 0, st,
+                               (const uint16_t*)h_gate, (const uint16_t*)h_up, T, Rg, Ru, ldg, ldu, (uint16_t*)Hs_g,
+                               (uint16_t*)Hs_u);
             BITSMOE_HIP_TRY(hipGetLastError());
         } else {
             Hs_g = (const uint16_t*)h_gate;
