@@ -43,11 +43,16 @@ __device__ inline void chunk_ranks(const IdT* __restrict__ selected, const int32
     const int lane = tid & 63;
     const int wave = tid >> 6;
     for (int e = tid; e < n_packed; e += ROUTE_THREADS) hist[e] = 0;
+    // all rounds' ids first: their (dependent) loads overlap instead of queueing behind the barriers
+#pragma unroll
+    for (int j = 0; j < ROUTE_ROUNDS; ++j)
+        local[j] = load_local_id<IdT>(selected, g2l, n_global, n_packed, chunk_base + (int64_t)j * ROUTE_THREADS + tid, n_flat);
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < ROUTE_ROUNDS; ++j) {
-        const int64_t idx = chunk_base + (int64_t)j * ROUTE_THREADS + tid;
-        const int id = load_local_id<IdT>(selected, g2l, n_global, n_packed, idx, n_flat);
+        rank[j] = 0;
+        if (chunk_base + (int64_t)j * ROUTE_THREADS >= n_flat) continue;     // (uniform) a round without entries
+        const int id = local[j];
         const uint64_t same = match_same_id(id, id_bits);
         const int before = __popcll(same & ((1ull << lane) - 1ull));
         const int count = __popcll(same);
@@ -59,9 +64,69 @@ __device__ inline void chunk_ranks(const IdT* __restrict__ selected, const int32
             if (wave == wv && last) hist[id] = old + count;
             __syncthreads();
         }
-        local[j] = id;
         rank[j] = old + before;
     }
+}
+
+// The same result with three barriers instead of two per (round, wavefront): every (round,
+// wavefront) pair counts into its own table, then one pass per expert turns the tables into
+// "entries of this expert before my (round, wavefront)".  tables: ROUTE_ROUNDS * 4 * n_packed ints.
+constexpr int ROUTE_TABLE_MAX_EXPERTS = 512;
+constexpr int ROUTE_G2L_LDS_MAX = 4096;      // global expert ids whose map is staged in LDS
+template <typename IdT>
+__device__ inline void chunk_ranks_tables(const IdT* __restrict__ selected, const int32_t* __restrict__ g2l,
+                                          int n_global, int n_packed, int id_bits, int64_t chunk_base,
+                                          int64_t n_flat, int* hist, int* tables, int* g2l_lds,
+                                          int (&local)[ROUTE_ROUNDS], int (&rank)[ROUTE_ROUNDS]) {
+    constexpr int WAVES = ROUTE_THREADS / 64;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int64_t left = n_flat - chunk_base;
+    const int rounds = (int)((left < ROUTE_CHUNK ? left : ROUTE_CHUNK) + ROUTE_THREADS - 1) / ROUTE_THREADS;   // uniform
+    for (int i = tid; i < rounds * WAVES * n_packed; i += ROUTE_THREADS) tables[i] = 0;
+    // the global-to-local map is copied to LDS (g2l_lds != nullptr) while the ids are on their
+    // way, so that the look-up is not a second global round trip
+    int64_t raw[ROUTE_ROUNDS];
+#pragma unroll
+    for (int j = 0; j < ROUTE_ROUNDS; ++j) {
+        const int64_t idx = chunk_base + (int64_t)j * ROUTE_THREADS + tid;
+        raw[j] = idx < n_flat ? (int64_t)selected[idx] : -1;
+    }
+    if (g2l_lds != nullptr) {
+        for (int i = tid; i < n_global; i += ROUTE_THREADS) g2l_lds[i] = g2l[i];
+        __syncthreads();
+    }
+#pragma unroll
+    for (int j = 0; j < ROUTE_ROUNDS; ++j) {
+        int l = -1;
+        if (raw[j] >= 0 && raw[j] < n_global) l = g2l_lds != nullptr ? g2l_lds[raw[j]] : g2l[raw[j]];
+        local[j] = (l >= 0 && l < n_packed) ? l : -1;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < ROUTE_ROUNDS; ++j) {
+        rank[j] = 0;
+        if (j >= rounds) continue;
+        const int id = local[j];
+        const uint64_t same = match_same_id(id, id_bits);
+        rank[j] = __popcll(same & ((1ull << lane) - 1ull));
+        if (id >= 0 && lane == 63 - __clzll((long long)same)) tables[(j * WAVES + wave) * n_packed + id] = __popcll(same);
+    }
+    __syncthreads();
+    for (int e = tid; e < n_packed; e += ROUTE_THREADS) {
+        int run = 0;
+        for (int t = 0; t < rounds * WAVES; ++t) {
+            const int c = tables[t * n_packed + e];
+            tables[t * n_packed + e] = run;
+            run += c;
+        }
+        hist[e] = run;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < ROUTE_ROUNDS; ++j)
+        if (j < rounds && local[j] >= 0) rank[j] += tables[(j * WAVES + wave) * n_packed + local[j]];
 }
 
 // Exclusive scan of data[0..n) in LDS by the whole workgroup; returns the total.
@@ -111,9 +176,21 @@ __global__ __launch_bounds__(ROUTE_THREADS) void k_route_fused(
     int* hist = lds;
     int* wave_sums = lds + n_packed;
     int local[ROUTE_ROUNDS], rank[ROUTE_ROUNDS];
-    chunk_ranks<IdT>(selected, g2l, n_global, n_packed, id_bits, 0, n_flat, hist, local, rank);
-    const int total = block_exclusive_scan(hist, n_packed, wave_sums);
     const int tid = threadIdx.x;
+    // the weights are only needed by the scatter: requested first, they arrive while the ranks are built
+    float w[ROUTE_ROUNDS];
+#pragma unroll
+    for (int j = 0; j < ROUTE_ROUNDS; ++j) {
+        const int64_t idx = (int64_t)j * ROUTE_THREADS + tid;
+        w[j] = idx < n_flat ? weights[idx] : 0.0f;
+    }
+    if (n_packed <= ROUTE_TABLE_MAX_EXPERTS)
+        chunk_ranks_tables<IdT>(selected, g2l, n_global, n_packed, id_bits, 0, n_flat, hist, lds + n_packed + 32,
+                                n_global <= ROUTE_G2L_LDS_MAX ? lds + n_packed + 32 + ROUTE_ROUNDS * (ROUTE_THREADS / 64) * n_packed : nullptr,
+                                local, rank);
+    else
+        chunk_ranks<IdT>(selected, g2l, n_global, n_packed, id_bits, 0, n_flat, hist, local, rank);
+    const int total = block_exclusive_scan(hist, n_packed, wave_sums);
     for (int e = tid; e < n_packed; e += ROUTE_THREADS) expert_offsets[e] = hist[e];
     if (tid == 0) expert_offsets[n_packed] = total;
 #pragma unroll
@@ -122,7 +199,7 @@ __global__ __launch_bounds__(ROUTE_THREADS) void k_route_fused(
             const int64_t idx = (int64_t)j * ROUTE_THREADS + tid;
             const int pos = hist[local[j]] + rank[j];
             token_indices[pos] = (int32_t)(idx / top_k);
-            route_flat[pos] = weights[idx];
+            route_flat[pos] = w[j];
         }
     }
 }
@@ -136,7 +213,12 @@ __global__ __launch_bounds__(ROUTE_THREADS) void k_route_count(
     int* hist = lds;
     int local[ROUTE_ROUNDS], rank[ROUTE_ROUNDS];
     const int64_t chunk_base = (int64_t)blockIdx.x * ROUTE_CHUNK;
-    chunk_ranks<IdT>(selected, g2l, n_global, n_packed, id_bits, chunk_base, n_flat, hist, local, rank);
+    if (n_packed <= ROUTE_TABLE_MAX_EXPERTS)
+        chunk_ranks_tables<IdT>(selected, g2l, n_global, n_packed, id_bits, chunk_base, n_flat, hist, lds + n_packed + 32,
+                                n_global <= ROUTE_G2L_LDS_MAX ? lds + n_packed + 32 + ROUTE_ROUNDS * (ROUTE_THREADS / 64) * n_packed : nullptr,
+                                local, rank);
+    else
+        chunk_ranks<IdT>(selected, g2l, n_global, n_packed, id_bits, chunk_base, n_flat, hist, local, rank);
     const int tid = threadIdx.x;
 #pragma unroll
     for (int j = 0; j < ROUTE_ROUNDS; ++j) {
@@ -191,8 +273,13 @@ static int route_impl(const IdT* selected, const float* weights, const int32_t* 
     int id_bits = 0;
     while ((1 << id_bits) < n_packed) ++id_bits;
     const size_t lds_bytes = (size_t)(n_packed + 32) * sizeof(int);
+    // histogram + wave sums, and the per-(round, wavefront) tables of the low-barrier variant
+    const size_t lds_rank_bytes = lds_bytes + (n_packed <= ROUTE_TABLE_MAX_EXPERTS
+                                                   ? ((size_t)ROUTE_ROUNDS * (ROUTE_THREADS / 64) * n_packed +
+                                                      (n_global <= ROUTE_G2L_LDS_MAX ? n_global : 0)) * sizeof(int)
+                                                   : 0);
     if (n_flat <= ROUTE_CHUNK) {
-        hipLaunchKernelGGL(k_route_fused<IdT>, dim3(1), dim3(ROUTE_THREADS), lds_bytes, st, selected, weights,
+        hipLaunchKernelGGL(k_route_fused<IdT>, dim3(1), dim3(ROUTE_THREADS), lds_rank_bytes, st, selected, weights,
                            g2l, n_global, n_flat, top_k, n_packed, id_bits, token_indices, expert_offsets,
                            route_flat);
         BITSMOE_HIP_TRY(hipGetLastError());
@@ -201,7 +288,7 @@ static int route_impl(const IdT* selected, const float* weights, const int32_t* 
     const int64_t n_chunks = (n_flat + ROUTE_CHUNK - 1) / ROUTE_CHUNK;
     int32_t* entry_rank = (int32_t*)workspace;
     int32_t* chunk_hist = entry_rank + ((n_flat + 63) / 64) * 64;
-    hipLaunchKernelGGL(k_route_count<IdT>, dim3((unsigned)n_chunks), dim3(ROUTE_THREADS), lds_bytes, st,
+    hipLaunchKernelGGL(k_route_count<IdT>, dim3((unsigned)n_chunks), dim3(ROUTE_THREADS), lds_rank_bytes, st,
                        selected, g2l, n_global, n_flat, n_packed, id_bits, entry_rank, chunk_hist);
     BITSMOE_HIP_TRY(hipGetLastError());
     hipLaunchKernelGGL(k_route_scan, dim3(1), dim3(1024), lds_bytes, st, chunk_hist, (int)n_chunks, n_packed,
