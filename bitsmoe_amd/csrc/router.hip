@@ -100,6 +100,78 @@ __global__ __launch_bounds__(256) void k_router_softmax_topk(const void* __restr
     }
 }
 
+// The same result for at most 256 experts without the k dependent arg-max rounds: every lane
+// counts, for each of its (up to four) logits, how many of the token's logits precede it in
+// the order (value descending, expert index ascending); that count is the position of the
+// expert in the top-k list.  The logits of a token sit in LDS and are read as broadcasts.
+// grid = ceil(T / 4), 256 threads (one wavefront per token).
+constexpr int ROUTER_RANK_PER_LANE = 4;
+template <int DT>
+__global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict__ logits, int T, int E, int k,
+                                                          int renorm, int round_dt, int32_t* __restrict__ sel32,
+                                                          int64_t* __restrict__ sel64, float* __restrict__ weights) {
+    // sort key of a logit: the float mapped to an unsigned integer of the same order, above the
+    // complemented expert index, so that one 64-bit comparison is "precedes in the top-k order"
+    __shared__ __attribute__((aligned(16))) uint64_t keys[4][64 * ROUTER_RANK_PER_LANE];
+    __shared__ float picked[4][64];
+    const int lane = threadIdx.x & 63;
+    const int wv = threadIdx.x >> 6;
+    const int tkn = blockIdx.x * 4 + wv;
+    if (tkn >= T) return;            // (no workgroup barrier below: a wavefront only reads what it wrote)
+    const int e2 = (E + 1) & ~1;
+    float v[ROUTER_RANK_PER_LANE];
+    uint64_t mine[ROUTER_RANK_PER_LANE];
+    float vmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) {
+        const int e = lane + 64 * i;
+        v[i] = e < E ? load_logit<DT>(logits, (int64_t)tkn * E + e) : -INFINITY;
+        vmax = fmaxf(vmax, v[i]);
+        const uint32_t bits = __float_as_uint(v[i] + 0.0f);      // (-0 and +0 are one value)
+        const uint32_t ordered = bits ^ ((bits >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+        mine[i] = e < E ? ((uint64_t)ordered << 32) | (uint32_t)(0xFFFFFFFFu - (uint32_t)e) : 0ull;   // padding sorts last
+        keys[wv][e] = mine[i];
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, d));
+    float pr[ROUTER_RANK_PER_LANE];
+    float part = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) {
+        pr[i] = (v[i] == -INFINITY) ? 0.0f : expf(v[i] - vmax);
+        part += pr[i];
+    }
+    const float denom = wave_sum(part);
+    int rank[ROUTER_RANK_PER_LANE] = {0, 0, 0, 0};
+#pragma unroll 4
+    for (int o = 0; o < e2; o += 2) {
+        const uint64_t q0 = keys[wv][o], q1 = keys[wv][o + 1];
+#pragma unroll
+        for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) rank[i] += (int)(q0 > mine[i]) + (int)(q1 > mine[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i)
+        if (lane + 64 * i < E && rank[i] < k) picked[wv][rank[i]] = pr[i] / denom;
+    // (LDS operations of one wavefront complete in order)
+    float picked_sum = 0.0f;
+    for (int j = 0; j < k; ++j) picked_sum += picked[wv][j];
+#pragma unroll
+    for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) {
+        if (lane + 64 * i < E && rank[i] < k) {
+            float w = pr[i] / denom;
+            if (renorm) w /= picked_sum;
+            if (round_dt == BITSMOE_DT_F16)
+                w = __half2float(__float2half(w));
+            else if (round_dt == BITSMOE_DT_BF16)
+                w = __bfloat162float(__float2bfloat16(w));
+            const int64_t o = (int64_t)tkn * k + rank[i];
+            if (sel32) sel32[o] = lane + 64 * i;
+            if (sel64) sel64[o] = lane + 64 * i;
+            weights[o] = w;
+        }
+    }
+}
+
 }  // namespace bitsmoe
 
 using namespace bitsmoe;
@@ -119,15 +191,18 @@ extern "C" int bitsmoe_router_softmax_topk(const void* logits, int32_t logits_dt
     int32_t* s32 = ids_are_i64 ? nullptr : (int32_t*)selected;
     int64_t* s64 = ids_are_i64 ? (int64_t*)selected : nullptr;
     const dim3 grid((unsigned)((n_tokens + 3) / 4));
-    if (logits_dtype == 0)
-        hipLaunchKernelGGL(k_router_softmax_topk<0>, grid, dim3(256), 0, st, logits, (int)n_tokens, n_experts, top_k,
-                           renormalize, round_dtype, s32, s64, weights);
-    else if (logits_dtype == 1)
-        hipLaunchKernelGGL(k_router_softmax_topk<1>, grid, dim3(256), 0, st, logits, (int)n_tokens, n_experts, top_k,
-                           renormalize, round_dtype, s32, s64, weights);
-    else
-        hipLaunchKernelGGL(k_router_softmax_topk<2>, grid, dim3(256), 0, st, logits, (int)n_tokens, n_experts, top_k,
-                           renormalize, round_dtype, s32, s64, weights);
+    const bool by_rank = n_experts <= 64 * ROUTER_RANK_PER_LANE;
+#define BITSMOE_ROUTER_LAUNCH(KERNEL)                                                                              \
+    hipLaunchKernelGGL(KERNEL, grid, dim3(256), 0, st, logits, (int)n_tokens, n_experts, top_k, renormalize, \
+                       round_dtype, s32, s64, weights)
+    if (logits_dtype == 0) {
+        if (by_rank) BITSMOE_ROUTER_LAUNCH(k_router_rank_topk<0>); else BITSMOE_ROUTER_LAUNCH(k_router_softmax_topk<0>);
+    } else if (logits_dtype == 1) {
+        if (by_rank) BITSMOE_ROUTER_LAUNCH(k_router_rank_topk<1>); else BITSMOE_ROUTER_LAUNCH(k_router_softmax_topk<1>);
+    } else {
+        if (by_rank) BITSMOE_ROUTER_LAUNCH(k_router_rank_topk<2>); else BITSMOE_ROUTER_LAUNCH(k_router_softmax_topk<2>);
+    }
+#undef BITSMOE_ROUTER_LAUNCH
     BITSMOE_HIP_TRY(hipGetLastError());
     return BITSMOE_OK;
 }

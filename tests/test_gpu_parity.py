@@ -385,7 +385,8 @@ def test_golden_vectors_dequant_on_device(cuda_device, name):
 
 
 @pytest.mark.parametrize("tokens,n_experts,top_k,renorm", [
-    (1, 128, 8, True), (64, 128, 8, True), (256, 512, 10, True), (16, 64, 6, False), (5, 8, 1, True), (37, 1000, 3, True)])
+    (1, 128, 8, True), (64, 128, 8, True), (256, 512, 10, True), (16, 64, 6, False), (5, 8, 1, True), (37, 1000, 3, True),
+    (9, 130, 4, True), (3, 256, 8, False), (33, 201, 64, True)])
 @pytest.mark.parametrize("logit_dtype", ["f32", "bf16"])
 def test_router_kernel_matches_oracle(cuda_device, tokens, n_experts, top_k, renorm, logit_dtype):
     """softmax / top-k / renormalise in one kernel: the picked experts are exactly the oracle's (in
