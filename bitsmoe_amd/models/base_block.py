@@ -270,10 +270,11 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         vh_gate, vh_up, _ = self._shared_basis(hidden_states.dtype)
         h_gate_proj = hidden_states @ vh_gate.T
         h_up_proj = hidden_states @ vh_up.T
-        final = torch.zeros((token_count, hidden_dim), dtype=hidden_states.dtype, device=hidden_states.device)
         flat_selected = selected_experts.reshape(-1)
         flat_w32 = routing_weights_fp32.reshape(-1)
+        final = None
         if self._super_expert_items:
+            final = torch.zeros((token_count, hidden_dim), dtype=hidden_states.dtype, device=hidden_states.device)
             self._run_super_experts(hidden_states, final, flat_selected,
                                     self._get_flat_token_ids(token_count, hidden_states.device),
                                     flat_w32.to(hidden_states.dtype))
@@ -281,6 +282,9 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         if routing is not None:
             token_indices, expert_offsets_t, route_flat = routing
             packed = self._packed_forward_grouped(h_gate_proj, h_up_proj, token_indices, expert_offsets_t,
-                                                  route_flat, token_count)
-            final = final + packed.to(hidden_states.dtype)
+                                                  route_flat, token_count).to(hidden_states.dtype)
+            # without dense experts the sum "zeros + packed" of the reference is `packed` itself
+            final = packed if final is None else final + packed
+        if final is None:
+            final = torch.zeros((token_count, hidden_dim), dtype=hidden_states.dtype, device=hidden_states.device)
         return final
