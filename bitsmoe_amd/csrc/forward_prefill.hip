@@ -24,6 +24,7 @@
 // does not depend on the order in which workgroups finish.
 // Operands are f16 for f16 and bf16 inputs alike (f16 keeps more mantissa than bf16).
 #include <algorithm>
+#include <type_traits>
 
 #include "fast_helpers.h"
 
@@ -268,23 +269,26 @@ __device__ inline int xcd_logical(int bid, int n_real) {
     return logical < n_real ? logical : -1;
 }
 
-// 128 x 64 16-bit activation piece: thread i owns rows i/8 + 32*j (j = 0..3), elements 8*(i%8)..+7
+// 128 x 64 16-bit activation piece: thread i owns rows i/8 + 32*j (j = 0..3), elements 8*(i%8)..+7.
+// NJ: how many of the four 32-row groups hold assignments (tiles of at most 32 rows: one).
 struct APiece {
     u32x4 v[4];
 };
+template <int NJ>
 __device__ __forceinline__ void load_piece(const uint16_t* __restrict__ src, int64_t ld, int a_begin, int rows, int col0, int tid,
                                   APiece& p) {
     const int r0 = tid >> 3, kc = (tid & 7) * 8;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NJ; ++j) {
         const int row = min(r0 + 32 * j, rows - 1);   // rows past the tile's end repeat the last one; never stored
         p.v[j] = *reinterpret_cast<const u32x4*>(src + (int64_t)(a_begin + row) * ld + col0 + kc);
     }
 }
+template <int NJ>
 __device__ __forceinline__ void store_piece(uint16_t* __restrict__ stage, int tid, const APiece& p) {
     const int r0 = tid >> 3, kc = (tid & 7) * 8;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(stage + (r0 + 32 * j) * PF_LDS_ROW + kc) = p.v[j];
+    for (int j = 0; j < NJ; ++j) *reinterpret_cast<u32x4*>(stage + (r0 + 32 * j) * PF_LDS_ROW + kc) = p.v[j];
 }
 
 __device__ __forceinline__ void zero_acc(f32x4 (&acc)[4][4]) {
@@ -308,15 +312,15 @@ struct GuFetch {
 // One slab (64 contraction rows, `bits` wide) for a wavefront's 128 x 64 tile; the weight
 // operand is the raw (2^bits + code), the scale already sits in the activations.
 // WU != 0: the width is a compile-time constant (experts whose slabs all share it).
-template <int WU>
+template <int WU, int NMB>
 __device__ __forceinline__ void gateup_slab_mfma(int bits, const uint16_t* __restrict__ stage,
-                                                 const uint32_t (&bw)[2][4], int lane, f32x4 (&acc)[8][4]) {
+                                                 const uint32_t (&bw)[2][4], int lane, f32x4 (&acc)[NMB][4]) {
     const int n = lane & 15, kg = lane >> 4;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-        u32x4 a[8];
+        u32x4 a[NMB];
 #pragma unroll
-        for (int mb = 0; mb < 8; ++mb)
+        for (int mb = 0; mb < NMB; ++mb)
             a[mb] = *reinterpret_cast<const u32x4*>(stage + (16 * mb + n) * PF_LDS_ROW + 16 * kg + 8 * ks);
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
@@ -332,7 +336,7 @@ __device__ __forceinline__ void gateup_slab_mfma(int bits, const uint16_t* __res
             else
                 b = decode_fields3<false>(w[nbl], 8 * ks, w[2 + nbl], 8 * (n >> 3) + 4 * ks);
 #pragma unroll
-            for (int mb = 0; mb < 8; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
+            for (int mb = 0; mb < NMB; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
         }
     }
 }
@@ -352,7 +356,7 @@ __device__ __forceinline__ void gateup_slab_mfma(int bits, const uint16_t* __res
 // token index (possible when every aligned run of 8 local rows is 8 consecutive logical ranks);
 // the per-row multiplier s is then taken from the folded scale table.  Otherwise Hs is the
 // pre-gathered [A, ld].  WU: the bit-width shared by every slab of the matrix, or 0 (mixed).
-template <bool DIRECT, int WU>
+template <bool DIRECT, int WU, int NMB>
 __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const FastSlab* __restrict__ fs_row, int nslabs,
                                                  const uint16_t* __restrict__ Hs, int ld,
                                                  const int32_t* __restrict__ token_indices, int T, int I, int n_tiles,
@@ -369,10 +373,11 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
 
     // this thread's four staging rows; DIRECT: their activation rows (invalid tokens read row 0:
     // the combine drops their outputs).  Element offsets: the launcher checks that they fit 32 bits.
+    constexpr int NJ = (NMB + 1) / 2;      // 32-row groups that hold assignments
     const int r0 = tid >> 3, kc = (tid & 7) * 8;
-    uint32_t rowbase[4];
+    uint32_t rowbase[NJ];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NJ; ++j) {
         const int a = a_begin + min(r0 + 32 * j, rows - 1);
         if constexpr (DIRECT) {
             const int tk = token_indices[a];
@@ -382,27 +387,27 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
         }
     }
 
-    f32x4 acc[8][4];
+    f32x4 acc[NMB][4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < NMB; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
     gptr<uint32_t> payload = as_global(fe.payload);
     gptr<__half> scale = as_global(DIRECT ? fe.scale_s : fe.scale);
     gptr<int32_t> rank_idx = as_global(fe.rank_idx);
     GuFetch f[1];              // the one slab in flight
-    float sum[2][4];           // [tile][row]
+    float sum[2][NJ];          // [tile][row]
 #pragma unroll
     for (int x = 0; x < 2; ++x)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) sum[x][j] = 0.0f;
+        for (int j = 0; j < NJ; ++j) sum[x][j] = 0.0f;
     auto slab_rec = [&](int s) { return s < nslabs ? load_fast_slab(fs_row, s) : FastSlab{0, 0, 0, 0}; };
     auto rank_base = [&](int s) { return (DIRECT && s < nslabs) ? rank_idx[s * SLAB_ROWS + kc] : 0; };
     auto issue = [&](GuFetch& dst, const FastSlab& r, int rbase, int s) {
         const int wb = WU != 0 ? WU : r.bits;
         const uint32_t col = DIRECT ? (uint32_t)rbase : (uint32_t)(s * SLAB_ROWS);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) dst.a.v[j] = *reinterpret_cast<const u32x4*>(Hs + (rowbase[j] + col));
+        for (int j = 0; j < NJ; ++j) dst.a.v[j] = *reinterpret_cast<const u32x4*>(Hs + (rowbase[j] + col));
         gptr<__half> sp = scale + (uint32_t)(r.scale_off + t0 * SLAB_ROWS + kc);
         dst.sc[0] = *reinterpret_cast<gptr_u32x4>(sp);
         dst.sc[1] = *reinterpret_cast<gptr_u32x4>(sp + (two_tiles ? SLAB_ROWS : 0));
@@ -421,7 +426,7 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
         for (int x = 0; x < 2; ++x) {
             if (x == 1 && !two_tiles) break;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < NJ; ++j) {
                 u32x4 v;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
@@ -472,7 +477,7 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
                     pending_rb = rank_base(s + 3);
                 }
             }
-            if (active && bits != 0) gateup_slab_mfma<WU>(bits, lds + ((s & 1) * 2 + tl) * GU_STAGE, bw, lane, acc);
+            if (active && bits != 0) gateup_slab_mfma<WU, NMB>(bits, lds + ((s & 1) * 2 + tl) * GU_STAGE, bw, lane, acc);
             __syncthreads();
             if (s + 1 < nslabs) {
 #pragma unroll
@@ -488,7 +493,7 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
 #pragma unroll
     for (int x = 0; x < 2; ++x)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < NJ; ++j) {
             float v = sum[x][j];
             v += __shfl_xor(v, 1);
             v += __shfl_xor(v, 2);
@@ -499,7 +504,7 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
     if (!active) return;
     // lane holds rows 16*mb + 4*kg + j, column 128*t + 64*wn + 16*nb + n
 #pragma unroll
-    for (int mb = 0; mb < 8; ++mb) {
+    for (int mb = 0; mb < NMB; ++mb) {
         if (16 * mb >= rows) break;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -546,9 +551,18 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     const int ld = proj ? ldu : ldg;
     uint16_t* __restrict__ out = proj ? U : G;
     const int w = __builtin_amdgcn_readfirstlane(fe.uniform_bits);
-#define BITSMOE_GU_BODY(W)                                                                                            \
-    gateup_tile_body<DIRECT, W>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out, a_begin, rows, 2 * tp, \
-                                lds, rowsum)
+    // tiles of at most 32 assignments (experts that see few tokens, remainders) run a body with a
+    // quarter of the accumulators, MFMAs and staging; complete bodies, so that no accumulator
+    // lives across the choice
+#define BITSMOE_GU_BODY(W)                                                                                           \
+    do {                                                                                                             \
+        if (rows <= 32)                                                                                              \
+            gateup_tile_body<DIRECT, W, 2>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out, a_begin,    \
+                                           rows, 2 * tp, lds, rowsum);                                               \
+        else                                                                                                         \
+            gateup_tile_body<DIRECT, W, 8>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out, a_begin,    \
+                                           rows, 2 * tp, lds, rowsum);                                               \
+    } while (0)
     if (w == 2)
         BITSMOE_GU_BODY(2);
     else if (w == 3)
@@ -587,16 +601,16 @@ constexpr int DN_SLABS_MFMA = 4;   // slabs (64 output rows each) per workgroup:
 // wavefront's 128 assignments x 64 output rows.  scp: this lane's row scale in both halves of a
 // pair, per 16-row block.  The weight operand is (code - 2^(W-1)) * scale rounded once to f16,
 // the operand the reference builds (bitsmoe/algorithms/cpp/mlp_forward.cu:1554-1694).
-template <int HH>
+template <int HH, int NMB>
 __device__ __forceinline__ void down_half_mfma(int bits, const uint16_t* __restrict__ stage, const Block16& blk,
-                                      const uint32_t (&scp)[4], int lane, f32x4 (&acc)[8][4]) {
+                                      const uint32_t (&scp)[4], int lane, f32x4 (&acc)[NMB][4]) {
     const int n = lane & 15, kg = lane >> 4;
 #pragma unroll
     for (int km = 0; km < 2; ++km) {
         const int m = 2 * HH + km;
-        u32x4 a[8];
+        u32x4 a[NMB];
 #pragma unroll
-        for (int mb = 0; mb < 8; ++mb)
+        for (int mb = 0; mb < NMB; ++mb)
             a[mb] = *reinterpret_cast<const u32x4*>(stage + (16 * mb + n) * PF_LDS_ROW + 32 * km + 8 * kg);
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
@@ -617,7 +631,7 @@ __device__ __forceinline__ void down_half_mfma(int bits, const uint16_t* __restr
 #pragma unroll
             for (int i = 0; i < 4; ++i) b[i] = pk_mul_f16(pk_add_f16(b[i], off), scp[nb]);
 #pragma unroll
-            for (int mb = 0; mb < 8; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
+            for (int mb = 0; mb < NMB; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
         }
     }
 }
@@ -625,9 +639,11 @@ __device__ __forceinline__ void down_half_mfma(int bits, const uint16_t* __restr
 // The column loop of one wavefront (fs.bits == 0: no slab, the wavefront only helps to stage).
 // Pieces of z (128 assignments x 64 columns) run two ahead of the MFMAs in two alternating
 // register sets, the payload block of the next tile one tile ahead.
+template <int NMB>
 __device__ __forceinline__ void down_tile_loop(gptr<uint32_t> payload, gptr<__half> scale, const FastSlab fs,
                                       const uint16_t* __restrict__ z, int I, int n_tiles, int a_begin, int rows,
-                                      uint16_t (*lds)[PF_M * PF_LDS_ROW], int tid, int lane, f32x4 (&acc)[8][4]) {
+                                      uint16_t (*lds)[PF_M * PF_LDS_ROW], int tid, int lane, f32x4 (&acc)[NMB][4]) {
+    constexpr int NJ = (NMB + 1) / 2;      // 32-row groups a thread stages
     const int n = lane & 15;
     const int W = fs.bits;
     APiece p0, p1;
@@ -648,22 +664,22 @@ __device__ __forceinline__ void down_tile_loop(gptr<uint32_t> payload, gptr<__ha
         }
     };
     const int n_halves = 2 * n_tiles;
-    load_piece(z, I, a_begin, rows, 0, tid, p0);
-    load_piece(z, I, a_begin, rows, 64, tid, p1);
+    load_piece<NJ>(z, I, a_begin, rows, 0, tid, p0);
+    load_piece<NJ>(z, I, a_begin, rows, 64, tid, p1);
     issue_b(0, blk, scp);
-    store_piece(lds[0], tid, p0);
+    store_piece<NJ>(lds[0], tid, p0);
     __syncthreads();
     for (int t = 0; t < n_tiles; ++t) {
         const int h = 2 * t;
         // first half of tile t is in lds[0], the second in flight in p1
-        if (h + 2 < n_halves) load_piece(z, I, a_begin, rows, 64 * (h + 2), tid, p0);
+        if (h + 2 < n_halves) load_piece<NJ>(z, I, a_begin, rows, 64 * (h + 2), tid, p0);
         if (t + 1 < n_tiles) issue_b(t + 1, blk_n, scp_n);
-        if (W != 0) down_half_mfma<0>(W, lds[0], blk, scp, lane, acc);
-        store_piece(lds[1], tid, p1);
+        if (W != 0) down_half_mfma<0, NMB>(W, lds[0], blk, scp, lane, acc);
+        store_piece<NJ>(lds[1], tid, p1);
         __syncthreads();
-        if (h + 3 < n_halves) load_piece(z, I, a_begin, rows, 64 * (h + 3), tid, p1);
-        if (W != 0) down_half_mfma<1>(W, lds[1], blk, scp, lane, acc);
-        if (h + 2 < n_halves) store_piece(lds[0], tid, p0);
+        if (h + 3 < n_halves) load_piece<NJ>(z, I, a_begin, rows, 64 * (h + 3), tid, p1);
+        if (W != 0) down_half_mfma<1, NMB>(W, lds[1], blk, scp, lane, acc);
+        if (h + 2 < n_halves) store_piece<NJ>(lds[0], tid, p0);
         __syncthreads();
         {
             if (W != 0 && t + 1 < n_tiles) {
@@ -716,28 +732,37 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
     gptr<uint32_t> payload = as_global(fe.payload);
     gptr<__half> scale = as_global(fe.scale);
 
-    f32x4 acc[8][4];
+    // tiles of at most 32 assignments run a body with a quarter of the accumulators and MFMAs:
+    // two complete bodies, so that no accumulator lives across the choice
+    auto run = [&](auto nmb_c) {
+        constexpr int NMB = decltype(nmb_c)::value;
+        f32x4 acc[NMB][4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < NMB; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
-    // wavefronts without a slab skip the MFMAs; all execute the same barriers
-    down_tile_loop(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, acc);
-    if (fs.bits == 0) return;
+            for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
+        // wavefronts without a slab skip the MFMAs; all execute the same barriers
+        down_tile_loop<NMB>(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, acc);
+        if (fs.bits == 0) return;
 
-    // lane holds assignments 16*mb + 4*kg + j, output rows 16*nb + n of the slab
-    _Float16* ycol = y + fs.rank_off + n;
+        // lane holds assignments 16*mb + 4*kg + j, output rows 16*nb + n of the slab
+        _Float16* ycol = y + fs.rank_off + n;
 #pragma unroll
-    for (int mb = 0; mb < 8; ++mb) {
-        if (16 * mb >= rows) break;
+        for (int mb = 0; mb < NMB; ++mb) {
+            if (16 * mb >= rows) break;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int r = 16 * mb + 4 * kg + j;
-            _Float16* dst = ycol + (int64_t)(r < rows ? a_begin + r : A) * ldy;
+            for (int j = 0; j < 4; ++j) {
+                const int r = 16 * mb + 4 * kg + j;
+                _Float16* dst = ycol + (int64_t)(r < rows ? a_begin + r : A) * ldy;
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb) dst[16 * nb] = (_Float16)acc[mb][nb][j];
+                for (int nb = 0; nb < 4; ++nb) dst[16 * nb] = (_Float16)acc[mb][nb][j];
+            }
         }
-    }
+    };
+    if (rows <= 32)
+        run(std::integral_constant<int, 2>{});
+    else
+        run(std::integral_constant<int, 8>{});
 }
 
 // ------------------------------------------------------------------------------- combine
