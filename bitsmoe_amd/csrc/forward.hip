@@ -34,9 +34,9 @@ static int resolve_path(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
         return BITSMOE_E_UNSUPPORTED;
     }
     if (path != BITSMOE_PATH_AUTO) return path;
-    // grouped GEMM from 36 assignments per expert on average (measured crossover: the decode kernels
+    // grouped GEMM from 32 assignments per expert on average (measured crossover: the decode kernels
     // re-stream the payload for every 16 assignments, the grouped GEMM pays for whole 128-row tiles)
-    if (mfma_ok && n_assign >= (int64_t)36 * gate->n_experts) return BITSMOE_PATH_MFMA;
+    if (mfma_ok && n_assign >= (int64_t)32 * gate->n_experts) return BITSMOE_PATH_MFMA;
     if (decode_ok) return BITSMOE_PATH_DECODE;
     if (mfma_ok && n_assign >= (int64_t)16 * gate->n_experts) return BITSMOE_PATH_MFMA;
     return BITSMOE_PATH_GENERIC;

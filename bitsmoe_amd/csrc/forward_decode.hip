@@ -65,6 +65,44 @@ __device__ inline int nth_active_expert(const int32_t* __restrict__ expert_offse
     return __builtin_amdgcn_readfirstlane(found);
 }
 
+// With many assignments an expert is served in chunks of 16; walking the chunks of a popular
+// expert one after the other inside a workgroup makes that expert the long pole of the launch.
+// The kernels can instead be launched over chunk slots: slot -> (expert, chunk) in expert order,
+// again by one wave-parallel pass over expert_offsets.  Returns expert -1 past the last chunk.
+struct ChunkRef {
+    int expert, chunk;
+};
+__device__ inline ChunkRef nth_chunk(const int32_t* __restrict__ expert_offsets, int E, int A, int slot, int lane) {
+    int found_e = -1, found_c = 0;
+    for (int e0 = 0; e0 < E && found_e < 0; e0 += 64) {
+        const int e = e0 + lane;
+        int chunks = 0;
+        if (e < E) {
+            const int b = max(expert_offsets[e], 0), en = min(expert_offsets[e + 1], A);
+            chunks = en > b ? (en - b + 15) >> 4 : 0;
+        }
+        int incl = chunks;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int v = __shfl_up(incl, d);
+            if (lane >= d) incl += v;
+        }
+        const int total = __shfl(incl, 63);
+        if (slot < total) {
+            const uint64_t hit = __ballot(slot >= incl - chunks && slot < incl);    // exactly one lane
+            const int l = (int)__builtin_ctzll(hit);
+            found_e = e0 + l;
+            found_c = slot - __shfl(incl - chunks, l);
+        }
+        slot -= total;
+    }
+    return ChunkRef{__builtin_amdgcn_readfirstlane(found_e), __builtin_amdgcn_readfirstlane(found_c)};
+}
+
+constexpr int GRID_EXPERTS = 0;   // the expert coordinate of the grid is the expert
+constexpr int GRID_ACTIVE = 1;    // ... counts active experts (nth_active_expert)
+constexpr int GRID_CHUNKS = 2;    // ... counts 16-assignment chunks (nth_chunk)
+
 // ------------------------------------------------------------------------------ gate / up
 // One (slab, tile) block restricted to one column-block pair: 2 column blocks x 2 k-steps,
 // plus the two MFMAs that accumulate the constant term.
@@ -102,8 +140,8 @@ __device__ __forceinline__ void gateup_pair(const uint32_t (&w)[4], u32x4 a0, u3
 // GENERAL == false: only the width-specialised bodies (groups of eight equal-width slabs that
 // follow each other in the payload); GENERAL == true: only the groups those skip.  Two kernels
 // instead of one keep the register budget of the common case free of the general body.
-// COMPACT: the expert coordinate of the grid counts active experts (see nth_active_expert).
-template <bool BF16, bool GENERAL, bool COMPACT>
+// MODE: what the expert coordinate of the grid counts (GRID_*).
+template <bool BF16, bool GENERAL, int MODE>
 __global__ __launch_bounds__(256) void k_gateup_decode(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
     const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
@@ -117,8 +155,14 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
     const int grp = (bid / n_tchunks) % n_groups;
     const int tid = threadIdx.x;
     int e = bid / (n_tchunks * n_groups);
-    if constexpr (COMPACT) {
+    int chunk = -1;
+    if constexpr (MODE == GRID_ACTIVE) {
         e = nth_active_expert(expert_offsets, E, A, e, tid & 63);
+        if (e < 0) return;
+    } else if constexpr (MODE == GRID_CHUNKS) {
+        const ChunkRef ref = nth_chunk(expert_offsets, E, A, e, tid & 63);
+        e = ref.expert;
+        chunk = ref.chunk;
         if (e < 0) return;
     }
     const int pair = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform
@@ -126,8 +170,12 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
     const int n = lane & 15, kg = lane >> 4;
 
     // one round trip: assignment range, expert record, the group's slab records
-    const int a_begin = max(expert_offsets[e], 0);
-    const int a_end = min(expert_offsets[e + 1], A);
+    int a_begin = max(expert_offsets[e], 0);
+    int a_end = min(expert_offsets[e + 1], A);
+    if (chunk >= 0) {      // this workgroup's chunk only
+        a_begin += MAX_A * chunk;
+        a_end = min(a_end, a_begin + MAX_A);
+    }
     const FastExpert* __restrict__ fe_tab = mt ? up_fe : gate_fe;
     const FastSlab* __restrict__ fs_tab = mt ? up_fs : gate_fs;
     const int max_slabs = mt ? up_max_slabs : gate_max_slabs;
@@ -470,7 +518,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
 // grid.x = E * n_groups * n_tchunks; 256 threads; dynamic LDS = 16 * (n_tiles * 128 + 8) * 2 bytes.
 // A workgroup takes four slabs of one expert and a run of tiles; with few active experts the
 // tiles are split over several workgroups (their partial sums meet in the atomics of the combine).
-template <bool BF16, bool COMPACT>
+template <bool BF16, int MODE>
 __global__ __launch_bounds__(256) void k_down_decode(
     const FastExpert* __restrict__ down_fe, const FastSlab* __restrict__ down_fs, int max_slabs,
     const float* __restrict__ G, const float* __restrict__ U, const float* __restrict__ route_w,
@@ -487,16 +535,27 @@ __global__ __launch_bounds__(256) void k_down_decode(
     const int grp = (bid / n_tchunks) % n_groups;
     const int e_slot = bid / (n_tchunks * n_groups);
     const int tid = threadIdx.x;
-    const int e = COMPACT ? nth_active_expert(expert_offsets, E, A, e_slot, tid & 63) : e_slot;
-    if (COMPACT && e < 0) return;
+    int e = e_slot, chunk = -1;
+    if constexpr (MODE == GRID_ACTIVE) {
+        e = nth_active_expert(expert_offsets, E, A, e_slot, tid & 63);
+    } else if constexpr (MODE == GRID_CHUNKS) {
+        const ChunkRef ref = nth_chunk(expert_offsets, E, A, e_slot, tid & 63);
+        e = ref.expert;
+        chunk = ref.chunk;
+    }
+    if (e < 0) return;
     const int tb = tchunk * tiles_per_wg;
     const int nt = min(tiles_per_wg, n_tiles - tb);
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int si = grp * DN_SLABS_PER_WG + wave;
 
-    const int a_begin = max(expert_offsets[e], 0);
-    const int a_end = min(expert_offsets[e + 1], A);
+    int a_begin = max(expert_offsets[e], 0);
+    int a_end = min(expert_offsets[e + 1], A);
+    if (chunk >= 0) {      // this workgroup's chunk only
+        a_begin += MAX_A * chunk;
+        a_end = min(a_end, a_begin + MAX_A);
+    }
     const FastExpert fe = down_fe[e];
     FastSlab fs = FastSlab{0, 0, 0, 0};
     if (si < max_slabs) fs = load_fast_slab(down_fs, e * max_slabs + si);
@@ -567,11 +626,16 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     // Tiles per workgroup: long runs amortise the start-up round trips, but the grid must
     // still hold a few workgroups per CU (two rounds of three per CU measured best).  At most min(E, A) experts can be active.
     const int64_t active_max = std::min<int64_t>(E, A);
-    // few assignments: launch over the experts that can be active at most, not over all of them
-    const bool compact = active_max * 2 <= E;
-    const int e_dim = compact ? (int)active_max : E;
+    // What the expert coordinate of the grids counts.  Few assignments: the experts that can be
+    // active at most, not all of them.  Sixteen or more assignments per expert on average: most
+    // experts have several 16-assignment chunks, one workgroup per chunk (below that the
+    // wave-parallel search of the chunk costs more than walking the few chunks in a loop).
+    const int mode = A >= (int64_t)16 * E ? GRID_CHUNKS : active_max * 2 <= E ? GRID_ACTIVE : GRID_EXPERTS;
+    const int e_dim = mode == GRID_CHUNKS ? (int)(active_max + A / MAX_A) : mode == GRID_ACTIVE ? (int)active_max : E;
+    // (expert, chunk) pairs expected to have work (e_dim is their upper bound in chunk mode)
+    const int64_t units = mode == GRID_CHUNKS ? A / MAX_A + active_max / 2 : active_max;
     int tiles_per_wg = n_tiles;
-    while (tiles_per_wg > 1 && active_max * 2 * gu_groups * ((n_tiles + tiles_per_wg - 1) / tiles_per_wg) < 1536)
+    while (tiles_per_wg > 1 && units * 2 * gu_groups * ((n_tiles + tiles_per_wg - 1) / tiles_per_wg) < 1536)
         tiles_per_wg = (tiles_per_wg + 1) / 2;
     const int n_tchunks = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
     dim3 grid((unsigned)(e_dim * gu_groups * n_tchunks), 2);
@@ -583,25 +647,30 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     };
     const bool need_general = !(gate->all_uniform8 && up->all_uniform8);
     const bool bf16 = act_dtype == BITSMOE_DT_BF16;
-    if (bf16 && compact) {
-        launch_gateup(k_gateup_decode<true, false, true>);
-        if (need_general) launch_gateup(k_gateup_decode<true, true, true>);
-    } else if (bf16) {
-        launch_gateup(k_gateup_decode<true, false, false>);
-        if (need_general) launch_gateup(k_gateup_decode<true, true, false>);
-    } else if (compact) {
-        launch_gateup(k_gateup_decode<false, false, true>);
-        if (need_general) launch_gateup(k_gateup_decode<false, true, true>);
-    } else {
-        launch_gateup(k_gateup_decode<false, false, false>);
-        if (need_general) launch_gateup(k_gateup_decode<false, true, false>);
-    }
+    auto launch_gateup_mode = [&](auto bf16_c, auto mode_c) {
+        constexpr bool B = decltype(bf16_c)::value;
+        constexpr int M = decltype(mode_c)::value;
+        launch_gateup(k_gateup_decode<B, false, M>);
+        if (need_general) launch_gateup(k_gateup_decode<B, true, M>);
+    };
+    auto with_mode = [&](auto fn, auto bf16_c) {
+        if (mode == GRID_CHUNKS)
+            fn(bf16_c, std::integral_constant<int, GRID_CHUNKS>{});
+        else if (mode == GRID_ACTIVE)
+            fn(bf16_c, std::integral_constant<int, GRID_ACTIVE>{});
+        else
+            fn(bf16_c, std::integral_constant<int, GRID_EXPERTS>{});
+    };
+    if (bf16)
+        with_mode(launch_gateup_mode, std::true_type{});
+    else
+        with_mode(launch_gateup_mode, std::false_type{});
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 2, st);
     const int dn_groups = (down->max_slabs + DN_SLABS_PER_WG - 1) / DN_SLABS_PER_WG;
     const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2;
     int dn_tiles_per_wg = n_tiles;
-    while (dn_tiles_per_wg > 1 && active_max * dn_groups * ((n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg) < 384)
+    while (dn_tiles_per_wg > 1 && units * dn_groups * ((n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg) < 384)
         dn_tiles_per_wg = (dn_tiles_per_wg + 1) / 2;
     const int dn_tchunks = (n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg;
     auto launch_down = [&](auto kernel) {
@@ -610,14 +679,13 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
                            down->d_fast_slabs, down->max_slabs, G, U, rw, tok, off, (int)T, (int)A, I, E, n_tiles,
                            dn_groups, dn_tchunks, dn_tiles_per_wg, n_work, rank_out, rank_accum);
     };
-    if (bf16 && compact)
-        launch_down(k_down_decode<true, true>);
-    else if (bf16)
-        launch_down(k_down_decode<true, false>);
-    else if (compact)
-        launch_down(k_down_decode<false, true>);
+    auto launch_down_mode = [&](auto bf16_c, auto mode_c) {
+        launch_down(k_down_decode<decltype(bf16_c)::value, decltype(mode_c)::value>);
+    };
+    if (bf16)
+        with_mode(launch_down_mode, std::true_type{});
     else
-        launch_down(k_down_decode<false, false>);
+        with_mode(launch_down_mode, std::false_type{});
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 3, st);
     if (prof) prof->recorded = true;
