@@ -6,7 +6,7 @@
 //   k_build_mtiles   expert_offsets -> list of (expert, first assignment, rows <= 128) tiles;
 //                    token_start = exclusive scan of the per-token assignment counts
 //   k_bf16_to_f16 /  activations as f16, read through the token index by the GEMM kernel, or
-//   k_pregather      Hs[a, k] = f16( h[tok_a, rank_idx[k]] * s[k] ) in expert-sorted assignment order
+//   k_pregather      Hs[a, k] = f16( h[tok_a, rank_idx[k]] ) in expert-sorted assignment order
 //   k_gateup_mfma    G = Hs_gate . W_gate, U = Hs_up . W_up as f16;  k_silu_mul_f16: z = silu(G) * U
 //   k_down_mfma      y[a, r] = sum_c W_down[r, c] z[a, c] as f16, and the per-token lists
 //   k_combine_tokens rank_accum[t, rank_idx[r]] = sum over the assignments of t of route_w * s[r] * y
@@ -15,10 +15,9 @@
 // workgroup.  The activation operand is staged through LDS in 128 x 64 pieces (double
 // buffered, one barrier per piece); the weight operand never touches LDS: every lane loads
 // its words of the prepared payload (wave_layout.h) and expands them to packed f16 pairs
-// (2^w + code) with a rotate and an and-or.  Gate/up multiply the activation rows by
-// scale * s while staging them and subtract 1.5 * 2^w * (weighted row sum) at the end; down
-// turns the pair into (code - 2^(w-1)) * scale with a packed add and a packed multiply --
-// the same "weight rounded to half" operand the reference's tensor-core path builds
+// (2^w + code) with a rotate and an and-or; a packed add and a packed multiply turn the pair
+// into (code - 2^(w-1)) * scale (gate/up: scale * s, folded once at prepare time) -- the same
+// "weight rounded to half" operand the reference's tensor-core path builds
 // (bitsmoe/algorithms/cpp/mlp_forward.cu:691-751, 1554-1694).  The top-k combine is a gather
 // per token instead of the reference's fp32 atomics (mlp_forward.cu:2036-2066): its result
 // does not depend on the order in which workgroups finish.
@@ -42,10 +41,6 @@ struct MTile {
     int32_t pad;
 };
 
-__device__ inline uint32_t pk_fma_f16(uint32_t a, uint32_t b, uint32_t c) {
-    const h2 r = __builtin_elementwise_fma(__builtin_bit_cast(h2, a), __builtin_bit_cast(h2, b), __builtin_bit_cast(h2, c));
-    return __builtin_bit_cast(uint32_t, r);
-}
 __device__ inline uint32_t pk_add_f16(uint32_t a, uint32_t b) {
     const h2 r = __builtin_bit_cast(h2, a) + __builtin_bit_cast(h2, b);
     return __builtin_bit_cast(uint32_t, r);
@@ -204,11 +199,9 @@ __global__ __launch_bounds__(256) void k_pregather(const FastExpert* __restrict_
     const int64_t hrow = (int64_t)(tok_ok ? tok : 0) * R;
     const int K = min(fe.num_slabs * SLAB_ROWS, ld);
     gptr<int32_t> rank_idx = as_global(fe.rank_idx);
-    gptr<__half> svec = as_global(fe.s);
     for (int k0 = lane * 8; k0 < K; k0 += 512) {
         const i32x4 r0 = *reinterpret_cast<const i32x4 __attribute__((address_space(1)))*>(rank_idx + k0);
         const i32x4 r1 = *reinterpret_cast<const i32x4 __attribute__((address_space(1)))*>(rank_idx + k0 + 4);
-        const u32x4 sv = *reinterpret_cast<gptr_u32x4>(svec + k0);
         uint32_t raw[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -219,9 +212,7 @@ __global__ __launch_bounds__(256) void k_pregather(const FastExpert* __restrict_
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int r = i < 4 ? r0[i] : r1[i - 4];
-            const uint32_t sw = sv[i >> 1];
-            const float sf = __half2float(__ushort_as_half((uint16_t)((i & 1) ? (sw >> 16) : (sw & 0xFFFFu))));
-            const float v = (tok_ok && r >= 0 && r < R) ? raw_to_f32<BF16>(raw[i]) * sf : 0.0f;
+            const float v = (tok_ok && r >= 0 && r < R) ? raw_to_f32<BF16>(raw[i]) : 0.0f;
             const uint32_t hb = __builtin_bit_cast(uint16_t, (_Float16)v);
             if (i & 1)
                 packed[i >> 1] |= hb << 16;
@@ -299,23 +290,28 @@ __device__ __forceinline__ void zero_acc(f32x4 (&acc)[4][4]) {
 }
 
 // ------------------------------------------------------------------------------ gate / up
-constexpr int GU_STAGE = PF_M * PF_LDS_ROW;   // 16-bit elements of one scaled 128 x 64 activation piece in LDS
-constexpr size_t GU_LDS_BYTES = (size_t)2 * 2 * GU_STAGE * 2 + 2 * PF_M * sizeof(float);
+constexpr int GU_STAGE = PF_M * PF_LDS_ROW;   // 16-bit elements of one 128 x 64 activation piece in LDS
 
 // Everything one thread fetches from global memory for one slab.
 struct GuFetch {
     APiece a;          // this thread's part of the 128 x 64 activation piece
-    u32x4 sc[2];       // scale pairs of contraction rows 8*(tid%8) .. +7 of the slab, for the two column tiles
+    u32x4 sc[2];       // scale pairs of the eight contraction rows this lane feeds per k-step (its own tile)
     uint32_t bw[2][4]; // payload words of the wavefront's two column-block pairs (its own tile)
 };
 
-// One slab (64 contraction rows, `bits` wide) for a wavefront's 128 x 64 tile; the weight
-// operand is the raw (2^bits + code), the scale already sits in the activations.
+// One slab (64 contraction rows, `bits` wide) for a wavefront's (16 * NMB) x 64 tile.  The weight
+// operand is (code - 2^(bits-1)) * scale_s rounded once to f16 -- the operand the reference
+// builds (bitsmoe/algorithms/cpp/mlp_forward.cu:691-751), with the per-row multiplier s folded
+// into the scale -- made from the raw field decode 2^bits + code by a packed add (exact) and a
+// packed multiply.  (One packed FMA with the constant -1.5 * 2^bits * scale_s would round that
+// constant: measured 4.5e-3 of error instead of 5e-4.)
 // WU != 0: the width is a compile-time constant (experts whose slabs all share it).
 template <int WU, int NMB>
-__device__ __forceinline__ void gateup_slab_mfma(int bits, const uint16_t* __restrict__ stage,
-                                                 const uint32_t (&bw)[2][4], int lane, f32x4 (&acc)[NMB][4]) {
+__device__ __forceinline__ void gateup_slab_mfma(int bits, const uint16_t* __restrict__ stage, const uint32_t (&bw)[2][4],
+                                                 const u32x4 (&sc)[2], int lane, f32x4 (&acc)[NMB][4]) {
     const int n = lane & 15, kg = lane >> 4;
+    const int wb = WU != 0 ? WU : bits;
+    const uint32_t neg = wb == 2 ? neg_offset_pair<2>() : wb == 3 ? neg_offset_pair<3>() : neg_offset_pair<4>();
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
         u32x4 a[NMB];
@@ -336,32 +332,29 @@ __device__ __forceinline__ void gateup_slab_mfma(int bits, const uint16_t* __res
             else
                 b = decode_fields3<false>(w[nbl], 8 * ks, w[2 + nbl], 8 * (n >> 3) + 4 * ks);
 #pragma unroll
+            for (int i = 0; i < 4; ++i) b[i] = pk_mul_f16(pk_add_f16(b[i], neg), sc[ks][i]);
+#pragma unroll
             for (int mb = 0; mb < NMB; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
         }
     }
 }
 
 // One workgroup = (assignment tile, projection, PAIR of 128-column tiles):
-// out[a, c] = f16 of sum_k A[a, k] * level[k, c] * scale[tile(c), k] over all slabs of the matrix.
-// Wavefront (tl, wn) owns all 128 assignments and columns 64*wn .. +63 of tile t0 + tl: a decoded
-// weight operand feeds eight MFMAs.
-//
-// The activation piece of a slab (128 x 64) is fetched once for both tiles.  The staging
-// threads multiply it by the slab's per-row scale of each tile (packed f16), write the two scaled
-// pieces to LDS and keep running sums of what they wrote, weighted with 1.5 * 2^W:
-// sum_k A'[a,k] * (2^W + code) - 1.5 * 2^W * sum_k A'[a,k] is the dot product with the true levels
-// code - 2^(W-1).  The loads of slab s + 2 are issued before slab s is multiplied.
+// out[a, c] = f16 of sum_k A[a, k] * f16(level[k, c] * scale_s[tile(c), k]) over all slabs of the matrix.
+// Wavefront (tl, wn) owns all assignments of the tile and columns 64*wn .. +63 of tile t0 + tl: a
+// decoded weight operand feeds NMB MFMAs.  The activation piece of a slab (128 x 64) is staged in
+// LDS once for both tiles; the loads of slab s + 2 are issued before slab s is multiplied.
 //
 // DIRECT: the activation rows are read straight from the f16 activations [T, ld] through the
 // token index (possible when every aligned run of 8 local rows is 8 consecutive logical ranks);
-// the per-row multiplier s is then taken from the folded scale table.  Otherwise Hs is the
-// pre-gathered [A, ld].  WU: the bit-width shared by every slab of the matrix, or 0 (mixed).
+// otherwise Hs is the pre-gathered [A, ld].  WU: the bit-width shared by every slab of the
+// matrix, or 0 (mixed).  NMB: 16-row blocks of the assignment tile that are computed.
 template <bool DIRECT, int WU, int NMB>
 __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const FastSlab* __restrict__ fs_row, int nslabs,
                                                  const uint16_t* __restrict__ Hs, int ld,
                                                  const int32_t* __restrict__ token_indices, int T, int I, int n_tiles,
                                                  uint16_t* __restrict__ out, int a_begin, int rows, int t0,
-                                                 uint16_t* __restrict__ lds, float* __restrict__ rowsum) {
+                                                 uint16_t* __restrict__ lds) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -371,8 +364,8 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
     const bool active = tl == 0 || two_tiles;        // a wavefront without a tile only helps to stage
     const int t = active ? t0 + tl : t0;             // (it re-reads tile t0: in bounds)
 
-    // this thread's four staging rows; DIRECT: their activation rows (invalid tokens read row 0:
-    // the combine drops their outputs).  Element offsets: the launcher checks that they fit 32 bits.
+    // this thread's staging rows; DIRECT: their activation rows (invalid tokens read row 0: the
+    // combine drops their outputs).  Element offsets: the launcher checks that they fit 32 bits.
     constexpr int NJ = (NMB + 1) / 2;      // 32-row groups that hold assignments
     const int r0 = tid >> 3, kc = (tid & 7) * 8;
     uint32_t rowbase[NJ];
@@ -393,14 +386,9 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
     gptr<uint32_t> payload = as_global(fe.payload);
-    gptr<__half> scale = as_global(DIRECT ? fe.scale_s : fe.scale);
+    gptr<__half> scale = as_global(fe.scale_s);
     gptr<int32_t> rank_idx = as_global(fe.rank_idx);
-    GuFetch f[1];              // the one slab in flight
-    float sum[2][NJ];          // [tile][row]
-#pragma unroll
-    for (int x = 0; x < 2; ++x)
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) sum[x][j] = 0.0f;
+    GuFetch F;                 // the one slab in flight
     auto slab_rec = [&](int s) { return s < nslabs ? load_fast_slab(fs_row, s) : FastSlab{0, 0, 0, 0}; };
     auto rank_base = [&](int s) { return (DIRECT && s < nslabs) ? rank_idx[s * SLAB_ROWS + kc] : 0; };
     auto issue = [&](GuFetch& dst, const FastSlab& r, int rbase, int s) {
@@ -408,9 +396,10 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
         const uint32_t col = DIRECT ? (uint32_t)rbase : (uint32_t)(s * SLAB_ROWS);
 #pragma unroll
         for (int j = 0; j < NJ; ++j) dst.a.v[j] = *reinterpret_cast<const u32x4*>(Hs + (rowbase[j] + col));
-        gptr<__half> sp = scale + (uint32_t)(r.scale_off + t0 * SLAB_ROWS + kc);
+        // the MFMA operand of k-step ks holds contraction rows 16*kg + 8*ks .. +7 of the slab
+        gptr<__half> sp = scale + (uint32_t)(r.scale_off + t * SLAB_ROWS + 16 * kg);
         dst.sc[0] = *reinterpret_cast<gptr_u32x4>(sp);
-        dst.sc[1] = *reinterpret_cast<gptr_u32x4>(sp + (two_tiles ? SLAB_ROWS : 0));
+        dst.sc[1] = *reinterpret_cast<gptr_u32x4>(sp + 8);
         gptr<uint32_t> blk = payload + (uint32_t)(r.pack_off + t * 256 * wb);
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
@@ -418,41 +407,26 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
             load_pair_role0(blk, wb, (uint32_t)(pair * 64 + lane), (uint32_t)hi_index0(kg, n, 2 * pair), dst.bw[p]);
         }
     };
-    // scale the fetched piece for both tiles, add the weighted row sums, write the two pieces to LDS
-    auto stage_piece = [&](const GuFetch& src, int bits, uint16_t* __restrict__ stage) {
-        const int wb = WU != 0 ? WU : bits;
-        const uint32_t cw = wb == 2 ? Codec<2, false>::CORR : wb == 3 ? Codec<3, false>::CORR : Codec<4, false>::CORR;
+    auto stage_piece = [&](const GuFetch& src, uint16_t* __restrict__ stage) {
 #pragma unroll
-        for (int x = 0; x < 2; ++x) {
-            if (x == 1 && !two_tiles) break;
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                u32x4 v;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const uint32_t raw = src.a.v[j][i];
-                    const uint32_t scaled = pk_mul_f16(raw, src.sc[x][i]);
-                    v[i] = scaled;
-                    sum[x][j] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, scaled), __builtin_bit_cast(h2, cw), sum[x][j], false);
-                }
-                *reinterpret_cast<u32x4*>(stage + x * GU_STAGE + (r0 + 32 * j) * PF_LDS_ROW + kc) = v;
-            }
-        }
+        for (int j = 0; j < NJ; ++j) *reinterpret_cast<u32x4*>(stage + (r0 + 32 * j) * PF_LDS_ROW + kc) = src.a.v[j];
     };
     if (nslabs > 0) {
         // prologue: slab 0 is fetched and staged, slab 1 requested
-        GuFetch& F = f[0];
-        uint32_t bw[2][4];       // payload words of the slab being multiplied
+        uint32_t bw[2][4];       // payload words and scales of the slab being multiplied
+        u32x4 sc[2];
         FastSlab rec = slab_rec(0);
         FastSlab pending = slab_rec(1);
         int pending_rb = rank_base(1);
         int bits = rec.bits;
         issue(F, rec, rank_base(0), 0);
-        stage_piece(F, bits, lds);
+        stage_piece(F, lds);
 #pragma unroll
-        for (int p = 0; p < 2; ++p)
+        for (int p = 0; p < 2; ++p) {
+            sc[p] = F.sc[p];
 #pragma unroll
             for (int i = 0; i < 4; ++i) bw[p][i] = F.bw[p][i];
+        }
         int bits_next = pending.bits;
         if (nslabs > 1) {
             issue(F, pending, pending_rb, 1);
@@ -464,43 +438,36 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
         // staged, slab s + 2 requested, then slab s is multiplied
         for (int s = 0; s < nslabs; ++s) {
             uint32_t bw_next[2][4];
+            u32x4 sc_next[2];
             const int bits_after = pending.bits;
             if (s + 1 < nslabs) {
-                stage_piece(F, bits_next, lds + ((s + 1) & 1) * 2 * GU_STAGE);
+                stage_piece(F, lds + ((s + 1) & 1) * GU_STAGE);
 #pragma unroll
-                for (int p = 0; p < 2; ++p)
+                for (int p = 0; p < 2; ++p) {
+                    sc_next[p] = F.sc[p];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) bw_next[p][i] = F.bw[p][i];
+                }
                 if (s + 2 < nslabs) {
                     issue(F, pending, pending_rb, s + 2);
                     pending = slab_rec(s + 3);
                     pending_rb = rank_base(s + 3);
                 }
             }
-            if (active && bits != 0) gateup_slab_mfma<WU, NMB>(bits, lds + ((s & 1) * 2 + tl) * GU_STAGE, bw, lane, acc);
+            if (active && bits != 0) gateup_slab_mfma<WU, NMB>(bits, lds + (s & 1) * GU_STAGE, bw, sc, lane, acc);
             __syncthreads();
             if (s + 1 < nslabs) {
 #pragma unroll
-                for (int p = 0; p < 2; ++p)
+                for (int p = 0; p < 2; ++p) {
+                    sc[p] = sc_next[p];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) bw[p][i] = bw_next[p][i];
+                }
                 bits = bits_next;
                 bits_next = bits_after;
             }
         }
     }
-    // row sums: the eight threads that share a row hold its eight 8-column parts
-#pragma unroll
-    for (int x = 0; x < 2; ++x)
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            float v = sum[x][j];
-            v += __shfl_xor(v, 1);
-            v += __shfl_xor(v, 2);
-            v += __shfl_xor(v, 4);
-            if ((tid & 7) == 0) rowsum[x * PF_M + r0 + 32 * j] = v;
-        }
-    __syncthreads();
     if (!active) return;
     // lane holds rows 16*mb + 4*kg + j, column 128*t + 64*wn + 16*nb + n
 #pragma unroll
@@ -510,16 +477,14 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
         for (int j = 0; j < 4; ++j) {
             const int row = 16 * mb + 4 * kg + j;
             if (row >= rows) continue;
-            const float c = rowsum[tl * PF_M + row];
             uint16_t* dst = out + (int64_t)(a_begin + row) * I + N_TILE * t + 64 * wn + n;
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb) dst[16 * nb] = __builtin_bit_cast(uint16_t, (_Float16)(acc[mb][nb][j] - c));
+            for (int nb = 0; nb < 4; ++nb) dst[16 * nb] = __builtin_bit_cast(uint16_t, (_Float16)acc[mb][nb][j]);
         }
     }
 }
 
-// grid.x = 8 * ceil(max_mtiles * 2 * ceil(n_tiles / 2) / 8), 256 threads, GU_LDS_BYTES of dynamic
-// LDS; G and U are f16 [A, I].
+// grid.x = 8 * ceil(max_mtiles * 2 * ceil(n_tiles / 2) / 8), 256 threads; G and U are f16 [A, I].
 template <bool DIRECT>
 __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
@@ -528,9 +493,7 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     const int32_t* __restrict__ token_indices, int T,
     const MTile* __restrict__ mtiles, const int32_t* __restrict__ n_mtiles, int I, int n_tiles,
     uint16_t* __restrict__ G, uint16_t* __restrict__ U) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char gu_smem[];
-    uint16_t* lds = reinterpret_cast<uint16_t*>(gu_smem);
-    float* rowsum = reinterpret_cast<float*>(gu_smem + (size_t)2 * 2 * GU_STAGE * 2);
+    __shared__ __attribute__((aligned(16))) uint16_t lds[2 * GU_STAGE];
     const int n_tp = (n_tiles + 1) >> 1;
     const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles) * 2 * n_tp);
     if (logical < 0) return;
@@ -558,10 +521,10 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     do {                                                                                                             \
         if (rows <= 32)                                                                                              \
             gateup_tile_body<DIRECT, W, 2>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out, a_begin,    \
-                                           rows, 2 * tp, lds, rowsum);                                               \
+                                           rows, 2 * tp, lds);                                                       \
         else                                                                                                         \
             gateup_tile_body<DIRECT, W, 8>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out, a_begin,    \
-                                           rows, 2 * tp, lds, rowsum);                                               \
+                                           rows, 2 * tp, lds);                                                       \
     } while (0)
     if (w == 2)
         BITSMOE_GU_BODY(2);
@@ -628,7 +591,6 @@ __device__ __forceinline__ void down_half_mfma(int bits, const uint16_t* __restr
                 b = decode_fields3<false>(blk.w[nb * 2 + HH], 8 * km, blk.w[8 + nb], 4 * m);
                 off = neg_offset_pair<3>();
             }
-#pragma unroll
             for (int i = 0; i < 4; ++i) b[i] = pk_mul_f16(pk_add_f16(b[i], off), scp[nb]);
 #pragma unroll
             for (int mb = 0; mb < NMB; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
@@ -978,14 +940,9 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
         const int n_tp = (n_tiles + 1) / 2;
         const int64_t wgs = (max_mtiles * 2 * n_tp + 7) / 8 * 8;
         auto launch = [&](auto kernel) -> hipError_t {
-            // more than 64 KB of LDS per workgroup has to be asked for explicitly (a property of
-            // the kernel, not a stream operation)
-            hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)GU_LDS_BYTES);
-            if (err != hipSuccess) return err;
-            hipLaunchKernelGGL(kernel, dim3((unsigned)wgs), dim3(256), GU_LDS_BYTES, st, gate->d_fast_experts,
-                               gate->d_fast_slabs, gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs,
-                               Hs_g, Hs_u, ldg, ldu, tok, (int)T, mtiles, n_mtiles, I, n_tiles, z, Ubuf);
+            hipLaunchKernelGGL(kernel, dim3((unsigned)wgs), dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs,
+                               gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs, Hs_g, Hs_u, ldg, ldu, tok,
+                               (int)T, mtiles, n_mtiles, I, n_tiles, z, Ubuf);
             return hipGetLastError();
         };
         BITSMOE_HIP_TRY(direct ? launch(k_gateup_mfma<true>) : launch(k_gateup_mfma<false>));
