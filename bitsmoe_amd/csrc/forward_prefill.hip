@@ -250,14 +250,19 @@ __global__ __launch_bounds__(256) void k_bf16_to_f16(const uint16_t* __restrict_
 }
 
 // --------------------------------------------------------------------------- shared GEMM parts
-// Workgroup id -> logical work index such that consecutive logical indices (which share the
-// activation tile) run on the same XCD: hardware places workgroup b on XCD b % 8.
-__device__ inline int xcd_logical(int bid, int n_real) {
-    const int per = (n_real + 7) >> 3;
+// Workgroup id -> logical work index = tile * units + unit.  Hardware places workgroup b on XCD
+// b % 8, and every XCD has its own L2: the `units` workgroups of one assignment tile (which share
+// its activations) get ids of one residue class, and the tiles are dealt to the XCDs two at a time
+// (neighbouring tiles mostly belong to one expert and share its weights), so that a long run of
+// heavy tiles (a popular expert) or of short ones does not land on one XCD.
+// The grid holds 32 * ceil(max tiles / 32) * units workgroups; -1: no such tile.
+constexpr int XCD_RUN = 2;
+__device__ inline int xcd_logical(int bid, int n_tiles_real, int units) {
     const int slot = bid >> 3;
-    if (slot >= per) return -1;
-    const int logical = (bid & 7) * per + slot;
-    return logical < n_real ? logical : -1;
+    const int q = slot / units;
+    const int tile = ((q / XCD_RUN) * 8 + (bid & 7)) * XCD_RUN + q % XCD_RUN;
+    if (tile >= n_tiles_real) return -1;
+    return tile * units + slot % units;
 }
 
 // 128 x 64 16-bit activation piece: thread i owns rows i/8 + 32*j (j = 0..3), elements 8*(i%8)..+7.
@@ -484,7 +489,7 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
     }
 }
 
-// grid.x = 8 * ceil(max_mtiles * 2 * ceil(n_tiles / 2) / 8), 256 threads; G and U are f16 [A, I].
+// grid.x = 32 * ceil(max_mtiles / 32) * 2 * ceil(n_tiles / 2), 256 threads; G and U are f16 [A, I].
 template <bool DIRECT>
 __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
@@ -495,7 +500,7 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     uint16_t* __restrict__ G, uint16_t* __restrict__ U) {
     __shared__ __attribute__((aligned(16))) uint16_t lds[2 * GU_STAGE];
     const int n_tp = (n_tiles + 1) >> 1;
-    const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles) * 2 * n_tp);
+    const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles), 2 * n_tp);
     if (logical < 0) return;
     // the tile pairs of one (assignment tile, projection) are neighbours: they share the activations
     const int tp = logical % n_tp;
@@ -653,7 +658,7 @@ __device__ __forceinline__ void down_tile_loop(gptr<uint32_t> payload, gptr<__ha
     }
 }
 
-// grid.x = 8 * ceil(max_mtiles * n_groups / 8); workgroup = (assignment tile, group of four
+// grid.x = 32 * ceil(max_mtiles / 32) * n_groups; workgroup = (assignment tile, group of four
 // slabs): wavefront w = all 128 assignments x the 64 output rows of slab 4*group + w.
 // Output: y[a, r] = sum_c W_down[r, c] z[a, c] as f16, r in the expert's own row order
 // (row `A` of y takes the stores of a tile's unused rows), and the per-token assignment lists
@@ -668,7 +673,7 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
                                                       int2* __restrict__ token_list, int A, int I, int n_tiles,
                                                       int n_groups, _Float16* __restrict__ y, int ldy) {
     __shared__ __attribute__((aligned(16))) uint16_t lds[2][PF_M * PF_LDS_ROW];
-    const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles) * n_groups);
+    const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles), n_groups);
     if (logical < 0) return;
     const int mt_i = logical / n_groups, grp = logical - mt_i * n_groups;
     const i32x4 tv = *reinterpret_cast<const i32x4*>(mtiles + mt_i);
@@ -938,7 +943,7 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     record(prof, 1, st);
     {
         const int n_tp = (n_tiles + 1) / 2;
-        const int64_t wgs = (max_mtiles * 2 * n_tp + 7) / 8 * 8;
+        const int64_t wgs = (max_mtiles + 31) / 32 * 32 * 2 * n_tp;
         auto launch = [&](auto kernel) -> hipError_t {
             hipLaunchKernelGGL(kernel, dim3((unsigned)wgs), dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs,
                                gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs, Hs_g, Hs_u, ldg, ldu, tok,
@@ -954,7 +959,7 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     record(prof, 2, st);
     {
         const int n_pairs = (down->max_slabs + DN_SLABS_MFMA - 1) / DN_SLABS_MFMA;
-        const int64_t wgs = (max_mtiles * n_pairs + 7) / 8 * 8;
+        const int64_t wgs = (max_mtiles + 31) / 32 * 32 * n_pairs;
         hipLaunchKernelGGL(k_down_mfma, dim3((unsigned)wgs), dim3(256), 0, st, down->d_fast_experts, down->d_fast_slabs,
                            down->max_slabs, z, mtiles, n_mtiles, tok, slot, token_start, token_list, (int)A, I, n_tiles,
                            n_pairs, y, ldy);
