@@ -128,7 +128,8 @@ def test_full_size_linear_in_route_weights(cuda_device, tokens):
     assert float(zero.abs().max()) == 0.0
 
 
-def test_full_size_dropped_assignments_do_not_contribute(cuda_device):
+@pytest.mark.parametrize("tokens", [64, 1024])      # decode kernels / grouped GEMM with the per-token gather
+def test_full_size_dropped_assignments_do_not_contribute(cuda_device, tokens):
     """Assignments routed to experts outside the packed set are dropped by the routing kernel:
     the output equals the one computed from the kept assignments alone."""
     import torch
@@ -138,7 +139,7 @@ def test_full_size_dropped_assignments_do_not_contribute(cuda_device):
 
     spec = SPECS["c2"]
     block = _layer("c2", cuda_device)
-    h_gate, h_up, selected, weights = _inputs(block, spec, 64, 9, cuda_device)
+    h_gate, h_up, selected, weights = _inputs(block, spec, tokens, 9, cuda_device)
     g2l = block._packed_global_to_local.clone()
     g2l[::3] = -1                                  # every third expert is "not packed"
     gate, up, down = block._ensure_matsets()
