@@ -214,18 +214,19 @@ HBM_TRAFFIC_BYTES = {"c2-t64": int((58021.9 * 2.0 + 12288.0) * 1024),        # k
                      "c3-t4096": int((191641.7 * 2.0 + 98304.0) * 1024)}     # k_gateup_mfma
 
 
-def roofline_of(res, inputs, bound):
+def roofline_of(res, inputs, bound, workload=None):
     work = inputs["work"]
+    traffic = HBM_TRAFFIC_BYTES.get(workload)
     if bound == "hbm":
         # dominant kernel at decode: the fused gate+up launch (two thirds of the weight bytes)
         achieved = res["gateup_GBps"]
         return {"bound": "hbm", "kernel": "gate_up", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                 "algorithmic_bytes_per_launch": work["bytes_gateup"], "launch_ms": res["kernel_ms"]["gate_up"],
                 "all_kernels_GBps": res["kernels_GBps"], "all_kernels_frac": res["kernels_GBps"] / HBM_PEAK_GBS}
     achieved = res["gateup_TFLOPs"]
     return {"bound": "mfma", "kernel": "gate_up", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
-            "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+            "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic,
             "algorithmic_flops_per_launch": work["flops_gateup"], "launch_ms": res["kernel_ms"]["gate_up"],
             "all_kernels_TFLOPs": res["kernels_TFLOPs"], "all_kernels_frac": res["kernels_TFLOPs"] / MFMA_BF16_PEAK_TFLOPS}
 
@@ -304,7 +305,7 @@ def main() -> int:
     build_s = time.perf_counter() - t0
 
     res, inputs = run_workload(block, SPECS[spec_key], tokens, args.steps, args.warmup, use_graph=not args.no_graph)
-    roof = roofline_of(res, inputs, bound)
+    roof = roofline_of(res, inputs, bound, args.workload)
     if args.copy_probe_mib > 0:
         n = args.copy_probe_mib * (1 << 20) // 4
         src = torch.ones(n, dtype=torch.float32, device=dev)
@@ -324,7 +325,7 @@ def main() -> int:
             # c2 and c3 are the same layer (same seed, shape and bit draw); only routing differs
             r, inp = run_workload(block, SPECS[skey], toks, max(5, args.steps // 2), max(2, args.warmup // 2),
                                   use_graph=not args.no_graph)
-            r["roofline"] = roofline_of(r, inp, bnd)
+            r["roofline"] = roofline_of(r, inp, bnd, name)
             extras[name] = r
     bits = block.expert_bits
     line = {
