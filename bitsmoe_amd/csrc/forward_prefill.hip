@@ -784,17 +784,31 @@ __global__ __launch_bounds__(256) void k_combine_tokens(const FastExpert* __rest
             __syncthreads();
             if (IDENTITY) {
                 const int r0 = c0 + tid * 8;
-                for (int i = 0; i < nl; ++i) {
-                    if (r0 >= nrow_s[i]) continue;
-                    const u32x4 yv = *reinterpret_cast<const u32x4*>(y_s[i] + r0);
-                    const u32x4 sv = *reinterpret_cast<gptr<u32x4>>(as_global(s_s[i]) + r0);
-                    const float rw = rw_s[i];
+                // four entries at a time: their eight loads are in flight together (an entry past
+                // the list or past its expert's rows loads from a valid address and is not added)
+                for (int i0 = 0; i0 < nl; i0 += 4) {
+                    u32x4 yv[4], sv[4];
+                    float rw[4];
+                    bool ok[4];
 #pragma unroll
-                    for (int k = 0; k < 8; ++k) {
-                        const uint32_t yw = yv[k >> 1], sw = sv[k >> 1];
-                        const h2 yp = __builtin_bit_cast(h2, yw);
-                        const h2 sp = __builtin_bit_cast(h2, sw);
-                        acc[k] += (float)yp[k & 1] * (float)sp[k & 1] * rw;
+                    for (int u = 0; u < 4; ++u) {
+                        const int i = min(i0 + u, nl - 1);
+                        ok[u] = i0 + u < nl && r0 < nrow_s[i];
+                        const int rr = ok[u] ? r0 : 0;
+                        yv[u] = *reinterpret_cast<const u32x4*>(y_s[i] + rr);
+                        sv[u] = *reinterpret_cast<gptr<u32x4>>(as_global(s_s[i]) + rr);
+                        rw[u] = rw_s[i];
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        if (!ok[u]) continue;
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) {
+                            const uint32_t yw = yv[u][k >> 1], sw = sv[u][k >> 1];
+                            const h2 yp = __builtin_bit_cast(h2, yw);
+                            const h2 sp = __builtin_bit_cast(h2, sw);
+                            acc[k] += (float)yp[k & 1] * (float)sp[k & 1] * rw[u];
+                        }
                     }
                 }
             } else {
