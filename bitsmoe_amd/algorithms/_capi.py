@@ -35,6 +35,7 @@ EXPORTED_SYMBOLS = (
     "bitsmoe_forward_workspace_bytes",
     "bitsmoe_forward_workspace_bytes_sets",
     "bitsmoe_moe_forward",
+    "bitsmoe_moe_forward_strided",
     "bitsmoe_profile_create",
     "bitsmoe_profile_destroy",
     "bitsmoe_profile_read",
@@ -106,6 +107,12 @@ def load() -> ctypes.CDLL:
     lib.bitsmoe_moe_forward.restype = c_int32
     lib.bitsmoe_moe_forward.argtypes = [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32,
+        c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32,
+        c_void_p, c_void_p, c_size_t, c_void_p, c_void_p,
+    ]
+    lib.bitsmoe_moe_forward_strided.restype = c_int32
+    lib.bitsmoe_moe_forward_strided.argtypes = [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_int64, c_int64,
         c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32,
         c_void_p, c_void_p, c_size_t, c_void_p, c_void_p,
     ]

@@ -216,7 +216,10 @@ def moe_forward_sets(h_gate: torch.Tensor, h_up: torch.Tensor, token_indices: to
                      up: MatrixSet, down: MatrixSet, rank_out: int, intermediate_size: int,
                      act_type: int = 0, path: int = _capi.PATH_AUTO,
                      profile: Optional[Profile] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The forward over explicit matrix sets.  Returns rank_accum fp32 [tokens, rank_out]."""
+    """The forward over explicit matrix sets.  Returns rank_accum fp32 [tokens, rank_out].
+    h_gate / h_up may be column ranges of a wider row-major tensor (unit column stride)."""
+    _check(h_gate.dim() == 2 and h_up.dim() == 2 and h_gate.stride(1) == 1 and h_up.stride(1) == 1,
+           "h_gate/h_up must be 2D with unit column stride")
     dev = h_gate.device
     n_tokens = int(h_gate.shape[0])
     n_assign = int(token_indices.numel())
@@ -233,9 +236,11 @@ def moe_forward_sets(h_gate: torch.Tensor, h_up: torch.Tensor, token_indices: to
                                                            n_assign, int(path)))
     ws = _workspace(dev, nbytes)
     with torch.cuda.device(dev):
-        _capi.check(_lib.bitsmoe_moe_forward(
+        _capi.check(_lib.bitsmoe_moe_forward_strided(
             gate.handle, up.handle, down.handle, h_gate.data_ptr(), h_up.data_ptr(), dt, n_tokens,
-            int(h_gate.shape[1]), int(h_up.shape[1]), token_indices.data_ptr(), expert_offsets.data_ptr(),
+            int(h_gate.shape[1]), int(h_up.shape[1]), int(h_gate.stride(0)) if n_tokens > 1 else int(h_gate.shape[1]),
+            int(h_up.stride(0)) if n_tokens > 1 else int(h_up.shape[1]),
+            token_indices.data_ptr(), expert_offsets.data_ptr(),
             route_weights.data_ptr(), n_assign, int(rank_out), int(intermediate_size), int(act_type),
             int(path), out.data_ptr(), ws.data_ptr(), ws.numel(),
             profile._handle if profile is not None else None, _stream_ptr(dev)))

@@ -63,18 +63,18 @@ struct SlabTask {              // one (expert, slab) unit of the down projection
 
 bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I);
 int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
-                          const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru,
-                          const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out, int I,
-                          float* rank_accum, float* G, float* U, int64_t inter_floats, bitsmoe_profile* prof,
+                          const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg,
+                          int64_t ldu, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
+                          int I, float* rank_accum, float* G, float* U, int64_t inter_floats, bitsmoe_profile* prof,
                           hipStream_t st);
 
 bool mfma_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I);
 size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int64_t T,
                             int64_t A, int I);
 int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
-                        const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru,
-                        const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out, int I,
-                        float* rank_accum, void* workspace, bitsmoe_profile* prof, hipStream_t st);
+                        const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg_in,
+                        int64_t ldu_in, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
+                        int I, float* rank_accum, void* workspace, bitsmoe_profile* prof, hipStream_t st);
 
 }  // namespace bitsmoe
 
@@ -179,7 +179,7 @@ __device__ inline float silu_f32(float x) { return x / (1.0f + __expf(-x)); }
 int launch_fill_zero(float* p, int64_t n, hipStream_t st);
 int launch_forward_generic(const bitsmoe_matset* gate, const bitsmoe_matset* up,
                            const bitsmoe_matset* down, const void* h_gate, const void* h_up,
-                           int act_dtype, int64_t T, int Rg, int Ru, const int32_t* tok,
+                           int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg, int64_t ldu, const int32_t* tok,
                            const int32_t* off, const float* rw, int64_t A, int rank_out, int I,
                            float* rank_accum, float* G, float* U, bitsmoe_profile* prof,
                            hipStream_t st);

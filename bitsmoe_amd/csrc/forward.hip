@@ -60,6 +60,21 @@ extern "C" int bitsmoe_moe_forward(const bitsmoe_matset* gate, const bitsmoe_mat
                                    int64_t n_assign, int32_t rank_out, int32_t intermediate_size,
                                    int32_t act_type, int32_t path, float* rank_accum, void* workspace,
                                    size_t workspace_bytes, bitsmoe_profile* profile, void* stream) {
+    return bitsmoe_moe_forward_strided(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, rank_gate,
+                                       rank_up, token_indices, expert_offsets, route_w, n_assign, rank_out,
+                                       intermediate_size, act_type, path, rank_accum, workspace, workspace_bytes, profile,
+                                       stream);
+}
+
+extern "C" int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                                           const bitsmoe_matset* down, const void* h_gate, const void* h_up,
+                                           int32_t act_dtype, int64_t n_tokens, int32_t rank_gate,
+                                           int32_t rank_up, int64_t ld_gate, int64_t ld_up,
+                                           const int32_t* token_indices, const int32_t* expert_offsets,
+                                           const float* route_w, int64_t n_assign, int32_t rank_out,
+                                           int32_t intermediate_size, int32_t act_type, int32_t path,
+                                           float* rank_accum, void* workspace, size_t workspace_bytes,
+                                           bitsmoe_profile* profile, void* stream) {
     hipStream_t st = (hipStream_t)stream;
     BITSMOE_REQUIRE(gate && up && down, "matrix sets must not be null");
     BITSMOE_REQUIRE(act_type == 0, "only SiLU act_type=0 is currently supported");
@@ -87,6 +102,7 @@ extern "C" int bitsmoe_moe_forward(const bitsmoe_matset* gate, const bitsmoe_mat
     }
     BITSMOE_REQUIRE(h_gate && h_up && token_indices && expert_offsets && route_w, "null input pointer");
     BITSMOE_REQUIRE(rank_gate > 0 && rank_up > 0, "rank_gate/rank_up must be > 0");
+    BITSMOE_REQUIRE(ld_gate >= rank_gate && ld_up >= rank_up, "ld_gate/ld_up must be at least rank_gate/rank_up");
     BITSMOE_REQUIRE(gate->max_rank_plus1 <= rank_gate && gate->min_rank >= 0,
                     "gate rank_idx references rank %d but h_gate has %d columns", gate->max_rank_plus1 - 1, rank_gate);
     BITSMOE_REQUIRE(up->max_rank_plus1 <= rank_up && up->min_rank >= 0,
@@ -101,17 +117,17 @@ extern "C" int bitsmoe_moe_forward(const bitsmoe_matset* gate, const bitsmoe_mat
     BITSMOE_REQUIRE(((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
 
     if (chosen == BITSMOE_PATH_MFMA)
-        return launch_forward_mfma(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, token_indices,
-                                   expert_offsets, route_w, n_assign, rank_out, intermediate_size, rank_accum, workspace,
-                                   profile, st);
+        return launch_forward_mfma(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
+                                   token_indices, expert_offsets, route_w, n_assign, rank_out, intermediate_size, rank_accum,
+                                   workspace, profile, st);
     const size_t inter = align_up((size_t)n_assign * (size_t)intermediate_size * sizeof(float), 256);
     float* G = (float*)workspace;
     float* U = (float*)((char*)workspace + inter);
     if (chosen == BITSMOE_PATH_DECODE)
-        return launch_forward_decode(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up,
+        return launch_forward_decode(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
                                      token_indices, expert_offsets, route_w, n_assign, rank_out, intermediate_size,
                                      rank_accum, G, U, (int64_t)(inter / sizeof(float)), profile, st);
-    return launch_forward_generic(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up,
+    return launch_forward_generic(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
                                   token_indices, expert_offsets, route_w, n_assign, rank_out,
                                   intermediate_size, rank_accum, G, U, profile, st);
 }

@@ -145,7 +145,7 @@ template <bool BF16, bool GENERAL, int MODE>
 __global__ __launch_bounds__(256) void k_gateup_decode(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
     const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
-    const uint16_t* __restrict__ h_gate, const uint16_t* __restrict__ h_up, int Rg, int Ru,
+    const uint16_t* __restrict__ h_gate, const uint16_t* __restrict__ h_up, int Rg, int Ru, int64_t ldg, int64_t ldu,
     const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
     int E, int n_tiles, int n_groups, int n_tchunks, int tiles_per_wg, float* __restrict__ G, float* __restrict__ U) {
     const int mt = blockIdx.y;
@@ -208,6 +208,7 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
     gptr<int32_t> rank_idx = as_global(fe.rank_idx);
     const uint16_t* __restrict__ h = mt ? h_up : h_gate;
     const int R = mt ? Ru : Rg;
+    const int64_t ld = mt ? ldu : ldg;      // elements from one activation row to the next
     float* __restrict__ out = mt ? U : G;
     const int t0_wg = tchunk * tiles_per_wg;
     const int t1 = min(t0_wg + tiles_per_wg, n_tiles);
@@ -284,7 +285,7 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
                     const int tk = __builtin_amdgcn_readlane(tok_lane, 8 * g + j);
                     const int tkc = min(max(tk, 0), T - 1);
 #pragma unroll
-                    for (int it = 0; it < 2; ++it) raw[it][j] = h[(int64_t)tkc * R + rkc[it]];
+                    for (int it = 0; it < 2; ++it) raw[it][j] = h[(int64_t)tkc * ld + rkc[it]];
                 }
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
@@ -605,9 +606,9 @@ bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up,
 }
 
 int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
-                          const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru,
-                          const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out, int I,
-                          float* rank_accum, float* G, float* U, int64_t inter_floats, bitsmoe_profile* prof,
+                          const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg,
+                          int64_t ldu, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
+                          int I, float* rank_accum, float* G, float* U, int64_t inter_floats, bitsmoe_profile* prof,
                           hipStream_t st) {
     const int E = gate->n_experts;
     const int n_tiles = gate->n_tiles;
@@ -642,7 +643,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     auto launch_gateup = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs, gate->max_slabs,
                            up->d_fast_experts, up->d_fast_slabs, up->max_slabs, (const uint16_t*)h_gate,
-                           (const uint16_t*)h_up, Rg, Ru, tok, off, (int)T, (int)A, I, E, n_tiles, gu_groups, n_tchunks,
+                           (const uint16_t*)h_up, Rg, Ru, ldg, ldu, tok, off, (int)T, (int)A, I, E, n_tiles, gu_groups, n_tchunks,
                            tiles_per_wg, G, U);
     };
     const bool need_general = !(gate->all_uniform8 && up->all_uniform8);

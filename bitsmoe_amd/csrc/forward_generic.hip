@@ -13,7 +13,7 @@ constexpr int AC = 8;  // assignments processed per pass over the weights
 template <typename HT>
 __global__ __launch_bounds__(256) void k_gateup_generic(
     const MatView* __restrict__ gate, const MatView* __restrict__ up,
-    const HT* __restrict__ h_gate, const HT* __restrict__ h_up, int Rg, int Ru,
+    const HT* __restrict__ h_gate, const HT* __restrict__ h_up, int Rg, int Ru, int64_t ldg, int64_t ldu,
     const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets,
     int T, int A, int I, int n_tiles, int ksplit, float* __restrict__ G, float* __restrict__ U) {
     const int mt = blockIdx.y;
@@ -28,6 +28,7 @@ __global__ __launch_bounds__(256) void k_gateup_generic(
     const MatView mv = (mt ? up : gate)[e];
     const HT* __restrict__ h = mt ? h_up : h_gate;
     const int R = mt ? Ru : Rg;
+    const int64_t ld = mt ? ldu : ldg;      // elements from one activation row to the next
     float* __restrict__ out = mt ? U : G;
 
     __shared__ uint32_t pk[K_STAGE * MICROS * 16];
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(256) void k_gateup_generic(
                         const int tok = token_indices[a0 + a];
                         const int rk = mv.rank_idx[rank_off + g0 + r];
                         if (tok >= 0 && tok < T && rk >= 0 && rk < R)
-                            v = to_f32<HT>(h[(int64_t)tok * R + rk]) * __half2float(mv.s[rank_off + g0 + r]);
+                            v = to_f32<HT>(h[(int64_t)tok * ld + rk]) * __half2float(mv.s[rank_off + g0 + r]);
                     }
                     hs[a][r] = v;
                 }
@@ -210,7 +211,7 @@ static inline void record(bitsmoe_profile* p, int i, hipStream_t st) {
 
 int launch_forward_generic(const bitsmoe_matset* gate, const bitsmoe_matset* up,
                            const bitsmoe_matset* down, const void* h_gate, const void* h_up,
-                           int act_dtype, int64_t T, int Rg, int Ru, const int32_t* tok,
+                           int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg, int64_t ldu, const int32_t* tok,
                            const int32_t* off, const float* rw, int64_t A, int rank_out, int I,
                            float* rank_accum, float* G, float* U, bitsmoe_profile* prof,
                            hipStream_t st) {
@@ -234,12 +235,12 @@ int launch_forward_generic(const bitsmoe_matset* gate, const bitsmoe_matset* up,
     dim3 grid((unsigned)(E * n_tiles * ksplit), 2);
     if (act_dtype == BITSMOE_DT_F16) {
         hipLaunchKernelGGL(k_gateup_generic<__half>, grid, dim3(256), 0, st, gate->d_views, up->d_views,
-                           (const __half*)h_gate, (const __half*)h_up, Rg, Ru, tok, off, (int)T, (int)A, I,
+                           (const __half*)h_gate, (const __half*)h_up, Rg, Ru, ldg, ldu, tok, off, (int)T, (int)A, I,
                            n_tiles, ksplit, G, U);
     } else {
         hipLaunchKernelGGL(k_gateup_generic<__hip_bfloat16>, grid, dim3(256), 0, st, gate->d_views,
                            up->d_views, (const __hip_bfloat16*)h_gate, (const __hip_bfloat16*)h_up, Rg, Ru,
-                           tok, off, (int)T, (int)A, I, n_tiles, ksplit, G, U);
+                           ldg, ldu, tok, off, (int)T, (int)A, I, n_tiles, ksplit, G, U);
     }
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 2, st);

@@ -173,8 +173,8 @@ template <bool BF16>
 __global__ __launch_bounds__(256) void k_pregather(const FastExpert* __restrict__ gate_fe,
                                                    const FastExpert* __restrict__ up_fe,
                                                    const uint16_t* __restrict__ h_gate,
-                                                   const uint16_t* __restrict__ h_up, int Rg, int Ru,
-                                                   const int32_t* __restrict__ token_indices,
+                                                   const uint16_t* __restrict__ h_up, int Rg, int Ru, int64_t sg,
+                                                   int64_t su, const int32_t* __restrict__ token_indices,
                                                    const int32_t* __restrict__ expert_offsets, int E, int T, int A,
                                                    uint16_t* __restrict__ Hs_g, uint16_t* __restrict__ Hs_u, int ldg,
                                                    int ldu) {
@@ -196,7 +196,7 @@ __global__ __launch_bounds__(256) void k_pregather(const FastExpert* __restrict_
     uint16_t* __restrict__ out = (mt ? Hs_u : Hs_g) + (int64_t)a * ld;
     const int tok = token_indices[a];
     const bool tok_ok = tok >= 0 && tok < T;
-    const int64_t hrow = (int64_t)(tok_ok ? tok : 0) * R;
+    const int64_t hrow = (int64_t)(tok_ok ? tok : 0) * (mt ? su : sg);      // sg, su: elements between activation rows
     const int K = min(fe.num_slabs * SLAB_ROWS, ld);
     gptr<int32_t> rank_idx = as_global(fe.rank_idx);
     for (int k0 = lane * 8; k0 < K; k0 += 512) {
@@ -223,15 +223,16 @@ __global__ __launch_bounds__(256) void k_pregather(const FastExpert* __restrict_
     }
 }
 
-// bf16 activations [T, R] -> f16 [T, ld] (columns < ld <= R); blockIdx.y = 0: gate, 1: up;
+// bf16 activations (rows sg / su elements apart) -> f16 [T, ld] (columns < ld); blockIdx.y = 0: gate, 1: up;
 // grid-stride over 8-element groups.
 __global__ __launch_bounds__(256) void k_bf16_to_f16(const uint16_t* __restrict__ src_g, const uint16_t* __restrict__ src_u,
-                                                     int64_t T, int Rg, int Ru, int ldg, int ldu,
+                                                     int64_t T, int64_t sg, int64_t su, int ldg, int ldu,
                                                      uint16_t* __restrict__ dst_g, uint16_t* __restrict__ dst_u) {
     const bool is_up = blockIdx.y != 0;
     const uint16_t* src = is_up ? src_u : src_g;
     uint16_t* dst = is_up ? dst_u : dst_g;
-    const int R = is_up ? Ru : Rg, ld = is_up ? ldu : ldg;
+    const int64_t R = is_up ? su : sg;      // elements between source rows
+    const int ld = is_up ? ldu : ldg;
     const int per_row = ld >> 3;
     const int64_t total = T * per_row;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
@@ -899,16 +900,18 @@ size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up
 }
 
 int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
-                        const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru,
-                        const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out, int I,
-                        float* rank_accum, void* workspace, bitsmoe_profile* prof, hipStream_t st) {
+                        const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg_in,
+                        int64_t ldu_in, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
+                        int I, float* rank_accum, void* workspace, bitsmoe_profile* prof, hipStream_t st) {
     const int E = gate->n_experts;
     const int n_tiles = gate->n_tiles;
     const int64_t max_mtiles = A / PF_M + E;
-    const bool direct = direct_ok(gate, up) && Rg % 8 == 0 && Ru % 8 == 0 && (((uintptr_t)h_gate | (uintptr_t)h_up) & 15) == 0 &&
-                        T * (int64_t)std::max(Rg, Ru) < ((int64_t)1 << 31);
-    const int ldg = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(gate) : Rg) : gate->max_slabs * SLAB_ROWS;
-    const int ldu = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(up) : Ru) : up->max_slabs * SLAB_ROWS;
+    // ldg_in / ldu_in: elements between the caller's activation rows (>= Rg / Ru)
+    const bool direct = direct_ok(gate, up) && Rg % 8 == 0 && Ru % 8 == 0 && ldg_in % 8 == 0 && ldu_in % 8 == 0 &&
+                        (((uintptr_t)h_gate | (uintptr_t)h_up) & 15) == 0 &&
+                        T * std::max(ldg_in, ldu_in) < ((int64_t)1 << 31);
+    const int ldg = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(gate) : (int)ldg_in) : gate->max_slabs * SLAB_ROWS;
+    const int ldu = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(up) : (int)ldu_in) : up->max_slabs * SLAB_ROWS;
     const MfmaWorkspace w = mfma_workspace(gate, up, down, T, A, I);
     char* ws = (char*)workspace;
     MTile* mtiles = (MTile*)(ws + w.mtiles);
@@ -935,7 +938,7 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
         if (act_dtype == BITSMOE_DT_BF16) {
             const int64_t groups = T * (std::max(ldg, ldu) / 8);
             hipLaunchKernelGGL(k_bf16_to_f16, dim3((unsigned)std::min<int64_t>((groups + 255) / 256, 2048), 2), dim3(256), 0, st,
-                               (const uint16_t*)h_gate, (const uint16_t*)h_up, T, Rg, Ru, ldg, ldu, (uint16_t*)Hs_g,
+                               (const uint16_t*)h_gate, (const uint16_t*)h_up, T, ldg_in, ldu_in, ldg, ldu, (uint16_t*)Hs_g,
                                (uint16_t*)Hs_u);
             BITSMOE_HIP_TRY(hipGetLastError());
         } else {
@@ -946,11 +949,11 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
         dim3 grid((unsigned)((A + 3) / 4), 2);
         if (act_dtype == BITSMOE_DT_BF16)
             hipLaunchKernelGGL((k_pregather<true>), grid, dim3(256), 0, st, gate->d_fast_experts, up->d_fast_experts,
-                               (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, tok, off, E, (int)T, (int)A,
+                               (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, ldg_in, ldu_in, tok, off, E, (int)T, (int)A,
                                (uint16_t*)Hs_g, (uint16_t*)Hs_u, ldg, ldu);
         else
             hipLaunchKernelGGL((k_pregather<false>), grid, dim3(256), 0, st, gate->d_fast_experts, up->d_fast_experts,
-                               (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, tok, off, E, (int)T, (int)A,
+                               (const uint16_t*)h_gate, (const uint16_t*)h_up, Rg, Ru, ldg_in, ldu_in, tok, off, E, (int)T, (int)A,
                                (uint16_t*)Hs_g, (uint16_t*)Hs_u, ldg, ldu);
         BITSMOE_HIP_TRY(hipGetLastError());
     }

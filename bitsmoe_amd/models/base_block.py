@@ -106,7 +106,7 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         self._cached_token_count = -1
         self._cached_flat_token_ids: Optional[torch.Tensor] = None
         self._matsets = None
-        self._basis_cache: Dict[torch.dtype, Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = {}
+        self._basis_cache: Dict[object, object] = {}      # per dtype: the three bases; ("stacked", dtype): gate over up
 
     def _ensure_runtime_cache(self, device: torch.device) -> None:
         if self._runtime_cache_ready and self._runtime_cache_device == device:
@@ -163,6 +163,16 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         if cached is None:
             cached = tuple(getattr(self, k).to(dtype).contiguous() for k in self._SHARED_BASIS_BUFFER_KEYS)
             self._basis_cache[dtype] = cached
+        return cached
+
+    def _shared_basis_stacked(self, dtype: torch.dtype) -> torch.Tensor:
+        """[rank_gate + rank_up, hidden]: the gate and up bases stacked, for one projection GEMM."""
+        key = ("stacked", dtype)
+        cached = self._basis_cache.get(key)
+        if cached is None:
+            vh_gate, vh_up, _ = self._shared_basis(dtype)
+            cached = torch.cat([vh_gate, vh_up], dim=0).contiguous()
+            self._basis_cache[key] = cached
         return cached
 
     def _get_flat_token_ids(self, token_count: int, device: torch.device) -> torch.Tensor:
@@ -267,9 +277,13 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         token_count, hidden_dim = hidden_states.shape
         if self.shared_vh_gate_proj.numel() == 0 or self.shared_vh_up_proj.numel() == 0:
             raise RuntimeError(f"Layer {self.layer_idx} missing shared_vh basis for packed routed experts.")
-        vh_gate, vh_up, _ = self._shared_basis(hidden_states.dtype)
-        h_gate_proj = hidden_states @ vh_gate.T
-        h_up_proj = hidden_states @ vh_up.T
+        # both shared-basis projections (bitsmoe/models/qwen3moe/bitsmoe_block.py:63-64) as ONE GEMM
+        # against the stacked bases; the operator reads the two halves as strided views
+        vh_both = self._shared_basis_stacked(hidden_states.dtype)
+        rank_gate = int(self.shared_vh_gate_proj.shape[0])
+        h_both = hidden_states @ vh_both.T
+        h_gate_proj = h_both[:, :rank_gate]
+        h_up_proj = h_both[:, rank_gate:]
         flat_selected = selected_experts.reshape(-1)
         flat_w32 = routing_weights_fp32.reshape(-1)
         final = None

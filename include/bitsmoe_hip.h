@@ -179,6 +179,23 @@ int bitsmoe_moe_forward(const bitsmoe_matset* gate, const bitsmoe_matset* up,
                         int64_t n_assign, int32_t rank_out, int32_t intermediate_size,
                         int32_t act_type, int32_t path, float* rank_accum, void* workspace,
                         size_t workspace_bytes, bitsmoe_profile* profile, void* stream);
+/*
+ * The same with the activation rows ld_gate / ld_up elements apart (>= rank_gate / rank_up), so
+ * that h_gate and h_up may be column ranges of one [T, rank_gate + rank_up] product of the two
+ * shared-basis projections (bitsmoe/models/qwen3moe/bitsmoe_block.py:63-64 computes them as two
+ * GEMMs; the reference's operator demands contiguous tensors,
+ * bitsmoe/algorithms/cpp/mlp_forward_binding.cpp:80-86).  bitsmoe_moe_forward is this call with
+ * ld_gate = rank_gate and ld_up = rank_up.
+ */
+int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                                const bitsmoe_matset* down, const void* h_gate, const void* h_up,
+                                int32_t act_dtype, int64_t n_tokens, int32_t rank_gate,
+                                int32_t rank_up, int64_t ld_gate, int64_t ld_up,
+                                const int32_t* token_indices, const int32_t* expert_offsets,
+                                const float* route_w, int64_t n_assign, int32_t rank_out,
+                                int32_t intermediate_size, int32_t act_type, int32_t path,
+                                float* rank_accum, void* workspace, size_t workspace_bytes,
+                                bitsmoe_profile* profile, void* stream);
 
 /*
  * Phase timing with HIP events recorded on the caller's stream between the kernels of

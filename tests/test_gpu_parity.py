@@ -322,6 +322,38 @@ def test_forward_mfma_path_token_with_many_assignments(cuda_device, scramble):
     assert helpers.norm_err(out, ref) < 3e-3
 
 
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+@pytest.mark.parametrize("path_name,tokens", [("generic", 24), ("decode", 24), ("mfma", 300)])
+def test_forward_accepts_column_slices_of_one_projection(cuda_device, path_name, tokens, dtype_name):
+    """h_gate and h_up as column ranges of one [T, rank_gate + rank_up] tensor (the two shared-basis
+    projections done as one GEMM) give the result of the contiguous tensors."""
+    import torch
+
+    from bitsmoe_amd.algorithms import _capi
+
+    hip = _hip()
+    path = {"generic": _capi.PATH_GENERIC, "decode": _capi.PATH_DECODE, "mfma": _capi.PATH_MFMA}[path_name]
+    rng = np.random.default_rng(91)
+    e, k, rin, rout, dim = 4, 2, 128, 128, 256
+    gate, up, down = helpers.make_experts(91, e, rin, rout, dim, slab_multiple=64)
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    both = torch.from_numpy(rng.normal(size=(tokens, 2 * rin + 8)).astype(np.float32)).to(dt).to(cuda_device)
+    h_gate_v, h_up_v = both[:, :rin], both[:, rin:2 * rin]
+    assert not h_gate_v.is_contiguous() and not h_up_v.is_contiguous()
+    idx, w = o.router_qwen(rng.normal(size=(tokens, e)).astype(np.float32), k)
+    tok, off, rw = (torch.from_numpy(x).to(cuda_device) for x in o.build_routing(idx, w, np.arange(e, dtype=np.int32), e))
+    sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=dim) for m in (gate, up, down)]
+    out_v = hip.moe_forward_sets(h_gate_v, h_up_v, tok, off, rw, sets[0], sets[1], sets[2], rout, dim, 0, path=path)
+    out_c = hip.moe_forward_sets(h_gate_v.contiguous(), h_up_v.contiguous(), tok, off, rw, sets[0], sets[1], sets[2],
+                                 rout, dim, 0, path=path)
+    scale = float(out_c.abs().max())
+    assert scale > 0
+    assert float((out_v - out_c).abs().max()) <= 1e-5 * scale      # (fp32 atomics of two runs may differ in order)
+    ref = o.moe_forward(h_gate_v.float().cpu().numpy(), h_up_v.float().cpu().numpy(), tok.cpu().numpy(),
+                        off.cpu().numpy(), rw.cpu().numpy(), gate, up, down, rout, dim)
+    assert helpers.norm_err(out_v.cpu().numpy(), ref) <= 1e-2
+
+
 def test_forward_mfma_path_needs_prepared_sets(cuda_device):
     import torch
 
