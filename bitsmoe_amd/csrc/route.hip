@@ -228,20 +228,50 @@ __global__ __launch_bounds__(ROUTE_THREADS) void k_route_count(
     for (int e = tid; e < n_packed; e += ROUTE_THREADS) chunk_hist[(int64_t)blockIdx.x * n_packed + e] = hist[e];
 }
 
+// One workgroup.  chunk_hist[b][e] (entries of expert e in chunk b) becomes the number of entries of
+// e in earlier chunks; expert_offsets the exclusive scan of the per-expert totals.  The chunks of an
+// expert are split over `parts` threads (parts * n_packed <= 1024) that first add up their runs.
 __global__ __launch_bounds__(1024) void k_route_scan(int32_t* __restrict__ chunk_hist, int n_chunks,
                                                       int n_packed, int32_t* __restrict__ expert_offsets) {
     extern __shared__ int lds[];
-    int* totals = lds;
-    int* wave_sums = lds + n_packed;
-    for (int e = threadIdx.x; e < n_packed; e += blockDim.x) {
-        int run = 0;
-        for (int b = 0; b < n_chunks; ++b) {
-            const int64_t i = (int64_t)b * n_packed + e;
-            const int c = chunk_hist[i];
-            chunk_hist[i] = run;  // entries of this expert in earlier chunks
-            run += c;
+    int* totals = lds;                       // [n_packed]
+    int* wave_sums = lds + n_packed;         // [32]
+    int* partial = lds + n_packed + 32;      // [parts][n_packed] when parts > 1
+    const int tid = threadIdx.x;
+    const int parts = n_packed <= 512 ? min(1024 / n_packed, 16) : 1;
+    if (parts > 1) {
+        const int per = (n_chunks + parts - 1) / parts;
+        const int e = tid % n_packed, p = tid / n_packed;
+        const bool worker = p < parts;
+        const int b0 = min(p * per, n_chunks), b1 = min(b0 + per, n_chunks);
+        int sum = 0;
+        if (worker) {
+            for (int b = b0; b < b1; ++b) sum += chunk_hist[(int64_t)b * n_packed + e];
+            partial[p * n_packed + e] = sum;
         }
-        totals[e] = run;
+        __syncthreads();
+        if (worker) {
+            int run = 0;
+            for (int q = 0; q < p; ++q) run += partial[q * n_packed + e];
+            if (p == parts - 1) totals[e] = run + sum;
+            for (int b = b0; b < b1; ++b) {
+                const int64_t i = (int64_t)b * n_packed + e;
+                const int c = chunk_hist[i];
+                chunk_hist[i] = run;
+                run += c;
+            }
+        }
+    } else {
+        for (int e = tid; e < n_packed; e += blockDim.x) {
+            int run = 0;
+            for (int b = 0; b < n_chunks; ++b) {
+                const int64_t i = (int64_t)b * n_packed + e;
+                const int c = chunk_hist[i];
+                chunk_hist[i] = run;  // entries of this expert in earlier chunks
+                run += c;
+            }
+            totals[e] = run;
+        }
     }
     __syncthreads();
     const int total = block_exclusive_scan(totals, n_packed, wave_sums);
@@ -291,8 +321,8 @@ static int route_impl(const IdT* selected, const float* weights, const int32_t* 
     hipLaunchKernelGGL(k_route_count<IdT>, dim3((unsigned)n_chunks), dim3(ROUTE_THREADS), lds_rank_bytes, st,
                        selected, g2l, n_global, n_flat, n_packed, id_bits, entry_rank, chunk_hist);
     BITSMOE_HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(k_route_scan, dim3(1), dim3(1024), lds_bytes, st, chunk_hist, (int)n_chunks, n_packed,
-                       expert_offsets);
+    hipLaunchKernelGGL(k_route_scan, dim3(1), dim3(1024), lds_bytes + (n_packed <= 512 ? (size_t)16 * n_packed * sizeof(int) : 0),
+                       st, chunk_hist, (int)n_chunks, n_packed, expert_offsets);
     BITSMOE_HIP_TRY(hipGetLastError());
     hipLaunchKernelGGL(k_route_scatter<IdT>, dim3((unsigned)((n_flat + ROUTE_THREADS - 1) / ROUTE_THREADS)),
                        dim3(ROUTE_THREADS), 0, st, selected, weights, g2l, n_global, n_flat, top_k, n_packed,
