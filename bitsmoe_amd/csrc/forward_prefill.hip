@@ -288,13 +288,6 @@ __device__ __forceinline__ void store_piece(uint16_t* __restrict__ stage, int ti
     for (int j = 0; j < NJ; ++j) *reinterpret_cast<u32x4*>(stage + (r0 + 32 * j) * PF_LDS_ROW + kc) = p.v[j];
 }
 
-__device__ __forceinline__ void zero_acc(f32x4 (&acc)[4][4]) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
-}
-
 // ------------------------------------------------------------------------------ gate / up
 constexpr int GU_STAGE = PF_M * PF_LDS_ROW;   // 16-bit elements of one 128 x 64 activation piece in LDS
 
