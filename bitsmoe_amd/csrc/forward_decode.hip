@@ -72,6 +72,22 @@ __device__ inline int nth_active_expert(const int32_t* __restrict__ expert_offse
 struct ChunkRef {
     int expert, chunk;
 };
+// v of lane i + (lanes selected by the DPP control whose source lane exists ? v of the source lane : 0)
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ inline int dpp_add(int v) {
+    return v + __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, false);
+}
+// Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves (no LDS round trips):
+// shifts by 1, 2, 4, 8 inside the rows of 16 lanes, then the row totals broadcast forward.
+__device__ inline int wave_inclusive_scan(int v) {
+    v = dpp_add<0x111>(v);          // row_shr:1
+    v = dpp_add<0x112>(v);          // row_shr:2
+    v = dpp_add<0x114>(v);          // row_shr:4
+    v = dpp_add<0x118>(v);          // row_shr:8
+    v = dpp_add<0x142, 0xa>(v);     // row_bcast:15 into rows 1 and 3
+    v = dpp_add<0x143, 0xc>(v);     // row_bcast:31 into rows 2 and 3
+    return v;
+}
 __device__ inline ChunkRef nth_chunk(const int32_t* __restrict__ expert_offsets, int E, int A, int slot, int lane) {
     int found_e = -1, found_c = 0;
     for (int e0 = 0; e0 < E && found_e < 0; e0 += 64) {
@@ -81,18 +97,13 @@ __device__ inline ChunkRef nth_chunk(const int32_t* __restrict__ expert_offsets,
             const int b = max(expert_offsets[e], 0), en = min(expert_offsets[e + 1], A);
             chunks = en > b ? (en - b + 15) >> 4 : 0;
         }
-        int incl = chunks;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const int v = __shfl_up(incl, d);
-            if (lane >= d) incl += v;
-        }
-        const int total = __shfl(incl, 63);
+        const int incl = wave_inclusive_scan(chunks);
+        const int total = __builtin_amdgcn_readlane(incl, 63);
         if (slot < total) {
             const uint64_t hit = __ballot(slot >= incl - chunks && slot < incl);    // exactly one lane
             const int l = (int)__builtin_ctzll(hit);
             found_e = e0 + l;
-            found_c = slot - __shfl(incl - chunks, l);
+            found_c = slot - __builtin_amdgcn_readlane(incl - chunks, l);
         }
         slot -= total;
     }
@@ -629,9 +640,11 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     const int64_t active_max = std::min<int64_t>(E, A);
     // What the expert coordinate of the grids counts.  Few assignments: the experts that can be
     // active at most, not all of them.  Sixteen or more assignments per expert on average: most
-    // experts have several 16-assignment chunks, one workgroup per chunk (below that the
-    // wave-parallel search of the chunk costs more than walking the few chunks in a loop).
-    const int mode = A >= (int64_t)16 * E ? GRID_CHUNKS : active_max * 2 <= E ? GRID_ACTIVE : GRID_EXPERTS;
+    // experts have several 16-assignment chunks, one workgroup per chunk.  Below that the search
+    // of the chunk (one more dependent round trip per workgroup, +10 %) costs more than walking
+    // an expert's few chunks in a loop, unless routing is skewed: with at most 64 experts (one
+    // search step) the chunk grid is already used from three assignments per expert on average.
+    const int mode = (A >= (int64_t)16 * E || (E <= 64 && A >= (int64_t)3 * E)) ? GRID_CHUNKS : active_max * 2 <= E ? GRID_ACTIVE : GRID_EXPERTS;
     const int e_dim = mode == GRID_CHUNKS ? (int)(active_max + A / MAX_A) : mode == GRID_ACTIVE ? (int)active_max : E;
     // (expert, chunk) pairs expected to have work (e_dim is their upper bound in chunk mode)
     const int64_t units = mode == GRID_CHUNKS ? A / MAX_A + active_max / 2 : active_max;
