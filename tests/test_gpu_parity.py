@@ -218,6 +218,8 @@ def test_irregular_sets_stay_on_generic_kernels(cuda_device):
     (8, 1, 4, 512, 256, 128),
     (6, 40, 3, 576, 192, 384),      # some experts get more than 16 assignments -> several passes
     (16, 64, 8, 1024, 512, 768),
+    (200, 500, 8, 64, 64, 128),     # chunk grid over more than 64 experts (several search steps)
+    (40, 60, 8, 64, 64, 128),       # chunk grid with at most 64 experts
 ])
 def test_forward_decode_path(cuda_device, shape, dtype_name):
     from bitsmoe_amd.algorithms import _capi
@@ -236,6 +238,7 @@ def test_forward_decode_path(cuda_device, shape, dtype_name):
     (3, 200, 2, 192, 192, 128),     # odd slab count in the down matrices: a slab pair with one slab
     (8, 20, 2, 128, 64, 384),       # a handful of rows per expert: half-empty tiles
     (2, 700, 1, 320, 256, 512),     # several full 128-row tiles per expert
+    (300, 900, 2, 64, 64, 128),     # more experts than the tile builder handles in one pass
 ])
 def test_forward_mfma_path(cuda_device, shape, dtype_name):
     from bitsmoe_amd.algorithms import _capi
