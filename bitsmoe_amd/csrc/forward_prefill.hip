@@ -289,7 +289,6 @@ __device__ __forceinline__ void store_piece(uint16_t* __restrict__ stage, int ti
 }
 
 // ------------------------------------------------------------------------------ gate / up
-constexpr int GU_STAGE = PF_M * PF_LDS_ROW;   // 16-bit elements of one 128 x 64 activation piece in LDS
 
 // Everything one thread fetches from global memory for one slab.
 struct GuFetch {
@@ -305,6 +304,11 @@ struct GuFetch {
 // packed multiply.  (One packed FMA with the constant -1.5 * 2^bits * scale_s would round that
 // constant: measured 4.5e-3 of error instead of 5e-4.)
 // WU != 0: the width is a compile-time constant (experts whose slabs all share it).
+// LDS element offset of the 16-byte chunk c (0..7) of row r in a stage written by LDS-direct loads:
+// rows are 128 bytes apart without padding, and the chunks of a row are permuted by the row index
+// so that the sixteen rows an MFMA operand load touches fall into different banks.
+__device__ __forceinline__ int dma_chunk_off(int r, int c) { return r * 64 + ((c ^ ((r >> 1) & 7)) << 3); }
+
 template <int WU, int NMB>
 __device__ __forceinline__ void gateup_slab_mfma(int bits, const uint16_t* __restrict__ stage, const uint32_t (&bw)[2][4],
                                                  const u32x4 (&sc)[2], int lane, f32x4 (&acc)[NMB][4]) {
@@ -316,7 +320,8 @@ __device__ __forceinline__ void gateup_slab_mfma(int bits, const uint16_t* __res
         u32x4 a[NMB];
 #pragma unroll
         for (int mb = 0; mb < NMB; ++mb)
-            a[mb] = *reinterpret_cast<const u32x4*>(stage + (16 * mb + n) * PF_LDS_ROW + 16 * kg + 8 * ks);
+            a[mb] = *reinterpret_cast<const u32x4*>(
+                stage + dma_chunk_off(16 * mb + n, 2 * kg + ks));
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
             const uint32_t(&w)[4] = bw[nb >> 1];
@@ -353,7 +358,7 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
                                                  const uint16_t* __restrict__ Hs, int ld,
                                                  const int32_t* __restrict__ token_indices, int T, int I, int n_tiles,
                                                  uint16_t* __restrict__ out, int a_begin, int rows, int t0,
-                                                 uint16_t* __restrict__ lds) {
+                                                 uint16_t* __restrict__ stage_even, uint16_t* __restrict__ stage_odd) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -408,7 +413,7 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
     };
     auto stage_piece = [&](const GuFetch& src, uint16_t* __restrict__ stage) {
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) *reinterpret_cast<u32x4*>(stage + (r0 + 32 * j) * PF_LDS_ROW + kc) = src.a.v[j];
+        for (int j = 0; j < NJ; ++j) *reinterpret_cast<u32x4*>(stage + dma_chunk_off(r0 + 32 * j, tid & 7)) = src.a.v[j];
     };
     if (nslabs > 0) {
         // prologue: slab 0 is fetched and staged, slab 1 requested
@@ -419,7 +424,7 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
         int pending_rb = rank_base(1);
         int bits = rec.bits;
         issue(F, rec, rank_base(0), 0);
-        stage_piece(F, lds);
+        stage_piece(F, stage_even);
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
             sc[p] = F.sc[p];
@@ -440,7 +445,7 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
             u32x4 sc_next[2];
             const int bits_after = pending.bits;
             if (s + 1 < nslabs) {
-                stage_piece(F, lds + ((s + 1) & 1) * GU_STAGE);
+                stage_piece(F, (s & 1) ? stage_even : stage_odd);
 #pragma unroll
                 for (int p = 0; p < 2; ++p) {
                     sc_next[p] = F.sc[p];
@@ -453,7 +458,8 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
                     pending_rb = rank_base(s + 3);
                 }
             }
-            if (active && bits != 0) gateup_slab_mfma<WU, NMB>(bits, lds + (s & 1) * GU_STAGE, bw, sc, lane, acc);
+            if (active && bits != 0)
+                gateup_slab_mfma<WU, NMB>(bits, (s & 1) ? stage_odd : stage_even, bw, sc, lane, acc);
             __syncthreads();
             if (s + 1 < nslabs) {
 #pragma unroll
@@ -483,6 +489,195 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
     }
 }
 
+// s_waitcnt that only waits for the vector-memory counter: at most `n` operations outstanding
+// (the counter is six bits wide, split over the immediate; the other counters are left alone).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
+}
+// Workgroup barrier without the wait for outstanding loads that __syncthreads implies.  The empty
+// asm statements keep the compiler from moving LDS accesses across it (the bare instruction is no
+// memory fence for the compiler).
+__device__ __forceinline__ void barrier_no_drain() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+constexpr int DMA_STAGES = 3;
+constexpr int DMA_MAX_SLABS = 64;       // per-slab tables in LDS
+constexpr int DMA_STAGE = PF_M * 64;    // 16-bit elements of one unpadded 128 x 64 activation piece
+constexpr int DMA_WSTAGE = 4 * 512;     // 32-bit words: payload of a (slab, tile) block as the four wavefronts fetch it
+constexpr int DMA_SSTAGE = 4 * 64;      // 16-bit scales: 64 contraction rows per wavefront
+
+// One stage of the ring: everything a workgroup needs for one slab.
+struct DmaStage {
+    uint16_t* a;     // [DMA_STAGE]
+    uint32_t* w;     // [DMA_WSTAGE]
+    uint16_t* sc;    // [DMA_SSTAGE]
+};
+
+// The same workgroup job as gateup_tile_body for experts of one bit-width, with EVERYTHING of a
+// slab -- activation piece, payload words, scales -- loaded straight from global memory into LDS
+// (global_load_lds: no registers, no staging instructions), two slabs ahead of the MFMAs in a ring
+// of three stages.  A wavefront's load instruction fills LDS in lane order; which 16-byte chunk of
+// its activation row a lane fetches is chosen so that the stage ends up in the bank-friendly order
+// of dma_chunk_off.  The loop contains no load into registers: the loads of a wavefront complete in
+// order, so "slab s + 1 has landed" is "at most the G loads of slab s + 2 are outstanding", waited
+// for with a bare s_waitcnt, and the workgroup barrier is the bare instruction (__syncthreads would
+// wait for every outstanding load).  Per-slab offsets come from small LDS tables built up front.
+template <bool DIRECT, int WU, int NMB>
+__device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const FastSlab* __restrict__ fs_row, int nslabs,
+                                                     const uint16_t* __restrict__ Hs, int ld,
+                                                     const int32_t* __restrict__ token_indices, int T, int I,
+                                                     int n_tiles, uint16_t* __restrict__ out, int a_begin, int rows,
+                                                     int t0, const DmaStage st0, const DmaStage st1, const DmaStage st2,
+                                                     int32_t* __restrict__ pack_tab, int32_t* __restrict__ scale_tab,
+                                                     int32_t* __restrict__ rank_tab) {
+    static_assert(WU == 2 || WU == 3 || WU == 4, "one bit-width per expert");
+    using gvoid = const void __attribute__((address_space(1)))*;
+    using lvoid = void __attribute__((address_space(3)))*;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tl = wave >> 1, wn = wave & 1;
+    const int n = lane & 15, kg = lane >> 4;
+    const bool two_tiles = t0 + 1 < n_tiles;
+    const bool active = tl == 0 || two_tiles;        // a wavefront without a tile only helps to stage
+    const int t = active ? t0 + tl : t0;             // (it re-reads tile t0: in bounds)
+
+    // this lane lands in row r0 + 32*j, chunk position tid % 8 of a stage; it fetches the chunk that
+    // belongs there (32*j does not change the permutation).  DIRECT: through the token index.
+    constexpr int NJ = (NMB + 1) / 2;      // 32-row groups that hold assignments
+    constexpr int NB = WU == 2 ? 1 : 2;    // payload load instructions per slab
+    constexpr int G = NJ + 1 + NB;         // load instructions per slab and wavefront
+    const int r0 = tid >> 3;
+    const int cpos = (tid & 7) ^ ((r0 >> 1) & 7);
+    uint32_t rowbase[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int a = a_begin + min(r0 + 32 * j, rows - 1);
+        if constexpr (DIRECT) {
+            const int tk = token_indices[a];
+            rowbase[j] = (uint32_t)((tk >= 0 && tk < T) ? tk : 0) * (uint32_t)ld;
+        } else {
+            rowbase[j] = (uint32_t)a * (uint32_t)ld + (uint32_t)(8 * cpos);
+        }
+    }
+    // per-slab tables (ordinary loads, finished before the first LDS-direct load is issued)
+    gptr<int32_t> rank_idx = as_global(fe.rank_idx);
+    for (int i = tid; i < nslabs; i += 256) {
+        const i32x4 r = *reinterpret_cast<const i32x4*>(fs_row + i);     // {bits, pack_off, scale_off, rank_off}
+        pack_tab[i] = r[1];
+        scale_tab[i] = r[2];
+    }
+    if constexpr (DIRECT)
+        for (int i = tid; i < nslabs * 8; i += 256) rank_tab[i] = rank_idx[(i >> 3) * SLAB_ROWS + (i & 7) * 8];
+    __syncthreads();
+
+    f32x4 acc[NMB][4];
+#pragma unroll
+    for (int i = 0; i < NMB; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
+    const uint32_t* __restrict__ payload = fe.payload;
+    const __half* __restrict__ scale = fe.scale_s;
+    // all loads of slab s into stage `st`: G instructions for every wavefront
+    auto request = [&](const DmaStage& st, int s) {
+        const uint32_t col = DIRECT ? (uint32_t)rank_tab[s * 8 + cpos] : (uint32_t)(s * SLAB_ROWS);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+            __builtin_amdgcn_global_load_lds((gvoid)(Hs + (rowbase[j] + col)), (lvoid)(st.a + j * 2048 + wave * 512), 16, 0, 0);
+        // scales of this wavefront's tile: 64 contraction rows, eight lanes of 16 bytes
+        if (lane < 8)
+            __builtin_amdgcn_global_load_lds((gvoid)(scale + (uint32_t)(scale_tab[s] + t * SLAB_ROWS + lane * 8)),
+                                             (lvoid)(st.sc + wave * 64), 16, 0, 0);
+        // payload of the wavefront's two column-block pairs, in memory order
+        const uint32_t* blk = payload + (uint32_t)(pack_tab[s] + t * 256 * WU);
+        if constexpr (WU == 4) {
+#pragma unroll
+            for (int p = 0; p < 2; ++p)
+                __builtin_amdgcn_global_load_lds((gvoid)(blk + ((2 * wn + p) * 64 + lane) * 4),
+                                                 (lvoid)(st.w + wave * 512 + p * 256), 16, 0, 0);
+        } else {
+            __builtin_amdgcn_global_load_lds((gvoid)(blk + 2 * wn * 128 + lane * 4), (lvoid)(st.w + wave * 512), 16, 0, 0);
+            if constexpr (WU == 3) {
+                if (lane < 32)
+                    __builtin_amdgcn_global_load_lds((gvoid)(blk + 512 + 2 * wn * 64 + lane * 4),
+                                                     (lvoid)(st.w + wave * 512 + 256), 16, 0, 0);
+            }
+        }
+    };
+    // payload words and scales of the slab in stage `st`, from LDS to this lane's registers
+    auto take = [&](const DmaStage& st, uint32_t (&bw)[2][4], u32x4 (&sc)[2]) {
+        const uint32_t* wbase = st.w + wave * 512;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            if constexpr (WU == 4) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(wbase + p * 256 + lane * 4);
+                bw[p][0] = v[0]; bw[p][1] = v[1]; bw[p][2] = v[2]; bw[p][3] = v[3];
+            } else {
+                const u32x2 v = *reinterpret_cast<const u32x2*>(wbase + p * 128 + lane * 2);
+                bw[p][0] = v[0]; bw[p][1] = v[1]; bw[p][2] = 0; bw[p][3] = 0;
+                if constexpr (WU == 3) {
+                    const u32x2 h = *reinterpret_cast<const u32x2*>(wbase + 256 + (p * 32 + kg * 8 + (n & 7)) * 2);
+                    bw[p][2] = h[0]; bw[p][3] = h[1];
+                }
+            }
+        }
+        // the MFMA operand of k-step ks holds contraction rows 16*kg + 8*ks .. +7 of the slab
+        sc[0] = *reinterpret_cast<const u32x4*>(st.sc + wave * 64 + 16 * kg);
+        sc[1] = *reinterpret_cast<const u32x4*>(st.sc + wave * 64 + 16 * kg + 8);
+    };
+    if (nslabs > 0) {
+        request(st0, 0);
+        if (nslabs > 1) request(st1, 1);
+        if (nslabs > 1)
+            wait_vmcnt<G>();
+        else
+            wait_vmcnt<0>();
+        barrier_no_drain();
+        // step s (s % 3 == U): slab s + 2 requested into the stage slab s - 1 used, slab s multiplied
+        auto step = [&](auto u_c, int s) {
+            constexpr int U = decltype(u_c)::value;
+            // (the stages are named statically: the compiler then knows that the LDS-direct loads in
+            // flight do not touch the stage being read and adds no wait of its own)
+            const DmaStage& cur = U == 0 ? st0 : U == 1 ? st1 : st2;
+            const DmaStage& nxt = U == 0 ? st2 : U == 1 ? st0 : st1;
+            uint32_t bw[2][4];
+            u32x4 sc[2];
+            take(cur, bw, sc);
+            if (s + 2 < nslabs) request(nxt, s + 2);
+            if (active) gateup_slab_mfma<WU, NMB>(WU, cur.a, bw, sc, lane, acc);
+            asm volatile("" ::: "memory");
+            if (s + 2 < nslabs)
+                wait_vmcnt<G>();      // slab s + 1 has landed; slab s + 2 may be in flight
+            else
+                wait_vmcnt<0>();
+            barrier_no_drain();
+        };
+        for (int s0 = 0; s0 < nslabs; s0 += DMA_STAGES) {
+            step(std::integral_constant<int, 0>{}, s0);
+            if (s0 + 1 < nslabs) step(std::integral_constant<int, 1>{}, s0 + 1);
+            if (s0 + 2 < nslabs) step(std::integral_constant<int, 2>{}, s0 + 2);
+        }
+    }
+    if (!active) return;
+    // lane holds rows 16*mb + 4*kg + j, column 128*t + 64*wn + 16*nb + n
+#pragma unroll
+    for (int mb = 0; mb < NMB; ++mb) {
+        if (16 * mb >= rows) break;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = 16 * mb + 4 * kg + j;
+            if (row >= rows) continue;
+            uint16_t* dst = out + (int64_t)(a_begin + row) * I + N_TILE * t + 64 * wn + n;
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) dst[16 * nb] = __builtin_bit_cast(uint16_t, (_Float16)acc[mb][nb][j]);
+        }
+    }
+}
+
 // grid.x = 32 * ceil(max_mtiles / 32) * 2 * ceil(n_tiles / 2), 256 threads; G and U are f16 [A, I].
 template <bool DIRECT>
 __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
@@ -492,7 +687,11 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     const int32_t* __restrict__ token_indices, int T,
     const MTile* __restrict__ mtiles, const int32_t* __restrict__ n_mtiles, int I, int n_tiles,
     uint16_t* __restrict__ G, uint16_t* __restrict__ U) {
-    __shared__ __attribute__((aligned(16))) uint16_t lds[2 * GU_STAGE];
+    // The ring of the LDS-direct bodies; the register-staged body uses two of the activation stages.
+    __shared__ __attribute__((aligned(16))) uint16_t sa0[DMA_STAGE], sa1[DMA_STAGE], sa2[DMA_STAGE];
+    __shared__ __attribute__((aligned(16))) uint32_t sw0[DMA_WSTAGE], sw1[DMA_WSTAGE], sw2[DMA_WSTAGE];
+    __shared__ __attribute__((aligned(16))) uint16_t ss0[DMA_SSTAGE], ss1[DMA_SSTAGE], ss2[DMA_SSTAGE];
+    __shared__ int32_t pack_tab[DMA_MAX_SLABS], scale_tab[DMA_MAX_SLABS], rank_tab[DMA_MAX_SLABS * 8];
     const int n_tp = (n_tiles + 1) >> 1;
     const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles), 2 * n_tp);
     if (logical < 0) return;
@@ -516,24 +715,38 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     // tiles of at most 32 assignments (experts that see few tokens, remainders) run a body with a
     // quarter of the accumulators, MFMAs and staging; complete bodies, so that no accumulator
     // lives across the choice
+    const DmaStage st0 = {sa0, sw0, ss0}, st1 = {sa1, sw1, ss1}, st2 = {sa2, sw2, ss2};
 #define BITSMOE_GU_BODY(W)                                                                                           \
     do {                                                                                                             \
         if (rows <= 32)                                                                                              \
-            gateup_tile_body<DIRECT, W, 2>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out, a_begin,    \
-                                           rows, 2 * tp, lds);                                                       \
+            gateup_tile_body_dma<DIRECT, W, 2>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out,         \
+                                               a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab); \
         else                                                                                                         \
-            gateup_tile_body<DIRECT, W, 8>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out, a_begin,    \
-                                           rows, 2 * tp, lds);                                                       \
+            gateup_tile_body_dma<DIRECT, W, 8>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out,         \
+                                               a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab); \
     } while (0)
-    if (w == 2)
+    // experts with mixed widths (or more slabs than the tables hold) take the register-staged body
+#define BITSMOE_GU_BODY_MIXED()                                                                                      \
+    do {                                                                                                             \
+        if (rows <= 32)                                                                                              \
+            gateup_tile_body<DIRECT, 0, 2>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out, a_begin,    \
+                                           rows, 2 * tp, sa0, sa1);                                                  \
+        else                                                                                                         \
+            gateup_tile_body<DIRECT, 0, 8>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out, a_begin,    \
+                                           rows, 2 * tp, sa0, sa1);                                                  \
+    } while (0)
+    if (nslabs > DMA_MAX_SLABS)
+        BITSMOE_GU_BODY_MIXED();
+    else if (w == 2)
         BITSMOE_GU_BODY(2);
     else if (w == 3)
         BITSMOE_GU_BODY(3);
     else if (w == 4)
         BITSMOE_GU_BODY(4);
     else
-        BITSMOE_GU_BODY(0);
+        BITSMOE_GU_BODY_MIXED();
 #undef BITSMOE_GU_BODY
+#undef BITSMOE_GU_BODY_MIXED
 }
 
 // z = f16( silu(G) * U ), written over G; 8 elements per thread and iteration.
