@@ -30,7 +30,6 @@
 namespace bitsmoe {
 
 constexpr int PF_M = 128;        // assignments per workgroup tile
-constexpr int PF_LDS_ROW = 72;   // 16-bit elements per LDS row: 64 + 8 (bank stagger, keeps 16-byte alignment)
 
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 
@@ -271,21 +270,37 @@ __device__ inline int xcd_logical(int bid, int n_tiles_real, int units) {
 struct APiece {
     u32x4 v[4];
 };
-template <int NJ>
-__device__ __forceinline__ void load_piece(const uint16_t* __restrict__ src, int64_t ld, int a_begin, int rows, int col0, int tid,
-                                  APiece& p) {
-    const int r0 = tid >> 3, kc = (tid & 7) * 8;
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-        const int row = min(r0 + 32 * j, rows - 1);   // rows past the tile's end repeat the last one; never stored
-        p.v[j] = *reinterpret_cast<const u32x4*>(src + (int64_t)(a_begin + row) * ld + col0 + kc);
-    }
+// LDS element offset of the 16-byte chunk c (0..7) of row r of a 128 x 64 stage: rows are 128
+// bytes apart without padding, and the chunks of a row are permuted by the row index so that the
+// sixteen rows an MFMA operand load touches fall into different banks.  (LDS-direct loads fill
+// LDS in lane order, which rules out padded rows.)
+__device__ __forceinline__ int dma_chunk_off(int r, int c) { return r * 64 + ((c ^ ((r >> 1) & 7)) << 3); }
+
+// s_waitcnt that only waits for the vector-memory counter: at most `n` operations outstanding
+// (the counter is six bits wide, split over the immediate; the other counters are left alone).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
 }
-template <int NJ>
-__device__ __forceinline__ void store_piece(uint16_t* __restrict__ stage, int tid, const APiece& p) {
-    const int r0 = tid >> 3, kc = (tid & 7) * 8;
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) *reinterpret_cast<u32x4*>(stage + (r0 + 32 * j) * PF_LDS_ROW + kc) = p.v[j];
+// Workgroup barrier without the wait for outstanding loads that __syncthreads implies.  The empty
+// asm statements keep the compiler from moving LDS accesses across it (the bare instruction is no
+// memory fence for the compiler).
+__device__ __forceinline__ void barrier_no_drain() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+constexpr int DMA_STAGE = PF_M * 64;    // 16-bit elements of one unpadded 128 x 64 activation piece
+
+// LDS-direct load: every active lane fetches 16 bytes from `src`, and the wavefront's data lands in
+// LDS at lds_base + 16 * lane (lds_base is wave-uniform).  Issued from an asm statement, so the
+// compiler keeps no book on it: it neither waits for these loads before LDS reads it cannot tell
+// apart from their destination, nor turns its other waits into waits for everything.  The caller
+// counts them (wait_vmcnt) and orders LDS accesses around them (barrier_no_drain).
+__device__ __forceinline__ void load_to_lds16(const void* src, void* lds_base) {
+    using lvoid = void __attribute__((address_space(3)))*;
+    const uint32_t l = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lvoid)lds_base);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(l) : "m0", "memory");
 }
 
 // ------------------------------------------------------------------------------ gate / up
@@ -304,11 +319,6 @@ struct GuFetch {
 // packed multiply.  (One packed FMA with the constant -1.5 * 2^bits * scale_s would round that
 // constant: measured 4.5e-3 of error instead of 5e-4.)
 // WU != 0: the width is a compile-time constant (experts whose slabs all share it).
-// LDS element offset of the 16-byte chunk c (0..7) of row r in a stage written by LDS-direct loads:
-// rows are 128 bytes apart without padding, and the chunks of a row are permuted by the row index
-// so that the sixteen rows an MFMA operand load touches fall into different banks.
-__device__ __forceinline__ int dma_chunk_off(int r, int c) { return r * 64 + ((c ^ ((r >> 1) & 7)) << 3); }
-
 template <int WU, int NMB>
 __device__ __forceinline__ void gateup_slab_mfma(int bits, const uint16_t* __restrict__ stage, const uint32_t (&bw)[2][4],
                                                  const u32x4 (&sc)[2], int lane, f32x4 (&acc)[NMB][4]) {
@@ -489,24 +499,8 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
     }
 }
 
-// s_waitcnt that only waits for the vector-memory counter: at most `n` operations outstanding
-// (the counter is six bits wide, split over the immediate; the other counters are left alone).
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
-}
-// Workgroup barrier without the wait for outstanding loads that __syncthreads implies.  The empty
-// asm statements keep the compiler from moving LDS accesses across it (the bare instruction is no
-// memory fence for the compiler).
-__device__ __forceinline__ void barrier_no_drain() {
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
-
 constexpr int DMA_STAGES = 3;
 constexpr int DMA_MAX_SLABS = 64;       // per-slab tables in LDS
-constexpr int DMA_STAGE = PF_M * 64;    // 16-bit elements of one unpadded 128 x 64 activation piece
 constexpr int DMA_WSTAGE = 4 * 512;     // 32-bit words: payload of a (slab, tile) block as the four wavefronts fetch it
 constexpr int DMA_SSTAGE = 4 * 64;      // 16-bit scales: 64 contraction rows per wavefront
 
@@ -777,7 +771,7 @@ constexpr int DN_SLABS_MFMA = 4;   // slabs (64 output rows each) per workgroup:
 // pair, per 16-row block.  The weight operand is (code - 2^(W-1)) * scale rounded once to f16,
 // the operand the reference builds (bitsmoe/algorithms/cpp/mlp_forward.cu:1554-1694).
 template <int HH, int NMB>
-__device__ __forceinline__ void down_half_mfma(int bits, const uint16_t* __restrict__ stage, const Block16& blk,
+__device__ __forceinline__ void down_half_mfma(int bits, const uint16_t* stage, const Block16& blk,
                                       const uint32_t (&scp)[4], int lane, f32x4 (&acc)[NMB][4]) {
     const int n = lane & 15, kg = lane >> 4;
 #pragma unroll
@@ -786,7 +780,7 @@ __device__ __forceinline__ void down_half_mfma(int bits, const uint16_t* __restr
         u32x4 a[NMB];
 #pragma unroll
         for (int mb = 0; mb < NMB; ++mb)
-            a[mb] = *reinterpret_cast<const u32x4*>(stage + (16 * mb + n) * PF_LDS_ROW + 32 * km + 8 * kg);
+            a[mb] = *reinterpret_cast<const u32x4*>(stage + dma_chunk_off(16 * mb + n, 4 * km + kg));
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
             // the width switch wraps one operand only: accumulators that flow through alternative
@@ -810,57 +804,123 @@ __device__ __forceinline__ void down_half_mfma(int bits, const uint16_t* __restr
     }
 }
 
+constexpr int DN_WBUF = 1024;    // 32-bit words: the payload block of one (slab, tile) as its wavefront fetches it
+constexpr int DN_SBUF = 64;      // 16-bit scales of one (slab, tile) block
+
 // The column loop of one wavefront (fs.bits == 0: no slab, the wavefront only helps to stage).
-// Pieces of z (128 assignments x 64 columns) run two ahead of the MFMAs in two alternating
-// register sets, the payload block of the next tile one tile ahead.
+// Everything comes straight from global memory into LDS (LDS-direct loads, no registers in
+// between): the pieces of z (128 assignments x 64 columns, chunk order of dma_chunk_off) into a
+// ring of three stages shared by the workgroup, two pieces ahead of the MFMAs; the payload block
+// and scales of the wavefront's next tile into a buffer of its own, from where they are taken
+// into registers when the tile begins.  The loads of a wavefront complete in order and every
+// wavefront issues the same number per step (four 16-byte payload loads whatever the width:
+// narrower blocks repeat an address), so "piece h + 1 has landed" is a count of outstanding
+// loads, waited for with a bare s_waitcnt before a bare barrier.
 template <int NMB>
-__device__ __forceinline__ void down_tile_loop(gptr<uint32_t> payload, gptr<__half> scale, const FastSlab fs,
-                                      const uint16_t* __restrict__ z, int I, int n_tiles, int a_begin, int rows,
-                                      uint16_t (*lds)[PF_M * PF_LDS_ROW], int tid, int lane, f32x4 (&acc)[NMB][4]) {
-    constexpr int NJ = (NMB + 1) / 2;      // 32-row groups a thread stages
+__device__ __forceinline__ void down_tile_loop(const uint32_t* __restrict__ payload, const __half* __restrict__ scale,
+                                      const FastSlab fs, const uint16_t* __restrict__ z, int I, int n_tiles, int a_begin, int rows,
+                                      uint16_t* st0, uint16_t* st1, uint16_t* st2, uint32_t* wbuf_all,
+                                      uint16_t* sbuf_all, int tid, int lane, f32x4 (&acc)[NMB][4]) {
+    constexpr int NJ = (NMB + 1) / 2;      // 32-row groups that hold assignments
+    constexpr int NP = 5;                  // payload and scale load instructions per tile
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15;
     const int W = fs.bits;
-    APiece p0, p1;
-    Block16 blk, blk_n;
-    uint32_t scp[4], scp_n[4];
-    auto issue_b = [&](int t, Block16& b, uint32_t(&s4)[4]) {
-        if (W != 0) {
-            gptr<uint32_t> src = payload + (uint32_t)(fs.pack_off + t * 256 * W);
-            if (W == 2)
-                load_block_role1<2>(src, lane, b);
-            else if (W == 3)
-                load_block_role1<3>(src, lane, b);
-            else
-                load_block_role1<4>(src, lane, b);
-            gptr<uint16_t> sp = reinterpret_cast<gptr<uint16_t>>(scale + (uint32_t)(fs.scale_off + t * SLAB_ROWS + n));
+    uint32_t* wbuf = wbuf_all + wave * DN_WBUF;
+    uint16_t* sbuf = sbuf_all + wave * DN_SBUF;
+    // this lane lands in row r0 + 32*j, chunk position tid % 8 of a stage and fetches the chunk
+    // that belongs there
+    const int r0 = tid >> 3;
+    const int cpos = (tid & 7) ^ ((r0 >> 1) & 7);
+    uint32_t rowbase[NJ];
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb) s4[nb] = (uint32_t)sp[16 * nb] * 0x10001u;
-        }
+    for (int j = 0; j < NJ; ++j)
+        rowbase[j] = (uint32_t)(a_begin + min(r0 + 32 * j, rows - 1)) * (uint32_t)I + (uint32_t)(8 * cpos);
+    auto request_z = [&](uint16_t* st, int h) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+            load_to_lds16(z + (rowbase[j] + (uint32_t)(64 * h)), st + j * 2048 + wave * 512);
     };
-    const int n_halves = 2 * n_tiles;
-    load_piece<NJ>(z, I, a_begin, rows, 0, tid, p0);
-    load_piece<NJ>(z, I, a_begin, rows, 64, tid, p1);
-    issue_b(0, blk, scp);
-    store_piece<NJ>(lds[0], tid, p0);
-    __syncthreads();
-    for (int t = 0; t < n_tiles; ++t) {
-        const int h = 2 * t;
-        // first half of tile t is in lds[0], the second in flight in p1
-        if (h + 2 < n_halves) load_piece<NJ>(z, I, a_begin, rows, 64 * (h + 2), tid, p0);
-        if (t + 1 < n_tiles) issue_b(t + 1, blk_n, scp_n);
-        if (W != 0) down_half_mfma<0, NMB>(W, lds[0], blk, scp, lane, acc);
-        store_piece<NJ>(lds[1], tid, p1);
-        __syncthreads();
-        if (h + 3 < n_halves) load_piece<NJ>(z, I, a_begin, rows, 64 * (h + 3), tid, p1);
-        if (W != 0) down_half_mfma<1, NMB>(W, lds[1], blk, scp, lane, acc);
-        if (h + 2 < n_halves) store_piece<NJ>(lds[0], tid, p0);
-        __syncthreads();
-        {
-            if (W != 0 && t + 1 < n_tiles) {
-                blk = blk_n;
+    // role 1 block: 2-bit 8 words per lane, 4-bit 16, 3-bit 8 low words + 4 high words
+    // (fast_helpers.h); load i fills words 4i .. 4i+3 of every lane's sixteen
+    const uint32_t lane_words = (uint32_t)lane * (W == 4 ? 16u : W != 0 ? 8u : 4u);
+    auto request_b = [&](int t) {
+        const uint32_t base = W != 0 ? (uint32_t)(fs.pack_off + t * 256 * W) : 0u;
+        const uint32_t o0 = base + lane_words;
+        const uint32_t o1 = W != 0 ? o0 + 4u : o0;
+        const uint32_t o2 = W == 4 ? o0 + 8u : W == 3 ? base + 512u + (uint32_t)lane * 4u : o0;
+        const uint32_t o3 = W == 4 ? o0 + 12u : o0;
+        load_to_lds16(payload + o0, wbuf);
+        load_to_lds16(payload + o1, wbuf + 256);
+        load_to_lds16(payload + o2, wbuf + 512);
+        load_to_lds16(payload + o3, wbuf + 768);
+        const uint32_t so = W != 0 ? (uint32_t)(fs.scale_off + t * SLAB_ROWS) : 0u;
+        if (lane < 8) load_to_lds16(scale + (so + (uint32_t)lane * 8u), sbuf);
+    };
+    Block16 blk;
+    uint32_t scp[4];
+    auto take_b = [&]() {
 #pragma unroll
-                for (int nb = 0; nb < 4; ++nb) scp[nb] = scp_n[nb];
-            }
+        for (int i = 0; i < 4; ++i) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(wbuf + i * 256 + lane * 4);
+            blk.w[4 * i] = v[0];
+            blk.w[4 * i + 1] = v[1];
+            blk.w[4 * i + 2] = v[2];
+            blk.w[4 * i + 3] = v[3];
+        }
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) scp[nb] = (uint32_t)sbuf[16 * nb + n] * 0x10001u;
+        // the buffer is requested again right away: its reads must have returned
+        __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0)
+        asm volatile("" ::: "memory");
+    };
+    const int n_halves = 2 * n_tiles;      // at least two
+    request_z(st0, 0);
+    request_b(0);
+    request_z(st1, 1);
+    wait_vmcnt<NJ>();                      // block 0 and piece 0 have landed
+    barrier_no_drain();
+    // step h (h % 3 == U, h % 2 == HH): (first half of a tile) the tile's block taken into
+    // registers; piece h + 2 requested into the stage piece h - 1 used, then (first half) the next
+    // tile's block; piece h multiplied
+    auto step = [&](auto u_c, auto hh_c, int h) {
+        constexpr int U = decltype(u_c)::value;
+        constexpr int HH = decltype(hh_c)::value;
+        // (the stages are named statically, so that the compiler can tell the stage being read
+        // from the ones being loaded)
+        uint16_t* cur = U == 0 ? st0 : U == 1 ? st1 : st2;
+        uint16_t* nxt = U == 0 ? st2 : U == 1 ? st0 : st1;
+        const bool more = h + 2 < n_halves;
+        if (HH == 0) take_b();
+        if (more) {
+            request_z(nxt, h + 2);
+            if (HH == 0) request_b((h >> 1) + 1);      // h + 2 < n_halves: there is a next tile
+        }
+        if (W != 0) down_half_mfma<HH, NMB>(W, cur, blk, scp, lane, acc);
+        asm volatile("" ::: "memory");
+        // piece h + 1 (and, after a second half, the next tile's block) must have landed; what this
+        // step requested may still be in flight
+        if (!more)
+            wait_vmcnt<0>();
+        else if (HH == 0)
+            wait_vmcnt<NJ + NP>();
+        else
+            wait_vmcnt<NJ>();
+        barrier_no_drain();
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    for (int h0 = 0; h0 < n_halves; h0 += 6) {
+        step(I0{}, I0{}, h0);
+        step(I1{}, I1{}, h0 + 1);
+        if (h0 + 2 < n_halves) {
+            step(I2{}, I0{}, h0 + 2);
+            step(I0{}, I1{}, h0 + 3);
+        }
+        if (h0 + 4 < n_halves) {
+            step(I1{}, I0{}, h0 + 4);
+            step(I2{}, I1{}, h0 + 5);
         }
     }
 }
@@ -879,7 +939,9 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
                                                       const int32_t* __restrict__ token_start,
                                                       int2* __restrict__ token_list, int A, int I, int n_tiles,
                                                       int n_groups, _Float16* __restrict__ y, int ldy) {
-    __shared__ __attribute__((aligned(16))) uint16_t lds[2][PF_M * PF_LDS_ROW];
+    __shared__ __attribute__((aligned(16))) uint16_t sz0[DMA_STAGE], sz1[DMA_STAGE], sz2[DMA_STAGE];
+    __shared__ __attribute__((aligned(16))) uint32_t wbuf[4 * DN_WBUF];
+    __shared__ __attribute__((aligned(16))) uint16_t sbuf[4 * DN_SBUF];
     const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles), n_groups);
     if (logical < 0) return;
     const int mt_i = logical / n_groups, grp = logical - mt_i * n_groups;
@@ -903,8 +965,6 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
     const int si = DN_SLABS_MFMA * grp + wave;
     FastSlab fs = FastSlab{0, 0, 0, 0};
     if (si < nslabs) fs = load_fast_slab(down_fs + (int64_t)e * max_slabs, si);
-    gptr<uint32_t> payload = as_global(fe.payload);
-    gptr<__half> scale = as_global(fe.scale);
 
     // tiles of at most 32 assignments run a body with a quarter of the accumulators and MFMAs:
     // two complete bodies, so that no accumulator lives across the choice
@@ -916,7 +976,7 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
         // wavefronts without a slab skip the MFMAs; all execute the same barriers
-        down_tile_loop<NMB>(payload, scale, fs, z, I, n_tiles, a_begin, rows, lds, tid, lane, acc);
+        down_tile_loop<NMB>(fe.payload, fe.scale, fs, z, I, n_tiles, a_begin, rows, sz0, sz1, sz2, wbuf, sbuf, tid, lane, acc);
         if (fs.bits == 0) return;
 
         // lane holds assignments 16*mb + 4*kg + j, output rows 16*nb + n of the slab
