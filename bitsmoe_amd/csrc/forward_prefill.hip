@@ -529,8 +529,6 @@ __device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const 
                                                      int32_t* __restrict__ pack_tab, int32_t* __restrict__ scale_tab,
                                                      int32_t* __restrict__ rank_tab) {
     static_assert(WU == 2 || WU == 3 || WU == 4, "one bit-width per expert");
-    using gvoid = const void __attribute__((address_space(1)))*;
-    using lvoid = void __attribute__((address_space(3)))*;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -581,24 +579,21 @@ __device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const 
         const uint32_t col = DIRECT ? (uint32_t)rank_tab[s * 8 + cpos] : (uint32_t)(s * SLAB_ROWS);
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
-            __builtin_amdgcn_global_load_lds((gvoid)(Hs + (rowbase[j] + col)), (lvoid)(st.a + j * 2048 + wave * 512), 16, 0, 0);
+            load_to_lds16(Hs + (rowbase[j] + col), st.a + j * 2048 + wave * 512);
         // scales of this wavefront's tile: 64 contraction rows, eight lanes of 16 bytes
         if (lane < 8)
-            __builtin_amdgcn_global_load_lds((gvoid)(scale + (uint32_t)(scale_tab[s] + t * SLAB_ROWS + lane * 8)),
-                                             (lvoid)(st.sc + wave * 64), 16, 0, 0);
+            load_to_lds16(scale + (uint32_t)(scale_tab[s] + t * SLAB_ROWS + lane * 8), st.sc + wave * 64);
         // payload of the wavefront's two column-block pairs, in memory order
         const uint32_t* blk = payload + (uint32_t)(pack_tab[s] + t * 256 * WU);
         if constexpr (WU == 4) {
 #pragma unroll
             for (int p = 0; p < 2; ++p)
-                __builtin_amdgcn_global_load_lds((gvoid)(blk + ((2 * wn + p) * 64 + lane) * 4),
-                                                 (lvoid)(st.w + wave * 512 + p * 256), 16, 0, 0);
+                load_to_lds16(blk + ((2 * wn + p) * 64 + lane) * 4, st.w + wave * 512 + p * 256);
         } else {
-            __builtin_amdgcn_global_load_lds((gvoid)(blk + 2 * wn * 128 + lane * 4), (lvoid)(st.w + wave * 512), 16, 0, 0);
+            load_to_lds16(blk + 2 * wn * 128 + lane * 4, st.w + wave * 512);
             if constexpr (WU == 3) {
                 if (lane < 32)
-                    __builtin_amdgcn_global_load_lds((gvoid)(blk + 512 + 2 * wn * 64 + lane * 4),
-                                                     (lvoid)(st.w + wave * 512 + 256), 16, 0, 0);
+                    load_to_lds16(blk + 512 + 2 * wn * 64 + lane * 4, st.w + wave * 512 + 256);
             }
         }
     };
@@ -634,8 +629,8 @@ __device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const 
         // step s (s % 3 == U): slab s + 2 requested into the stage slab s - 1 used, slab s multiplied
         auto step = [&](auto u_c, int s) {
             constexpr int U = decltype(u_c)::value;
-            // (the stages are named statically: the compiler then knows that the LDS-direct loads in
-            // flight do not touch the stage being read and adds no wait of its own)
+            // (the stages are named statically, so that the compiler can tell the stage being read
+            // from the ones being loaded)
             const DmaStage& cur = U == 0 ? st0 : U == 1 ? st1 : st2;
             const DmaStage& nxt = U == 0 ? st2 : U == 1 ? st0 : st1;
             uint32_t bw[2][4];
