@@ -3,10 +3,10 @@
 // of one expert.  See wave_layout.h for the layout and the (2^w + code) operand trick.
 //
 //   k_gateup_decode   G[a,c] / U[a,c] += sum_k  hs'[a,k] * level[k,c]
-//                     hs'[a,k] = h[tok_a, rank_idx[k]] * s[k] * scale[tile(c), k]  (16-bit operand)
+//                     hs'[a,k] = h[tok_a, rank_idx[k]] * s[k] * scale[tile(c), k]  (f16 operand)
 //   k_down_decode     rank_accum[tok_a, rank_idx[r]] += route_w[a] * s[r] *
 //                         sum_tiles scale[tile, r] * sum_{c in tile} level[r,c] * z[a,c]
-//                     z = silu(G) * U  (16-bit operand)
+//                     z = silu(G) * U  (f16 operand)
 //
 // MFMA operands: A = activations (row index = assignment), B = weights (column index =
 // output column / output rank row); D[4*(lane/16)+j][lane%16].
@@ -117,26 +117,26 @@ constexpr int GRID_CHUNKS = 2;    // ... counts 16-assignment chunks (nth_chunk)
 // ------------------------------------------------------------------------------ gate / up
 // One (slab, tile) block restricted to one column-block pair: 2 column blocks x 2 k-steps,
 // plus the two MFMAs that accumulate the constant term.
-template <int W, bool BF16>
+template <int W>
 __device__ __forceinline__ void gateup_pair(const uint32_t (&w)[4], u32x4 a0, u32x4 a1, int upper, f32x4 (&acc)[2], f32x4& corr) {
-    const u32x4 bc = corr_operand<W, BF16>();
-    corr = mfma16<BF16>(a0, bc, corr);
-    corr = mfma16<BF16>(a1, bc, corr);
+    const u32x4 bc = corr_operand<W, false>();
+    corr = mfma16<false>(a0, bc, corr);
+    corr = mfma16<false>(a1, bc, corr);
 #pragma unroll
     for (int nbl = 0; nbl < 2; ++nbl) {
         u32x4 b0, b1;
         if constexpr (W == 2) {
-            b0 = decode_fields2<2, BF16>(w[nbl], 0);
-            b1 = decode_fields2<2, BF16>(w[nbl], 8);
+            b0 = decode_fields2<2, false>(w[nbl], 0);
+            b1 = decode_fields2<2, false>(w[nbl], 8);
         } else if constexpr (W == 4) {
-            b0 = decode_fields4<BF16>(w[2 * nbl]);
-            b1 = decode_fields4<BF16>(w[2 * nbl + 1]);
+            b0 = decode_fields4<false>(w[2 * nbl]);
+            b1 = decode_fields4<false>(w[2 * nbl + 1]);
         } else {
-            b0 = decode_fields3<BF16>(w[nbl], 0, w[2 + nbl], 8 * upper);
-            b1 = decode_fields3<BF16>(w[nbl], 8, w[2 + nbl], 8 * upper + 4);
+            b0 = decode_fields3<false>(w[nbl], 0, w[2 + nbl], 8 * upper);
+            b1 = decode_fields3<false>(w[nbl], 8, w[2 + nbl], 8 * upper + 4);
         }
-        acc[nbl] = mfma16<BF16>(a0, b0, acc[nbl]);
-        acc[nbl] = mfma16<BF16>(a1, b1, acc[nbl]);
+        acc[nbl] = mfma16<false>(a0, b0, acc[nbl]);
+        acc[nbl] = mfma16<false>(a1, b1, acc[nbl]);
     }
 }
 
@@ -306,6 +306,13 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
                     for (int it = 0; it < 2; ++it)
                         if (!(tk_ok && rk[it] >= 0)) raw[it][j] = 0;
                 }
+                if constexpr (BF16) {      // the MFMA operands are f16 whatever the activations are
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+#pragma unroll
+                        for (int it = 0; it < 2; ++it)
+                            raw[it][j] = __builtin_bit_cast(uint16_t, (_Float16)__uint_as_float(raw[it][j] << 16));
+                }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     hp[0][4 * g + j] = raw[0][2 * j] | (raw[0][2 * j + 1] << 16);
@@ -326,14 +333,14 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
 #pragma unroll
             for (int it = 0; it < 2; ++it) {
                 if (mine[it].bits == 0) continue;
-                const float sv = srow[it] * sc_cur[it];
+                // two assignments per packed multiply; rows without an assignment hold zeros
+                const uint32_t sv = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)(srow[it] * sc_cur[it])) * 0x10001u;
                 uint16_t* dst = &hs[(pair + 4 * it) * SLAB_ROWS + lane];
 #pragma unroll
                 for (int ap = 0; ap < MAX_A / 2; ++ap) {
-                    if (2 * ap < n_a) {
-                        dst[(2 * ap) * GU_STRIDE] = to_operand<BF16>(operand_to_f32<BF16>((uint16_t)(hp[it][ap] & 0xFFFFu)) * sv);
-                        dst[(2 * ap + 1) * GU_STRIDE] = to_operand<BF16>(operand_to_f32<BF16>((uint16_t)(hp[it][ap] >> 16)) * sv);
-                    }
+                    const uint32_t v = pk_mul_f16(hp[it][ap], sv);
+                    dst[(2 * ap) * GU_STRIDE] = (uint16_t)(v & 0xFFFFu);
+                    dst[(2 * ap + 1) * GU_STRIDE] = (uint16_t)(v >> 16);
                 }
             }
             __syncthreads();   // hs'(t) is complete
@@ -347,11 +354,11 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
                 const u32x4 a_lo = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS);
                 const u32x4 a_hi = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS + 8);
                 if (bq == 2)
-                    gateup_pair<2, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
+                    gateup_pair<2>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
                 else if (bq == 3)
-                    gateup_pair<3, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
+                    gateup_pair<3>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
                 else
-                    gateup_pair<4, BF16>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
+                    gateup_pair<4>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
                 // the buffer is free again: fetch the same slab's block of the next tile
                 if (more) issue(qc, t + 1, bq, q_pack(q));
             }, std::make_integer_sequence<int, GU_SLABS>{});
@@ -696,10 +703,8 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     auto launch_down_mode = [&](auto bf16_c, auto mode_c) {
         launch_down(k_down_decode<decltype(bf16_c)::value, decltype(mode_c)::value>);
     };
-    if (bf16)
-        with_mode(launch_down_mode, std::true_type{});
-    else
-        with_mode(launch_down_mode, std::false_type{});
+    // (G and U are fp32 and the operands f16 whatever the activation type was)
+    with_mode(launch_down_mode, std::false_type{});
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 3, st);
     if (prof) prof->recorded = true;

@@ -31,23 +31,12 @@ namespace bitsmoe {
 
 constexpr int PF_M = 128;        // assignments per workgroup tile
 
-typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-
 struct MTile {
     int32_t expert;   // -1: unused slot
     int32_t a_begin;
     int32_t rows;
     int32_t pad;
 };
-
-__device__ inline uint32_t pk_add_f16(uint32_t a, uint32_t b) {
-    const h2 r = __builtin_bit_cast(h2, a) + __builtin_bit_cast(h2, b);
-    return __builtin_bit_cast(uint32_t, r);
-}
-__device__ inline uint32_t pk_mul_f16(uint32_t a, uint32_t b) {
-    const h2 r = __builtin_bit_cast(h2, a) * __builtin_bit_cast(h2, b);
-    return __builtin_bit_cast(uint32_t, r);
-}
 
 // -(1.5 * 2^W) as a packed f16 pair: times the scale it is the constant that turns
 // (2^W + code) * scale into (code - 2^(W-1)) * scale.

@@ -142,6 +142,17 @@ __device__ inline u32x4 decode_fields3(uint32_t z, int first, uint32_t hi, int h
     return r;
 }
 
+// Packed f16 arithmetic on two values in one 32-bit register.
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+__device__ inline uint32_t pk_add_f16(uint32_t a, uint32_t b) {
+    const h2 r = __builtin_bit_cast(h2, a) + __builtin_bit_cast(h2, b);
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ inline uint32_t pk_mul_f16(uint32_t a, uint32_t b) {
+    const h2 r = __builtin_bit_cast(h2, a) * __builtin_bit_cast(h2, b);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
 template <bool BF16>
 __device__ inline f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
     if constexpr (BF16)
