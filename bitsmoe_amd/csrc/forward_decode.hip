@@ -3,7 +3,8 @@
 // of one expert.  See wave_layout.h for the layout and the (2^w + code) operand trick.
 //
 //   k_gateup_decode   G[a,c] / U[a,c] += sum_k  hs'[a,k] * level[k,c]
-//                     hs'[a,k] = h[tok_a, rank_idx[k]] * s[k] * scale[tile(c), k]  (f16 operand)
+//                     hs'[a,k] = h[tok_a, rank_idx[k]] * s[k] * scale[tile(c), k]  (f16 operand,
+//                     times the power of two by which the staggered field decode shrinks the code)
 //   k_down_decode     rank_accum[tok_a, rank_idx[r]] += route_w[a] * s[r] *
 //                         sum_tiles scale[tile, r] * sum_{c in tile} level[r,c] * z[a,c]
 //                     z = silu(G) * U  (f16 operand)
@@ -116,24 +117,25 @@ constexpr int GRID_CHUNKS = 2;    // ... counts 16-assignment chunks (nth_chunk)
 
 // ------------------------------------------------------------------------------ gate / up
 // One (slab, tile) block restricted to one column-block pair: 2 column blocks x 2 k-steps,
-// plus the two MFMAs that accumulate the constant term.
+// plus the two MFMAs that accumulate the constant term.  The decoded registers hold
+// 2^W + code / f_i (staggered fields, wave_layout.h); the activations carry f_i.
 template <int W>
 __device__ __forceinline__ void gateup_pair(const uint32_t (&w)[4], u32x4 a0, u32x4 a1, int upper, f32x4 (&acc)[2], f32x4& corr) {
-    const u32x4 bc = corr_operand<W, false>();
+    const u32x4 bc = offset0_regs<W>();
     corr = mfma16<false>(a0, bc, corr);
     corr = mfma16<false>(a1, bc, corr);
 #pragma unroll
     for (int nbl = 0; nbl < 2; ++nbl) {
         u32x4 b0, b1;
         if constexpr (W == 2) {
-            b0 = decode_fields2<2, false>(w[nbl], 0);
-            b1 = decode_fields2<2, false>(w[nbl], 8);
+            b0 = decode0_lo<2>(w[nbl], 0);
+            b1 = decode0_lo<2>(w[nbl], 1);
         } else if constexpr (W == 4) {
-            b0 = decode_fields4<false>(w[2 * nbl]);
-            b1 = decode_fields4<false>(w[2 * nbl + 1]);
+            b0 = decode0_fields4(w[2 * nbl]);
+            b1 = decode0_fields4(w[2 * nbl + 1]);
         } else {
-            b0 = decode_fields3<false>(w[nbl], 0, w[2 + nbl], 8 * upper);
-            b1 = decode_fields3<false>(w[nbl], 8, w[2 + nbl], 8 * upper + 4);
+            b0 = decode0_fields3(w[nbl], 0, w[2 + nbl], upper);
+            b1 = decode0_fields3(w[nbl], 1, w[2 + nbl], upper);
         }
         acc[nbl] = mfma16<false>(a0, b0, acc[nbl]);
         acc[nbl] = mfma16<false>(a1, b1, acc[nbl]);
@@ -334,7 +336,9 @@ __global__ __launch_bounds__(256) void k_gateup_decode(
             for (int it = 0; it < 2; ++it) {
                 if (mine[it].bits == 0) continue;
                 // two assignments per packed multiply; rows without an assignment hold zeros
-                const uint32_t sv = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)(srow[it] * sc_cur[it])) * 0x10001u;
+                // (times the stagger factor of the row: the decoded weight carries its inverse)
+                const float fac = (float)stagger_factor(mine[it].bits, lane);
+                const uint32_t sv = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)(srow[it] * sc_cur[it] * fac)) * 0x10001u;
                 uint16_t* dst = &hs[(pair + 4 * it) * SLAB_ROWS + lane];
 #pragma unroll
                 for (int ap = 0; ap < MAX_A / 2; ++ap) {

@@ -304,8 +304,8 @@ struct GuFetch {
 // One slab (64 contraction rows, `bits` wide) for a wavefront's (16 * NMB) x 64 tile.  The weight
 // operand is (code - 2^(bits-1)) * scale_s rounded once to f16 -- the operand the reference
 // builds (bitsmoe/algorithms/cpp/mlp_forward.cu:691-751), with the per-row multiplier s folded
-// into the scale -- made from the raw field decode 2^bits + code by a packed add (exact) and a
-// packed multiply.  (One packed FMA with the constant -1.5 * 2^bits * scale_s would round that
+// into the scale -- made from the raw field decode 2^bits + code / f (f: the row's stagger factor,
+// a power of two that the scale table carries) by a packed add (exact) and a packed multiply.  (One packed FMA with the constant -1.5 * 2^bits * scale_s would round that
 // constant: measured 4.5e-3 of error instead of 5e-4.)
 // WU != 0: the width is a compile-time constant (experts whose slabs all share it).
 template <int WU, int NMB>
@@ -313,7 +313,11 @@ __device__ __forceinline__ void gateup_slab_mfma(int bits, const uint16_t* __res
                                                  const u32x4 (&sc)[2], int lane, f32x4 (&acc)[NMB][4]) {
     const int n = lane & 15, kg = lane >> 4;
     const int wb = WU != 0 ? WU : bits;
-    const uint32_t neg = wb == 2 ? neg_offset_pair<2>() : wb == 3 ? neg_offset_pair<3>() : neg_offset_pair<4>();
+    // minus (2^w + 2^(w-1) / f_i): leaves (code - 2^(w-1)) / f_i of the staggered decode (wave_layout.h);
+    // the scale table carries f_i
+    u32x4 neg = wb == 2 ? offset0_regs<2>() : wb == 3 ? offset0_regs<3>() : offset0_regs<4>();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) neg[i] |= 0x80008000u;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
         u32x4 a[NMB];
@@ -329,13 +333,13 @@ __device__ __forceinline__ void gateup_slab_mfma(int bits, const uint16_t* __res
             // do not flow through alternative paths (which multiplies the register demand)
             u32x4 b;
             if (WU == 2 || (WU == 0 && bits == 2))
-                b = decode_fields2<2, false>(w[nbl], 8 * ks);
+                b = decode0_lo<2>(w[nbl], ks);
             else if (WU == 4 || (WU == 0 && bits == 4))
-                b = decode_fields4<false>(w[2 * nbl + ks]);
+                b = decode0_fields4(w[2 * nbl + ks]);
             else
-                b = decode_fields3<false>(w[nbl], 8 * ks, w[2 + nbl], 8 * (n >> 3) + 4 * ks);
+                b = decode0_fields3(w[nbl], ks, w[2 + nbl], n >> 3);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) b[i] = pk_mul_f16(pk_add_f16(b[i], neg), sc[ks][i]);
+            for (int i = 0; i < 4; ++i) b[i] = pk_mul_f16(pk_add_f16(b[i], neg[i]), sc[ks][i]);
 #pragma unroll
             for (int mb = 0; mb < NMB; ++mb) acc[mb][nb] = mfma16<false>(a[mb], b, acc[mb][nb]);
         }

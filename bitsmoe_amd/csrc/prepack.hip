@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src
                     for (int x = 0; x < 16; ++x) {
                         int row, col;
                         run_element(role, nb, kg, n8 + 8 * upper, x, &row, &col);
-                        word |= ((ref_code(in, w, row, col) >> 2) & 1u) << (pos1(x) + 8 * upper);
+                        word |= ((ref_code(in, w, row, col) >> 2) & 1u) << pos1s(x, upper);
                     }
             } else {                      // j = l*4 + nb
                 const int nb = j & 3, l = j >> 2, n = l & 15, kg = l >> 4;
@@ -88,7 +88,9 @@ __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src
             int row, col;
             run_element(role, nb, kg, n, x, &row, &col);
             const uint32_t u = ref_code(in, w, row, col);
-            if (fb == 4)
+            if (role == ROLE_GATE_UP)      // staggered fields; one may wrap around bit 31
+                word |= rotl32(fb == 4 ? (u & 15u) : (u & 3u), fb == 4 ? pos4s(i) : pos2s(w, i));
+            else if (fb == 4)
                 word |= (u & 15u) << pos4(i);
             else
                 word |= (u & 3u) << pos2(i);
@@ -122,16 +124,18 @@ __global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* payload 
         const int unit = (role == ROLE_GATE_UP) ? idx2_role0(nb, l) : (l * nbs + nb);
         if (w == 4) {
             const int per = run / 8;
-            u = (blk[unit * per + (x >> 3)] >> pos4(x & 7)) & 15u;
+            const uint32_t word = blk[unit * per + (x >> 3)];
+            u = (role == ROLE_GATE_UP ? rotr32(word, pos4s(x & 7)) : word >> pos4(x & 7)) & 15u;
         } else {
             const int per = run / 16;
-            u = (blk[unit * per + (x >> 4)] >> pos2(x & 15)) & 3u;
+            const uint32_t word = blk[unit * per + (x >> 4)];
+            u = (role == ROLE_GATE_UP ? rotr32(word, pos2s(w, x & 15)) : word >> pos2(x & 15)) & 3u;
             if (w == 3) {
                 uint32_t hi;
                 int p;
                 if (role == ROLE_GATE_UP) {
                     hi = blk[512 + hi_index0(kg, n, nb)];
-                    p = pos1(x) + 8 * (n >> 3);
+                    p = pos1s(x, n >> 3);
                 } else {
                     hi = blk[512 + l * 4 + nb];
                     p = pos1(x);
@@ -147,7 +151,8 @@ __global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* payload 
     }
 }
 
-// scale_s[scale_off(slab, tile) + row] = scale[...] * s[rank_off(slab) + row], rounded once to fp16.
+// scale_s[scale_off(slab, tile) + row] = scale[...] * s[rank_off(slab) + row], rounded once to fp16,
+// times the row's stagger factor (a power of two: the decoded weight carries its inverse).
 // grid (slab tasks, tiles), 64 threads.
 __global__ __launch_bounds__(64) void k_fold_scale_s(const MatView* __restrict__ views, const SlabTask* __restrict__ tasks,
                                                      const int64_t* __restrict__ out_offsets, __half* __restrict__ out) {
@@ -159,7 +164,8 @@ __global__ __launch_bounds__(64) void k_fold_scale_s(const MatView* __restrict__
     const int scale_off = mv.tile_meta[t * 3 + 1];
     const int row = threadIdx.x;
     const float v = __half2float(mv.scale[scale_off + row]) * __half2float(mv.s[rank_off + row]);
-    out[out_offsets[task.expert] + scale_off + row] = __float2half(v);
+    const int w = mv.slab_meta[si * 4 + 0];
+    out[out_offsets[task.expert] + scale_off + row] = __float2half(v * (float)stagger_factor(w, row));
 }
 
 }  // namespace bitsmoe

@@ -15,15 +15,27 @@
 //   role 1 (down: contraction over columns, outputs are rows; nb = 0..3)
 //     output row 16*nb + n, columns 32*m + 8*kg + e', m = 0..3, e' = 0..7   (32 codes)
 //
-//   A run of 16 codes with index x = 0..15 sits in a word at bit 2*(x/2)... precisely:
+//   Role 1: a run of 16 codes with index x = 0..15 sits in a word, precisely:
 //     2-bit fields:  field LSB at  (x & ~1) + 16*(x & 1)
 //     4-bit fields:  8 codes per word, field LSB at 4*(x'/2) + 16*(x' & 1), x' = x % 8
 //     3-bit codes :  low two bits as 2-bit fields, bit 2 as single bits at
-//                    (y/2) + 16*(y & 1) of a separate word (y = index in a run of 32;
-//                    role 0 shares one such word between lanes n and n+8: the upper lane
-//                    uses the positions + 8)
+//                    (y/2) + 16*(y & 1) of a separate word (y = index in a run of 32)
 //   so that ONE rotate and ONE and-or turn a word into a packed pair of 16-bit floats
 //   (2^w + code) for two neighbouring contraction indices: the pair lives 16 bits apart.
+//
+//   Role 0 staggers the fields so that most rotates disappear.  The MFMA operand of one k-step
+//   is four registers i = 0..3 (contraction indices 2i, 2i+1 of the lane's run of eight).  The
+//   field of register i sits 2i bits (4-bit codes: 4*(i%2) bits) BELOW the place where it would
+//   read as 2^w + code in an f16 mantissa, so the four registers of a k-step come out of the
+//   same word with four different masks and no rotate, as 2^w + code / f_i with
+//   f_i = 4^i (2- and 3-bit) or 16^(i%2) (4-bit).  The other k-step (4-bit: the registers 2, 3)
+//   sits 8 bits further up: one rotate by 8 serves its four (two) registers.  The factor f_i
+//   is a power of two and moves exactly into the other operand's scale (stagger_factor).
+//     2/3-bit fields: field LSB at (10 - w - 2i + 16*(x&1) + 8*ks) mod 32, x = 8*ks + 2i + (x&1)
+//     4-bit fields  : field LSB at (6 - 4*(i%2) + 16*(x'&1) + 8*(i/2)) mod 32, x' = 2i + (x'&1)
+//     3-bit, bit 2  : (9 - 2i + 16*(x&1) + 8*upper + ks) mod 32 of a separate word shared by
+//                     lanes n and n+8 (upper = n/8): one rotate by 8*upper + ks
+//   (a field may wrap around bit 31).  Role 0 operands are f16 (a bf16 mantissa is too short).
 //
 // Word order inside a block (every lane reads one contiguous run):
 //   role 0: the four wavefronts of a workgroup own the column-block PAIRS nbp = nb/2, so
@@ -62,6 +74,26 @@ __host__ __device__ inline int pos4(int x) { return 4 * (x >> 1) + 16 * (x & 1);
 // index y (0..31) of a run of 32 single bits (role 1) / (0..15) + 8*upper (role 0)
 __host__ __device__ inline int pos1(int y) { return (y >> 1) + 16 * (y & 1); }
 
+// role 0 (staggered): field LSB of code x (0..15) of a run in a two-bit field word, w = 2 or 3
+__host__ __device__ inline int pos2s(int w, int x) {
+    const int p = x >> 1;
+    return (10 - w - 2 * (p & 3) + 16 * (x & 1) + 8 * (p >> 2)) & 31;
+}
+// role 0 (staggered): field LSB of code x' (0..7) of a four-bit field word
+__host__ __device__ inline int pos4s(int x) {
+    const int i = x >> 1;
+    return (6 - 4 * (i & 1) + 16 * (x & 1) + 8 * (i >> 1)) & 31;
+}
+// role 0 (staggered): bit 2 of code x (0..15) of the run of lane n (upper = n / 8)
+__host__ __device__ inline int pos1s(int x, int upper) {
+    const int p = x >> 1;
+    return (9 - 2 * (p & 3) + 16 * (x & 1) + 8 * upper + (p >> 2)) & 31;
+}
+// role 0: the decoded value of row k of a w-bit slab is 2^w + code / stagger_factor(w, k)
+__host__ __device__ inline int stagger_factor(int w, int k) {
+    return w == 4 ? (((k >> 1) & 1) ? 16 : 1) : 1 << (2 * ((k & 7) >> 1));
+}
+
 // role 0: word index of column block nb for lane l (two-bit field words)
 __host__ __device__ inline int idx2_role0(int nb, int l) { return ((nb >> 1) * 64 + l) * 2 + (nb & 1); }
 // role 0, 3-bit: word index (inside the 256-word high region) shared by lanes n and n+8
@@ -89,6 +121,7 @@ struct Codec {
 };
 
 __device__ inline uint32_t rotr32(uint32_t x, int s) { return __builtin_amdgcn_alignbit(x, x, (uint32_t)(s & 31)); }
+__device__ inline uint32_t rotl32(uint32_t x, int s) { return rotr32(x, 32 - (s & 31)); }
 
 // Pointers that come out of a table in memory are generic; the hot kernels cast them to the
 // global address space so that loads become global_load / s_load instead of flat_load.
@@ -140,6 +173,42 @@ __device__ inline u32x4 decode_fields3(uint32_t z, int first, uint32_t hi, int h
         r[i] = (rotr32(hi, hi_first + i - (C::POS + 2)) & mh) | lo;
     }
     return r;
+}
+
+// ---- role 0 (staggered fields, f16 operands) ----
+// The k-step's four registers from a two-bit field word (W = 2 or 3), ks = 0 or 1.
+template <int W>
+__device__ inline u32x4 decode0_lo(uint32_t z, int ks) {
+    const uint32_t zz = ks ? rotr32(z, 8) : z;
+    const uint32_t magic = vreg(Codec<W, false>::MAGIC);
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = (zz & ((3u << (10 - W - 2 * i)) * 0x10001u)) | magic;
+    return r;
+}
+__device__ inline u32x4 decode0_fields4(uint32_t z) {
+    const uint32_t zz = rotr32(z, 8);
+    const uint32_t magic = vreg(Codec<4, false>::MAGIC);
+    const uint32_t m0 = (15u << 6) * 0x10001u, m1 = (15u << 2) * 0x10001u;
+    u32x4 r = {(z & m0) | magic, (z & m1) | magic, (zz & m0) | magic, (zz & m1) | magic};
+    return r;
+}
+__device__ inline u32x4 decode0_fields3(uint32_t z, int ks, uint32_t hi, int upper) {
+    u32x4 r = decode0_lo<3>(z, ks);
+    const uint32_t hh = rotr32(hi, 8 * upper + ks);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = (hh & ((1u << (9 - 2 * i)) * 0x10001u)) | r[i];
+    return r;
+}
+// What has to be subtracted from the decoded registers to leave (code - 2^(W-1)) / f_i:
+// 2^W + 2^(W-1) / f_i as a packed f16 pair per register (mantissa 512 / f_i).
+template <int W>
+__device__ inline u32x4 offset0_regs() {
+    constexpr uint32_t magic = Codec<W, false>::MAGIC;
+    if constexpr (W == 4)
+        return u32x4{magic | 512u * 0x10001u, magic | 32u * 0x10001u, magic | 512u * 0x10001u, magic | 32u * 0x10001u};
+    else
+        return u32x4{magic | 512u * 0x10001u, magic | 128u * 0x10001u, magic | 32u * 0x10001u, magic | 8u * 0x10001u};
 }
 
 // Packed f16 arithmetic on two values in one 32-bit register.
