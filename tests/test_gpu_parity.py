@@ -250,6 +250,30 @@ def test_forward_mfma_path(cuda_device, shape, dtype_name):
     assert err < 3e-3      # f16 operands: well inside the 1e-2 bar
 
 
+@pytest.mark.parametrize("tokens", [9, 40, 300])        # tiles of <= 32 rows, of 33..128 rows, several tiles
+@pytest.mark.parametrize("slabs", [1, 2, 3, 4, 7])      # the three-stage ring at every phase of its wrap-around
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_forward_mfma_path_one_width_per_expert(cuda_device, bits, slabs, tokens):
+    """Experts whose slabs all share one bit-width run the bodies that load everything straight
+    into LDS, one compiled per width; tile counts 1, 2 and 3 leave wavefronts without a tile."""
+    from bitsmoe_amd.algorithms import _capi
+
+    for dim in ((128, 384) if slabs == 2 else (256,)):
+        err = _forward_case(cuda_device, 500 + 10 * bits + slabs, 2, tokens, 1, 64 * slabs, 64 * slabs, dim, "f16", (bits,),
+                            path=_capi.PATH_MFMA, tol=1e-2, uniform_bits=True)
+        assert err < 3e-3
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_forward_decode_path_one_width_per_expert(cuda_device, bits):
+    """The decode kernels' width-specialised bodies (eight equal slabs in a row), per width."""
+    from bitsmoe_amd.algorithms import _capi
+
+    err = _forward_case(cuda_device, 600 + bits, 3, 20, 2, 512, 256, 256, "bf16", (bits,), path=_capi.PATH_DECODE,
+                        tol=1e-2, uniform_bits=True)
+    assert err < 3e-3
+
+
 @pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
 def test_forward_mfma_path_scattered_ranks(cuda_device, dtype_name):
     """rank_idx without runs of eight consecutive ranks: the activations are gathered first."""
