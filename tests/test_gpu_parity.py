@@ -264,6 +264,15 @@ def test_forward_mfma_path_one_width_per_expert(cuda_device, bits, slabs, tokens
         assert err < 3e-3
 
 
+def test_forward_mfma_path_more_slabs_than_the_slab_tables_hold(cuda_device):
+    """65 slabs of one width: past the per-slab tables of the LDS-direct body, the register-staged body runs."""
+    from bitsmoe_amd.algorithms import _capi
+
+    err = _forward_case(cuda_device, 650, 2, 40, 1, 65 * 64, 64, 128, "bf16", (3,), path=_capi.PATH_MFMA, tol=1e-2,
+                        uniform_bits=True)
+    assert err < 3e-3
+
+
 @pytest.mark.parametrize("bits", [2, 3, 4])
 def test_forward_decode_path_one_width_per_expert(cuda_device, bits):
     """The decode kernels' width-specialised bodies (eight equal slabs in a row), per width."""
