@@ -694,14 +694,17 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     const int ld = proj ? ldu : ldg;
     uint16_t* __restrict__ out = proj ? U : G;
     const int w = __builtin_amdgcn_readfirstlane(fe.uniform_bits);
-    // tiles of at most 32 assignments (experts that see few tokens, remainders) run a body with a
-    // quarter of the accumulators, MFMAs and staging; complete bodies, so that no accumulator
-    // lives across the choice
+    // tiles of at most 32 (64) assignments (experts that see few tokens, remainders) run a body with
+    // a quarter (half) of the accumulators, MFMAs and staging; complete bodies, so that no
+    // accumulator lives across the choice
     const DmaStage st0 = {sa0, sw0, ss0}, st1 = {sa1, sw1, ss1}, st2 = {sa2, sw2, ss2};
 #define BITSMOE_GU_BODY(W)                                                                                           \
     do {                                                                                                             \
         if (rows <= 32)                                                                                              \
             gateup_tile_body_dma<DIRECT, W, 2>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out,         \
+                                               a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab); \
+        else if (rows <= 64)                                                                                         \
+            gateup_tile_body_dma<DIRECT, W, 4>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out,         \
                                                a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab); \
         else                                                                                                         \
             gateup_tile_body_dma<DIRECT, W, 8>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out,         \
@@ -954,8 +957,8 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
     FastSlab fs = FastSlab{0, 0, 0, 0};
     if (si < nslabs) fs = load_fast_slab(down_fs + (int64_t)e * max_slabs, si);
 
-    // tiles of at most 32 assignments run a body with a quarter of the accumulators and MFMAs:
-    // two complete bodies, so that no accumulator lives across the choice
+    // tiles of at most 32 (64) assignments run a body with a quarter (half) of the accumulators and
+    // MFMAs: complete bodies, so that no accumulator lives across the choice
     auto run = [&](auto nmb_c) {
         constexpr int NMB = decltype(nmb_c)::value;
         f32x4 acc[NMB][4];
@@ -983,6 +986,8 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
     };
     if (rows <= 32)
         run(std::integral_constant<int, 2>{});
+    else if (rows <= 64)
+        run(std::integral_constant<int, 4>{});
     else
         run(std::integral_constant<int, 8>{});
 }
