@@ -215,7 +215,11 @@ __global__ __launch_bounds__(256) void k_pregather(const FastExpert* __restrict_
 // grid-stride over 8-element groups.
 __global__ __launch_bounds__(256) void k_bf16_to_f16(const uint16_t* __restrict__ src_g, const uint16_t* __restrict__ src_u,
                                                      int64_t T, int64_t sg, int64_t su, int ldg, int ldu,
-                                                     uint16_t* __restrict__ dst_g, uint16_t* __restrict__ dst_u) {
+                                                     uint16_t* __restrict__ dst_g, uint16_t* __restrict__ dst_u,
+                                                     int32_t* __restrict__ zero, int n_zero) {
+    // (also clears the per-token counters: one launch less in front of the GEMM)
+    if (blockIdx.y == 0)
+        for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n_zero; i += gridDim.x * blockDim.x) zero[i] = 0;
     const bool is_up = blockIdx.y != 0;
     const uint16_t* src = is_up ? src_u : src_g;
     uint16_t* dst = is_up ? dst_u : dst_g;
@@ -1187,20 +1191,23 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     const int ldy = down->max_slabs * SLAB_ROWS;
 
     record(prof, 0, st);
-    BITSMOE_REQUIRE(launch_fill_zero((float*)token_count, T + 1, st) == BITSMOE_OK, "zero fill failed");
+    const bool convert = direct && act_dtype == BITSMOE_DT_BF16;
+    if (convert) {      // the conversion pass clears the per-token counters on its way
+        const int64_t groups = T * (std::max(ldg, ldu) / 8);
+        hipLaunchKernelGGL(k_bf16_to_f16, dim3((unsigned)std::min<int64_t>((groups + 255) / 256, 2048), 2), dim3(256), 0, st,
+                           (const uint16_t*)h_gate, (const uint16_t*)h_up, T, ldg_in, ldu_in, ldg, ldu, (uint16_t*)Hs_g,
+                           (uint16_t*)Hs_u, token_count, (int)(T + 1));
+        BITSMOE_HIP_TRY(hipGetLastError());
+    } else {
+        BITSMOE_REQUIRE(launch_fill_zero((float*)token_count, T + 1, st) == BITSMOE_OK, "zero fill failed");
+    }
     hipLaunchKernelGGL(k_token_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, st, tok, off, E, (int)A, (int)T,
                        token_count, slot);
     hipLaunchKernelGGL(k_build_mtiles, dim3(1), dim3(256), 0, st, off, E, (int)A, (int)max_mtiles, mtiles, n_mtiles,
                        token_count, (int)T, token_start);
     BITSMOE_HIP_TRY(hipGetLastError());
     if (direct) {
-        if (act_dtype == BITSMOE_DT_BF16) {
-            const int64_t groups = T * (std::max(ldg, ldu) / 8);
-            hipLaunchKernelGGL(k_bf16_to_f16, dim3((unsigned)std::min<int64_t>((groups + 255) / 256, 2048), 2), dim3(256), 0, st,
-                               (const uint16_t*)h_gate, (const uint16_t*)h_up, T, ldg_in, ldu_in, ldg, ldu, (uint16_t*)Hs_g,
-                               (uint16_t*)Hs_u);
-            BITSMOE_HIP_TRY(hipGetLastError());
-        } else {
+        if (!convert) {
             Hs_g = (const uint16_t*)h_gate;
             Hs_u = (const uint16_t*)h_up;
         }
