@@ -275,6 +275,9 @@ template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
 }
+// s_waitcnt lgkmcnt(0) alone: every LDS read of the wavefront has returned (the vector-memory and
+// export counters are left at their maxima).
+__device__ __forceinline__ void wait_lds_reads() { __builtin_amdgcn_s_waitcnt(0xC07F); }
 // Workgroup barrier without the wait for outstanding loads that __syncthreads implies.  The empty
 // asm statements keep the compiler from moving LDS accesses across it (the bare instruction is no
 // memory fence for the compiler).
@@ -866,7 +869,7 @@ __device__ __forceinline__ void down_tile_loop(const uint32_t* __restrict__ payl
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) scp[nb] = (uint32_t)sbuf[16 * nb + n] * 0x10001u;
         // the buffer is requested again right away: its reads must have returned
-        __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0)
+        wait_lds_reads();
         asm volatile("" ::: "memory");
     };
     const int n_halves = 2 * n_tiles;      // at least two
