@@ -8,8 +8,8 @@
 //   k_bf16_to_f16 /  activations as f16, read through the token index by the GEMM kernel, or
 //   k_pregather      Hs[a, k] = f16( h[tok_a, rank_idx[k]] ) in expert-sorted assignment order
 //   k_gateup_mfma    G = Hs_gate . W_gate, U = Hs_up . W_up as f16;  k_silu_mul_f16: z = silu(G) * U
-//   k_down_mfma      y[a, r] = sum_c W_down[r, c] z[a, c] as f16, and the per-token lists
-//   k_combine_tokens rank_accum[t, rank_idx[r]] = sum over the assignments of t of route_w * s[r] * y
+//   k_down_mfma      y[a, r] = s[r] * sum_c W_down[r, c] z[a, c] as f16, and the per-token lists
+//   k_combine_tokens rank_accum[t, rank_idx[r]] = sum over the assignments of t of route_w * y
 //
 // Both GEMM kernels use 16x16x32 f16 MFMA with four wavefronts of 128 rows x 64 columns per
 // workgroup.  The activation operand is staged through LDS in 128 x 64 pieces (double
@@ -925,7 +925,7 @@ __device__ __forceinline__ void down_tile_loop(const uint32_t* __restrict__ payl
 
 // grid.x = 32 * ceil(max_mtiles / 32) * n_groups; workgroup = (assignment tile, group of four
 // slabs): wavefront w = all 128 assignments x the 64 output rows of slab 4*group + w.
-// Output: y[a, r] = sum_c W_down[r, c] z[a, c] as f16, r in the expert's own row order
+// Output: y[a, r] = s[r] * sum_c W_down[r, c] z[a, c] as f16, r in the expert's own row order
 // (row `A` of y takes the stores of a tile's unused rows), and the per-token assignment lists
 // token_list[token_start[tok_a] + slot[a]] = (a, expert) that k_combine_tokens walks.
 __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restrict__ down_fe,
@@ -977,7 +977,11 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
         down_tile_loop<NMB>(fe.payload, fe.scale, fs, z, I, n_tiles, a_begin, rows, sz0, sz1, sz2, wbuf, sbuf, tid, lane, acc);
         if (fs.bits == 0) return;
 
-        // lane holds assignments 16*mb + 4*kg + j, output rows 16*nb + n of the slab
+        // lane holds assignments 16*mb + 4*kg + j, output rows 16*nb + n of the slab; the rows'
+        // multipliers s[r] go into y here, so that the combine reads one operand per assignment
+        float srow[4];
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) srow[nb] = __half2float(fe.s[fs.rank_off + 16 * nb + n]);
         _Float16* ycol = y + fs.rank_off + n;
 #pragma unroll
         for (int mb = 0; mb < NMB; ++mb) {
@@ -987,7 +991,7 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
                 const int r = 16 * mb + 4 * kg + j;
                 _Float16* dst = ycol + (int64_t)(r < rows ? a_begin + r : A) * ldy;
 #pragma unroll
-                for (int nb = 0; nb < 4; ++nb) dst[16 * nb] = (_Float16)acc[mb][nb][j];
+                for (int nb = 0; nb < 4; ++nb) dst[16 * nb] = (_Float16)(acc[mb][nb][j] * srow[nb]);
             }
         }
     };
@@ -1004,7 +1008,7 @@ constexpr int CB_COLS = 4096;    // output columns one pass of the general form 
 constexpr int CB_SORT = 256;     // list entries ordered at a time
 
 // rank_accum[t, rank_idx_e[r]] = sum over the assignments (a, e) of token t, in ascending a,
-// of route_w[a] * s_e[r] * y[a, r].  One workgroup per token; it writes every column of its
+// of route_w[a] * y[a, r] (y carries the row multiplier s_e[r]).  One workgroup per token; it writes every column of its
 // row, so rank_accum needs no zero fill.  IDENTITY: rank_idx_e[r] == r in every expert, and a
 // thread keeps its eight columns in registers; otherwise the row is accumulated in LDS, one
 // assignment after the other.
@@ -1018,7 +1022,6 @@ __global__ __launch_bounds__(256) void k_combine_tokens(const FastExpert* __rest
     __shared__ __attribute__((aligned(16))) float out_s[IDENTITY ? 4 : CB_COLS];
     __shared__ int2 raw_s[CB_SORT];
     __shared__ const _Float16* y_s[CB_SORT];
-    __shared__ const __half* s_s[CB_SORT];
     __shared__ const int32_t* idx_s[CB_SORT];
     __shared__ int nrow_s[CB_SORT];
     __shared__ float rw_s[CB_SORT];
@@ -1043,7 +1046,6 @@ __global__ __launch_bounds__(256) void k_combine_tokens(const FastExpert* __rest
                 for (int i = 0; i < nl; ++i) pos += raw_s[i].x < mine.x;
                 const FastExpert fe = down_fe[mine.y];
                 y_s[pos] = y + (int64_t)mine.x * ldy;
-                s_s[pos] = fe.s;
                 idx_s[pos] = fe.rank_idx;
                 nrow_s[pos] = min(fe.num_slabs, max_slabs) * SLAB_ROWS;
                 rw_s[pos] = route_w[mine.x];
@@ -1054,7 +1056,7 @@ __global__ __launch_bounds__(256) void k_combine_tokens(const FastExpert* __rest
                 // four entries at a time: their eight loads are in flight together (an entry past
                 // the list or past its expert's rows loads from a valid address and is not added)
                 for (int i0 = 0; i0 < nl; i0 += 4) {
-                    u32x4 yv[4], sv[4];
+                    u32x4 yv[4];
                     float rw[4];
                     bool ok[4];
 #pragma unroll
@@ -1063,7 +1065,6 @@ __global__ __launch_bounds__(256) void k_combine_tokens(const FastExpert* __rest
                         ok[u] = i0 + u < nl && r0 < nrow_s[i];
                         const int rr = ok[u] ? r0 : 0;
                         yv[u] = *reinterpret_cast<const u32x4*>(y_s[i] + rr);
-                        sv[u] = *reinterpret_cast<gptr<u32x4>>(as_global(s_s[i]) + rr);
                         rw[u] = rw_s[i];
                     }
 #pragma unroll
@@ -1071,10 +1072,9 @@ __global__ __launch_bounds__(256) void k_combine_tokens(const FastExpert* __rest
                         if (!ok[u]) continue;
 #pragma unroll
                         for (int k = 0; k < 8; ++k) {
-                            const uint32_t yw = yv[u][k >> 1], sw = sv[u][k >> 1];
+                            const uint32_t yw = yv[u][k >> 1];
                             const h2 yp = __builtin_bit_cast(h2, yw);
-                            const h2 sp = __builtin_bit_cast(h2, sw);
-                            acc[k] += (float)yp[k & 1] * (float)sp[k & 1] * rw[u];
+                            acc[k] += (float)yp[k & 1] * rw[u];
                         }
                     }
                 }
@@ -1083,20 +1083,17 @@ __global__ __launch_bounds__(256) void k_combine_tokens(const FastExpert* __rest
                     const int nrow = nrow_s[i];
                     const float rw = rw_s[i];
                     gptr<int32_t> rank_idx = as_global(idx_s[i]);
-                    gptr<__half> svec = as_global(s_s[i]);
                     const _Float16* yrow = y_s[i];
                     for (int r0 = tid * 8; r0 < nrow; r0 += 256 * 8) {
                         const u32x4 yv = *reinterpret_cast<const u32x4*>(yrow + r0);
-                        const u32x4 sv = *reinterpret_cast<gptr<u32x4>>(svec + r0);
                         const i32x4 ia = *reinterpret_cast<gptr<i32x4>>(rank_idx + r0);
                         const i32x4 ib = *reinterpret_cast<gptr<i32x4>>(rank_idx + r0 + 4);
 #pragma unroll
                         for (int k = 0; k < 8; ++k) {
-                            const uint32_t yw = yv[k >> 1], sw = sv[k >> 1];
+                            const uint32_t yw = yv[k >> 1];
                             const h2 yp = __builtin_bit_cast(h2, yw);
-                            const h2 sp = __builtin_bit_cast(h2, sw);
                             const int col = (k < 4 ? ia[k & 3] : ib[k & 3]) - c0;
-                            if (col >= 0 && col < cols) atomicAdd(out_s + col, (float)yp[k & 1] * (float)sp[k & 1] * rw);
+                            if (col >= 0 && col < cols) atomicAdd(out_s + col, (float)yp[k & 1] * rw);
                         }
                     }
                     __syncthreads();    // entries are added one after the other: the sum has one order
