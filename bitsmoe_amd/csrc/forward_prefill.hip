@@ -63,40 +63,79 @@ __global__ __launch_bounds__(256) void k_token_count(const int32_t* __restrict__
 
 // One workgroup: the list of (expert, first assignment, rows <= 128) tiles from
 // expert_offsets, then token_start = exclusive scan of token_count (T + 1 entries).
+// The list is ordered by decreasing cost (a counting sort over a few cost classes: the body the
+// tile runs -- full, half or quarter height -- then the bit-widths of the expert's gate and up
+// matrices): workgroups start in list order, so the long ones run first and the short ones fill
+// the end of the launch.  Which of two tiles of one class comes first is left to the LDS atomics:
+// no result depends on the order.
+constexpr int MT_KEYS = 32;
+__device__ inline int mtile_key(int rows, int wsum) {      // 0 = most expensive
+    const int c = rows > 64 ? 0 : rows > 32 ? 1 : 2;
+    return c * 8 + (7 - min(max(wsum - 1, 0), 7));           // wsum: 4 .. 8, or 0 (mixed widths: taken as the most expensive)
+}
 __global__ __launch_bounds__(256) void k_build_mtiles(const int32_t* __restrict__ expert_offsets, int E, int A,
                                                       int max_tiles, MTile* __restrict__ tiles,
                                                       int32_t* __restrict__ n_tiles_out,
                                                       const int32_t* __restrict__ token_count, int T,
-                                                      int32_t* __restrict__ token_start) {
+                                                      int32_t* __restrict__ token_start,
+                                                      const FastExpert* __restrict__ gate_fe,
+                                                      const FastExpert* __restrict__ up_fe) {
     __shared__ int scan[256];
+    __shared__ int hist[MT_KEYS], cursor[MT_KEYS];
     __shared__ int base_s;
     const int tid = threadIdx.x;
-    if (tid == 0) base_s = 0;
+    if (tid < MT_KEYS) hist[tid] = 0;
     __syncthreads();
+    auto expert_tiles = [&](int e, int* begin, int* cnt, int* k_full, int* k_last) {
+        *begin = 0;
+        *cnt = 0;
+        *k_full = 0;
+        *k_last = 0;
+        if (e >= E) return;
+        *begin = min(max(expert_offsets[e], 0), A);
+        const int end = min(max(expert_offsets[e + 1], 0), A);
+        *cnt = max(end - *begin, 0);
+        if (*cnt == 0) return;
+        const int wg = gate_fe ? gate_fe[e].uniform_bits : 2, wu = up_fe ? up_fe[e].uniform_bits : 2;
+        const int wsum = (wg == 0 || wu == 0) ? 8 : wg + wu;
+        *k_full = mtile_key(PF_M, wsum);
+        *k_last = mtile_key(*cnt - (*cnt - 1) / PF_M * PF_M, wsum);
+    };
+    // pass 1: tiles per cost class
+    for (int e0 = 0; e0 < E; e0 += 256) {
+        int begin, cnt, k_full, k_last;
+        expert_tiles(e0 + tid, &begin, &cnt, &k_full, &k_last);
+        const int nt = (cnt + PF_M - 1) / PF_M;
+        if (nt > 1) atomicAdd(&hist[k_full], nt - 1);
+        if (nt > 0) atomicAdd(&hist[k_last], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int k = 0; k < MT_KEYS; ++k) {
+            cursor[k] = run;
+            run += hist[k];
+        }
+        base_s = run;
+    }
+    __syncthreads();
+    // pass 2: every expert claims places for its tiles
     for (int e0 = 0; e0 < E; e0 += 256) {
         const int e = e0 + tid;
-        int begin = 0, cnt = 0;
-        if (e < E) {
-            begin = min(max(expert_offsets[e], 0), A);
-            const int end = min(max(expert_offsets[e + 1], 0), A);
-            cnt = max(end - begin, 0);
-        }
+        int begin, cnt, k_full, k_last;
+        expert_tiles(e, &begin, &cnt, &k_full, &k_last);
         const int nt = (cnt + PF_M - 1) / PF_M;
-        scan[tid] = nt;
-        __syncthreads();
-        for (int d = 1; d < 256; d <<= 1) {
-            const int v = tid >= d ? scan[tid - d] : 0;
-            __syncthreads();
-            scan[tid] += v;
-            __syncthreads();
+        if (nt > 1) {
+            const int at = atomicAdd(&cursor[k_full], nt - 1);
+            for (int j = 0; j < nt - 1; ++j)
+                if (at + j < max_tiles) tiles[at + j] = MTile{e, begin + j * PF_M, PF_M, 0};
         }
-        const int excl = scan[tid] - nt + base_s;
-        for (int j = 0; j < nt; ++j)
-            if (excl + j < max_tiles) tiles[excl + j] = MTile{e, begin + j * PF_M, min(PF_M, cnt - j * PF_M), 0};
-        __syncthreads();
-        if (tid == 255) base_s += scan[255];
-        __syncthreads();
+        if (nt > 0) {
+            const int at = atomicAdd(&cursor[k_last], 1);
+            if (at < max_tiles) tiles[at] = MTile{e, begin + (nt - 1) * PF_M, cnt - (nt - 1) * PF_M, 0};
+        }
     }
+    __syncthreads();
     const int total = min(base_s, max_tiles);
     for (int i = total + tid; i < max_tiles; i += 256) tiles[i] = MTile{-1, 0, 0, 0};
     if (tid == 0) *n_tiles_out = total;
@@ -245,15 +284,14 @@ __global__ __launch_bounds__(256) void k_bf16_to_f16(const uint16_t* __restrict_
 // --------------------------------------------------------------------------- shared GEMM parts
 // Workgroup id -> logical work index = tile * units + unit.  Hardware places workgroup b on XCD
 // b % 8, and every XCD has its own L2: the `units` workgroups of one assignment tile (which share
-// its activations) get ids of one residue class, and the tiles are dealt to the XCDs two at a time
-// (neighbouring tiles mostly belong to one expert and share its weights), so that a long run of
-// heavy tiles (a popular expert) or of short ones does not land on one XCD.
+// its activations) get ids of one residue class.  The tile list is ordered by decreasing cost; it
+// is dealt to the XCDs back and forth (tiles 0..7 to XCDs 0..7, tiles 8..15 to XCDs 7..0, ...), so
+// that every XCD gets the same mix and starts its own share in order of decreasing cost.
 // The grid holds 32 * ceil(max tiles / 32) * units workgroups; -1: no such tile.
-constexpr int XCD_RUN = 2;
 __device__ inline int xcd_logical(int bid, int n_tiles_real, int units) {
-    const int slot = bid >> 3;
+    const int slot = bid >> 3, x = bid & 7;
     const int q = slot / units;
-    const int tile = ((q / XCD_RUN) * 8 + (bid & 7)) * XCD_RUN + q % XCD_RUN;
+    const int tile = q * 8 + ((q & 1) ? 7 - x : x);
     if (tile >= n_tiles_real) return -1;
     return tile * units + slot % units;
 }
@@ -1204,7 +1242,7 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     hipLaunchKernelGGL(k_token_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, st, tok, off, E, (int)A, (int)T,
                        token_count, slot);
     hipLaunchKernelGGL(k_build_mtiles, dim3(1), dim3(256), 0, st, off, E, (int)A, (int)max_mtiles, mtiles, n_mtiles,
-                       token_count, (int)T, token_start);
+                       token_count, (int)T, token_start, gate->d_fast_experts, up->d_fast_experts);
     BITSMOE_HIP_TRY(hipGetLastError());
     if (direct) {
         if (!convert) {
