@@ -211,7 +211,7 @@ def run_workload(block, spec, tokens, steps, warmup, seed=42, use_graph=True):
 # each scaled by what it reads for a 256 MiB copy); collected offline with rocprofv3 --pmc on
 # this same script (profiles/*_hbm_traffic_counters.txt), None where not collected.
 HBM_TRAFFIC_BYTES = {"c2-t64": int((58349.4 * 2.0 + 18742.4) * 1024),        # k_gateup_decode
-                     "c3-t4096": int((250824.8 * 2.0 + 98304.0) * 1024)}     # k_gateup_mfma
+                     "c3-t4096": int((268721.1 * 2.0 + 98304.0) * 1024)}     # k_gateup_mfma
 
 
 def roofline_of(res, inputs, bound, workload=None):
