@@ -56,6 +56,12 @@ struct FastSlab {              // tile t of the slab: payload word pack_off + t*
     int32_t rank_off;
 };
 
+// Kernel argument (by value): the expert a grid coordinate stands for.
+constexpr int EXPERT_ORDER_MAX = 256;
+struct ExpertOrder {
+    unsigned char e[EXPERT_ORDER_MAX];
+};
+
 struct SlabTask {              // one (expert, slab) unit of the down projection
     int32_t expert;
     int32_t slab;
@@ -96,6 +102,10 @@ struct bitsmoe_matset {
     __half* d_scale_s = nullptr;      // gate/up sets: scale folded with the per-row multiplier s
     bool vector_aligned = false;      // scale / s / rank_idx of every expert start on 16-byte boundaries
     bool all_uniform8 = false;        // role 0: every aligned group of 8 slabs has one width and is contiguous
+    // experts by decreasing payload size (prepared sets of at most EXPERT_ORDER_MAX experts): the
+    // decode kernels start the expensive experts' workgroups first
+    bool has_cost_order = false;
+    unsigned char cost_order[256] = {};
     uint32_t* d_prepared = nullptr;   // wave-native copy of every payload (see wave_layout.h)
     bitsmoe::MatView* d_views_prepared = nullptr;
     bitsmoe::FastExpert* d_fast_experts = nullptr;   // [n_experts]

@@ -162,7 +162,8 @@ __global__ __launch_bounds__(256, 4) void k_gateup_decode(
     const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
     const uint16_t* __restrict__ h_gate, const uint16_t* __restrict__ h_up, int Rg, int Ru, int64_t ldg, int64_t ldu,
     const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
-    int E, int n_tiles, int n_groups, int n_tchunks, int tiles_per_wg, float* __restrict__ G, float* __restrict__ U) {
+    int E, int n_tiles, int n_groups, int n_tchunks, int tiles_per_wg, float* __restrict__ G, float* __restrict__ U,
+    const ExpertOrder gate_order, const ExpertOrder up_order) {
     const int mt = blockIdx.y;
     // (consecutive workgroups land on different XCDs: that spreads experts of different cost)
     const int bid = blockIdx.x;
@@ -171,7 +172,9 @@ __global__ __launch_bounds__(256, 4) void k_gateup_decode(
     const int tid = threadIdx.x;
     int e = bid / (n_tchunks * n_groups);
     int chunk = -1;
-    if constexpr (MODE == GRID_ACTIVE) {
+    if constexpr (MODE == GRID_EXPERTS) {      // expensive experts first (the identity when there is no order)
+        if (E <= EXPERT_ORDER_MAX) e = mt ? up_order.e[e] : gate_order.e[e];
+    } else if constexpr (MODE == GRID_ACTIVE) {
         e = nth_active_expert(expert_offsets, E, A, e, tid & 63);
         if (e < 0) return;
     } else if constexpr (MODE == GRID_CHUNKS) {
@@ -666,11 +669,18 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         tiles_per_wg = (tiles_per_wg + 1) / 2;
     const int n_tchunks = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
     dim3 grid((unsigned)(e_dim * gu_groups * n_tchunks), 2);
+    // the expert a grid coordinate stands for: by decreasing payload size, or the identity
+    auto order_of = [&](const bitsmoe_matset* set) {
+        ExpertOrder o;
+        for (int i = 0; i < EXPERT_ORDER_MAX; ++i) o.e[i] = set->has_cost_order && i < E ? set->cost_order[i] : (unsigned char)i;
+        return o;
+    };
+    const ExpertOrder gate_order = order_of(gate), up_order = order_of(up);
     auto launch_gateup = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs, gate->max_slabs,
                            up->d_fast_experts, up->d_fast_slabs, up->max_slabs, (const uint16_t*)h_gate,
                            (const uint16_t*)h_up, Rg, Ru, ldg, ldu, tok, off, (int)T, (int)A, I, E, n_tiles, gu_groups, n_tchunks,
-                           tiles_per_wg, G, U);
+                           tiles_per_wg, G, U, gate_order, up_order);
     };
     const bool need_general = !(gate->all_uniform8 && up->all_uniform8);
     const bool bf16 = act_dtype == BITSMOE_DT_BF16;

@@ -286,6 +286,18 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
         for (int si = 1; si < f.num_slabs; ++si)
             if (set->slab_meta_host[e][si * 4] != f.uniform_bits) f.uniform_bits = 0;
     }
+    set->has_cost_order = set->n_experts <= EXPERT_ORDER_MAX;
+    if (set->has_cost_order) {
+        std::vector<int> order(set->n_experts);
+        for (int e = 0; e < set->n_experts; ++e) order[e] = e;
+        auto words = [&](int e) {       // payload words per tile of expert e
+            int64_t w = 0;
+            for (int si = 0; si < set->descs[e].num_slabs; ++si) w += set->slab_meta_host[e][si * 4];
+            return w;
+        };
+        std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return words(a) > words(b); });
+        for (int e = 0; e < set->n_experts; ++e) set->cost_order[e] = (unsigned char)order[e];
+    }
     BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_fast_experts, sizeof(FastExpert) * fexp.size()));
     BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_fast_experts, fexp.data(), sizeof(FastExpert) * fexp.size(), hipMemcpyHostToDevice, st));
     BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_fast_slabs, sizeof(FastSlab) * fslabs.size()));
