@@ -210,7 +210,7 @@ def run_workload(block, spec, tokens, steps, warmup, seed=42, use_graph=True):
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE,
 # each scaled by what it reads for a 256 MiB copy); collected offline with rocprofv3 --pmc on
 # this same script (profiles/*_hbm_traffic_counters.txt), None where not collected.
-HBM_TRAFFIC_BYTES = {"c2-t64": int((58349.4 * 2.0 + 18742.4) * 1024),        # k_gateup_decode
+HBM_TRAFFIC_BYTES = {"c2-t64": int((58445.4 * 2.0 + 18742.4) * 1024),        # k_gateup_decode
                      "c3-t4096": int((268721.1 * 2.0 + 98304.0) * 1024)}     # k_gateup_mfma
 
 
