@@ -57,9 +57,9 @@ struct FastSlab {              // tile t of the slab: payload word pack_off + t*
 };
 
 // Kernel argument (by value): the expert a grid coordinate stands for.
-constexpr int EXPERT_ORDER_MAX = 256;
+constexpr int EXPERT_ORDER_MAX = 512;
 struct ExpertOrder {
-    unsigned char e[EXPERT_ORDER_MAX];
+    uint16_t e[EXPERT_ORDER_MAX];
 };
 
 struct SlabTask {              // one (expert, slab) unit of the down projection
@@ -105,7 +105,7 @@ struct bitsmoe_matset {
     // experts by decreasing payload size (prepared sets of at most EXPERT_ORDER_MAX experts): the
     // decode kernels start the expensive experts' workgroups first
     bool has_cost_order = false;
-    unsigned char cost_order[256] = {};
+    uint16_t cost_order[512] = {};
     uint32_t* d_prepared = nullptr;   // wave-native copy of every payload (see wave_layout.h)
     bitsmoe::MatView* d_views_prepared = nullptr;
     bitsmoe::FastExpert* d_fast_experts = nullptr;   // [n_experts]

@@ -672,7 +672,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     // the expert a grid coordinate stands for: by decreasing payload size, or the identity
     auto order_of = [&](const bitsmoe_matset* set) {
         ExpertOrder o;
-        for (int i = 0; i < EXPERT_ORDER_MAX; ++i) o.e[i] = set->has_cost_order && i < E ? set->cost_order[i] : (unsigned char)i;
+        for (int i = 0; i < EXPERT_ORDER_MAX; ++i) o.e[i] = set->has_cost_order && i < E ? set->cost_order[i] : (uint16_t)i;
         return o;
     };
     const ExpertOrder gate_order = order_of(gate), up_order = order_of(up);

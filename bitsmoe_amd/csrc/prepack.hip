@@ -296,7 +296,7 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
             return w;
         };
         std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return words(a) > words(b); });
-        for (int e = 0; e < set->n_experts; ++e) set->cost_order[e] = (unsigned char)order[e];
+        for (int e = 0; e < set->n_experts; ++e) set->cost_order[e] = (uint16_t)order[e];
     }
     BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_fast_experts, sizeof(FastExpert) * fexp.size()));
     BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_fast_experts, fexp.data(), sizeof(FastExpert) * fexp.size(), hipMemcpyHostToDevice, st));
