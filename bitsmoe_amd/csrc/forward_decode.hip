@@ -28,18 +28,9 @@ constexpr int GU_STRIDE = GU_SLABS * SLAB_ROWS + 8;  // 16-bit elements; +8 stag
 constexpr int DN_SLABS_PER_WG = 4;                 // one slab per wavefront
 constexpr int MAX_A = 16;                          // assignments per MFMA pass
 
-// raw 16-bit activation -> fp32
-template <bool BF16>
-__device__ inline float operand_to_f32(uint16_t v) {
-    if constexpr (BF16)
-        return __uint_as_float((uint32_t)v << 16);
-    else
-        return __half2float(__ushort_as_half(v));
-}
-
-template <int W, bool BF16>
+template <int W>
 __device__ inline u32x4 corr_operand() {
-    const uint32_t c = Codec<W, BF16>::CORR;
+    const uint32_t c = Codec<W, false>::CORR;
     u32x4 r = {c, c, c, c};
     return r;
 }
@@ -404,12 +395,12 @@ __global__ __launch_bounds__(256, 4) void k_gateup_decode(
 
 // ----------------------------------------------------------------------------------- down
 // One (slab, tile) block of a down matrix: 4 row blocks x 4 k-steps (micro-tiles).
-template <int W, bool BF16>
+template <int W>
 __device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4], const float (&sc)[4], f32x4 (&acc)[4]) {
-    const u32x4 bc = corr_operand<W, BF16>();
+    const u32x4 bc = corr_operand<W>();
     f32x4 corr = {0, 0, 0, 0};
 #pragma unroll
-    for (int m = 0; m < 4; ++m) corr = mfma16<BF16>(az[m], bc, corr);
+    for (int m = 0; m < 4; ++m) corr = mfma16<false>(az[m], bc, corr);
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) {
         f32x4 t = {0, 0, 0, 0};
@@ -417,12 +408,12 @@ __device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4
         for (int m = 0; m < 4; ++m) {
             u32x4 bw;
             if constexpr (W == 2)
-                bw = decode_fields2<2, BF16>(b.w[nb * 2 + (m >> 1)], 8 * (m & 1));
+                bw = decode_fields2<2, false>(b.w[nb * 2 + (m >> 1)], 8 * (m & 1));
             else if constexpr (W == 4)
-                bw = decode_fields4<BF16>(b.w[nb * 4 + m]);
+                bw = decode_fields4<false>(b.w[nb * 4 + m]);
             else
-                bw = decode_fields3<BF16>(b.w[nb * 2 + (m >> 1)], 8 * (m & 1), b.w[8 + nb], 4 * m);
-            t = mfma16<BF16>(az[m], bw, t);
+                bw = decode_fields3<false>(b.w[nb * 2 + (m >> 1)], 8 * (m & 1), b.w[8 + nb], 4 * m);
+            t = mfma16<false>(az[m], bw, t);
         }
         acc[nb] += (t - corr) * sc[nb];
     }
@@ -433,7 +424,7 @@ __device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4
 // The payload of the first two tiles is requested BEFORE z is built, so that the weights
 // are in flight while G and U are read and SiLU is evaluated; afterwards the tiles stream
 // through three register buffers, two tiles ahead of the one being computed.
-template <int W, bool BF16>
+template <int W>
 __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gptr<__half> svec, gptr<int32_t> rank_idx,
                                  const FastSlab fs, const float* __restrict__ G, const float* __restrict__ U,
                                  const float* __restrict__ route_w, const int32_t* __restrict__ token_indices,
@@ -468,7 +459,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
             const uint16_t* zp = z + n * z_stride + (tb + i) * N_TILE + 8 * kg;
 #pragma unroll
             for (int m = 0; m < 4; ++m) az[m] = *reinterpret_cast<const u32x4*>(zp + 32 * m);
-            down_block<WL, BF16>(buf[B], az, sc[B], acc);
+            down_block<WL>(buf[B], az, sc[B], acc);
         };
         int lr[4];
         float sv[4];
@@ -504,10 +495,10 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                 for (int j = 0; j < 4; ++j) {
                     if (ab + j < n_a) {
                         u32x2 packed;
-                        packed[0] = (uint32_t)to_operand<BF16>(silu_f32(gv[j][0]) * uv[j][0]) |
-                                    ((uint32_t)to_operand<BF16>(silu_f32(gv[j][1]) * uv[j][1]) << 16);
-                        packed[1] = (uint32_t)to_operand<BF16>(silu_f32(gv[j][2]) * uv[j][2]) |
-                                    ((uint32_t)to_operand<BF16>(silu_f32(gv[j][3]) * uv[j][3]) << 16);
+                        packed[0] = (uint32_t)to_operand<false>(silu_f32(gv[j][0]) * uv[j][0]) |
+                                    ((uint32_t)to_operand<false>(silu_f32(gv[j][1]) * uv[j][1]) << 16);
+                        packed[1] = (uint32_t)to_operand<false>(silu_f32(gv[j][2]) * uv[j][2]) |
+                                    ((uint32_t)to_operand<false>(silu_f32(gv[j][3]) * uv[j][3]) << 16);
                         *reinterpret_cast<u32x2*>(z + (ab + j) * z_stride + c) = packed;
                     }
                 }
@@ -546,7 +537,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
 // grid.x = E * n_groups * n_tchunks; 256 threads; dynamic LDS = 16 * (n_tiles * 128 + 8) * 2 bytes.
 // A workgroup takes four slabs of one expert and a run of tiles; with few active experts the
 // tiles are split over several workgroups (their partial sums meet in the atomics of the combine).
-template <bool BF16, int MODE>
+template <int MODE>
 __global__ __launch_bounds__(256) void k_down_decode(
     const FastExpert* __restrict__ down_fe, const FastSlab* __restrict__ down_fs, int max_slabs,
     const float* __restrict__ G, const float* __restrict__ U, const float* __restrict__ route_w,
@@ -601,16 +592,16 @@ __global__ __launch_bounds__(256) void k_down_decode(
     // the four wavefronts may run four different instantiations; every one of them executes
     // the same two workgroup barriers per assignment chunk
     if (fs.bits == 2)
-        down_wave<2, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
+        down_wave<2>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, tid, lane);
     else if (fs.bits == 3)
-        down_wave<3, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
+        down_wave<3>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, tid, lane);
     else if (fs.bits == 4)
-        down_wave<4, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
+        down_wave<4>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, tid, lane);
     else
-        down_wave<0, BF16>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
+        down_wave<0>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, tid, lane);
 }
 
@@ -716,9 +707,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
                            down->d_fast_slabs, down->max_slabs, G, U, rw, tok, off, (int)T, (int)A, I, E, n_tiles,
                            dn_groups, dn_tchunks, dn_tiles_per_wg, n_work, rank_out, rank_accum);
     };
-    auto launch_down_mode = [&](auto bf16_c, auto mode_c) {
-        launch_down(k_down_decode<decltype(bf16_c)::value, decltype(mode_c)::value>);
-    };
+    auto launch_down_mode = [&](auto, auto mode_c) { launch_down(k_down_decode<decltype(mode_c)::value>); };
     // (G and U are fp32 and the operands f16 whatever the activation type was)
     with_mode(launch_down_mode, std::false_type{});
     BITSMOE_HIP_TRY(hipGetLastError());
