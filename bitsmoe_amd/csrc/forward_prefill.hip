@@ -565,8 +565,8 @@ __device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const 
                                                      int n_tiles, uint16_t* __restrict__ out, int a_begin, int rows,
                                                      int t0, const DmaStage st0, const DmaStage st1, const DmaStage st2,
                                                      int32_t* __restrict__ pack_tab, int32_t* __restrict__ scale_tab,
-                                                     int32_t* __restrict__ rank_tab) {
-    static_assert(WU == 2 || WU == 3 || WU == 4, "one bit-width per expert");
+                                                     int32_t* __restrict__ rank_tab, int32_t* __restrict__ bits_tab) {
+    static_assert(WU == 0 || WU == 2 || WU == 3 || WU == 4, "a bit-width, or 0 for widths that differ from slab to slab");
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -579,7 +579,8 @@ __device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const 
     // this lane lands in row r0 + 32*j, chunk position tid % 8 of a stage; it fetches the chunk that
     // belongs there (32*j does not change the permutation).  DIRECT: through the token index.
     constexpr int NJ = (NMB + 1) / 2;      // 32-row groups that hold assignments
-    constexpr int NB = WU == 2 ? 1 : 2;    // payload load instructions per slab
+    constexpr int NB = WU == 2 ? 1 : 2;    // payload load instructions per slab (mixed widths: always two, so that
+                                           // one wait count serves every slab; a 2-bit slab repeats its load)
     constexpr int G = NJ + 1 + NB;         // load instructions per slab and wavefront
     const int r0 = tid >> 3;
     const int cpos = (tid & 7) ^ ((r0 >> 1) & 7);
@@ -600,6 +601,7 @@ __device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const 
         const i32x4 r = *reinterpret_cast<const i32x4*>(fs_row + i);     // {bits, pack_off, scale_off, rank_off}
         pack_tab[i] = r[1];
         scale_tab[i] = r[2];
+        if constexpr (WU == 0) bits_tab[i] = r[0];
     }
     if constexpr (DIRECT)
         for (int i = tid; i < nslabs * 8; i += 256) rank_tab[i] = rank_idx[(i >> 3) * SLAB_ROWS + (i & 7) * 8];
@@ -622,6 +624,15 @@ __device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const 
         if (lane < 8)
             load_to_lds16(scale + (uint32_t)(scale_tab[s] + t * SLAB_ROWS + lane * 8), st.sc + wave * 64);
         // payload of the wavefront's two column-block pairs, in memory order
+        if constexpr (WU == 0) {
+            const int W = __builtin_amdgcn_readfirstlane(bits_tab[s]);
+            const uint32_t* blk = payload + (uint32_t)(pack_tab[s] + t * 256 * W);
+            const uint32_t first = W == 4 ? (uint32_t)((2 * wn * 64 + lane) * 4) : (uint32_t)(2 * wn * 128 + lane * 4);
+            const uint32_t second = W == 4 ? first + 256u : W == 3 ? (uint32_t)(512 + 2 * wn * 64 + lane * 4) : first;
+            load_to_lds16(blk + first, st.w + wave * 512);
+            if (W != 3 || lane < 32) load_to_lds16(blk + second, st.w + wave * 512 + 256);
+            return;
+        }
         const uint32_t* blk = payload + (uint32_t)(pack_tab[s] + t * 256 * WU);
         if constexpr (WU == 4) {
 #pragma unroll
@@ -636,17 +647,17 @@ __device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const 
         }
     };
     // payload words and scales of the slab in stage `st`, from LDS to this lane's registers
-    auto take = [&](const DmaStage& st, uint32_t (&bw)[2][4], u32x4 (&sc)[2]) {
+    auto take = [&](const DmaStage& st, int W, uint32_t (&bw)[2][4], u32x4 (&sc)[2]) {
         const uint32_t* wbase = st.w + wave * 512;
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
-            if constexpr (WU == 4) {
+            if (WU == 4 || (WU == 0 && W == 4)) {
                 const u32x4 v = *reinterpret_cast<const u32x4*>(wbase + p * 256 + lane * 4);
                 bw[p][0] = v[0]; bw[p][1] = v[1]; bw[p][2] = v[2]; bw[p][3] = v[3];
             } else {
                 const u32x2 v = *reinterpret_cast<const u32x2*>(wbase + p * 128 + lane * 2);
                 bw[p][0] = v[0]; bw[p][1] = v[1]; bw[p][2] = 0; bw[p][3] = 0;
-                if constexpr (WU == 3) {
+                if (WU == 3 || (WU == 0 && W == 3)) {
                     const u32x2 h = *reinterpret_cast<const u32x2*>(wbase + 256 + (p * 32 + kg * 8 + (n & 7)) * 2);
                     bw[p][2] = h[0]; bw[p][3] = h[1];
                 }
@@ -673,9 +684,10 @@ __device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const 
             const DmaStage& nxt = U == 0 ? st2 : U == 1 ? st0 : st1;
             uint32_t bw[2][4];
             u32x4 sc[2];
-            take(cur, bw, sc);
+            const int W = WU != 0 ? WU : __builtin_amdgcn_readfirstlane(bits_tab[s]);
+            take(cur, W, bw, sc);
             if (s + 2 < nslabs) request(nxt, s + 2);
-            if (active) gateup_slab_mfma<WU, NMB>(WU, cur.a, bw, sc, lane, acc);
+            if (active) gateup_slab_mfma<WU, NMB>(W, cur.a, bw, sc, lane, acc);
             asm volatile("" ::: "memory");
             if (s + 2 < nslabs)
                 wait_vmcnt<G>();      // slab s + 1 has landed; slab s + 2 may be in flight
@@ -718,7 +730,7 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     __shared__ __attribute__((aligned(16))) uint16_t sa0[DMA_STAGE], sa1[DMA_STAGE], sa2[DMA_STAGE];
     __shared__ __attribute__((aligned(16))) uint32_t sw0[DMA_WSTAGE], sw1[DMA_WSTAGE], sw2[DMA_WSTAGE];
     __shared__ __attribute__((aligned(16))) uint16_t ss0[DMA_SSTAGE], ss1[DMA_SSTAGE], ss2[DMA_SSTAGE];
-    __shared__ int32_t pack_tab[DMA_MAX_SLABS], scale_tab[DMA_MAX_SLABS], rank_tab[DMA_MAX_SLABS * 8];
+    __shared__ int32_t pack_tab[DMA_MAX_SLABS], scale_tab[DMA_MAX_SLABS], rank_tab[DMA_MAX_SLABS * 8], bits_tab[DMA_MAX_SLABS];
     const int n_tp = (n_tiles + 1) >> 1;
     const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles), 2 * n_tp);
     if (logical < 0) return;
@@ -747,15 +759,15 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     do {                                                                                                             \
         if (rows <= 32)                                                                                              \
             gateup_tile_body_dma<DIRECT, W, 2>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out,         \
-                                               a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab); \
+                                               a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab, bits_tab); \
         else if (rows <= 64)                                                                                         \
             gateup_tile_body_dma<DIRECT, W, 4>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out,         \
-                                               a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab); \
+                                               a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab, bits_tab); \
         else                                                                                                         \
             gateup_tile_body_dma<DIRECT, W, 8>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out,         \
-                                               a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab); \
+                                               a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab, bits_tab); \
     } while (0)
-    // experts with mixed widths (or more slabs than the tables hold) take the register-staged body
+    // experts with more slabs than the tables hold take the register-staged body
 #define BITSMOE_GU_BODY_MIXED()                                                                                      \
     do {                                                                                                             \
         if (rows <= 32)                                                                                              \
@@ -774,7 +786,7 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     else if (w == 4)
         BITSMOE_GU_BODY(4);
     else
-        BITSMOE_GU_BODY_MIXED();
+        BITSMOE_GU_BODY(0);
 #undef BITSMOE_GU_BODY
 #undef BITSMOE_GU_BODY_MIXED
 }
