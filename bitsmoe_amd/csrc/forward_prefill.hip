@@ -64,13 +64,13 @@ __global__ __launch_bounds__(256) void k_token_count(const int32_t* __restrict__
 // One workgroup: the list of (expert, first assignment, rows <= 128) tiles from
 // expert_offsets, then token_start = exclusive scan of token_count (T + 1 entries).
 // The list is ordered by decreasing cost (a counting sort over a few cost classes: the body the
-// tile runs -- full, half or quarter height -- then the bit-widths of the expert's gate and up
+// tile runs -- full to quarter height -- then the bit-widths of the expert's gate and up
 // matrices): workgroups start in list order, so the long ones run first and the short ones fill
 // the end of the launch.  Which of two tiles of one class comes first is left to the LDS atomics:
 // no result depends on the order.
 constexpr int MT_KEYS = 32;
 __device__ inline int mtile_key(int rows, int wsum) {      // 0 = most expensive
-    const int c = rows > 64 ? 0 : rows > 32 ? 1 : 2;
+    const int c = rows > 96 ? 0 : rows > 64 ? 1 : rows > 32 ? 2 : 3;
     return c * 8 + (7 - min(max(wsum - 1, 0), 7));           // wsum: 4 .. 8, or 0 (mixed widths: taken as the most expensive)
 }
 __global__ __launch_bounds__(256) void k_build_mtiles(const int32_t* __restrict__ expert_offsets, int E, int A,
@@ -751,9 +751,9 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     const int ld = proj ? ldu : ldg;
     uint16_t* __restrict__ out = proj ? U : G;
     const int w = __builtin_amdgcn_readfirstlane(fe.uniform_bits);
-    // tiles of at most 32 (64) assignments (experts that see few tokens, remainders) run a body with
-    // a quarter (half) of the accumulators, MFMAs and staging; complete bodies, so that no
-    // accumulator lives across the choice
+    // tiles of at most 32 / 64 / 96 assignments (experts that see few tokens, remainders) run a body
+    // with a quarter / half / three quarters of the accumulators, MFMAs and staging; complete
+    // bodies, so that no accumulator lives across the choice
     const DmaStage st0 = {sa0, sw0, ss0}, st1 = {sa1, sw1, ss1}, st2 = {sa2, sw2, ss2};
 #define BITSMOE_GU_BODY(W)                                                                                           \
     do {                                                                                                             \
@@ -762,6 +762,9 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
                                                a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab, bits_tab); \
         else if (rows <= 64)                                                                                         \
             gateup_tile_body_dma<DIRECT, W, 4>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out,         \
+                                               a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab, bits_tab); \
+        else if (rows <= 96)                                                                                         \
+            gateup_tile_body_dma<DIRECT, W, 6>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out,         \
                                                a_begin, rows, 2 * tp, st0, st1, st2, pack_tab, scale_tab, rank_tab, bits_tab); \
         else                                                                                                         \
             gateup_tile_body_dma<DIRECT, W, 8>(fe, fs_row, nslabs, Hs, ld, token_indices, T, I, n_tiles, out,         \
@@ -1014,8 +1017,8 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
     FastSlab fs = FastSlab{0, 0, 0, 0};
     if (si < nslabs) fs = load_fast_slab(down_fs + (int64_t)e * max_slabs, si);
 
-    // tiles of at most 32 (64) assignments run a body with a quarter (half) of the accumulators and
-    // MFMAs: complete bodies, so that no accumulator lives across the choice
+    // tiles of at most 32 / 64 / 96 assignments run a body with a quarter / half / three quarters of
+    // the accumulators and MFMAs: complete bodies, so that no accumulator lives across the choice
     auto run = [&](auto nmb_c) {
         constexpr int NMB = decltype(nmb_c)::value;
         f32x4 acc[NMB][4];
@@ -1049,6 +1052,8 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
         run(std::integral_constant<int, 2>{});
     else if (rows <= 64)
         run(std::integral_constant<int, 4>{});
+    else if (rows <= 96)
+        run(std::integral_constant<int, 6>{});
     else
         run(std::integral_constant<int, 8>{});
 }
