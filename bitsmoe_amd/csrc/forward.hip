@@ -34,13 +34,12 @@ static int resolve_path(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
         return BITSMOE_E_UNSUPPORTED;
     }
     if (path != BITSMOE_PATH_AUTO) return path;
-    // grouped GEMM from 24 assignments per expert on average, 16 with many experts (measured
-    // crossovers on layers of 64, 128 and 512 experts: the decode kernels re-stream the payload for
-    // every 16 assignments, the grouped GEMM pays for whole 128-row tiles and a longer launch chain)
-    const int64_t per_expert = gate->n_experts >= 128 ? 16 : 24;
-    if (mfma_ok && n_assign >= per_expert * gate->n_experts) return BITSMOE_PATH_MFMA;
+    // grouped GEMM from 14 assignments per expert on average (measured crossovers on layers of 64,
+    // 128 and 512 experts: 12 to 16; the decode kernels re-stream the payload for every 16
+    // assignments, the grouped GEMM pays for a longer launch chain)
+    if (mfma_ok && n_assign >= (int64_t)14 * gate->n_experts) return BITSMOE_PATH_MFMA;
     if (decode_ok) return BITSMOE_PATH_DECODE;
-    if (mfma_ok && n_assign >= (int64_t)16 * gate->n_experts) return BITSMOE_PATH_MFMA;
+    if (mfma_ok) return BITSMOE_PATH_MFMA;      // (an intermediate size beyond the decode kernels' LDS budget)
     return BITSMOE_PATH_GENERIC;
 }
 
