@@ -102,6 +102,8 @@ struct bitsmoe_matset {
     __half* d_scale_s = nullptr;      // gate/up sets: scale folded with the per-row multiplier s
     bool vector_aligned = false;      // scale / s / rank_idx of every expert start on 16-byte boundaries
     bool all_uniform8 = false;        // role 0: every aligned group of 8 slabs has one width and is contiguous
+    bool all_affine = false;          // role 0: every expert has max_slabs slabs of ONE width whose payload, scale and
+                                      // rank offsets advance by a whole slab from one slab to the next
     // experts by decreasing payload size (prepared sets of at most EXPERT_ORDER_MAX experts): the
     // decode kernels start the expensive experts' workgroups first
     bool has_cost_order = false;

@@ -17,6 +17,7 @@
 // addressable from its block index (FastExpert / FastSlab tables: one round trip, not a
 // chain of five), (2) every workgroup walks several tiles and keeps the payload of the next
 // tile in flight while it computes the current one.
+#include <cstdlib>
 #include <type_traits>
 #include <utility>
 
@@ -27,6 +28,7 @@ namespace bitsmoe {
 constexpr int GU_STRIDE = GU_SLABS * SLAB_ROWS + 8;  // 16-bit elements; +8 staggers LDS banks
 constexpr int DN_SLABS_PER_WG = 4;                 // one slab per wavefront
 constexpr int MAX_A = 16;                          // assignments per MFMA pass
+constexpr int64_t WALK_MIN_WGS = 512;              // walking gate/up kernel: fewest (expert, projection, tile) units
 
 template <int W>
 __device__ inline u32x4 corr_operand() {
@@ -393,6 +395,196 @@ __global__ __launch_bounds__(256, 4) void k_gateup_decode(
     }
 }
 
+// ------------------------------------------------------- gate / up, one workgroup per tile
+// The same contraction for sets in which every expert is one affine run of equal-width slabs
+// (bitsmoe_matset::all_affine) whose rank_idx maps every aligned run of eight rows to eight
+// consecutive ranks (rank_chunked8): a workgroup takes one expert, one projection and ONE
+// 128-column tile and walks all slab groups, keeping the tile's accumulators in registers.
+//  * Every output element has exactly one owner: plain stores instead of fp32 atomics, no zero
+//    fill of G / U beforehand.
+//  * The payload stream of a wavefront runs on across the group boundaries (the block addresses
+//    are affine in group, slab and tile).
+//  * The activation operand of a group is built with 16-byte accesses: wavefront w serves the
+//    assignments w, w+4, w+8, w+12 of the chunk; its lane l loads rows 8l .. 8l+7 of the group for
+//    one assignment as ONE 16-byte load (eight consecutive ranks of the token's row), the eight
+//    folded scales as another, multiplies and writes one 16-byte piece of the LDS operand.  Only
+//    assignments that exist are touched (an MFMA output row depends on its own operand row
+//    only, and rows past the chunk's assignments are never stored).
+//  * Nothing a group needs is fetched when the group begins: the rank of a lane's rows arrives
+//    two groups ahead, its scales one group ahead, and the activations of the wavefront's first
+//    two assignments are requested right after the previous group's operand has been staged, so
+//    they return behind that group's MFMAs.
+// A token index out of range is clamped for the address: the down kernel ignores such an
+// assignment, whatever its G / U rows hold.
+// The kernel also clears `zero_out` (the forward's accumulator, added into by the down kernel).
+// grid.x = (expert coordinate) * n_tiles, grid.y = 2 (gate, up); 256 threads = 4 wavefronts.
+template <bool BF16>
+__device__ __forceinline__ u32x4 scaled_f16x8(u32x4 raw, u32x4 sc) {
+    u32x4 out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t v = raw[i];
+        if constexpr (BF16) {      // bf16 -> f16 is exact inside the f16 range (8 significant bits into 11)
+            typedef __fp16 h2v __attribute__((ext_vector_type(2)));
+            const h2v c = __builtin_amdgcn_cvt_pkrtz(__uint_as_float(v << 16), __uint_as_float(v & 0xFFFF0000u));
+            v = __builtin_bit_cast(uint32_t, c);
+        }
+        out[i] = pk_mul_f16(v, sc[i]);
+    }
+    return out;
+}
+
+template <bool BF16, int MODE>
+__global__ __launch_bounds__(256, 4) void k_gateup_walk(
+    const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
+    const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
+    const uint16_t* __restrict__ h_gate, const uint16_t* __restrict__ h_up, int64_t ldg, int64_t ldu,
+    const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
+    int E, int n_tiles, float* __restrict__ G, float* __restrict__ U, float* __restrict__ zero_out,
+    int64_t zero_n, const ExpertOrder gate_order, const ExpertOrder up_order) {
+    const int mt = blockIdx.y;
+    const int bid = blockIdx.x;
+    const int tid = threadIdx.x;
+    {   // this workgroup's share of the accumulator (before any exit)
+        const int64_t total = (int64_t)gridDim.x * 2 * 256;
+        for (int64_t i = ((int64_t)mt * gridDim.x + bid) * 256 + tid; i < zero_n; i += total) zero_out[i] = 0.0f;
+    }
+    const int t = bid % n_tiles;
+    int e = bid / n_tiles;
+    int chunk = -1;
+    if constexpr (MODE == GRID_EXPERTS) {      // expensive experts first (the identity when there is no order)
+        if (E <= EXPERT_ORDER_MAX) e = mt ? up_order.e[e] : gate_order.e[e];
+    } else if constexpr (MODE == GRID_ACTIVE) {
+        e = nth_active_expert(expert_offsets, E, A, e, tid & 63);
+        if (e < 0) return;
+    } else if constexpr (MODE == GRID_CHUNKS) {
+        const ChunkRef ref = nth_chunk(expert_offsets, E, A, e, tid & 63);
+        e = ref.expert;
+        chunk = ref.chunk;
+        if (e < 0) return;
+    }
+    const int pair = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform
+    const int lane = tid & 63;
+    const int n = lane & 15, kg = lane >> 4;
+
+    // one round trip: assignment range, expert record, the record of the expert's first slab
+    int a_begin = max(expert_offsets[e], 0);
+    int a_end = min(expert_offsets[e + 1], A);
+    if (chunk >= 0) {
+        a_begin += MAX_A * chunk;
+        a_end = min(a_end, a_begin + MAX_A);
+    }
+    const FastExpert* __restrict__ fe_tab = mt ? up_fe : gate_fe;
+    const FastSlab* __restrict__ fs_tab = mt ? up_fs : gate_fs;
+    const int max_slabs = mt ? up_max_slabs : gate_max_slabs;
+    const FastExpert fe = fe_tab[e];
+    const FastSlab first = load_fast_slab(fs_tab, e * max_slabs);
+    if (a_end <= a_begin || first.bits == 0) return;
+    const int n_groups = max_slabs / GU_SLABS;
+
+    gptr<uint32_t> payload = as_global(fe.payload);
+    gptr<__half> scale_s = as_global(fe.scale_s);
+    gptr<int32_t> rank_idx = as_global(fe.rank_idx);
+    const uint16_t* __restrict__ h = mt ? h_up : h_gate;
+    const int64_t ld = mt ? ldu : ldg;
+    float* __restrict__ out = mt ? U : G;
+    const uint32_t unit = (uint32_t)(pair * 64 + lane);
+    const uint32_t hi_unit = (uint32_t)hi_index0(kg, n, 2 * pair);
+
+    __shared__ __attribute__((aligned(16))) uint16_t hs[MAX_A * GU_STRIDE];
+
+    auto body = [&](auto w_c) {
+    constexpr int W = decltype(w_c)::value;
+    const int slab_words = n_tiles * 256 * W;       // payload words from one slab to the next
+    for (int a0 = a_begin; a0 < a_end; a0 += MAX_A) {
+        const int n_a = min(MAX_A, a_end - a0);
+        int chunk_zero = 0;
+        asm volatile("" : "+s"(chunk_zero));   // keeps this chunk's address arithmetic inside the loop
+        const int pack0 = first.pack_off + t * 256 * W + chunk_zero;
+
+        uint32_t pw[GU_SLABS][4];   // slab q's block of the current group; refilled for the next group right after use
+        auto issue = [&](auto q_c, int g) {
+            constexpr int q = decltype(q_c)::value;
+            load_pair_role0(payload + (uint32_t)(pack0 + (g * GU_SLABS + q) * slab_words), W, unit, hi_unit, pw[q]);
+        };
+        static_for([&](auto qc) { issue(qc, 0); }, std::make_integer_sequence<int, GU_SLABS>{});
+
+        // the rows of this wavefront's assignments pair, pair + 4, pair + 8, pair + 12 (wave-uniform)
+        const uint16_t* trow[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int a = pair + 4 * i;
+            const int tk = a < n_a ? __builtin_amdgcn_readfirstlane(token_indices[a0 + a]) : 0;
+            trow[i] = h + (int64_t)min(max(tk, 0), T - 1) * ld;
+        }
+        // rows 8*lane .. 8*lane + 7 of group g: first logical rank, the f16 bits of their eight
+        // scale * s * stagger factor (folded once when the set was prepared), the activations
+        auto rank_at = [&](int g) { return rank_idx[first.rank_off + g * (GU_SLABS * SLAB_ROWS) + 8 * lane]; };
+        auto scale_at = [&](int g) {
+            return *reinterpret_cast<gptr_u32x4>(
+                scale_s + (uint32_t)(first.scale_off + ((g * GU_SLABS + (lane >> 3)) * n_tiles + t) * SLAB_ROWS + 8 * (lane & 7)));
+        };
+        auto act_at = [&](int i, int rank) { return *reinterpret_cast<const u32x4*>(trow[i] + rank); };
+        auto stage = [&](int i, u32x4 raw, u32x4 sc) {
+            *reinterpret_cast<u32x4*>(&hs[(pair + 4 * i) * GU_STRIDE + 8 * lane]) = scaled_f16x8<BF16>(raw, sc);
+        };
+        int rank_cur = rank_at(0);
+        int rank_nxt = n_groups > 1 ? rank_at(1) : 0;
+        u32x4 sc_cur = scale_at(0);
+        u32x4 raw0 = {0, 0, 0, 0}, raw1 = {0, 0, 0, 0};
+        if (pair < n_a) raw0 = act_at(0, rank_cur);
+        if (pair + 4 < n_a) raw1 = act_at(1, rank_cur);
+        f32x4 acc[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+        f32x4 corr = {0, 0, 0, 0};
+        for (int g = 0; g < n_groups; ++g) {
+            const bool more = g + 1 < n_groups;
+            int rank_nxt2 = 0;
+            if (g + 2 < n_groups) rank_nxt2 = rank_at(g + 2);
+            u32x4 sc_nxt = {0, 0, 0, 0};
+            if (more) sc_nxt = scale_at(g + 1);
+            __syncthreads();   // every wavefront is done reading the previous group's operand
+            if (pair < n_a) stage(0, raw0, sc_cur);
+            if (pair + 4 < n_a) stage(1, raw1, sc_cur);
+            if (pair + 8 < n_a) stage(2, act_at(2, rank_cur), sc_cur);      // (rare: fetched here, not ahead)
+            if (pair + 12 < n_a) stage(3, act_at(3, rank_cur), sc_cur);
+            __syncthreads();   // the operand is complete
+            if (more) {
+                if (pair < n_a) raw0 = act_at(0, rank_nxt);
+                if (pair + 4 < n_a) raw1 = act_at(1, rank_nxt);
+            }
+            const uint16_t* ap16 = &hs[n * GU_STRIDE + 16 * kg];
+            static_for([&](auto qc) {
+                constexpr int q = decltype(qc)::value;
+                const u32x4 a_lo = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS);
+                const u32x4 a_hi = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS + 8);
+                gateup_pair<W>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
+                if (more) issue(qc, g + 1);
+            }, std::make_integer_sequence<int, GU_SLABS>{});
+            sc_cur = sc_nxt;
+            rank_cur = rank_nxt;
+            rank_nxt = rank_nxt2;
+        }
+        // remove the constant term; lane holds rows a = 4*kg + j of column 32*pair + 16*nbl + n
+#pragma unroll
+        for (int nbl = 0; nbl < 2; ++nbl) {
+            const int c = t * N_TILE + 32 * pair + 16 * nbl + n;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int a = 4 * kg + j;
+                if (a < n_a && c < I) out[(int64_t)(a0 + a) * I + c] = acc[nbl][j] - corr[j];
+            }
+        }
+    }
+    };   // body
+
+    if (first.bits == 2)
+        body(std::integral_constant<int, 2>{});
+    else if (first.bits == 3)
+        body(std::integral_constant<int, 3>{});
+    else if (first.bits == 4)
+        body(std::integral_constant<int, 4>{});
+}
+
 // ----------------------------------------------------------------------------------- down
 // One (slab, tile) block of a down matrix: 4 row blocks x 4 k-steps (micro-tiles).
 template <int W>
@@ -631,7 +823,26 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     const int E = gate->n_experts;
     const int n_tiles = gate->n_tiles;
     record(prof, 0, st);
-    {
+    // What the expert coordinate of the grids counts.  Few assignments: the experts that can be
+    // active at most, not all of them.  Sixteen or more assignments per expert on average: most
+    // experts have several 16-assignment chunks, one workgroup per chunk.  Below that the search
+    // of the chunk (one more dependent round trip per workgroup, +10 %) costs more than walking
+    // an expert's few chunks in a loop, unless routing is skewed: with at most 64 experts (one
+    // search step) the chunk grid is already used from three assignments per expert on average.
+    // At most min(E, A) experts can be active.
+    const int64_t active_max = std::min<int64_t>(E, A);
+    const int mode = (A >= (int64_t)16 * E || (E <= 64 && A >= (int64_t)3 * E)) ? GRID_CHUNKS : active_max * 2 <= E ? GRID_ACTIVE : GRID_EXPERTS;
+    const int e_dim = mode == GRID_CHUNKS ? (int)(active_max + A / MAX_A) : mode == GRID_ACTIVE ? (int)active_max : E;
+    // (expert, chunk) pairs expected to have work (e_dim is their upper bound in chunk mode)
+    const int64_t units = mode == GRID_CHUNKS ? A / MAX_A + active_max / 2 : active_max;
+    // Sets of affine single-width experts, enough (expert, tile) pairs to fill the chip: the
+    // walking gate/up kernel, which also clears rank_accum and needs no cleared G / U.
+    // (its 16-byte activation loads also need rank_idx in runs of eight and aligned rows)
+    auto rows16 = [](const void* p, int64_t ld) { return ((uintptr_t)p & 15) == 0 && ld % 8 == 0; };
+    int walk_tpw = gate->all_affine && up->all_affine && gate->rank_chunked8 && up->rank_chunked8 &&
+                   rows16(h_gate, ldg) && rows16(h_up, ldu) && units * 2 * n_tiles >= WALK_MIN_WGS;
+    if (const char* ev = getenv("BITSMOE_WALK_TPW")) walk_tpw = atoi(ev);
+    if (walk_tpw == 0) {
         // G and U are adjacent in the workspace: one range; rank_accum is the second
         const int64_t n1 = inter_floats + A * (int64_t)I;
         const int64_t n2 = T * (int64_t)rank_out;
@@ -643,18 +854,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     const int max_slabs = std::max(gate->max_slabs, up->max_slabs);
     const int gu_groups = (max_slabs + GU_SLABS - 1) / GU_SLABS;
     // Tiles per workgroup: long runs amortise the start-up round trips, but the grid must
-    // still hold a few workgroups per CU (two rounds of three per CU measured best).  At most min(E, A) experts can be active.
-    const int64_t active_max = std::min<int64_t>(E, A);
-    // What the expert coordinate of the grids counts.  Few assignments: the experts that can be
-    // active at most, not all of them.  Sixteen or more assignments per expert on average: most
-    // experts have several 16-assignment chunks, one workgroup per chunk.  Below that the search
-    // of the chunk (one more dependent round trip per workgroup, +10 %) costs more than walking
-    // an expert's few chunks in a loop, unless routing is skewed: with at most 64 experts (one
-    // search step) the chunk grid is already used from three assignments per expert on average.
-    const int mode = (A >= (int64_t)16 * E || (E <= 64 && A >= (int64_t)3 * E)) ? GRID_CHUNKS : active_max * 2 <= E ? GRID_ACTIVE : GRID_EXPERTS;
-    const int e_dim = mode == GRID_CHUNKS ? (int)(active_max + A / MAX_A) : mode == GRID_ACTIVE ? (int)active_max : E;
-    // (expert, chunk) pairs expected to have work (e_dim is their upper bound in chunk mode)
-    const int64_t units = mode == GRID_CHUNKS ? A / MAX_A + active_max / 2 : active_max;
+    // still hold a few workgroups per CU (two rounds of three per CU measured best).
     int tiles_per_wg = n_tiles;
     while (tiles_per_wg > 1 && units * 2 * gu_groups * ((n_tiles + tiles_per_wg - 1) / tiles_per_wg) < 1536)
         tiles_per_wg = (tiles_per_wg + 1) / 2;
@@ -689,10 +889,23 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         else
             fn(bf16_c, std::integral_constant<int, GRID_EXPERTS>{});
     };
-    if (bf16)
+    auto launch_walk_mode = [&](auto bf16_c, auto mode_c) {
+        hipLaunchKernelGGL((k_gateup_walk<decltype(bf16_c)::value, decltype(mode_c)::value>), dim3((unsigned)(e_dim * n_tiles), 2),
+                           dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs, gate->max_slabs, up->d_fast_experts,
+                           up->d_fast_slabs, up->max_slabs, (const uint16_t*)h_gate, (const uint16_t*)h_up, ldg, ldu,
+                           tok, off, (int)T, (int)A, I, E, n_tiles, G, U, rank_accum, T * (int64_t)rank_out, gate_order,
+                           up_order);
+    };
+    if (walk_tpw != 0) {
+        if (bf16)
+            with_mode(launch_walk_mode, std::true_type{});
+        else
+            with_mode(launch_walk_mode, std::false_type{});
+    } else if (bf16) {
         with_mode(launch_gateup_mode, std::true_type{});
-    else
+    } else {
         with_mode(launch_gateup_mode, std::false_type{});
+    }
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 2, st);
     const int dn_groups = (down->max_slabs + DN_SLABS_PER_WG - 1) / DN_SLABS_PER_WG;

@@ -233,6 +233,18 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
         }
     }
     set->all_uniform8 = all_uniform;
+    // is every expert one affine run of equal-width slabs (what the walking gate/up kernel assumes)?
+    bool all_affine = all_uniform;
+    for (int e = 0; e < set->n_experts && all_affine; ++e) {
+        const FastSlab& first = fslabs[(size_t)e * set->max_slabs];
+        for (int si = 1; si < set->max_slabs; ++si) {
+            const FastSlab& f = fslabs[(size_t)e * set->max_slabs + si];
+            if (f.bits != first.bits || f.pack_off != first.pack_off + si * set->n_tiles * 256 * first.bits ||
+                f.scale_off != first.scale_off + si * set->n_tiles * SLAB_ROWS || f.rank_off != first.rank_off + si * SLAB_ROWS)
+                all_affine = false;
+        }
+    }
+    set->all_affine = all_affine;
     bool aligned = true;
     for (int e = 0; e < set->n_experts; ++e) {
         const bitsmoe_matrix_desc& d = set->descs[e];
