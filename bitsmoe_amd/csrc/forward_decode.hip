@@ -17,7 +17,6 @@
 // addressable from its block index (FastExpert / FastSlab tables: one round trip, not a
 // chain of five), (2) every workgroup walks several tiles and keeps the payload of the next
 // tile in flight while it computes the current one.
-#include <cstdlib>
 #include <type_traits>
 #include <utility>
 
@@ -491,7 +490,8 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const uint32_t unit = (uint32_t)(pair * 64 + lane);
     const uint32_t hi_unit = (uint32_t)hi_index0(kg, n, 2 * pair);
 
-    __shared__ __attribute__((aligned(16))) uint16_t hs[MAX_A * GU_STRIDE];
+    // two copies of the operand, used in turn: one workgroup barrier per group instead of two
+    __shared__ __attribute__((aligned(16))) uint16_t hs_all[2 * MAX_A * GU_STRIDE];
 
     auto body = [&](auto w_c) {
     constexpr int W = decltype(w_c)::value;
@@ -525,6 +525,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
                 scale_s + (uint32_t)(first.scale_off + ((g * GU_SLABS + (lane >> 3)) * n_tiles + t) * SLAB_ROWS + 8 * (lane & 7)));
         };
         auto act_at = [&](int i, int rank) { return *reinterpret_cast<const u32x4*>(trow[i] + rank); };
+        uint16_t* hs = hs_all;
         auto stage = [&](int i, u32x4 raw, u32x4 sc) {
             *reinterpret_cast<u32x4*>(&hs[(pair + 4 * i) * GU_STRIDE + 8 * lane]) = scaled_f16x8<BF16>(raw, sc);
         };
@@ -542,7 +543,11 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
             if (g + 2 < n_groups) rank_nxt2 = rank_at(g + 2);
             u32x4 sc_nxt = {0, 0, 0, 0};
             if (more) sc_nxt = scale_at(g + 1);
-            __syncthreads();   // every wavefront is done reading the previous group's operand
+            // Group g writes copy g mod 2.  Its last readers (group g - 2) are done: every wavefront
+            // passed the barrier of group g - 1 after its MFMAs of group g - 2.  Only a new chunk
+            // needs a barrier of its own before the first write.
+            hs = hs_all + (g & 1) * (MAX_A * GU_STRIDE);
+            if (g == 0) __syncthreads();
             if (pair < n_a) stage(0, raw0, sc_cur);
             if (pair + 4 < n_a) stage(1, raw1, sc_cur);
             if (pair + 8 < n_a) stage(2, act_at(2, rank_cur), sc_cur);      // (rare: fetched here, not ahead)
@@ -839,10 +844,9 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     // walking gate/up kernel, which also clears rank_accum and needs no cleared G / U.
     // (its 16-byte activation loads also need rank_idx in runs of eight and aligned rows)
     auto rows16 = [](const void* p, int64_t ld) { return ((uintptr_t)p & 15) == 0 && ld % 8 == 0; };
-    int walk_tpw = gate->all_affine && up->all_affine && gate->rank_chunked8 && up->rank_chunked8 &&
+    const bool walk = gate->all_affine && up->all_affine && gate->rank_chunked8 && up->rank_chunked8 &&
                    rows16(h_gate, ldg) && rows16(h_up, ldu) && units * 2 * n_tiles >= WALK_MIN_WGS;
-    if (const char* ev = getenv("BITSMOE_WALK_TPW")) walk_tpw = atoi(ev);
-    if (walk_tpw == 0) {
+    if (!walk) {
         // G and U are adjacent in the workspace: one range; rank_accum is the second
         const int64_t n1 = inter_floats + A * (int64_t)I;
         const int64_t n2 = T * (int64_t)rank_out;
@@ -896,7 +900,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
                            tok, off, (int)T, (int)A, I, E, n_tiles, G, U, rank_accum, T * (int64_t)rank_out, gate_order,
                            up_order);
     };
-    if (walk_tpw != 0) {
+    if (walk) {
         if (bf16)
             with_mode(launch_walk_mode, std::true_type{});
         else

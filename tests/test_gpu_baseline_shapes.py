@@ -153,3 +153,47 @@ def test_full_size_dropped_assignments_do_not_contribute(cuda_device, tokens):
     tok2, off2, rw2 = hip.route(selected, w2, block._packed_global_to_local, block._packed_expert_count)
     out2 = hip.moe_forward_sets(h_gate, h_up, tok2, off2, rw2, gate, up, down, rank_out, isz, 0)
     assert float((out - out2).abs().max()) <= 1e-5 * float(out2.abs().max())
+
+
+@pytest.mark.parametrize("dtype_name", ["bfloat16", "float16"])
+def test_walking_gateup_popular_expert_and_offset_rows(cuda_device, dtype_name):
+    """The decode gate/up kernel that walks all slab groups of a tile: one expert that every token
+    selects (64 assignments = four 16-assignment chunks served in a loop), one with 12 to 16, the
+    others with fewer, for bf16 and f16 activations; and the same batch with activation rows that do not start on
+    16-byte boundaries, which takes the kernel with 2-byte gathers instead: same result."""
+    import torch
+
+    from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
+    from bitsmoe_amd.synth import SPECS
+
+    spec = SPECS["c2"]
+    block = _layer("c2", cuda_device)
+    dtype = getattr(torch, dtype_name)
+    h_gate, h_up, selected, weights = _inputs(block, spec, 64, 77, cuda_device)
+    h_gate, h_up = h_gate.to(dtype), h_up.to(dtype)
+    selected = selected.clone()
+    popular = 5
+    for row in range(selected.shape[0]):            # expert 5 in every token's selection, once
+        if not bool((selected[row] == popular).any()):
+            selected[row, 0] = popular
+    second = 9
+    for row in range(12):                           # expert 9 in the first twelve tokens' selections
+        if not bool((selected[row] == second).any()):
+            selected[row, 1 if int(selected[row, 1]) != popular else 2] = second
+    tok, off, rw, out = _run(block, h_gate, h_up, selected, weights)
+    counts = (off[1:] - off[:-1]).cpu().numpy()
+    assert counts[popular] == 64 and 12 <= counts[second] <= 16
+    ref = _oracle(block, h_gate, h_up, *(t.cpu().numpy() for t in (tok, off, rw)))
+    err = float(np.abs(out.cpu().numpy() - ref).max()) / float(np.abs(ref).max())
+    assert err <= 1e-2, f"normalised error {err:.3e}"
+    # rows shifted by one element inside a wider buffer: 2-byte aligned only
+    gate, up, down = block._ensure_matsets()
+    wide = torch.zeros((64, 2 * h_gate.shape[1] + 16), dtype=dtype, device=cuda_device)
+    hg = wide[:, 1:1 + h_gate.shape[1]]
+    hu = wide[:, 9 + h_gate.shape[1]:9 + h_gate.shape[1] + h_up.shape[1]]
+    hg.copy_(h_gate)
+    hu.copy_(h_up)
+    assert hg.data_ptr() % 16 != 0
+    out2 = hip.moe_forward_sets(hg, hu, tok, off, rw, gate, up, down, int(block.shared_u_down.shape[1]),
+                                int(block._packed_intermediate_size), 0)
+    assert float((out2 - out).abs().max()) <= 2e-3 * float(out.abs().max())
