@@ -144,21 +144,23 @@ def run_workload(block, spec, tokens, steps, warmup, seed=42, use_graph=True):
         except Exception as exc:   # noqa: BLE001 - the eager figure stands
             print(f"bench.py: graph replay unavailable ({exc}); reporting eager launches", file=sys.stderr)
     phases = [p.read() for p in profiles]
-    ms_fill = sum(p[0] for p in phases) / steps
-    ms_gateup = sum(p[1] for p in phases) / steps
-    ms_down = sum(p[2] for p in phases) / steps
+    # phases of the operator: preparation (with the routing launch before it), gate/up kernel,
+    # SiLU pass, down kernel, combine (third and fifth: launches of their own at prefill only)
+    ms_fill, ms_gateup, ms_silu, ms_down, ms_combine = (sum(p[i] for p in phases) / steps for i in range(5))
+    ms_all = ms_fill + ms_gateup + ms_silu + ms_down + ms_combine
     counts = (off[1:] - off[:-1]).cpu().tolist()
     work = algorithmic_work(block, counts, tokens, int(tok.numel()))
     res = {
         "tokens": tokens, "ms_per_step": elapsed / steps * 1e3, "tokens_per_s": tokens * steps / elapsed,
         "launch": launch, "eager_ms_per_step": eager / steps * 1e3, "hipgraph_ms_per_step": graph_ms,
-        "kernel_ms": {"zero_fill": ms_fill, "gate_up": ms_gateup, "down": ms_down},
+        "kernel_ms": {"prepare": ms_fill, "gate_up": ms_gateup, "silu_mul": ms_silu, "down": ms_down,
+                      "combine": ms_combine},
         "active_experts": work["active_experts"], "algorithmic_bytes": work["bytes_total"],
         "algorithmic_flops": work["flops"],
         "gateup_GBps": work["bytes_gateup"] / (ms_gateup * 1e-3) / 1e9 if ms_gateup > 0 else None,
         "down_GBps": work["bytes_down"] / (ms_down * 1e-3) / 1e9 if ms_down > 0 else None,
-        "kernels_GBps": work["bytes_total"] / ((ms_gateup + ms_down + ms_fill) * 1e-3) / 1e9,
-        "kernels_TFLOPs": work["flops"] / ((ms_gateup + ms_down + ms_fill) * 1e-3) / 1e12,
+        "kernels_GBps": work["bytes_total"] / (ms_all * 1e-3) / 1e9,
+        "kernels_TFLOPs": work["flops"] / (ms_all * 1e-3) / 1e12,
         "gateup_TFLOPs": work["flops_gateup"] / (ms_gateup * 1e-3) / 1e12 if ms_gateup > 0 else None,
         "down_TFLOPs": work["flops_down"] / (ms_down * 1e-3) / 1e12 if ms_down > 0 else None,
     }

@@ -17,7 +17,7 @@ PATH_AUTO = 0
 PATH_GENERIC = 1
 PATH_DECODE = 2
 PATH_MFMA = 3
-PROFILE_PHASES = 3
+PROFILE_PHASES = 5
 
 # every extern "C" symbol include/bitsmoe_hip.h declares
 EXPORTED_SYMBOLS = (

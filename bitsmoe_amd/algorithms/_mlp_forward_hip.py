@@ -133,14 +133,15 @@ class MatrixSet:
 
 
 class Profile:
-    """Per-phase HIP-event timing of one forward (zero-fill, gate+up, down), in ms."""
+    """Per-phase HIP-event timing of one forward, in ms: preparation, gate/up kernel, SiLU pass,
+    down kernel, combine (the third and fifth are launches of their own only on the grouped-GEMM path)."""
 
     def __init__(self):
         h = ctypes.c_void_p()
         _capi.check(_lib.bitsmoe_profile_create(ctypes.byref(h)))
         self._handle = h
 
-    def read(self) -> Tuple[float, float, float]:
+    def read(self) -> Tuple[float, ...]:
         ms = (ctypes.c_float * _capi.PROFILE_PHASES)()
         _capi.check(_lib.bitsmoe_profile_read(self._handle, ms))
         return tuple(float(v) for v in ms)

@@ -912,6 +912,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     }
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 2, st);
+    record(prof, 3, st);      // (SiLU happens inside the down kernel)
     const int dn_groups = (down->max_slabs + DN_SLABS_PER_WG - 1) / DN_SLABS_PER_WG;
     const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2;
     int dn_tiles_per_wg = n_tiles;
@@ -928,7 +929,8 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     // (G and U are fp32 and the operands f16 whatever the activation type was)
     with_mode(launch_down_mode, std::false_type{});
     BITSMOE_HIP_TRY(hipGetLastError());
-    record(prof, 3, st);
+    record(prof, 4, st);
+    record(prof, 5, st);      // (the combine too)
     if (prof) prof->recorded = true;
     return BITSMOE_OK;
 }

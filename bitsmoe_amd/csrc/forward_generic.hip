@@ -244,12 +244,14 @@ int launch_forward_generic(const bitsmoe_matset* gate, const bitsmoe_matset* up,
     }
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 2, st);
+    record(prof, 3, st);
     if (down->total_slabs > 0) {
         hipLaunchKernelGGL(k_down_generic, dim3((unsigned)down->total_slabs), dim3(256), 0, st, down->d_views,
                            down->d_slab_tasks, G, U, rw, tok, off, (int)T, (int)A, I, rank_out, rank_accum);
         BITSMOE_HIP_TRY(hipGetLastError());
     }
-    record(prof, 3, st);
+    record(prof, 4, st);
+    record(prof, 5, st);
     if (prof) prof->recorded = true;
     return BITSMOE_OK;
 }

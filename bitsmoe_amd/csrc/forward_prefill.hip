@@ -1289,18 +1289,20 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
             return hipGetLastError();
         };
         BITSMOE_HIP_TRY(direct ? launch(k_gateup_mfma<true>) : launch(k_gateup_mfma<false>));
+        record(prof, 2, st);
         const int64_t n8 = A * (int64_t)I / 8;
         hipLaunchKernelGGL(k_silu_mul_f16, dim3((unsigned)std::min<int64_t>((n8 + 255) / 256, 4096)), dim3(256), 0, st, z,
                            Ubuf, n8);
         BITSMOE_HIP_TRY(hipGetLastError());
     }
-    record(prof, 2, st);
+    record(prof, 3, st);
     {
         const int n_pairs = (down->max_slabs + DN_SLABS_MFMA - 1) / DN_SLABS_MFMA;
         const int64_t wgs = (max_mtiles + 31) / 32 * 32 * n_pairs;
         hipLaunchKernelGGL(k_down_mfma, dim3((unsigned)wgs), dim3(256), 0, st, down->d_fast_experts, down->d_fast_slabs,
                            down->max_slabs, z, mtiles, n_mtiles, tok, slot, token_start, token_list, (int)A, I, n_tiles,
                            n_pairs, y, ldy);
+        record(prof, 4, st);
         if (down->rank_identity)
             hipLaunchKernelGGL(k_combine_tokens<true>, dim3((unsigned)T), dim3(256), 0, st, down->d_fast_experts,
                                down->max_slabs, y, ldy, token_start, token_list, rw, rank_out, rank_accum);
@@ -1309,7 +1311,7 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
                                down->max_slabs, y, ldy, token_start, token_list, rw, rank_out, rank_accum);
         BITSMOE_HIP_TRY(hipGetLastError());
     }
-    record(prof, 3, st);
+    record(prof, 5, st);
     if (prof) prof->recorded = true;
     return BITSMOE_OK;
 }

@@ -202,9 +202,12 @@ int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bitsmoe_matset
  * one bitsmoe_moe_forward call (no reference counterpart: the reference has no
  * profiling hooks in the op).  After the stream has been synchronised,
  * bitsmoe_profile_read returns milliseconds for phase i:
- *   0 = zero-fill, 1 = gate+up kernels, 2 = down kernel(s).
+ *   0 = preparation (zero fill; grouped GEMM: activation conversion, tile and token lists),
+ *   1 = the gate/up kernel, 2 = the SiLU-and-multiply pass (its own launch only on the grouped
+ *   GEMM path, else 0), 3 = the down kernel, 4 = the per-token combine (its own launch only on
+ *   the grouped GEMM path, else 0).
  */
-#define BITSMOE_PROFILE_PHASES 3
+#define BITSMOE_PROFILE_PHASES 5
 int bitsmoe_profile_create(bitsmoe_profile** out);
 void bitsmoe_profile_destroy(bitsmoe_profile* p);
 int bitsmoe_profile_read(bitsmoe_profile* p, float ms[BITSMOE_PROFILE_PHASES]);
