@@ -111,11 +111,16 @@ constexpr int GRID_CHUNKS = 2;    // ... counts 16-assignment chunks (nth_chunk)
 // One (slab, tile) block restricted to one column-block pair: 2 column blocks x 2 k-steps,
 // plus the two MFMAs that accumulate the constant term.  The decoded registers hold
 // 2^W + code / f_i (staggered fields, wave_layout.h); the activations carry f_i.
-template <int W>
-__device__ __forceinline__ void gateup_pair(const uint32_t (&w)[4], u32x4 a0, u32x4 a1, int upper, f32x4 (&acc)[2], f32x4& corr) {
-    const u32x4 bc = offset0_regs<W>();
-    corr = mfma16<false>(a0, bc, corr);
-    corr = mfma16<false>(a1, bc, corr);
+// CONST_TERM == false leaves the constant term to the caller (the walking kernel sums it while it
+// stages the operand).
+template <int W, bool CONST_TERM = true>
+__device__ __forceinline__ void gateup_pair(const uint32_t (&w)[4], u32x4 a0, u32x4 a1, int upper, f32x4 (&acc)[2], f32x4& corr,
+                                            const Masks3* m3 = nullptr) {
+    if constexpr (CONST_TERM) {
+        const u32x4 bc = offset0_regs<W>();
+        corr = mfma16<false>(a0, bc, corr);
+        corr = mfma16<false>(a1, bc, corr);
+    }
 #pragma unroll
     for (int nbl = 0; nbl < 2; ++nbl) {
         u32x4 b0, b1;
@@ -125,6 +130,9 @@ __device__ __forceinline__ void gateup_pair(const uint32_t (&w)[4], u32x4 a0, u3
         } else if constexpr (W == 4) {
             b0 = decode0_fields4(w[2 * nbl]);
             b1 = decode0_fields4(w[2 * nbl + 1]);
+        } else if (m3) {
+            b0 = decode0_fields3(w[nbl], 0, w[2 + nbl], upper, *m3);
+            b1 = decode0_fields3(w[nbl], 1, w[2 + nbl], upper, *m3);
         } else {
             b0 = decode0_fields3(w[nbl], 0, w[2 + nbl], upper);
             b1 = decode0_fields3(w[nbl], 1, w[2 + nbl], upper);
@@ -417,6 +425,34 @@ __global__ __launch_bounds__(256, 4) void k_gateup_decode(
 // assignment, whatever its G / U rows hold.
 // The kernel also clears `zero_out` (the forward's accumulator, added into by the down kernel).
 // grid.x = (expert coordinate) * n_tiles, grid.y = 2 (gate, up); 256 threads = 4 wavefronts.
+// Sum of v over the 64 lanes, valid in lane 63 (the data-parallel-primitive moves of wave_inclusive_scan).
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ inline float dpp_add_f32(float v) {
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ inline float wave_sum_lane63(float v) {
+    v = dpp_add_f32<0x111>(v);
+    v = dpp_add_f32<0x112>(v);
+    v = dpp_add_f32<0x114>(v);
+    v = dpp_add_f32<0x118>(v);
+    v = dpp_add_f32<0x142, 0xa>(v);
+    v = dpp_add_f32<0x143, 0xc>(v);
+    return v;
+}
+// sum over a lane's eight staged operands of operand * (what offset0_regs holds for its register)
+template <int W>
+__device__ __forceinline__ float const_term_partial(u32x4 staged) {
+    typedef __fp16 h2v __attribute__((ext_vector_type(2)));
+    const u32x4 bc = offset0_regs<W>();
+    const uint32_t s0 = staged[0], s1 = staged[1], s2 = staged[2], s3 = staged[3];
+    const uint32_t c0 = bc[0], c1 = bc[1], c2 = bc[2], c3 = bc[3];
+    float p = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2v, s0), __builtin_bit_cast(h2v, c0), 0.0f, false);
+    p = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2v, s1), __builtin_bit_cast(h2v, c1), p, false);
+    p = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2v, s2), __builtin_bit_cast(h2v, c2), p, false);
+    p = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2v, s3), __builtin_bit_cast(h2v, c3), p, false);
+    return p;
+}
+
 template <bool BF16>
 __device__ __forceinline__ u32x4 scaled_f16x8(u32x4 raw, u32x4 sc) {
     u32x4 out;
@@ -433,6 +469,12 @@ __device__ __forceinline__ u32x4 scaled_f16x8(u32x4 raw, u32x4 sc) {
     return out;
 }
 
+#ifdef EXP_TIMING
+__device__ unsigned long long g_timing[8192 * 8];
+#define TSTAMP(i) do { if (tid == 0) g_timing[(((size_t)mt * gridDim.x + bid) & 8191) * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define TSTAMP(i) do {} while (0)
+#endif
 template <bool BF16, int MODE>
 __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
@@ -448,6 +490,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
         const int64_t total = (int64_t)gridDim.x * 2 * 256;
         for (int64_t i = ((int64_t)mt * gridDim.x + bid) * 256 + tid; i < zero_n; i += total) zero_out[i] = 0.0f;
     }
+    TSTAMP(0);
     const int t = bid % n_tiles;
     int e = bid / n_tiles;
     int chunk = -1;
@@ -479,6 +522,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const FastExpert fe = fe_tab[e];
     const FastSlab first = load_fast_slab(fs_tab, e * max_slabs);
     if (a_end <= a_begin || first.bits == 0) return;
+    TSTAMP(1);
     const int n_groups = max_slabs / GU_SLABS;
 
     gptr<uint32_t> payload = as_global(fe.payload);
@@ -492,10 +536,13 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
 
     // two copies of the operand, used in turn: one workgroup barrier per group instead of two
     __shared__ __attribute__((aligned(16))) uint16_t hs_all[2 * MAX_A * GU_STRIDE];
+    __shared__ float cterm_lds[MAX_A];
 
     auto body = [&](auto w_c) {
     constexpr int W = decltype(w_c)::value;
     const int slab_words = n_tiles * 256 * W;       // payload words from one slab to the next
+    Masks3 m3;
+    if constexpr (W == 3) m3 = masks3_role0();
     for (int a0 = a_begin; a0 < a_end; a0 += MAX_A) {
         const int n_a = min(MAX_A, a_end - a0);
         int chunk_zero = 0;
@@ -526,9 +573,20 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
         };
         auto act_at = [&](int i, int rank) { return *reinterpret_cast<const u32x4*>(trow[i] + rank); };
         uint16_t* hs = hs_all;
-        auto stage = [&](int i, u32x4 raw, u32x4 sc) {
-            *reinterpret_cast<u32x4*>(&hs[(pair + 4 * i) * GU_STRIDE + 8 * lane]) = scaled_f16x8<BF16>(raw, sc);
+        // The decoded weights are 2^W + code / f, the levels (code - 2^(W-1)) / f: the difference times
+        // the operand, summed over all rows, is the same for every column.  The wavefront that
+        // stages an assignment sums it on the way (lane 63 holds the wave's total).
+        float cterm[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        auto stage = [&](auto i_c, u32x4 raw, u32x4 sc) {
+            constexpr int i = decltype(i_c)::value;
+            const u32x4 v = scaled_f16x8<BF16>(raw, sc);
+            *reinterpret_cast<u32x4*>(&hs[(pair + 4 * i) * GU_STRIDE + 8 * lane]) = v;
+            cterm[i] += wave_sum_lane63(const_term_partial<W>(v));
         };
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        using I3 = std::integral_constant<int, 3>;
         int rank_cur = rank_at(0);
         int rank_nxt = n_groups > 1 ? rank_at(1) : 0;
         u32x4 sc_cur = scale_at(0);
@@ -548,11 +606,12 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
             // needs a barrier of its own before the first write.
             hs = hs_all + (g & 1) * (MAX_A * GU_STRIDE);
             if (g == 0) __syncthreads();
-            if (pair < n_a) stage(0, raw0, sc_cur);
-            if (pair + 4 < n_a) stage(1, raw1, sc_cur);
-            if (pair + 8 < n_a) stage(2, act_at(2, rank_cur), sc_cur);      // (rare: fetched here, not ahead)
-            if (pair + 12 < n_a) stage(3, act_at(3, rank_cur), sc_cur);
+            if (pair < n_a) stage(I0{}, raw0, sc_cur);
+            if (pair + 4 < n_a) stage(I1{}, raw1, sc_cur);
+            if (pair + 8 < n_a) stage(I2{}, act_at(2, rank_cur), sc_cur);      // (rare: fetched here, not ahead)
+            if (pair + 12 < n_a) stage(I3{}, act_at(3, rank_cur), sc_cur);
             __syncthreads();   // the operand is complete
+            if (g == 0) TSTAMP(2);
             if (more) {
                 if (pair < n_a) raw0 = act_at(0, rank_nxt);
                 if (pair + 4 < n_a) raw1 = act_at(1, rank_nxt);
@@ -562,13 +621,23 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
                 constexpr int q = decltype(qc)::value;
                 const u32x4 a_lo = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS);
                 const u32x4 a_hi = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS + 8);
-                gateup_pair<W>(pw[q], a_lo, a_hi, n >> 3, acc, corr);
+                gateup_pair<W, false>(pw[q], a_lo, a_hi, n >> 3, acc, corr, W == 3 ? &m3 : nullptr);
                 if (more) issue(qc, g + 1);
             }, std::make_integer_sequence<int, GU_SLABS>{});
             sc_cur = sc_nxt;
             rank_cur = rank_nxt;
             rank_nxt = rank_nxt2;
+            if (g == 0) TSTAMP(3);
         }
+        TSTAMP(4);
+        // the constant terms of the chunk's assignments, from the wavefronts that staged them
+        if (lane == 63) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) cterm_lds[pair + 4 * i] = cterm[i];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) corr[j] = cterm_lds[4 * kg + j];
         // remove the constant term; lane holds rows a = 4*kg + j of column 32*pair + 16*nbl + n
 #pragma unroll
         for (int nbl = 0; nbl < 2; ++nbl) {
@@ -588,7 +657,26 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
         body(std::integral_constant<int, 3>{});
     else if (first.bits == 4)
         body(std::integral_constant<int, 4>{});
+#ifdef EXP_TIMING
+    if (tid == 0) {
+        g_timing[(((size_t)mt * gridDim.x + bid) & 8191) * 8 + 5] = wall_clock64();
+        g_timing[(((size_t)mt * gridDim.x + bid) & 8191) * 8 + 6] = first.bits;
+        g_timing[(((size_t)mt * gridDim.x + bid) & 8191) * 8 + 7] = 1;
+    }
+#endif
 }
+#ifdef EXP_TIMING
+}  // namespace bitsmoe
+extern "C" void bitsmoe_debug_timing(unsigned long long* out, int reset) {
+    (void)hipDeviceSynchronize();
+    (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(bitsmoe::g_timing), sizeof(unsigned long long) * 8192 * 8);
+    if (reset) {
+        static unsigned long long zeros[8192 * 8];
+        (void)hipMemcpyToSymbol(HIP_SYMBOL(bitsmoe::g_timing), zeros, sizeof(zeros));
+    }
+}
+namespace bitsmoe {
+#endif
 
 // ----------------------------------------------------------------------------------- down
 // One (slab, tile) block of a down matrix: 4 row blocks x 4 k-steps (micro-tiles).

@@ -200,6 +200,39 @@ __device__ inline u32x4 decode0_fields3(uint32_t z, int ks, uint32_t hi, int upp
     for (int i = 0; i < 4; ++i) r[i] = (hh & ((1u << (9 - 2 * i)) * 0x10001u)) | r[i];
     return r;
 }
+// The same decode with the eight field masks held in scalar registers by the caller
+// (masks3_role0): gfx950's three-operand and-or takes no literal, and with literal masks the
+// compiler falls back to two ands and an or3 per register; with scalar masks it is one and-or
+// for the two low bits and one for the high bit.
+struct Masks3 {
+    uint32_t lo[4], hi[4];
+};
+__device__ __forceinline__ Masks3 masks3_role0() {
+    Masks3 m;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        m.lo[i] = (3u << (7 - 2 * i)) * 0x10001u;
+        m.hi[i] = (1u << (9 - 2 * i)) * 0x10001u;
+        asm volatile("" : "+s"(m.lo[i]));      // opaque: stays a scalar register, not a literal
+        asm volatile("" : "+s"(m.hi[i]));
+    }
+    return m;
+}
+__device__ __forceinline__ u32x4 decode0_fields3(uint32_t z, int ks, uint32_t hi, int upper, const Masks3& m) {
+    const uint32_t zz = ks ? rotr32(z, 8) : z;
+    const uint32_t hh = rotr32(hi, 8 * upper + ks);
+    const uint32_t magic = vreg(Codec<3, false>::MAGIC);
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        // (written out: from the C expression the compiler selects and + and + or3)
+        uint32_t low, both;
+        asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(low) : "v"(zz), "s"(m.lo[i]), "v"(magic));
+        asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(both) : "v"(hh), "s"(m.hi[i]), "v"(low));
+        r[i] = both;
+    }
+    return r;
+}
 // What has to be subtracted from the decoded registers to leave (code - 2^(W-1)) / f_i:
 // 2^W + 2^(W-1) / f_i as a packed f16 pair per register (mantissa 512 / f_i).
 template <int W>
