@@ -475,7 +475,7 @@ __device__ unsigned long long g_timing[8192 * 8];
 #else
 #define TSTAMP(i) do {} while (0)
 #endif
-template <bool BF16, int MODE>
+template <bool BF16, int MODE, bool IDENT>
 __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
     const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
@@ -554,19 +554,21 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
             constexpr int q = decltype(q_c)::value;
             load_pair_role0(payload + (uint32_t)(pack0 + (g * GU_SLABS + q) * slab_words), W, unit, hi_unit, pw[q]);
         };
-        static_for([&](auto qc) { issue(qc, 0); }, std::make_integer_sequence<int, GU_SLABS>{});
-
         // the rows of this wavefront's assignments pair, pair + 4, pair + 8, pair + 12 (wave-uniform)
         const uint16_t* trow[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int a = pair + 4 * i;
-            const int tk = a < n_a ? __builtin_amdgcn_readfirstlane(token_indices[a0 + a]) : 0;
+            // (index clamped instead of a branch: four scalar loads in flight together)
+            const int tk = __builtin_amdgcn_readfirstlane(token_indices[min(a0 + pair + 4 * i, A - 1)]);
             trow[i] = h + (int64_t)min(max(tk, 0), T - 1) * ld;
         }
         // rows 8*lane .. 8*lane + 7 of group g: first logical rank, the f16 bits of their eight
         // scale * s * stagger factor (folded once when the set was prepared), the activations
-        auto rank_at = [&](int g) { return rank_idx[first.rank_off + g * (GU_SLABS * SLAB_ROWS) + 8 * lane]; };
+        auto rank_at = [&](int g) {
+            const int k = first.rank_off + g * (GU_SLABS * SLAB_ROWS) + 8 * lane;
+            if constexpr (IDENT) return k;      // rank_idx[k] == k in every expert of both sets
+            else return (int)rank_idx[k];
+        };
         auto scale_at = [&](int g) {
             return *reinterpret_cast<gptr_u32x4>(
                 scale_s + (uint32_t)(first.scale_off + ((g * GU_SLABS + (lane >> 3)) * n_tiles + t) * SLAB_ROWS + 8 * (lane & 7)));
@@ -591,16 +593,24 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
         int rank_nxt = n_groups > 1 ? rank_at(1) : 0;
         u32x4 sc_cur = scale_at(0);
         u32x4 raw0 = {0, 0, 0, 0}, raw1 = {0, 0, 0, 0};
-        if (pair < n_a) raw0 = act_at(0, rank_cur);
-        if (pair + 4 < n_a) raw1 = act_at(1, rank_cur);
+        // (requested whether or not the assignments exist -- a row of token 0 otherwise -- so that
+        // the number of loads in flight does not depend on the path and the waits can be counted)
+        raw0 = act_at(0, rank_cur);
+        raw1 = act_at(1, rank_cur);
+        // The payload of the first group is requested only now: loads return in order, so anything
+        // requested behind it would be held back until it has arrived from HBM, and the first
+        // operand could not be staged in the meantime.
+        static_for([&](auto qc) { issue(qc, 0); }, std::make_integer_sequence<int, GU_SLABS>{});
         f32x4 acc[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
         f32x4 corr = {0, 0, 0, 0};
-        for (int g = 0; g < n_groups; ++g) {
-            const bool more = g + 1 < n_groups;
+        // (MORE: another group follows -- compiled twice, so that the eight blocks of a group are
+        // one straight run of code the compiler can schedule across)
+        auto group_step = [&](auto more_c, int g) {
+            constexpr bool more = decltype(more_c)::value;
             int rank_nxt2 = 0;
             if (g + 2 < n_groups) rank_nxt2 = rank_at(g + 2);
             u32x4 sc_nxt = {0, 0, 0, 0};
-            if (more) sc_nxt = scale_at(g + 1);
+            if constexpr (more) sc_nxt = scale_at(g + 1);
             // Group g writes copy g mod 2.  Its last readers (group g - 2) are done: every wavefront
             // passed the barrier of group g - 1 after its MFMAs of group g - 2.  Only a new chunk
             // needs a barrier of its own before the first write.
@@ -612,9 +622,9 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
             if (pair + 12 < n_a) stage(I3{}, act_at(3, rank_cur), sc_cur);
             __syncthreads();   // the operand is complete
             if (g == 0) TSTAMP(2);
-            if (more) {
-                if (pair < n_a) raw0 = act_at(0, rank_nxt);
-                if (pair + 4 < n_a) raw1 = act_at(1, rank_nxt);
+            if constexpr (more) {
+                raw0 = act_at(0, rank_nxt);
+                raw1 = act_at(1, rank_nxt);
             }
             const uint16_t* ap16 = &hs[n * GU_STRIDE + 16 * kg];
             static_for([&](auto qc) {
@@ -622,13 +632,15 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
                 const u32x4 a_lo = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS);
                 const u32x4 a_hi = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS + 8);
                 gateup_pair<W, false>(pw[q], a_lo, a_hi, n >> 3, acc, corr, W == 3 ? &m3 : nullptr);
-                if (more) issue(qc, g + 1);
+                if constexpr (more) issue(qc, g + 1);
             }, std::make_integer_sequence<int, GU_SLABS>{});
             sc_cur = sc_nxt;
             rank_cur = rank_nxt;
             rank_nxt = rank_nxt2;
             if (g == 0) TSTAMP(3);
-        }
+        };
+        for (int g = 0; g + 1 < n_groups; ++g) group_step(std::true_type{}, g);
+        group_step(std::false_type{}, n_groups - 1);
         TSTAMP(4);
         // the constant terms of the chunk's assignments, from the wavefronts that staged them
         if (lane == 63) {
@@ -982,7 +994,9 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
             fn(bf16_c, std::integral_constant<int, GRID_EXPERTS>{});
     };
     auto launch_walk_mode = [&](auto bf16_c, auto mode_c) {
-        hipLaunchKernelGGL((k_gateup_walk<decltype(bf16_c)::value, decltype(mode_c)::value>), dim3((unsigned)(e_dim * n_tiles), 2),
+        auto kern = k_gateup_walk<decltype(bf16_c)::value, decltype(mode_c)::value, false>;
+        if (gate->rank_identity && up->rank_identity) kern = k_gateup_walk<decltype(bf16_c)::value, decltype(mode_c)::value, true>;
+        hipLaunchKernelGGL(kern, dim3((unsigned)(e_dim * n_tiles), 2),
                            dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs, gate->max_slabs, up->d_fast_experts,
                            up->d_fast_slabs, up->max_slabs, (const uint16_t*)h_gate, (const uint16_t*)h_up, ldg, ldu,
                            tok, off, (int)T, (int)A, I, E, n_tiles, G, U, rank_accum, T * (int64_t)rank_out, gate_order,
