@@ -555,13 +555,11 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
             load_pair_role0(payload + (uint32_t)(pack0 + (g * GU_SLABS + q) * slab_words), W, unit, hi_unit, pw[q]);
         };
         // the rows of this wavefront's assignments pair, pair + 4, pair + 8, pair + 12 (wave-uniform)
-        const uint16_t* trow[4];
+        // (indices clamped instead of branches, and all four requested before the first is used:
+        // scalar loads in flight together)
+        int tki[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            // (index clamped instead of a branch: four scalar loads in flight together)
-            const int tk = __builtin_amdgcn_readfirstlane(token_indices[min(a0 + pair + 4 * i, A - 1)]);
-            trow[i] = h + (int64_t)min(max(tk, 0), T - 1) * ld;
-        }
+        for (int i = 0; i < 4; ++i) tki[i] = token_indices[min(a0 + pair + 4 * i, A - 1)];
         // rows 8*lane .. 8*lane + 7 of group g: first logical rank, the f16 bits of their eight
         // scale * s * stagger factor (folded once when the set was prepared), the activations
         auto rank_at = [&](int g) {
@@ -573,6 +571,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
             return *reinterpret_cast<gptr_u32x4>(
                 scale_s + (uint32_t)(first.scale_off + ((g * GU_SLABS + (lane >> 3)) * n_tiles + t) * SLAB_ROWS + 8 * (lane & 7)));
         };
+        const uint16_t* trow[4];
         auto act_at = [&](int i, int rank) { return *reinterpret_cast<const u32x4*>(trow[i] + rank); };
         uint16_t* hs = hs_all;
         // The decoded weights are 2^W + code / f, the levels (code - 2^(W-1)) / f: the difference times
@@ -592,6 +591,9 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
         int rank_cur = rank_at(0);
         int rank_nxt = n_groups > 1 ? rank_at(1) : 0;
         u32x4 sc_cur = scale_at(0);
+        // (the token indices are first used here, behind the requests that do not depend on them)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) trow[i] = h + (int64_t)min(max(__builtin_amdgcn_readfirstlane(tki[i]), 0), T - 1) * ld;
         u32x4 raw0 = {0, 0, 0, 0}, raw1 = {0, 0, 0, 0};
         // (requested whether or not the assignments exist -- a row of token 0 otherwise -- so that
         // the number of loads in flight does not depend on the path and the waits can be counted)
