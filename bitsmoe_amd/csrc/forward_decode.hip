@@ -27,14 +27,7 @@ namespace bitsmoe {
 constexpr int GU_STRIDE = GU_SLABS * SLAB_ROWS + 8;  // 16-bit elements; +8 staggers LDS banks
 constexpr int DN_SLABS_PER_WG = 4;                 // one slab per wavefront
 constexpr int MAX_A = 16;                          // assignments per MFMA pass
-constexpr int64_t WALK_MIN_WGS = 512;              // walking gate/up kernel: fewest (expert, projection, tile) units
-
-template <int W>
-__device__ inline u32x4 corr_operand() {
-    const uint32_t c = Codec<W, false>::CORR;
-    u32x4 r = {c, c, c, c};
-    return r;
-}
+constexpr int ZSUM_STRIDE = 16;                    // tiles per assignment row of the down kernel's z sums (I <= 1920)
 
 // With few assignments most experts are idle; launching a workgroup per (expert, ...) then
 // costs more than the work.  The kernels can instead be launched over `slots` and let every
@@ -694,12 +687,11 @@ namespace bitsmoe {
 
 // ----------------------------------------------------------------------------------- down
 // One (slab, tile) block of a down matrix: 4 row blocks x 4 k-steps (micro-tiles).
+// `corr`: 1.5 * 2^W times the sum of the tile's z over its 128 columns, per assignment row of the
+// lane (the constant term of the decoded operands 2^W + code; the z rows are summed once, when z
+// is built, instead of by four more MFMAs per block).
 template <int W>
-__device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4], const float (&sc)[4], f32x4 (&acc)[4]) {
-    const u32x4 bc = corr_operand<W>();
-    f32x4 corr = {0, 0, 0, 0};
-#pragma unroll
-    for (int m = 0; m < 4; ++m) corr = mfma16<false>(az[m], bc, corr);
+__device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4], const float (&sc)[4], f32x4 corr, f32x4 (&acc)[4]) {
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) {
         f32x4 t = {0, 0, 0, 0};
@@ -728,7 +720,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                                  const FastSlab fs, const float* __restrict__ G, const float* __restrict__ U,
                                  const float* __restrict__ route_w, const int32_t* __restrict__ token_indices,
                                  int a_begin, int a_end, int T, int I, int tb, int nt, int rank_out,
-                                 float* __restrict__ rank_accum, uint16_t* __restrict__ z, int z_stride, int tid, int lane) {
+                                 float* __restrict__ rank_accum, uint16_t* __restrict__ z, int z_stride, float* __restrict__ zsum, int tid, int lane) {
     const int n = lane & 15, kg = lane >> 4, g4 = kg * 4;
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
@@ -758,7 +750,10 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
             const uint16_t* zp = z + n * z_stride + (tb + i) * N_TILE + 8 * kg;
 #pragma unroll
             for (int m = 0; m < 4; ++m) az[m] = *reinterpret_cast<const u32x4*>(zp + 32 * m);
-            down_block<WL>(buf[B], az, sc[B], acc);
+            f32x4 corr;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) corr[j] = zsum[(g4 + j) * ZSUM_STRIDE + tb + i] * (1.5f * (float)(1 << WL));
+            down_block<WL>(buf[B], az, sc[B], corr, acc);
         };
         int lr[4];
         float sv[4];
@@ -793,12 +788,25 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     if (ab + j < n_a) {
+                        uint16_t zb[4];
+                        float part = 0.0f;      // sum of the four operands as rounded
+#pragma unroll
+                        for (int x = 0; x < 4; ++x) {
+                            zb[x] = to_operand<false>(silu_f32(gv[j][x]) * uv[j][x]);
+                            part += __half2float(__ushort_as_half(zb[x]));
+                        }
                         u32x2 packed;
-                        packed[0] = (uint32_t)to_operand<false>(silu_f32(gv[j][0]) * uv[j][0]) |
-                                    ((uint32_t)to_operand<false>(silu_f32(gv[j][1]) * uv[j][1]) << 16);
-                        packed[1] = (uint32_t)to_operand<false>(silu_f32(gv[j][2]) * uv[j][2]) |
-                                    ((uint32_t)to_operand<false>(silu_f32(gv[j][3]) * uv[j][3]) << 16);
+                        packed[0] = (uint32_t)zb[0] | ((uint32_t)zb[1] << 16);
+                        packed[1] = (uint32_t)zb[2] | ((uint32_t)zb[3] << 16);
                         *reinterpret_cast<u32x2*>(z + (ab + j) * z_stride + c) = packed;
+                        // the 32 lanes of a half wavefront hold one tile's 128 columns: their sum
+                        // arrives in lanes 31 and 63 (whole rows of 16 lanes are active or not)
+                        part = dpp_add_f32<0x111>(part);
+                        part = dpp_add_f32<0x112>(part);
+                        part = dpp_add_f32<0x114>(part);
+                        part = dpp_add_f32<0x118>(part);
+                        part = dpp_add_f32<0x142, 0xa>(part);
+                        if ((lane & 31) == 31) zsum[(ab + j) * ZSUM_STRIDE + c / N_TILE] = part;
                     }
                 }
             }
@@ -887,21 +895,22 @@ __global__ __launch_bounds__(256) void k_down_decode(
     extern __shared__ __attribute__((aligned(16))) unsigned char dsmem[];
     uint16_t* z = reinterpret_cast<uint16_t*>(dsmem);
     const int z_stride = n_tiles * N_TILE + 8;
+    float* zsum = reinterpret_cast<float*>(dsmem + (size_t)MAX_A * z_stride * 2);      // [assignment][tile]
 
     // the four wavefronts may run four different instantiations; every one of them executes
     // the same two workgroup barriers per assignment chunk
     if (fs.bits == 2)
         down_wave<2>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
-                           rank_out, rank_accum, z, z_stride, tid, lane);
+                           rank_out, rank_accum, z, z_stride, zsum, tid, lane);
     else if (fs.bits == 3)
         down_wave<3>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
-                           rank_out, rank_accum, z, z_stride, tid, lane);
+                           rank_out, rank_accum, z, z_stride, zsum, tid, lane);
     else if (fs.bits == 4)
         down_wave<4>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
-                           rank_out, rank_accum, z, z_stride, tid, lane);
+                           rank_out, rank_accum, z, z_stride, zsum, tid, lane);
     else
         down_wave<0>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
-                           rank_out, rank_accum, z, z_stride, tid, lane);
+                           rank_out, rank_accum, z, z_stride, zsum, tid, lane);
 }
 
 __global__ void k_fill_zero2(float* __restrict__ p1, int64_t n1, float* __restrict__ p2, int64_t n2) {
@@ -917,8 +926,8 @@ static inline void record(bitsmoe_profile* p, int i, hipStream_t st) {
 
 bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I) {
     const int n_tiles = (I + N_TILE - 1) / N_TILE;
-    const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2;
-    return gate->role == ROLE_GATE_UP && up->role == ROLE_GATE_UP && down->role == ROLE_DOWN && z_bytes <= 65536 &&
+    const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4;
+    return n_tiles <= ZSUM_STRIDE && gate->role == ROLE_GATE_UP && up->role == ROLE_GATE_UP && down->role == ROLE_DOWN && z_bytes <= 65536 &&
            I % N_TILE == 0;
 }
 
@@ -947,7 +956,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     // (its 16-byte activation loads also need rank_idx in runs of eight and aligned rows)
     auto rows16 = [](const void* p, int64_t ld) { return ((uintptr_t)p & 15) == 0 && ld % 8 == 0; };
     const bool walk = gate->all_affine && up->all_affine && gate->rank_chunked8 && up->rank_chunked8 &&
-                   rows16(h_gate, ldg) && rows16(h_up, ldu) && units * 2 * n_tiles >= WALK_MIN_WGS;
+                   rows16(h_gate, ldg) && rows16(h_up, ldu);
     if (!walk) {
         // G and U are adjacent in the workspace: one range; rank_accum is the second
         const int64_t n1 = inter_floats + A * (int64_t)I;
@@ -1018,7 +1027,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     record(prof, 2, st);
     record(prof, 3, st);      // (SiLU happens inside the down kernel)
     const int dn_groups = (down->max_slabs + DN_SLABS_PER_WG - 1) / DN_SLABS_PER_WG;
-    const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2;
+    const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4;
     int dn_tiles_per_wg = n_tiles;
     while (dn_tiles_per_wg > 1 && units * dn_groups * ((n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg) < 384)
         dn_tiles_per_wg = (dn_tiles_per_wg + 1) / 2;
