@@ -27,6 +27,7 @@ namespace bitsmoe {
 constexpr int GU_STRIDE = GU_SLABS * SLAB_ROWS + 8;  // 16-bit elements; +8 staggers LDS banks
 constexpr int DN_SLABS_PER_WG = 4;                 // one slab per wavefront
 constexpr int MAX_A = 16;                          // assignments per MFMA pass
+constexpr int ZROWS = 2;                           // assignment rows of G / U the down kernel's z build fetches together
 constexpr int ZSUM_STRIDE = 16;                    // tiles per assignment row of the down kernel's z sums (I <= 1920)
 
 // With few assignments most experts are idle; launching a workgroup per (expert, ...) then
@@ -462,12 +463,6 @@ __device__ __forceinline__ u32x4 scaled_f16x8(u32x4 raw, u32x4 sc) {
     return out;
 }
 
-#ifdef EXP_TIMING
-__device__ unsigned long long g_timing[8192 * 8];
-#define TSTAMP(i) do { if (tid == 0) g_timing[(((size_t)mt * gridDim.x + bid) & 8191) * 8 + (i)] = wall_clock64(); } while (0)
-#else
-#define TSTAMP(i) do {} while (0)
-#endif
 template <bool BF16, int MODE, bool IDENT>
 __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
@@ -483,7 +478,6 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
         const int64_t total = (int64_t)gridDim.x * 2 * 256;
         for (int64_t i = ((int64_t)mt * gridDim.x + bid) * 256 + tid; i < zero_n; i += total) zero_out[i] = 0.0f;
     }
-    TSTAMP(0);
     const int t = bid % n_tiles;
     int e = bid / n_tiles;
     int chunk = -1;
@@ -515,7 +509,6 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const FastExpert fe = fe_tab[e];
     const FastSlab first = load_fast_slab(fs_tab, e * max_slabs);
     if (a_end <= a_begin || first.bits == 0) return;
-    TSTAMP(1);
     const int n_groups = max_slabs / GU_SLABS;
 
     gptr<uint32_t> payload = as_global(fe.payload);
@@ -616,7 +609,6 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
             if (pair + 8 < n_a) stage(I2{}, act_at(2, rank_cur), sc_cur);      // (rare: fetched here, not ahead)
             if (pair + 12 < n_a) stage(I3{}, act_at(3, rank_cur), sc_cur);
             __syncthreads();   // the operand is complete
-            if (g == 0) TSTAMP(2);
             if constexpr (more) {
                 raw0 = act_at(0, rank_nxt);
                 raw1 = act_at(1, rank_nxt);
@@ -632,11 +624,9 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
             sc_cur = sc_nxt;
             rank_cur = rank_nxt;
             rank_nxt = rank_nxt2;
-            if (g == 0) TSTAMP(3);
         };
         for (int g = 0; g + 1 < n_groups; ++g) group_step(std::true_type{}, g);
         group_step(std::false_type{}, n_groups - 1);
-        TSTAMP(4);
         // the constant terms of the chunk's assignments, from the wavefronts that staged them
         if (lane == 63) {
 #pragma unroll
@@ -664,26 +654,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
         body(std::integral_constant<int, 3>{});
     else if (first.bits == 4)
         body(std::integral_constant<int, 4>{});
-#ifdef EXP_TIMING
-    if (tid == 0) {
-        g_timing[(((size_t)mt * gridDim.x + bid) & 8191) * 8 + 5] = wall_clock64();
-        g_timing[(((size_t)mt * gridDim.x + bid) & 8191) * 8 + 6] = first.bits;
-        g_timing[(((size_t)mt * gridDim.x + bid) & 8191) * 8 + 7] = 1;
-    }
-#endif
 }
-#ifdef EXP_TIMING
-}  // namespace bitsmoe
-extern "C" void bitsmoe_debug_timing(unsigned long long* out, int reset) {
-    (void)hipDeviceSynchronize();
-    (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(bitsmoe::g_timing), sizeof(unsigned long long) * 8192 * 8);
-    if (reset) {
-        static unsigned long long zeros[8192 * 8];
-        (void)hipMemcpyToSymbol(HIP_SYMBOL(bitsmoe::g_timing), zeros, sizeof(zeros));
-    }
-}
-namespace bitsmoe {
-#endif
 
 // ----------------------------------------------------------------------------------- down
 // One (slab, tile) block of a down matrix: 4 row blocks x 4 k-steps (micro-tiles).
@@ -714,13 +685,18 @@ __device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4
 // per bit-width of the wavefront's slab (W == 0: no slab, the wavefront only helps to build z).
 // The payload of the first two tiles is requested BEFORE z is built, so that the weights
 // are in flight while G and U are read and SiLU is evaluated; afterwards the tiles stream
-// through three register buffers, two tiles ahead of the one being computed.
+// through three register buffers, two tiles ahead of the one being computed (4-bit slabs, 16
+// registers per tile: two buffers, one tile ahead).  The register budget is 128, so that all four
+// workgroups of a CU -- on the 64-token benchmark layer the whole grid -- are resident at once:
+// what only the epilogue needs (rank and multiplier of the rows, token and weight of the
+// assignments) waits in LDS, and z is built two assignment rows at a time.
 template <int W>
 __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gptr<__half> svec, gptr<int32_t> rank_idx,
                                  const FastSlab fs, const float* __restrict__ G, const float* __restrict__ U,
                                  const float* __restrict__ route_w, const int32_t* __restrict__ token_indices,
                                  int a_begin, int a_end, int T, int I, int tb, int nt, int rank_out,
-                                 float* __restrict__ rank_accum, uint16_t* __restrict__ z, int z_stride, float* __restrict__ zsum, int tid, int lane) {
+                                 float* __restrict__ rank_accum, uint16_t* __restrict__ z, int z_stride, float* __restrict__ zsum,
+                                 int2* __restrict__ rows, int2* __restrict__ assigns, int tid, int lane) {
     const int n = lane & 15, kg = lane >> 4, g4 = kg * 4;
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
@@ -755,38 +731,36 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
             for (int j = 0; j < 4; ++j) corr[j] = zsum[(g4 + j) * ZSUM_STRIDE + tb + i] * (1.5f * (float)(1 << WL));
             down_block<WL>(buf[B], az, sc[B], corr, acc);
         };
-        int lr[4];
-        float sv[4];
+        // logical rank and multiplier of the slab's row `lane`: needed by the epilogue only, kept
+        // in LDS until then (one wavefront's own 64 entries: no barrier involved)
+        int row_rank = -1;
+        float row_s = 0.0f;
         if constexpr (W != 0) {
             issue(I0{}, 0);
             if (nt > 1) issue(I1{}, 1);
-            // logical rank and multiplier of this lane's four output rows (needed by the epilogue)
-#pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
-                const int row = fs.rank_off + 16 * nb + n;
-                lr[nb] = rank_idx[row];
-                sv[nb] = gload_half(svec + row);
-            }
+            row_rank = rank_idx[fs.rank_off + lane];
+            row_s = gload_half(svec + fs.rank_off + lane);
         }
-        // token ids and routing weights of the chunk (lane a holds assignment a)
+        // token ids and routing weights of the chunk (lane a holds assignment a): for the epilogue,
+        // kept in LDS until then (every wavefront writes the same sixteen entries)
         const int tok_lane = (lane < n_a) ? token_indices[a0 + lane] : -1;
         const float rw_lane = (lane < n_a) ? route_w[a0 + lane] : 0.0f;
         __syncthreads();   // the previous chunk is done with z
         // z[a][c] = silu(G) * U as 16-bit operands for the rows a < n_a (other rows feed
         // output rows that are never stored).  Each thread owns four neighbouring columns
-        // and walks the assignments four at a time, all eight vector loads issued together.
+        // and walks the assignments ZROWS at a time, their vector loads issued together.
         for (int c = tb * N_TILE + tid * 4; c < min((tb + nt) * N_TILE, I); c += 1024) {
-            for (int ab = 0; ab < n_a; ab += 4) {
-                f32x4 gv[4], uv[4];
+            for (int ab = 0; ab < n_a; ab += ZROWS) {
+                f32x4 gv[ZROWS], uv[ZROWS];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
+                for (int j = 0; j < ZROWS; ++j) {
                     const int a = min(ab + j, n_a - 1);
                     const int64_t gi = (int64_t)(a0 + a) * I + c;
                     gv[j] = *reinterpret_cast<const f32x4*>(G + gi);
                     uv[j] = *reinterpret_cast<const f32x4*>(U + gi);
                 }
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
+                for (int j = 0; j < ZROWS; ++j) {
                     if (ab + j < n_a) {
                         uint16_t zb[4];
                         float part = 0.0f;      // sum of the four operands as rounded
@@ -811,8 +785,20 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                 }
             }
         }
+        if constexpr (W != 0) rows[lane] = int2{row_rank, __float_as_int(row_s)};
+        if (lane < MAX_A) assigns[lane] = int2{tok_lane, __float_as_int(rw_lane)};
         __syncthreads();
-        if constexpr (W != 0) {
+        if constexpr (W == 4) {
+            // (16 payload registers per tile: two buffers, one tile ahead)
+            for (int i = 0; i < nt; i += 2) {
+                compute(I0{}, i);
+                if (i + 1 < nt) {
+                    if (i + 2 < nt) issue(I0{}, i + 2);
+                    compute(I1{}, i + 1);
+                    if (i + 3 < nt) issue(I1{}, i + 3);
+                }
+            }
+        } else if constexpr (W != 0) {
             for (int i = 0; i < nt; i += 3) {
                 if (i + 2 < nt) issue(I2{}, i + 2);
                 compute(I0{}, i);
@@ -825,27 +811,34 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                     compute(I2{}, i + 2);
                 }
             }
+        }
+        if constexpr (W != 0) {
             // combine: rows of this slab are distinct output ranks; lane holds assignments 4*kg + j
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) {
+                const int2 rs = rows[16 * nb + n];
+                const int lr = rs.x;
+                const float sv = __int_as_float(rs.y);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int a = g4 + j;
-                    const int tk = __shfl(tok_lane, a);
-                    const float rw = __shfl(rw_lane, a);
-                    if (lr[nb] >= 0 && lr[nb] < rank_out && a < n_a && tk >= 0 && tk < T)
-                        atomicAdd(&rank_accum[(int64_t)tk * rank_out + lr[nb]], acc[nb][j] * sv[nb] * rw);
+                    const int2 tr = assigns[a];
+                    const int tk = tr.x;
+                    const float rw = __int_as_float(tr.y);
+                    if (lr >= 0 && lr < rank_out && a < n_a && tk >= 0 && tk < T)
+                        atomicAdd(&rank_accum[(int64_t)tk * rank_out + lr], acc[nb][j] * sv * rw);
                 }
             }
         }
     }
 }
 
-// grid.x = E * n_groups * n_tchunks; 256 threads; dynamic LDS = 16 * (n_tiles * 128 + 8) * 2 bytes.
+// grid.x = E * n_groups * n_tchunks; 256 threads; dynamic LDS = z (16 * (n_tiles * 128 + 8) * 2 bytes), the
+// per-tile sums of its rows, the epilogue's row and assignment records.
 // A workgroup takes four slabs of one expert and a run of tiles; with few active experts the
 // tiles are split over several workgroups (their partial sums meet in the atomics of the combine).
 template <int MODE>
-__global__ __launch_bounds__(256) void k_down_decode(
+__global__ __launch_bounds__(256, 4) void k_down_decode(
     const FastExpert* __restrict__ down_fe, const FastSlab* __restrict__ down_fs, int max_slabs,
     const float* __restrict__ G, const float* __restrict__ U, const float* __restrict__ route_w,
     const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
@@ -891,26 +884,27 @@ __global__ __launch_bounds__(256) void k_down_decode(
     gptr<__half> scale = as_global(fe.scale);
     gptr<__half> svec = as_global(fe.s);
     gptr<int32_t> rank_idx = as_global(fe.rank_idx);
-
     extern __shared__ __attribute__((aligned(16))) unsigned char dsmem[];
     uint16_t* z = reinterpret_cast<uint16_t*>(dsmem);
     const int z_stride = n_tiles * N_TILE + 8;
     float* zsum = reinterpret_cast<float*>(dsmem + (size_t)MAX_A * z_stride * 2);      // [assignment][tile]
+    int2* rows = reinterpret_cast<int2*>(zsum + MAX_A * ZSUM_STRIDE) + wave * SLAB_ROWS;     // this wavefront's (rank, multiplier) per row
+    int2* assigns = reinterpret_cast<int2*>(zsum + MAX_A * ZSUM_STRIDE) + DN_SLABS_PER_WG * SLAB_ROWS;    // (token, routing weight) per assignment
 
     // the four wavefronts may run four different instantiations; every one of them executes
     // the same two workgroup barriers per assignment chunk
     if (fs.bits == 2)
         down_wave<2>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
-                           rank_out, rank_accum, z, z_stride, zsum, tid, lane);
+                           rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else if (fs.bits == 3)
         down_wave<3>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
-                           rank_out, rank_accum, z, z_stride, zsum, tid, lane);
+                           rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else if (fs.bits == 4)
         down_wave<4>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
-                           rank_out, rank_accum, z, z_stride, zsum, tid, lane);
+                           rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else
         down_wave<0>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
-                           rank_out, rank_accum, z, z_stride, zsum, tid, lane);
+                           rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
 }
 
 __global__ void k_fill_zero2(float* __restrict__ p1, int64_t n1, float* __restrict__ p2, int64_t n2) {
@@ -926,7 +920,7 @@ static inline void record(bitsmoe_profile* p, int i, hipStream_t st) {
 
 bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I) {
     const int n_tiles = (I + N_TILE - 1) / N_TILE;
-    const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4;
+    const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4 + DN_SLABS_PER_WG * SLAB_ROWS * 8 + MAX_A * 8;
     return n_tiles <= ZSUM_STRIDE && gate->role == ROLE_GATE_UP && up->role == ROLE_GATE_UP && down->role == ROLE_DOWN && z_bytes <= 65536 &&
            I % N_TILE == 0;
 }
@@ -1027,7 +1021,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     record(prof, 2, st);
     record(prof, 3, st);      // (SiLU happens inside the down kernel)
     const int dn_groups = (down->max_slabs + DN_SLABS_PER_WG - 1) / DN_SLABS_PER_WG;
-    const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4;
+    const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4 + DN_SLABS_PER_WG * SLAB_ROWS * 8 + MAX_A * 8;
     int dn_tiles_per_wg = n_tiles;
     while (dn_tiles_per_wg > 1 && units * dn_groups * ((n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg) < 384)
         dn_tiles_per_wg = (dn_tiles_per_wg + 1) / 2;
