@@ -212,8 +212,8 @@ def run_workload(block, spec, tokens, steps, warmup, seed=42, use_graph=True):
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE,
 # each scaled by what it reads for a 256 MiB copy); collected offline with rocprofv3 --pmc on
 # this same script (profiles/*_hbm_traffic_counters.txt), None where not collected.
-HBM_TRAFFIC_BYTES = {"c2-t64": int((58445.4 * 2.0 + 18742.4) * 1024),        # k_gateup_decode
-                     "c3-t4096": int((268721.1 * 2.0 + 98304.0) * 1024)}     # k_gateup_mfma
+HBM_TRAFFIC_BYTES = {"c2-t64": int((59366.5 * 2.0 + 3584.0) * 1024),         # k_gateup_walk
+                     "c3-t4096": int((268522.9 * 2.0 + 98304.0) * 1024)}     # k_gateup_mfma
 
 
 def roofline_of(res, inputs, bound, workload=None):
