@@ -1023,7 +1023,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     const int dn_groups = (down->max_slabs + DN_SLABS_PER_WG - 1) / DN_SLABS_PER_WG;
     const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4 + DN_SLABS_PER_WG * SLAB_ROWS * 8 + MAX_A * 8;
     int dn_tiles_per_wg = n_tiles;
-    while (dn_tiles_per_wg > 1 && units * dn_groups * ((n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg) < 384)
+    while (dn_tiles_per_wg > 1 && units * dn_groups * ((n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg) < 600)
         dn_tiles_per_wg = (dn_tiles_per_wg + 1) / 2;
     const int dn_tchunks = (n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg;
     auto launch_down = [&](auto kernel) {
