@@ -276,8 +276,8 @@ def cpu_baseline(block, inputs, tokens, budget_s=12.0):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=400)      # (the closing synchronize costs as much as several steps)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c2-t64", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extras", action="store_true", help="measure the primary workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
