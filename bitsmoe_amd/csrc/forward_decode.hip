@@ -2,7 +2,10 @@
 // prepared payload, field decode in registers, 16x16x32 MFMA against up to 16 assignments
 // of one expert.  See wave_layout.h for the layout and the (2^w + code) operand trick.
 //
-//   k_gateup_decode   G[a,c] / U[a,c] += sum_k  hs'[a,k] * level[k,c]
+//   k_gateup_walk     G[a,c] / U[a,c]  = sum_k  hs'[a,k] * level[k,c]   (one workgroup per expert,
+//                     projection and 128-column tile over all rows k: plain stores; the default)
+//   k_gateup_decode   G[a,c] / U[a,c] += sum_k  hs'[a,k] * level[k,c]   (split over groups of 512 rows,
+//                     fp32 atomics into cleared outputs: sets the walking kernel cannot take)
 //                     hs'[a,k] = h[tok_a, rank_idx[k]] * s[k] * scale[tile(c), k]  (f16 operand,
 //                     times the power of two by which the staggered field decode shrinks the code)
 //   k_down_decode     rank_accum[tok_a, rank_idx[r]] += route_w[a] * s[r] *
@@ -12,11 +15,12 @@
 // MFMA operands: A = activations (row index = assignment), B = weights (column index =
 // output column / output rank row); D[4*(lane/16)+j][lane%16].
 //
-// Both kernels are latency-engineered rather than compute-engineered: one memory round
+// The kernels are latency-engineered rather than compute-engineered: one memory round
 // trip costs 1-2 us on a loaded MI355X, so (1) all metadata a workgroup needs is
 // addressable from its block index (FastExpert / FastSlab tables: one round trip, not a
-// chain of five), (2) every workgroup walks several tiles and keeps the payload of the next
-// tile in flight while it computes the current one.
+// chain of five), (2) every workgroup keeps the payload of its next step in flight while it
+// computes the current one, (3) requests are ordered by when their data is needed: loads
+// return in order, so a small request behind a large one waits for the large one.
 #include <type_traits>
 #include <utility>
 
