@@ -13,6 +13,7 @@ bitsmoe/algorithms/cpp/mlp_forward.cu:2464-2503), `route`, `dequant_matrix`.
 from __future__ import annotations
 
 import ctypes
+from collections import OrderedDict
 from typing import List, Optional, Sequence, Tuple
 
 import torch
@@ -50,6 +51,9 @@ class MatrixSet:
                           (scale, "scale"), (s, "s")):
             _check(len(lst) == n, f"{name}: {what} list length {len(lst)} != {n}")
         self._keep = (tuple(payload), tuple(rank_idx), tuple(tile_meta), tuple(slab_meta), tuple(scale), tuple(s))
+        self._keep_lists = self._keep
+        self._name = name
+        self._fingerprint = fingerprint(self._keep)
         self.n_experts = n
         self.intermediate_size = int(intermediate_size)
         self.device = payload[0].device if n else torch.device("cuda", torch.cuda.current_device())
@@ -101,6 +105,19 @@ class MatrixSet:
             _capi.check(_lib.bitsmoe_matset_prepare(self._handle, int(role), _stream_ptr(self.device)))
         self.role = int(role)
         return True
+
+    def is_current(self) -> bool:
+        """False once any buffer the set was built from has been written in place since (the set
+        is a snapshot: validated metadata, prepared payload copy, folded scales)."""
+        return self._fingerprint == fingerprint(self._keep)
+
+    def refresh(self) -> None:
+        """Rebuild the snapshot from the buffers' current contents (same tensors, same role)."""
+        role = self.role
+        self.close()
+        self.__init__(*self._keep, intermediate_size=self.intermediate_size, name=self._name)
+        if role >= 0:
+            self.prepare(role)
 
     def dequant_prepared(self, expert: int) -> torch.Tensor:
         """Dense fp32 matrix decoded from the prepared (wave-native) copy."""
@@ -158,44 +175,47 @@ class Profile:
 # ----------------------------------------------------------------------------------------
 # matrix-set cache for the list-based reference signature
 # ----------------------------------------------------------------------------------------
-_SET_CACHE: List[Tuple[tuple, MatrixSet]] = []
-_SET_BY_ADDRESS = {}
-_SET_CACHE_LIMIT = 4096
+# A MatrixSet is a SNAPSHOT of the caller's buffers: creation validates and caches the metadata,
+# prepare() makes a re-laid-out copy of the payload and a folded scale table.  The reference keeps
+# only meta tables per raw pointer and reads the payload live
+# (bitsmoe/algorithms/cpp/mlp_forward.cu:2464-2503, 2608-2619), so a caller of the list signature
+# may overwrite or swap buffers between calls.  The cache key therefore holds the address, size and
+# version counter of EVERY tensor of EVERY expert: a swapped middle expert or an in-place write
+# (`copy_`, `load_state_dict` on a child module) misses the cache and builds a fresh set.
+_SET_CACHE: "OrderedDict[tuple, MatrixSet]" = OrderedDict()
+_SET_CACHE_LIMIT = int(os.environ.get("BITSMOE_SET_CACHE_LIMIT", "384"))     # sets kept (each pins its GPU copy)
 
 
 def clear_matset_cache() -> None:
+    for ms in _SET_CACHE.values():
+        ms.close()
     _SET_CACHE.clear()
-    _SET_BY_ADDRESS.clear()
 
 
-def _address_key(lists: tuple, intermediate_size: int) -> tuple:
-    """Addresses and sizes of the six buffers of the first and the last expert: what identifies a
-    set when the sequences arrive as fresh list objects (calls through the dispatcher)."""
-    n = len(lists[0])
-    ends = (0, n - 1) if n > 1 else (0,)
-    return (n, int(intermediate_size)) + tuple((seq[i].data_ptr(), seq[i].numel()) for i in ends for seq in lists)
+def fingerprint(lists: Sequence[Sequence[torch.Tensor]]) -> tuple:
+    """(address, element count, version counter) of every tensor of the six buffer lists."""
+    return tuple((t.data_ptr(), t.numel(), t._version) for seq in lists for t in seq)
 
 
 def _lookup_set(lists: tuple, intermediate_size: int, name: str) -> MatrixSet:
-    # Fast path: the caller passes the same tuple objects every call (the host block keeps
-    # them in its runtime cache), so identity of the six sequences decides.
-    for key, ms in _SET_CACHE:
-        if all(a is b for a, b in zip(key, lists)) and ms.intermediate_size == intermediate_size:
-            return ms
-    akey = _address_key(lists, intermediate_size) if len(lists[0]) else None
-    ms = _SET_BY_ADDRESS.get(akey) if akey is not None else None
+    key = (len(lists[0]), int(intermediate_size), fingerprint(lists))
+    ms = _SET_CACHE.get(key)
     if ms is not None:
+        _SET_CACHE.move_to_end(key)
         return ms
+    # a set built from the same list objects or the same first payload address whose key no longer
+    # matches is stale (its buffers were overwritten or swapped): release its GPU copy now
+    for old_key, old in list(_SET_CACHE.items()):
+        if all(a is b for a, b in zip(old._keep_lists, lists)) or (
+                len(lists[0]) and old.n_experts and old._keep[0][0].data_ptr() == lists[0][0].data_ptr()):
+            old.close()
+            del _SET_CACHE[old_key]
     ms = MatrixSet(*lists, intermediate_size=intermediate_size, name=name)
-    if len(_SET_CACHE) >= _SET_CACHE_LIMIT:
-        dropped = _SET_CACHE.pop(0)[1]
-        for k in [k for k, v in _SET_BY_ADDRESS.items() if v is dropped]:
-            del _SET_BY_ADDRESS[k]
-    # the cache holds the sequences themselves, so neither their ids nor the buffer addresses
-    # can be recycled while the entry lives
-    _SET_CACHE.append((lists, ms))
-    if akey is not None:
-        _SET_BY_ADDRESS[akey] = ms
+    ms._keep_lists = lists
+    while len(_SET_CACHE) >= max(_SET_CACHE_LIMIT, 1):
+        _SET_CACHE.popitem(last=False)[1].close()
+    # the set holds the tensors themselves, so no address of the key can be recycled while it lives
+    _SET_CACHE[key] = ms
     return ms
 
 

@@ -142,6 +142,11 @@ __global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict
         part += pr[i];
     }
     const float denom = wave_sum(part);
+    // the other lanes' keys are read below: order the LDS writes above before those reads whatever
+    // the compiler's schedule (one wavefront: a wave-scope fence and a wave barrier, no s_barrier)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     int rank[ROUTER_RANK_PER_LANE] = {0, 0, 0, 0};
 #pragma unroll 4
     for (int o = 0; o < e2; o += 2) {
@@ -152,7 +157,9 @@ __global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict
 #pragma unroll
     for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i)
         if (lane + 64 * i < E && rank[i] < k) picked[wv][rank[i]] = pr[i] / denom;
-    // (LDS operations of one wavefront complete in order)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     float picked_sum = 0.0f;
     for (int j = 0; j < k; ++j) picked_sum += picked[wv][j];
 #pragma unroll

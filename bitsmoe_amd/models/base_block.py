@@ -22,6 +22,7 @@ import torch
 import torch.nn as nn
 
 from bitsmoe_amd.algorithms import _HAS_MLP_FORWARD_CUDA, mlp_forward_cuda
+from bitsmoe_amd.models.base_mlp import buffer_generation
 
 _BUFFER_NAMES = ("payload", "rank_idx", "tile_meta", "slab_meta", "scale", "s")
 
@@ -106,11 +107,32 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         self._cached_token_count = -1
         self._cached_flat_token_ids: Optional[torch.Tensor] = None
         self._matsets = None
+        self._buffer_generation_seen = -1
         self._basis_cache: Dict[object, object] = {}      # per dtype: the three bases; ("stacked", dtype): gate over up
 
     def _ensure_runtime_cache(self, device: torch.device) -> None:
         if self._runtime_cache_ready and self._runtime_cache_device == device:
-            return
+            if self._buffer_generation_seen == buffer_generation():
+                return
+            # Some expert container (of this block or another) rebound or reloaded a buffer since the
+            # tuples and matrix sets were built.  The sets are snapshots: keep them only if every
+            # tensor they were built from is still the bound one and unwritten.
+            self._buffer_generation_seen = buffer_generation()
+            fresh = all(
+                len(getattr(self, f"_{proj}_{name}_static")) == self._packed_expert_count
+                for proj in ("gate", "up", "down") for name in _BUFFER_NAMES)
+            if fresh:
+                packed = [layer for idx, layer in enumerate(self.experts)
+                          if layer is not None and idx not in self._super_expert_set]
+                for proj in ("gate", "up", "down"):
+                    for name in _BUFFER_NAMES:
+                        held = getattr(self, f"_{proj}_{name}_static")
+                        fresh = fresh and len(packed) == len(held) and all(
+                            getattr(e, f"{proj}_{name}_buffer" if name != "s" else f"{proj}_s_buffer") is t
+                            for e, t in zip(packed, held))
+            if fresh and (self._matsets is None or all(ms.is_current() for ms in self._matsets)):
+                return
+            self._invalidate_runtime_cache()
         super_items: List[Tuple[int, nn.Module]] = []
         packed_items: List[Tuple[int, nn.Module]] = []
         for expert_idx, layer in enumerate(self.experts):
@@ -145,6 +167,12 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         self._runtime_cache_ready = True
         self._runtime_cache_device = device
         self._runtime_warmed = False
+        self._buffer_generation_seen = buffer_generation()
+
+    def refresh_packed_weights(self) -> None:
+        """Call after writing into packed buffers in place by other means than the expert containers'
+        own loaders (`tensor.copy_()`, custom kernels): the matrix sets are snapshots."""
+        self._invalidate_runtime_cache()
 
     def _static_lists(self, proj: str) -> Tuple[Sequence[torch.Tensor], ...]:
         return tuple(getattr(self, f"_{proj}_{name}_static") for name in _BUFFER_NAMES)

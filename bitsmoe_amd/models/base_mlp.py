@@ -16,6 +16,15 @@ import torch
 import torch.nn as nn
 
 
+# Bumped whenever any expert container rebinds or reloads a buffer: blocks compare it with the value
+# they saw when they built their matrix sets (snapshots of the buffers) and rebuild stale ones.
+_BUFFER_GENERATION = [0]
+
+
+def buffer_generation() -> int:
+    return _BUFFER_GENERATION[0]
+
+
 class BitsMoE_BaseMoeMLP(nn.Module):
     _MTYPE_TO_TAG = {"gate_proj": "gate", "up_proj": "up", "down_proj": "down"}
     _RUNTIME_BUFFER_DTYPES = {
@@ -64,6 +73,7 @@ class BitsMoE_BaseMoeMLP(nn.Module):
                 self.register_buffer(f"{tag}_{name}", init, persistent=True)
 
     def _bind(self, name: str, tensor: torch.Tensor) -> None:
+        _BUFFER_GENERATION[0] += 1
         if name in self._buffers:
             self._buffers[name] = tensor
         else:
@@ -146,6 +156,7 @@ class BitsMoE_BaseMoeMLP(nn.Module):
                 continue
             self._bind(leaf, tensor.detach() if assign else torch.empty_like(tensor))
         super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs)
+        _BUFFER_GENERATION[0] += 1      # (the generic loader copies in place into buffers of matching shape)
         self.is_bitsmoe_packed = all(
             isinstance(getattr(self, f"{tag}_payload_buffer", None), torch.Tensor)
             and getattr(self, f"{tag}_payload_buffer").numel() > 0

@@ -149,9 +149,14 @@ class _SourceBlock(nn.Module):
         self.experts = nn.ModuleList([None] * n_experts)
 
 
+_BASIS_CACHE: Dict[Tuple[int, int, str], torch.Tensor] = {}
+
+
 def make_layer(spec: LayerSpec, device="cuda", dtype=torch.bfloat16, seed: int = 42, layer_idx: int = 0,
-               s_mode: str = "ones") -> nn.Module:
-    """A ready-to-run sparse-MoE block of `spec`'s family on `device`."""
+               s_mode: str = "ones", basis_seed: Optional[int] = None) -> nn.Module:
+    """A ready-to-run sparse-MoE block of `spec`'s family on `device`.  `basis_seed`: take the three
+    shared bases from this seed instead of the layer's own (layers of a stack may share them: the
+    host factorisation of three 2048 x 2048 matrices per layer dominates the build otherwise)."""
     from bitsmoe_amd.models.deepseekv2.bitsmoe_block import BitsMoE_DeepSeekSparseMoeBlock
     from bitsmoe_amd.models.deepseekv2.bitsmoe_mlp import BitsMoE_DeepSeekMLP
     from bitsmoe_amd.models.qwen3moe.bitsmoe_block import BitsMoE_Qwen3MoeSparseMoeBlock
@@ -191,8 +196,17 @@ def make_layer(spec: LayerSpec, device="cuda", dtype=torch.bfloat16, seed: int =
     for e, mod in enumerate(experts):
         block.set_expert(e, mod, packed=True)
     r = int(spec.rank or h)
-    block.set_shared_basis(orthonormal(h, seed * 31 + 1, device)[:r], orthonormal(h, seed * 31 + 2, device)[:r],
-                           orthonormal(h, seed * 31 + 3, device)[:, :r])
+    bseed = seed if basis_seed is None else int(basis_seed)
+
+    def basis(j: int) -> torch.Tensor:
+        key = (h, bseed * 31 + j, str(device))
+        if key not in _BASIS_CACHE:
+            if len(_BASIS_CACHE) >= 12:
+                _BASIS_CACHE.clear()
+            _BASIS_CACHE[key] = orthonormal(h, bseed * 31 + j, device)
+        return _BASIS_CACHE[key]
+
+    block.set_shared_basis(basis(1)[:r], basis(2)[:r], basis(3)[:, :r])
     block.expert_bits = bits
     block.spec = spec
     return block.to(device)

@@ -404,6 +404,25 @@ def test_forward_mfma_path_needs_prepared_sets(cuda_device):
                              sets[0], sets[1], sets[2], 80, 128, 0, path=_capi.PATH_MFMA)
 
 
+def test_forward_rejects_a_rank_out_no_down_row_writes_into(cuda_device):
+    """Down rows whose rank_idx lies outside [0, rank_out) are skipped, as in the reference
+    (bitsmoe/algorithms/cpp/mlp_forward.cu:1782); a rank_out that EVERY row misses is an error."""
+    import torch
+
+    hip = _hip()
+    gate, up, down = helpers.make_experts(6, 2, 64, 64, 128, choices=(2,), uniform_bits=True)
+    for m in down:
+        m["rank_idx"] = (m["rank_idx"] + 64).astype(np.int32)      # ranks 64..127
+    sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=128) for m in (gate, up, down)]
+    z = lambda *s, dt=torch.float16: torch.zeros(s, dtype=dt, device=cuda_device)
+    args = (z(4, 64), z(4, 64), z(4, dt=torch.int32), torch.tensor([0, 2, 4], dtype=torch.int32, device=cuda_device),
+            z(4, dt=torch.float32))
+    with pytest.raises(RuntimeError, match="no row of the down matrices writes"):
+        hip.moe_forward_sets(*args, sets[0], sets[1], sets[2], 64, 128, 0)
+    out = hip.moe_forward_sets(*args, sets[0], sets[1], sets[2], 128, 128, 0)      # rank_out that holds them
+    assert out.shape == (4, 128)
+
+
 def test_dispatcher_operator_equals_direct_call(cuda_device):
     """torch.ops.bitsmoe.moe_packed_forward (fresh list objects on every call) and the module-level
     function give the same result and share one matrix set."""
@@ -427,7 +446,7 @@ def test_dispatcher_operator_equals_direct_call(cuda_device):
     n_sets = len(hip._SET_CACHE)
     via_op = torch.ops.bitsmoe.moe_packed_forward(h_gate, h_up, tok, off, rw, *flat, 64, 256, 0)
     again = torch.ops.bitsmoe.moe_packed_forward(h_gate, h_up, tok, off, rw, *flat, 64, 256, 0)
-    assert len(hip._SET_CACHE) == n_sets == 3            # found by buffer address, not rebuilt
+    assert len(hip._SET_CACHE) == n_sets == 3            # found by the buffers' fingerprint, not rebuilt
     scale = float(direct.abs().max())
     assert float((via_op - direct).abs().max()) <= 1e-5 * scale and float((again - direct).abs().max()) <= 1e-5 * scale
 
