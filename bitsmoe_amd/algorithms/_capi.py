@@ -36,6 +36,8 @@ EXPORTED_SYMBOLS = (
     "bitsmoe_forward_workspace_bytes_sets",
     "bitsmoe_moe_forward",
     "bitsmoe_moe_forward_strided",
+    "bitsmoe_static_scratch_bytes",
+    "bitsmoe_moe_forward_static",
     "bitsmoe_profile_create",
     "bitsmoe_profile_destroy",
     "bitsmoe_profile_read",
@@ -115,6 +117,13 @@ def load() -> ctypes.CDLL:
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_int64, c_int64,
         c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32,
         c_void_p, c_void_p, c_size_t, c_void_p, c_void_p,
+    ]
+    lib.bitsmoe_static_scratch_bytes.restype = c_size_t
+    lib.bitsmoe_static_scratch_bytes.argtypes = []
+    lib.bitsmoe_moe_forward_static.restype = c_int32
+    lib.bitsmoe_moe_forward_static.argtypes = [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_int64, c_int64,
+        c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p,
     ]
     lib.bitsmoe_profile_create.restype = c_int32
     lib.bitsmoe_profile_create.argtypes = [POINTER(c_void_p)]

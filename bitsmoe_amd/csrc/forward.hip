@@ -4,6 +4,42 @@
 
 using namespace bitsmoe;
 
+#include <mutex>
+
+// Intermediates of bitsmoe_moe_forward_static: one array per GPU, held until the process ends.
+// In host code the array's name is only a stand-in for the symbol; its address on a device comes
+// from hipGetSymbolAddress, made once per device with that device current.
+static __device__ __align__(256) unsigned char scratch[BITSMOE_STATIC_SCRATCH_BYTES];
+
+static constexpr int MAX_DEVICES = 64;
+static void* g_scratch_ptr[MAX_DEVICES] = {};
+static std::mutex g_scratch_mutex;
+
+// The current device's copy of `scratch` (device address), or nullptr with the error set.
+static void* scratch_of_current_device() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        hip_fail(e, "hipGetDevice");
+        return nullptr;
+    }
+    if (dev < 0 || dev >= MAX_DEVICES) {
+        set_error("device index %d outside [0, %d)", dev, MAX_DEVICES);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            hip_fail(e, "hipGetSymbolAddress(scratch)");
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 extern "C" size_t bitsmoe_forward_workspace_bytes(int64_t n_tokens, int64_t n_assign,
@@ -108,6 +144,12 @@ extern "C" int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bit
                     "gate rank_idx references rank %d but h_gate has %d columns", gate->max_rank_plus1 - 1, rank_gate);
     BITSMOE_REQUIRE(up->max_rank_plus1 <= rank_up && up->min_rank >= 0,
                     "up rank_idx references rank %d but h_up has %d columns", up->max_rank_plus1 - 1, rank_up);
+    // (rows whose rank_idx lies outside [0, rank_out) are skipped by design -- the reference does the same,
+    // bitsmoe/algorithms/cpp/mlp_forward.cu:1782 -- but a down set whose EVERY reference is out of range is
+    // a rank_out that does not belong to these matrices)
+    BITSMOE_REQUIRE(down->total_slabs == 0 || (down->min_rank < rank_out && down->max_rank_plus1 > 0),
+                    "down rank_idx references ranks [%d, %d] but rank_out is %d: no row of the down matrices writes "
+                    "into rank_accum", down->min_rank, down->max_rank_plus1 - 1, rank_out);
     const int chosen = resolve_path(gate, up, down, n_assign, intermediate_size, path);
     if (chosen < 0) return chosen;
     const size_t need = bitsmoe_forward_workspace_bytes_sets(gate, up, down, n_tokens, n_assign, chosen);
@@ -131,4 +173,35 @@ extern "C" int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bit
     return launch_forward_generic(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
                                   token_indices, expert_offsets, route_w, n_assign, rank_out,
                                   intermediate_size, rank_accum, G, U, profile, st);
+}
+
+extern "C" size_t bitsmoe_static_scratch_bytes(void) { return (size_t)BITSMOE_STATIC_SCRATCH_BYTES; }
+
+extern "C" int bitsmoe_moe_forward_static(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                                          const bitsmoe_matset* down, const void* h_gate, const void* h_up,
+                                          int32_t act_dtype, int64_t n_tokens, int32_t rank_gate, int32_t rank_up,
+                                          int64_t ld_gate, int64_t ld_up, const int32_t* token_indices,
+                                          const int32_t* expert_offsets, const float* route_w, int64_t n_assign,
+                                          int32_t rank_out, int32_t intermediate_size, int32_t act_type, int32_t path,
+                                          float* rank_accum, void* stream) {
+    BITSMOE_REQUIRE(gate && up && down, "matrix sets must not be null");
+    BITSMOE_REQUIRE(n_assign >= 0 && n_tokens >= 0, "negative token or assignment count");
+    BITSMOE_REQUIRE(path >= BITSMOE_PATH_AUTO && path <= BITSMOE_PATH_MFMA, "unknown path %d", path);
+    // the size check comes first: a call that cannot be served touches nothing
+    const int chosen = resolve_path(gate, up, down, n_assign, gate->intermediate_size, path);
+    if (chosen < 0) return chosen;
+    const size_t need = bitsmoe_forward_workspace_bytes_sets(gate, up, down, n_tokens, n_assign, chosen);
+    if (need > (size_t)BITSMOE_STATIC_SCRATCH_BYTES) {
+        set_error("bitsmoe_moe_forward_static: this call needs %zu bytes of intermediates, the static scratch holds %zu "
+                  "(use bitsmoe_moe_forward with a caller-owned workspace)", need, (size_t)BITSMOE_STATIC_SCRATCH_BYTES);
+        return BITSMOE_E_WORKSPACE;
+    }
+    void* ptr = scratch_of_current_device();
+    if (!ptr) return BITSMOE_E_HIP;
+    // Every path clears what it needs cleared with its own kernels (the array keeps the previous
+    // call's contents), so the shared entry point can run on it as on any workspace.
+    return bitsmoe_moe_forward_strided(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
+                                       token_indices, expert_offsets, route_w, n_assign, rank_out, intermediate_size,
+                                       act_type, chosen, rank_accum, ptr, (size_t)BITSMOE_STATIC_SCRATCH_BYTES, nullptr,
+                                       stream);
 }

@@ -198,6 +198,27 @@ int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bitsmoe_matset
                                 bitsmoe_profile* profile, void* stream);
 
 /*
+ * The forward for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): bitsmoe_moe_forward_strided without the
+ * workspace argument.  No counterpart in the reference, whose operator allocates its
+ * intermediates from the framework's allocator on every call.  The intermediates live in a
+ * static device array of BITSMOE_STATIC_SCRATCH_BYTES that every GPU the library runs on holds
+ * until the process ends; the call allocates nothing (no hipMalloc / hipFree, no framework
+ * allocator).  A call whose path needs more (bitsmoe_forward_workspace_bytes_sets) fails with
+ * BITSMOE_E_WORKSPACE before anything is launched.  All calls on one GPU share that GPU's array:
+ * calls that overlap on one GPU (two streams, two threads) race; serialise them.
+ */
+#define BITSMOE_STATIC_SCRATCH_BYTES (32u << 20)
+size_t bitsmoe_static_scratch_bytes(void);
+int bitsmoe_moe_forward_static(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                               const bitsmoe_matset* down, const void* h_gate, const void* h_up,
+                               int32_t act_dtype, int64_t n_tokens, int32_t rank_gate, int32_t rank_up,
+                               int64_t ld_gate, int64_t ld_up, const int32_t* token_indices,
+                               const int32_t* expert_offsets, const float* route_w, int64_t n_assign,
+                               int32_t rank_out, int32_t intermediate_size, int32_t act_type,
+                               int32_t path, float* rank_accum, void* stream);
+
+/*
  * Phase timing with HIP events recorded on the caller's stream between the kernels of
  * one bitsmoe_moe_forward call (no reference counterpart: the reference has no
  * profiling hooks in the op).  After the stream has been synchronised,
