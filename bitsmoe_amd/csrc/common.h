@@ -106,6 +106,7 @@ struct bitsmoe_matset {
                                       // rank offsets advance by a whole slab from one slab to the next
     // experts by decreasing payload size (prepared sets of at most EXPERT_ORDER_MAX experts): the
     // decode kernels start the expensive experts' workgroups first
+    std::vector<uint8_t> expert_bits;   // prepared sets: the bit-width all slabs of an expert share, or 0
     bool has_cost_order = false;
     uint16_t cost_order[512] = {};
     uint32_t* d_prepared = nullptr;   // wave-native copy of every payload (see wave_layout.h)

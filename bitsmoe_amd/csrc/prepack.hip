@@ -285,6 +285,7 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
         BITSMOE_HIP_TRY(sync_err);
     }
     std::vector<FastExpert> fexp(set->n_experts);
+    set->expert_bits.assign(set->n_experts, 0);
     for (int e = 0; e < set->n_experts; ++e) {
         FastExpert& f = fexp[e];
         memset(&f, 0, sizeof(f));
@@ -297,6 +298,7 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
         f.uniform_bits = f.num_slabs > 0 ? set->slab_meta_host[e][0] : 0;
         for (int si = 1; si < f.num_slabs; ++si)
             if (set->slab_meta_host[e][si * 4] != f.uniform_bits) f.uniform_bits = 0;
+        set->expert_bits[e] = (uint8_t)f.uniform_bits;
     }
     set->has_cost_order = set->n_experts <= EXPERT_ORDER_MAX;
     if (set->has_cost_order) {

@@ -284,6 +284,20 @@ def test_forward_decode_path_one_width_per_expert(cuda_device, bits):
 
 
 @pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_forward_decode_path_both_projections_in_one_workgroup(cuda_device, bits, dtype_name, monkeypatch):
+    """BITSMOE_DECODE_FUSED_Z=1: one workgroup forms gate AND up of a tile and hands z = silu(G) * U to the
+    down kernel as 16-bit operands (plus the row sums of its decode's constant term); 40 tokens over 3
+    experts: chunks of 16 assignments and a ragged last chunk."""
+    from bitsmoe_amd.algorithms import _capi
+
+    monkeypatch.setenv("BITSMOE_DECODE_FUSED_Z", "1")
+    err = _forward_case(cuda_device, 700 + bits, 3, 40, 2, 1024, 256, 384, dtype_name, (bits,), path=_capi.PATH_DECODE,
+                        tol=1e-2, uniform_bits=True)
+    assert err < 3e-3
+
+
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
 def test_forward_mfma_path_scattered_ranks(cuda_device, dtype_name):
     """rank_idx without runs of eight consecutive ranks: the activations are gathered first."""
     from bitsmoe_amd.algorithms import _capi
