@@ -95,6 +95,7 @@ struct bitsmoe_matset {
     int32_t min_rank = 0;             // smallest logical rank
     bool regular = false;             // every matrix: 2/3/4-bit, k_slab % 16 == 0, full tiles
     bool regular64 = false;           // ... and every slab has exactly 64 rows, payload 16-byte aligned
+    bool fast_ok = false;             // every slab 2/3/4-bit over full 128-column tiles: bitsmoe_matset_prepare can take the set
     int role = -1;                    // -1: not prepared; 0: gate/up layout; 1: down layout
     bool rank_chunked8 = false;       // slab i holds local rows 64*i.., and every aligned run of 8 local rows
                                       // maps to 8 consecutive logical ranks starting at a multiple of 8
@@ -109,11 +110,12 @@ struct bitsmoe_matset {
     std::vector<uint8_t> expert_bits;   // prepared sets: the bit-width all slabs of an expert share, or 0
     bool has_cost_order = false;
     uint16_t cost_order[512] = {};
-    uint32_t* d_prepared = nullptr;   // wave-native copy of every payload (see wave_layout.h)
-    bitsmoe::MatView* d_views_prepared = nullptr;
+    uint32_t* d_prepared = nullptr;   // wave-native copy of every payload (see wave_layout.h), every slab padded to 64 rows
+    void* d_prepared_rows = nullptr;  // the prepared copy's row tables: rank_idx', s', scale' (padded the same way)
+    std::vector<bitsmoe::FastExpert> fast_experts_host;
+    std::vector<std::vector<int32_t>> rank_idx_host;
     bitsmoe::FastExpert* d_fast_experts = nullptr;   // [n_experts]
     bitsmoe::FastSlab* d_fast_slabs = nullptr;       // [n_experts][max_slabs]
-    std::vector<int64_t> prepared_offsets;
     int device = -1;
     std::vector<bitsmoe_matrix_desc> descs;
     std::vector<std::vector<int32_t>> slab_meta_host;

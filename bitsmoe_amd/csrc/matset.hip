@@ -78,7 +78,7 @@ extern "C" const char* bitsmoe_version(void) { return "bitsmoe_hip 0.1 (gfx950)"
 
 static int validate_matrix(const bitsmoe_matrix_desc& d, int e, int I,
                            const std::vector<int32_t>& slab, const std::vector<int32_t>& tile,
-                           bool* regular, bool* regular64) {
+                           bool* regular, bool* regular64, bool* fast_ok) {
     const int n_tiles_mat = (I + N_TILE - 1) / N_TILE;
     int64_t rows_seen = 0;
     for (int s = 0; s < d.num_slabs; ++s) {
@@ -97,6 +97,7 @@ static int validate_matrix(const bitsmoe_matrix_desc& d, int e, int I,
         if (!(bits == 2 || bits == 3 || bits == 4) || (k_slab % K_STAGE) != 0 ||
             tile_end - tile_off != n_tiles_mat)
             *regular = false;
+        if (!(bits == 2 || bits == 3 || bits == 4) || tile_end - tile_off != n_tiles_mat) *fast_ok = false;
         if (k_slab != K_SLAB) *regular64 = false;
         const int64_t words_tile = (int64_t)k_slab * MICROS * words_per_row(bits);
         for (int t = tile_off; t < tile_end; ++t) {
@@ -109,6 +110,7 @@ static int validate_matrix(const bitsmoe_matrix_desc& d, int e, int I,
                             "expert %d tile %d: scale range exceeds scale size %lld", e, t, (long long)d.scale_len);
             BITSMOE_REQUIRE(n_valid >= 1 && n_valid <= N_TILE, "expert %d tile %d: n_valid=%d outside [1,128]", e, t, n_valid);
             if (n_valid != N_TILE || (pack_off & 3) != 0) *regular = false;
+            if (n_valid != N_TILE) *fast_ok = false;
         }
         rows_seen += k_slab;
     }
@@ -140,6 +142,8 @@ extern "C" int bitsmoe_matset_create(const bitsmoe_matrix_desc* descs, int32_t n
     set->tile_meta_host.resize(n_experts);
     set->regular = n_experts > 0;
     set->regular64 = n_experts > 0;
+    set->fast_ok = n_experts > 0;
+    set->rank_idx_host.resize(n_experts);
 
     std::vector<MatView> views(n_experts);
     std::vector<SlabTask> tasks;
@@ -166,9 +170,11 @@ extern "C" int bitsmoe_matset_create(const bitsmoe_matrix_desc* descs, int32_t n
         if (!rk.empty())
             BITSMOE_HIP_TRY(hipMemcpyAsync(rk.data(), d.rank_idx, rk.size() * 4, hipMemcpyDeviceToHost, st));
         BITSMOE_HIP_TRY(hipStreamSynchronize(st));
-        bool regular = true, regular64 = true;
-        const int rc = validate_matrix(d, e, intermediate_size, slab, tile, &regular, &regular64);
+        bool regular = true, regular64 = true, fast_ok = true;
+        const int rc = validate_matrix(d, e, intermediate_size, slab, tile, &regular, &regular64, &fast_ok);
         if (rc != BITSMOE_OK) return rc;
+        if (!fast_ok || d.num_slabs == 0) set->fast_ok = false;
+        set->rank_idx_host[e] = rk;
         if (!regular || d.num_slabs == 0) set->regular = false;
         if (!regular || !regular64 || d.num_slabs == 0 || ((uintptr_t)d.payload & 15) != 0) set->regular64 = false;
         for (int32_t v : rk) {
@@ -224,7 +230,7 @@ extern "C" void bitsmoe_matset_destroy(bitsmoe_matset* set) {
     if (set->d_slab_tasks) (void)hipFree(set->d_slab_tasks);
     if (set->d_prepared) (void)hipFree(set->d_prepared);
     if (set->d_scale_s) (void)hipFree(set->d_scale_s);
-    if (set->d_views_prepared) (void)hipFree(set->d_views_prepared);
+    if (set->d_prepared_rows) (void)hipFree(set->d_prepared_rows);
     if (set->d_fast_experts) (void)hipFree(set->d_fast_experts);
     if (set->d_fast_slabs) (void)hipFree(set->d_fast_slabs);
     delete set;
@@ -239,7 +245,7 @@ extern "C" int bitsmoe_matset_info(const bitsmoe_matset* set, int64_t info[8]) {
     info[4] = set->regular ? 1 : 0;
     info[5] = set->max_slabs;
     info[6] = set->min_rank;
-    info[7] = (set->regular64 ? 1 : 0) | (set->role >= 0 ? 2 : 0);
+    info[7] = (set->fast_ok ? 1 : 0) | (set->role >= 0 ? 2 : 0) | (set->role == 0 && set->all_affine && set->rank_chunked8 ? 4 : 0);
     return BITSMOE_OK;
 }
 

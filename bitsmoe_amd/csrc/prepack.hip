@@ -7,11 +7,14 @@
 
 namespace bitsmoe {
 
-// code (unsigned, before the level offset) of element (row, col) of a (slab, tile) block
-// in the reference bit-plane layout; `blk` points at the block's first word, rows = 64.
-__device__ inline uint32_t ref_code(const uint32_t* __restrict__ blk, int w, int row, int col) {
+// code (unsigned, before the level offset) of element (row, col) of a (slab, tile) block of `k_slab`
+// rows in the reference bit-plane layout; `blk` points at the block's first word.  Rows past
+// k_slab (a ragged slab is padded to 64 rows in the prepared copy) read as the code of level zero.
+__device__ inline uint32_t ref_code(const uint32_t* __restrict__ blk, int w, int k_slab, int row, int col) {
+    if (row >= k_slab) return (uint32_t)level_offset(w);
     const int stage = row >> 4, r = row & 15, micro = col >> 5, lane = col & 31;
-    const uint32_t* words = blk + stage * (K_STAGE * MICROS * w) + micro * (K_STAGE * w) + r * w;
+    const int rows_cur = min(K_STAGE, k_slab - stage * K_STAGE);
+    const uint32_t* words = blk + stage * (K_STAGE * MICROS * w) + micro * (rows_cur * w) + r * w;
     uint32_t u = 0;
     for (int p = 0; p < w; ++p) u |= ((words[p] >> lane) & 1u) << p;
     return u;
@@ -28,18 +31,22 @@ __device__ inline void run_element(int role, int nb, int kg, int n, int x, int* 
     }
 }
 
-// grid: (slab tasks, tiles); every thread builds whole output words of one block.
-__global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src, const MatView* __restrict__ dst,
+// grid: (slab tasks, tiles); every thread builds whole output words of one block.  Reads the caller's
+// reference layout (through its own tile_meta / slab_meta), writes the prepared copy at the offsets of
+// the FastSlab table.
+__global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src, const FastExpert* __restrict__ fexp,
+                                                 const FastSlab* __restrict__ fslabs, int max_slabs,
                                                  const SlabTask* __restrict__ tasks, int role) {
     const SlabTask task = tasks[blockIdx.x];
     const MatView mv = src[task.expert];
     const int si = task.slab;
     const int w = mv.slab_meta[si * 4 + 0];
+    const int k_slab = mv.slab_meta[si * 4 + 1];
     const int tile_off = mv.slab_meta[si * 4 + 3];
     const int t = tile_off + blockIdx.y;
-    const int pack_off = mv.tile_meta[t * 3 + 0];
-    const uint32_t* __restrict__ in = mv.payload + pack_off;
-    uint32_t* __restrict__ out = const_cast<uint32_t*>(dst[task.expert].payload) + pack_off;
+    const uint32_t* __restrict__ in = mv.payload + mv.tile_meta[t * 3 + 0];
+    const FastSlab fs = fslabs[(int64_t)task.expert * max_slabs + si];
+    uint32_t* __restrict__ out = const_cast<uint32_t*>(fexp[task.expert].payload) + fs.pack_off + (int)blockIdx.y * 256 * w;
     const int nbs = (role == ROLE_GATE_UP) ? 8 : 4;        // output blocks per lane
     const int run = (role == ROLE_GATE_UP) ? 16 : 32;      // contraction indices per (lane, nb)
     const int n_words = 256 * w;
@@ -55,14 +62,14 @@ __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src
                     for (int x = 0; x < 16; ++x) {
                         int row, col;
                         run_element(role, nb, kg, n8 + 8 * upper, x, &row, &col);
-                        word |= ((ref_code(in, w, row, col) >> 2) & 1u) << pos1s(x, upper);
+                        word |= ((ref_code(in, w, k_slab, row, col) >> 2) & 1u) << pos1s(x, upper);
                     }
             } else {                      // j = l*4 + nb
                 const int nb = j & 3, l = j >> 2, n = l & 15, kg = l >> 4;
                 for (int x = 0; x < 32; ++x) {
                     int row, col;
                     run_element(role, nb, kg, n, x, &row, &col);
-                    word |= ((ref_code(in, w, row, col) >> 2) & 1u) << pos1(x);
+                    word |= ((ref_code(in, w, k_slab, row, col) >> 2) & 1u) << pos1(x);
                 }
             }
             out[idx] = word;
@@ -87,7 +94,7 @@ __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src
             const int x = sub * codes + i;
             int row, col;
             run_element(role, nb, kg, n, x, &row, &col);
-            const uint32_t u = ref_code(in, w, row, col);
+            const uint32_t u = ref_code(in, w, k_slab, row, col);
             if (role == ROLE_GATE_UP)      // staggered fields; one may wrap around bit 31
                 word |= rotl32(fb == 4 ? (u & 15u) : (u & 3u), fb == 4 ? pos4s(i) : pos2s(w, i));
             else if (fb == 4)
@@ -99,17 +106,44 @@ __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src
     }
 }
 
-// Dense fp32 dequantisation FROM THE PREPARED LAYOUT, written to mirror the decode of the
-// hot kernels (fields, not planes); output identical to k_dequant_matrix.
-__global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* payload = prepared */, int role, int I,
+// The per-row tables of the prepared copy, every slab padded to 64 rows: s' (multiplier), scale'
+// [(slab, tile)][64] and, for gate/up sets, scale_s' = scale * s * stagger factor (a power of two: the
+// decoded weight carries its inverse), each rounded once to fp16.  Padding rows get zeros, so whatever
+// the kernels read for them contributes nothing.  grid (slab tasks, tiles), 64 threads.
+__global__ __launch_bounds__(64) void k_prepare_rows(const MatView* __restrict__ views, const FastExpert* __restrict__ fexp,
+                                                     const FastSlab* __restrict__ fslabs, int max_slabs,
+                                                     const SlabTask* __restrict__ tasks) {
+    const SlabTask task = tasks[blockIdx.x];
+    const MatView mv = views[task.expert];
+    const FastExpert fe = fexp[task.expert];
+    const int si = task.slab;
+    const int w = mv.slab_meta[si * 4 + 0];
+    const int k_slab = mv.slab_meta[si * 4 + 1];
+    const int rank_off = mv.slab_meta[si * 4 + 2];
+    const int t = mv.slab_meta[si * 4 + 3] + blockIdx.y;
+    const int scale_off = mv.tile_meta[t * 3 + 1];
+    const FastSlab fs = fslabs[(int64_t)task.expert * max_slabs + si];
+    const int row = threadIdx.x;
+    const bool valid = row < k_slab;
+    const float sv = valid ? __half2float(mv.s[rank_off + row]) : 0.0f;
+    const float sc = valid ? __half2float(mv.scale[scale_off + row]) : 0.0f;
+    const int out_sc = fs.scale_off + (int)blockIdx.y * SLAB_ROWS + row;
+    const_cast<__half*>(fe.scale)[out_sc] = __float2half(sc);
+    if (fe.scale_s) const_cast<__half*>(fe.scale_s)[out_sc] = __float2half(sc * sv * (float)stagger_factor(w, row));
+    if (blockIdx.y == 0) const_cast<__half*>(fe.s)[fs.rank_off + row] = __float2half(sv);
+}
+
+// Dense fp32 dequantisation FROM THE PREPARED COPY, written to mirror the decode of the hot kernels
+// (fields, not planes); rows in the caller's local row order, output identical to k_dequant_matrix.
+__global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* the caller's tables */, FastExpert fe,
+                                                          const FastSlab* __restrict__ fs_row, int role, int I,
                                                           float* __restrict__ out) {
     const int si = blockIdx.x;
     const int w = mv.slab_meta[si * 4 + 0];
+    const int k_slab = mv.slab_meta[si * 4 + 1];
     const int rank_off = mv.slab_meta[si * 4 + 2];
-    const int t = mv.slab_meta[si * 4 + 3] + blockIdx.y;
-    const int pack_off = mv.tile_meta[t * 3 + 0];
-    const int scale_off = mv.tile_meta[t * 3 + 1];
-    const uint32_t* __restrict__ blk = mv.payload + pack_off;
+    const FastSlab fs = fs_row[si];
+    const uint32_t* __restrict__ blk = fe.payload + fs.pack_off + (int)blockIdx.y * 256 * w;
     const int nbs = (role == ROLE_GATE_UP) ? 8 : 4;
     const int run = (role == ROLE_GATE_UP) ? 16 : 32;
     for (int idx = threadIdx.x; idx < SLAB_ROWS * N_TILE; idx += blockDim.x) {
@@ -144,28 +178,11 @@ __global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* payload 
             }
         }
         const int c = blockIdx.y * N_TILE + col;
-        if (c < I) {
+        if (c < I && row < k_slab) {
             const float q = (float)((int)u - level_offset(w));
-            out[(int64_t)(rank_off + row) * I + c] = q * __half2float(mv.scale[scale_off + row]);
+            out[(int64_t)(rank_off + row) * I + c] = q * __half2float(fe.scale[fs.scale_off + (int)blockIdx.y * SLAB_ROWS + row]);
         }
     }
-}
-
-// scale_s[scale_off(slab, tile) + row] = scale[...] * s[rank_off(slab) + row], rounded once to fp16,
-// times the row's stagger factor (a power of two: the decoded weight carries its inverse).
-// grid (slab tasks, tiles), 64 threads.
-__global__ __launch_bounds__(64) void k_fold_scale_s(const MatView* __restrict__ views, const SlabTask* __restrict__ tasks,
-                                                     const int64_t* __restrict__ out_offsets, __half* __restrict__ out) {
-    const SlabTask task = tasks[blockIdx.x];
-    const MatView mv = views[task.expert];
-    const int si = task.slab;
-    const int rank_off = mv.slab_meta[si * 4 + 2];
-    const int t = mv.slab_meta[si * 4 + 3] + blockIdx.y;
-    const int scale_off = mv.tile_meta[t * 3 + 1];
-    const int row = threadIdx.x;
-    const float v = __half2float(mv.scale[scale_off + row]) * __half2float(mv.s[rank_off + row]);
-    const int w = mv.slab_meta[si * 4 + 0];
-    out[out_offsets[task.expert] + scale_off + row] = __float2half(v * (float)stagger_factor(w, row));
 }
 
 }  // namespace bitsmoe
@@ -182,8 +199,8 @@ extern "C" int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* s
     const int rc = prepare_impl(set, role, (hipStream_t)stream);
     if (rc != BITSMOE_OK) {
         // nothing of a failed attempt stays behind: the set remains usable by the generic kernels
-        void** owned[] = {(void**)&set->d_prepared, (void**)&set->d_views_prepared, (void**)&set->d_fast_experts,
-                          (void**)&set->d_fast_slabs, (void**)&set->d_scale_s};
+        void** owned[] = {(void**)&set->d_prepared, (void**)&set->d_fast_experts, (void**)&set->d_fast_slabs,
+                          (void**)&set->d_scale_s, (void**)&set->d_prepared_rows};
         for (void** p : owned) {
             if (*p) (void)hipFree(*p);
             *p = nullptr;
@@ -193,134 +210,135 @@ extern "C" int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* s
     return rc;
 }
 
+static inline int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
 static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
-    if (!set->regular64 || set->total_slabs == 0) {
-        set_error("matrix set is not regular (every slab 64 rows of 2/3/4 bits, full 128-column tiles): "
+    if (!set->fast_ok || set->total_slabs == 0) {
+        set_error("matrix set holds slabs of other widths than 2, 3 or 4 bits, or tiles of fewer than 128 columns: "
                   "only the generic kernels can run it");
         return BITSMOE_E_UNSUPPORTED;
     }
-    // the flattened tables assume the tiles of a slab follow each other in payload and scale
-    std::vector<FastSlab> fslabs((size_t)set->n_experts * set->max_slabs, FastSlab{0, 0, 0, 0});
-    for (int e = 0; e < set->n_experts; ++e) {
+    const int E = set->n_experts, n_tiles = set->n_tiles, max_slabs = set->max_slabs;
+    // Offsets of the prepared copy: every slab is a full 64-row slab there (a ragged slab of the caller's
+    // layout is padded), so slab si of an expert holds local rows [64 si, 64 si + 64), its tiles follow
+    // each other in payload' (256 w words each) and in scale' (64 each).
+    std::vector<FastSlab> fslabs((size_t)E * max_slabs, FastSlab{0, 0, 0, 0});
+    std::vector<int64_t> pay_off(E), row_off(E), sc_off(E);
+    int64_t pay_words = 0, rows_total = 0, scale_total = 0;
+    for (int e = 0; e < E; ++e) {
+        pay_off[e] = pay_words;
+        row_off[e] = rows_total;
+        sc_off[e] = scale_total;
         const auto& slab = set->slab_meta_host[e];
-        const auto& tile = set->tile_meta_host[e];
+        int64_t words = 0;
+        const int ns = set->descs[e].num_slabs;
+        for (int si = 0; si < ns; ++si) {
+            const int bits = slab[si * 4 + 0];
+            BITSMOE_REQUIRE(words < ((int64_t)1 << 31) - (int64_t)n_tiles * 256 * 4, "expert %d: prepared payload exceeds int32 word offsets", e);
+            fslabs[(size_t)e * max_slabs + si] = FastSlab{bits, (int32_t)words, si * n_tiles * SLAB_ROWS, si * SLAB_ROWS};
+            words += (int64_t)n_tiles * 256 * bits;
+        }
+        pay_words += round_up(words, 64);                               // keep every matrix 256-byte aligned
+        rows_total += round_up((int64_t)ns * SLAB_ROWS, 64);
+        scale_total += round_up((int64_t)ns * n_tiles * SLAB_ROWS, 128);
+    }
+    // rank_idx' on the host (the kernels' eligibility flags are read off it): a padding row reads rank -1,
+    // which every kernel treats as "no such row" -- except whole padded runs of eight rows, which read the
+    // ranks 0..7 (their scale is zero) so that they do not break the runs-of-eight property below.
+    std::vector<int32_t> rank_rows((size_t)std::max<int64_t>(rows_total, 1), -1);
+    for (int e = 0; e < E; ++e) {
+        const auto& slab = set->slab_meta_host[e];
+        const auto& rk = set->rank_idx_host[e];
         for (int si = 0; si < set->descs[e].num_slabs; ++si) {
-            const int bits = slab[si * 4 + 0], tile_off = slab[si * 4 + 3];
-            for (int t = 0; t < set->n_tiles; ++t) {
-                if (tile[(tile_off + t) * 3 + 0] != tile[tile_off * 3 + 0] + t * 256 * bits ||
-                    tile[(tile_off + t) * 3 + 1] != tile[tile_off * 3 + 1] + t * SLAB_ROWS) {
-                    set_error("expert %d slab %d: tiles are not contiguous in payload/scale; only the generic "
-                              "kernels can run this set", e, si);
-                    return BITSMOE_E_UNSUPPORTED;
-                }
+            const int k_slab = slab[si * 4 + 1], rank_off = slab[si * 4 + 2];
+            int32_t* dst = rank_rows.data() + row_off[e] + (int64_t)si * SLAB_ROWS;
+            for (int r = 0; r < SLAB_ROWS; ++r) {
+                if (r < k_slab)
+                    dst[r] = rk[rank_off + r];
+                else if ((r & ~7) >= k_slab && set->max_rank_plus1 >= 8)
+                    dst[r] = r & 7;
             }
-            fslabs[(size_t)e * set->max_slabs + si] =
-                FastSlab{bits, tile[tile_off * 3 + 0], tile[tile_off * 3 + 1], slab[si * 4 + 2]};
         }
     }
-    // does every aligned group of GU_SLABS slabs have one width and follow each other in the payload?
-    // (the same test the gate/up kernel applies per workgroup)
-    bool all_uniform = set->max_slabs % GU_SLABS == 0;
-    for (int e = 0; e < set->n_experts && all_uniform; ++e) {
-        if (set->descs[e].num_slabs != set->max_slabs) all_uniform = false;
-        for (int s0 = 0; s0 < set->descs[e].num_slabs && all_uniform; s0 += GU_SLABS) {
-            const FastSlab& first = fslabs[(size_t)e * set->max_slabs + s0];
-            for (int q = 1; q < GU_SLABS; ++q) {
-                const FastSlab& f = fslabs[(size_t)e * set->max_slabs + s0 + q];
-                if (f.bits != first.bits || f.pack_off != first.pack_off + q * set->n_tiles * 256 * first.bits)
-                    all_uniform = false;
-            }
+    // every aligned run of 8 rows = 8 consecutive logical ranks starting at a multiple of 8?  rank'[k] == k?
+    bool chunked8 = E > 0, identity = E > 0;
+    for (int e = 0; e < E && (chunked8 || identity); ++e) {
+        const int64_t n = (int64_t)set->descs[e].num_slabs * SLAB_ROWS;
+        const int32_t* r = rank_rows.data() + row_off[e];
+        for (int64_t k = 0; k < n; ++k) {
+            if (r[k] != (int32_t)k) identity = false;
+            if ((k & 7) == 0 ? (r[k] < 0 || (r[k] & 7) != 0) : (r[k] != r[k - 1] + 1)) chunked8 = false;
+        }
+    }
+    set->rank_chunked8 = chunked8;
+    set->rank_identity = identity;
+    // does every aligned group of GU_SLABS slabs have one width (the same test the split gate/up kernel
+    // applies per workgroup), and is every expert ONE run of equal-width slabs (what the walking kernel assumes)?
+    bool all_uniform = max_slabs % GU_SLABS == 0, all_affine = max_slabs % GU_SLABS == 0;
+    for (int e = 0; e < E && all_uniform; ++e) {
+        if (set->descs[e].num_slabs != max_slabs) all_uniform = all_affine = false;
+        for (int si = 0; si < set->descs[e].num_slabs && all_uniform; ++si) {
+            const int bits = fslabs[(size_t)e * max_slabs + si].bits;
+            if (bits != fslabs[(size_t)e * max_slabs + si / GU_SLABS * GU_SLABS].bits) all_uniform = false;
+            if (bits != fslabs[(size_t)e * max_slabs].bits) all_affine = false;
         }
     }
     set->all_uniform8 = all_uniform;
-    // is every expert one affine run of equal-width slabs (what the walking gate/up kernel assumes)?
-    bool all_affine = all_uniform;
-    for (int e = 0; e < set->n_experts && all_affine; ++e) {
-        const FastSlab& first = fslabs[(size_t)e * set->max_slabs];
-        for (int si = 1; si < set->max_slabs; ++si) {
-            const FastSlab& f = fslabs[(size_t)e * set->max_slabs + si];
-            if (f.bits != first.bits || f.pack_off != first.pack_off + si * set->n_tiles * 256 * first.bits ||
-                f.scale_off != first.scale_off + si * set->n_tiles * SLAB_ROWS || f.rank_off != first.rank_off + si * SLAB_ROWS)
-                all_affine = false;
-        }
-    }
-    set->all_affine = all_affine;
-    bool aligned = true;
-    for (int e = 0; e < set->n_experts; ++e) {
-        const bitsmoe_matrix_desc& d = set->descs[e];
-        if ((((uintptr_t)d.scale) | ((uintptr_t)d.s) | ((uintptr_t)d.rank_idx)) & 15) aligned = false;
-    }
-    set->vector_aligned = aligned;
-    int64_t total_words = 0;
-    std::vector<int64_t> offs(set->n_experts);
-    for (int e = 0; e < set->n_experts; ++e) {
-        offs[e] = total_words;
-        total_words += (set->descs[e].payload_words + 63) / 64 * 64;    // keep every matrix 256-byte aligned
-    }
-    BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_prepared, (size_t)total_words * 4));
-    std::vector<MatView> views(set->n_experts);
-    BITSMOE_HIP_TRY(hipMemcpyAsync(views.data(), set->d_views, sizeof(MatView) * set->n_experts, hipMemcpyDeviceToHost, st));
-    BITSMOE_HIP_TRY(hipStreamSynchronize(st));
-    for (int e = 0; e < set->n_experts; ++e) views[e].payload = set->d_prepared + offs[e];
-    BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_views_prepared, sizeof(MatView) * set->n_experts));
-    BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_views_prepared, views.data(), sizeof(MatView) * set->n_experts, hipMemcpyHostToDevice, st));
-    // gate/up sets also get a copy of the scales folded with the per-row multiplier
-    std::vector<int64_t> sc_offs(set->n_experts, 0);
-    if (role == ROLE_GATE_UP) {
-        int64_t total_scale = 0;
-        for (int e = 0; e < set->n_experts; ++e) {
-            sc_offs[e] = total_scale;
-            total_scale += (set->descs[e].scale_len + 127) / 128 * 128;    // keep every expert 256-byte aligned
-        }
-        int64_t* d_offs = nullptr;
-        BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_scale_s, (size_t)std::max<int64_t>(total_scale, 1) * 2));
-        BITSMOE_HIP_TRY(hipMalloc((void**)&d_offs, sizeof(int64_t) * set->n_experts));
-        BITSMOE_HIP_TRY(hipMemcpyAsync(d_offs, sc_offs.data(), sizeof(int64_t) * set->n_experts, hipMemcpyHostToDevice, st));
-        hipLaunchKernelGGL(k_fold_scale_s, dim3((unsigned)set->total_slabs, set->n_tiles), dim3(64), 0, st, set->d_views,
-                           set->d_slab_tasks, d_offs, set->d_scale_s);
-        const hipError_t launch_err = hipGetLastError();
-        const hipError_t sync_err = hipStreamSynchronize(st);
-        (void)hipFree(d_offs);
-        BITSMOE_HIP_TRY(launch_err);
-        BITSMOE_HIP_TRY(sync_err);
-    }
-    std::vector<FastExpert> fexp(set->n_experts);
-    set->expert_bits.assign(set->n_experts, 0);
-    for (int e = 0; e < set->n_experts; ++e) {
+    set->all_affine = all_uniform && all_affine;
+    set->vector_aligned = true;       // (the prepared tables are the library's own, 256-byte aligned allocations)
+
+    BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_prepared, (size_t)std::max<int64_t>(pay_words, 1) * 4));
+    // one allocation for the row tables: rank' (i32), s' (f16), scale' (f16)
+    const size_t rows_bytes = (size_t)round_up(rows_total * 4, 256) + (size_t)round_up(rows_total * 2, 256) +
+                              (size_t)round_up(scale_total * 2, 256);
+    BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_prepared_rows, std::max<size_t>(rows_bytes, 256)));
+    int32_t* d_rank = (int32_t*)set->d_prepared_rows;
+    __half* d_s = (__half*)((char*)set->d_prepared_rows + round_up(rows_total * 4, 256));
+    __half* d_scale = (__half*)((char*)d_s + round_up(rows_total * 2, 256));
+    if (role == ROLE_GATE_UP)
+        BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_scale_s, (size_t)std::max<int64_t>(scale_total, 1) * 2));
+    BITSMOE_HIP_TRY(hipMemcpyAsync(d_rank, rank_rows.data(), (size_t)rows_total * 4, hipMemcpyHostToDevice, st));
+
+    std::vector<FastExpert> fexp(E);
+    set->expert_bits.assign(E, 0);
+    for (int e = 0; e < E; ++e) {
         FastExpert& f = fexp[e];
         memset(&f, 0, sizeof(f));
-        f.scale_s = set->d_scale_s ? set->d_scale_s + sc_offs[e] : nullptr;
-        f.payload = set->d_prepared + offs[e];
-        f.scale = (const __half*)set->descs[e].scale;
-        f.s = (const __half*)set->descs[e].s;
-        f.rank_idx = (const int32_t*)set->descs[e].rank_idx;
+        f.payload = set->d_prepared + pay_off[e];
+        f.scale = d_scale + sc_off[e];
+        f.s = d_s + row_off[e];
+        f.rank_idx = d_rank + row_off[e];
+        f.scale_s = set->d_scale_s ? set->d_scale_s + sc_off[e] : nullptr;
         f.num_slabs = set->descs[e].num_slabs;
         f.uniform_bits = f.num_slabs > 0 ? set->slab_meta_host[e][0] : 0;
         for (int si = 1; si < f.num_slabs; ++si)
             if (set->slab_meta_host[e][si * 4] != f.uniform_bits) f.uniform_bits = 0;
         set->expert_bits[e] = (uint8_t)f.uniform_bits;
     }
-    set->has_cost_order = set->n_experts <= EXPERT_ORDER_MAX;
+    set->has_cost_order = E <= EXPERT_ORDER_MAX;
     if (set->has_cost_order) {
-        std::vector<int> order(set->n_experts);
-        for (int e = 0; e < set->n_experts; ++e) order[e] = e;
+        std::vector<int> order(E);
+        for (int e = 0; e < E; ++e) order[e] = e;
         auto words = [&](int e) {       // payload words per tile of expert e
             int64_t w = 0;
             for (int si = 0; si < set->descs[e].num_slabs; ++si) w += set->slab_meta_host[e][si * 4];
             return w;
         };
         std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return words(a) > words(b); });
-        for (int e = 0; e < set->n_experts; ++e) set->cost_order[e] = (uint16_t)order[e];
+        for (int e = 0; e < E; ++e) set->cost_order[e] = (uint16_t)order[e];
     }
     BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_fast_experts, sizeof(FastExpert) * fexp.size()));
     BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_fast_experts, fexp.data(), sizeof(FastExpert) * fexp.size(), hipMemcpyHostToDevice, st));
     BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_fast_slabs, sizeof(FastSlab) * fslabs.size()));
     BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_fast_slabs, fslabs.data(), sizeof(FastSlab) * fslabs.size(), hipMemcpyHostToDevice, st));
-    hipLaunchKernelGGL(k_prepack, dim3((unsigned)set->total_slabs, set->n_tiles), dim3(256), 0, st, set->d_views,
-                       set->d_views_prepared, set->d_slab_tasks, role);
+    hipLaunchKernelGGL(k_prepare_rows, dim3((unsigned)set->total_slabs, n_tiles), dim3(64), 0, st, set->d_views,
+                       set->d_fast_experts, set->d_fast_slabs, max_slabs, set->d_slab_tasks);
     BITSMOE_HIP_TRY(hipGetLastError());
-    BITSMOE_HIP_TRY(hipStreamSynchronize(st));
-    set->prepared_offsets = offs;
+    hipLaunchKernelGGL(k_prepack, dim3((unsigned)set->total_slabs, n_tiles), dim3(256), 0, st, set->d_views,
+                       set->d_fast_experts, set->d_fast_slabs, max_slabs, set->d_slab_tasks, role);
+    BITSMOE_HIP_TRY(hipGetLastError());
+    BITSMOE_HIP_TRY(hipStreamSynchronize(st));      // (the host vectors above are read by the copies until here)
+    set->fast_experts_host = fexp;
     set->role = role;
     return BITSMOE_OK;
 }
@@ -331,8 +349,9 @@ extern "C" int bitsmoe_dequant_matrix_prepared(const bitsmoe_matset* set, int32_
     BITSMOE_REQUIRE(set->role >= 0, "matrix set is not prepared");
     hipStream_t st = (hipStream_t)stream;
     const bitsmoe_matrix_desc& d = set->descs[expert];
+    if (d.num_slabs == 0) return BITSMOE_OK;
     MatView mv;
-    mv.payload = set->d_prepared + set->prepared_offsets[expert];
+    mv.payload = (const uint32_t*)d.payload;
     mv.rank_idx = (const int32_t*)d.rank_idx;
     mv.tile_meta = (const int32_t*)d.tile_meta;
     mv.slab_meta = (const int32_t*)d.slab_meta;
@@ -342,7 +361,8 @@ extern "C" int bitsmoe_dequant_matrix_prepared(const bitsmoe_matset* set, int32_
     mv.num_tiles = d.num_tiles;
     mv.rank_len = d.rank_len;
     mv.flags = 1;
-    hipLaunchKernelGGL(k_dequant_prepared, dim3(d.num_slabs, set->n_tiles), dim3(256), 0, st, mv, set->role,
+    hipLaunchKernelGGL(k_dequant_prepared, dim3(d.num_slabs, set->n_tiles), dim3(256), 0, st, mv,
+                       set->fast_experts_host[expert], set->d_fast_slabs + (int64_t)expert * set->max_slabs, set->role,
                        set->intermediate_size, out_device);
     BITSMOE_HIP_TRY(hipGetLastError());
     return BITSMOE_OK;

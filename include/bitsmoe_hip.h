@@ -79,14 +79,17 @@ int bitsmoe_matset_create(const bitsmoe_matrix_desc* descs, int32_t n_experts,
                           int32_t intermediate_size, void* stream, bitsmoe_matset** out);
 void bitsmoe_matset_destroy(bitsmoe_matset* set);
 /*
- * One-time re-layout of a set's payload into the wave64-native field layout the fast
- * kernels read (same byte count as the reference payload; the caller's buffers are not
- * modified, the library allocates the copy once and frees it in bitsmoe_matset_destroy).
+ * One-time re-layout of a set into the wave64-native copy the fast kernels read: the payload as
+ * bit FIELDS in MFMA operand order, every slab padded to 64 rows (a bit bucket whose row count is
+ * not a multiple of 64 ends in a ragged slab: bitsmoe/quant/packer.py:636-643), with row tables of
+ * its own (rank_idx, s, scale padded the same way; padding rows carry zero scales).  The caller's
+ * buffers are not modified; the library allocates the copy once and frees it in
+ * bitsmoe_matset_destroy.  The copy is a SNAPSHOT: buffers overwritten afterwards need a new set.
  * role 0: gate / up (contraction over rows), role 1: down (contraction over columns).
  * Plays the part of the reference's one-time meta build
- * (bitsmoe/algorithms/cpp/mlp_forward.cu:2529-2697).  Returns BITSMOE_E_UNSUPPORTED for
- * sets that are not "regular" (every slab 64 rows of 2/3/4 bits, full 128-column tiles,
- * 16-byte aligned payload): those run on the generic kernels only.  Synchronises `stream`.
+ * (bitsmoe/algorithms/cpp/mlp_forward.cu:2529-2697).  Returns BITSMOE_E_UNSUPPORTED for sets that
+ * hold slabs of other widths than 2, 3 or 4 bits or tiles of fewer than 128 columns: those run
+ * on the generic kernels only.  Synchronises `stream`.
  */
 int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* stream);
 /* Dense fp32 dequantisation read back FROM THE PREPARED LAYOUT (parity check of it). */
@@ -95,8 +98,9 @@ int bitsmoe_dequant_matrix_prepared(const bitsmoe_matset* set, int32_t expert, f
 
 /* info[0]=n_experts, [1]=intermediate_size, [2]=total slabs, [3]=max logical rank + 1,
  * [4]=1 if every matrix has slabs of 16-row multiples, 2/3/4-bit, full tiles,
- * [5]=largest slab count, [6]=smallest logical rank, [7]=bit0: fast kernels applicable,
- * bit1: prepared */
+ * [5]=largest slab count, [6]=smallest logical rank, [7]=bit0: bitsmoe_matset_prepare can take the
+ * set (fast kernels applicable), bit1: prepared, bit2: prepared for role 0 and every expert is one
+ * run of equal-width slabs whose rows sit in aligned runs of eight ranks (the walking gate/up kernel) */
 int bitsmoe_matset_info(const bitsmoe_matset* set, int64_t info[8]);
 
 /*

@@ -206,9 +206,32 @@ def test_prepared_layout_dequant_bit_exact(cuda_device, role, dim):
 def test_irregular_sets_stay_on_generic_kernels(cuda_device):
     hip = _hip()
     rng = np.random.default_rng(1)
-    mats = [helpers.make_matrix(rng, 80, 128, [(2, (0, 80))])]       # 64 + 16 rows: not regular
-    ms = hip.MatrixSet(*helpers.to_device_lists(mats, cuda_device), intermediate_size=128)
-    assert not ms.fast_capable and not ms.prepare(0)
+    for mats in ([helpers.make_matrix(rng, 80, 160, [(2, (0, 80))])],            # a tail tile of 32 columns
+                 [helpers.make_matrix(rng, 128, 128, [(8, (0, 64)), (2, (64, 128))])]):      # an 8-bit slab
+        ms = hip.MatrixSet(*helpers.to_device_lists(mats, cuda_device), intermediate_size=int(mats[0]["dim"]))
+        assert not ms.fast_capable and not ms.prepare(0)
+
+
+@pytest.mark.parametrize("role", [0, 1])
+def test_prepared_layout_pads_ragged_slabs(cuda_device, role):
+    """Bit buckets whose row counts are not multiples of 64 end in ragged slabs (1, 15, 17, 36, 63 rows,
+    also not multiples of the 16-row stage): the prepared copy pads them to 64 rows and decodes to
+    exactly the oracle's values."""
+    hip = _hip()
+    rng = np.random.default_rng(40 + role)
+    dim = 256
+    cases = [[(4, (0, 100)), (3, (100, 163)), (2, (163, 180))],      # 64+36 | 63 | 17
+             [(2, (0, 1))],                                            # one row
+             [(3, (0, 79)), (0, (79, 90)), (4, (90, 233))],            # 64+15 | dropped | 64+64+15
+             [(4, (0, 64)), (2, (64, 192))]]                           # nothing ragged
+    mats = [helpers.make_matrix(rng, segs[-1][1][1], dim, segs) for segs in cases]
+    ms = hip.MatrixSet(*helpers.to_device_lists(mats, cuda_device), intermediate_size=dim)
+    assert ms.fast_capable and ms.prepare(role)
+    for e, m in enumerate(mats):
+        ref = o.dequant_matrix(m, dim)
+        got = ms.dequant_prepared(e).cpu().numpy()
+        assert got.shape == ref.shape
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), f"expert {e}: prepared copy decodes differently"
 
 
 @pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
@@ -305,6 +328,56 @@ def test_forward_mfma_path_scattered_ranks(cuda_device, dtype_name):
     err = _forward_case(cuda_device, 311, 3, 260, 2, 192, 128, 256, dtype_name, (2, 3, 4),
                         path=_capi.PATH_MFMA, tol=1e-2, slab_multiple=64, scramble_ranks=True)
     assert err < 3e-3
+
+
+def _checkpoint_shaped_experts(seed, n_experts, rank, dim):
+    """Experts packed the way a checkpoint's are (bitsmoe/quant/packer.py:566-589, 615-643): per matrix three
+    width buckets in descending order of width whose sizes are no multiples of 64 (ragged last slabs), about
+    5 % of the ranks dropped (0-bit segment), and the kept rows in a permuted order of ranks."""
+    rng = np.random.default_rng(seed)
+    mats = ([], [], [])
+    for _ in range(n_experts):
+        for lst in mats:
+            perm = rng.permutation(rank)
+            n_drop = max(1, rank // 20)
+            cut1 = int(rng.integers(rank // 8, rank // 4))
+            cut2 = int(rng.integers(rank // 3, rank // 2))
+            segs = [(4, (0, cut1)), (3, (cut1, cut2)), (2, (cut2, rank - n_drop)), (0, (rank - n_drop, rank))]
+            m = helpers.make_matrix(rng, rank, dim, segs)
+            # the packer keeps rows in segment order; give them a permuted set of logical ranks
+            m["rank_idx"] = perm[m["rank_idx"]].astype(np.int32)
+            lst.append(m)
+    return mats
+
+
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+@pytest.mark.parametrize("path_name,tokens", [("decode", 9), ("decode", 70), ("mfma", 300), ("auto", 40)])
+def test_forward_checkpoint_shaped_layout_on_fast_paths(cuda_device, path_name, tokens, dtype_name):
+    """Several width buckets per expert with ragged slabs, dropped and permuted ranks: the matrix sets are
+    prepared (padded copy) and the decode / grouped-GEMM kernels run them -- not the generic fallback."""
+    import torch
+
+    from bitsmoe_amd.algorithms import _capi
+
+    hip = _hip()
+    path = {"decode": _capi.PATH_DECODE, "mfma": _capi.PATH_MFMA, "auto": _capi.PATH_AUTO}[path_name]
+    e, k, rank, dim = 6, 2, 300, 256
+    gate, up, down = _checkpoint_shaped_experts(900 + tokens, e, rank, dim)
+    rng = np.random.default_rng(tokens)
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    h_gate = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(dt)
+    h_up = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(dt)
+    idx, w = o.router_qwen(rng.normal(size=(tokens, e)).astype(np.float32), k)
+    tok, off, rw = o.build_routing(idx, w, np.arange(e, dtype=np.int32), e)
+    ref = o.moe_forward(h_gate.float().numpy(), h_up.float().numpy(), tok, off, rw, gate, up, down, rank, dim)
+    sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=dim) for m in (gate, up, down)]
+    assert all(s.fast_capable and not s.regular for s in sets)
+    out = hip.moe_forward_sets(h_gate.to(cuda_device), h_up.to(cuda_device), torch.from_numpy(tok).to(cuda_device),
+                               torch.from_numpy(off).to(cuda_device), torch.from_numpy(rw).to(cuda_device),
+                               sets[0], sets[1], sets[2], rank, dim, 0, path=path)
+    assert sets[0].role == 0 and sets[1].role == 0 and sets[2].role == 1      # prepared: the fast kernels ran
+    err = helpers.norm_err(out.cpu().numpy(), ref)
+    assert err <= 3e-3, f"normalised error {err:.3e}"
 
 
 def _scramble_down_ranks(rng, down, rank_out):
@@ -410,7 +483,7 @@ def test_forward_mfma_path_needs_prepared_sets(cuda_device):
     from bitsmoe_amd.algorithms import _capi
 
     hip = _hip()
-    gate, up, down = helpers.make_experts(5, 2, 80, 80, 128, choices=(2,), uniform_bits=True)   # 64 + 16 rows
+    gate, up, down = helpers.make_experts(5, 2, 80, 80, 128, choices=(8,), uniform_bits=True)   # 8-bit slabs: generic only
     sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=128) for m in (gate, up, down)]
     z = lambda *s, dt=torch.float16: torch.zeros(s, dtype=dt, device=cuda_device)
     with pytest.raises(RuntimeError, match="MFMA path needs"):
