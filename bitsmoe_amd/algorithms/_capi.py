@@ -43,6 +43,8 @@ EXPORTED_SYMBOLS = (
     "bitsmoe_profile_read",
     "bitsmoe_pack_bitplanes",
     "bitsmoe_unpack_bitplanes",
+    "bitsmoe_quantize_tiles",
+    "bitsmoe_pack_slabs",
 )
 
 
@@ -135,6 +137,10 @@ def load() -> ctypes.CDLL:
     lib.bitsmoe_pack_bitplanes.argtypes = [c_void_p, c_int64, c_int64, c_int32, c_void_p, c_void_p]
     lib.bitsmoe_unpack_bitplanes.restype = c_int32
     lib.bitsmoe_unpack_bitplanes.argtypes = [c_void_p, c_int64, c_int64, c_int32, c_void_p, c_void_p]
+    lib.bitsmoe_quantize_tiles.restype = c_int32
+    lib.bitsmoe_quantize_tiles.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p]
+    lib.bitsmoe_pack_slabs.restype = c_int32
+    lib.bitsmoe_pack_slabs.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_int32, c_void_p, c_void_p, c_void_p]
     _lib = lib
     return lib
 

@@ -376,6 +376,38 @@ def unpack_bitplanes(words: torch.Tensor, bits: int) -> torch.Tensor:
     return out
 
 
+def quantize_tiles(rows: torch.Tensor, bits: int, iters: int = 50) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp32 [k, dim] -> (levels int8 [k, ceil(dim/128)*128], scale fp32 [k, ceil(dim/128)]): the symmetric
+    quantiser per (row, 128-column tile), one wavefront each."""
+    _check(rows.dim() == 2 and rows.is_cuda and rows.dtype == torch.float32 and rows.stride(1) == 1,
+           "rows must be a CUDA fp32 matrix with unit column stride")
+    k, dim = int(rows.shape[0]), int(rows.shape[1])
+    n_tiles = (dim + 127) // 128
+    levels = torch.empty((k, n_tiles * 128), dtype=torch.int8, device=rows.device)
+    scale = torch.empty((k, n_tiles), dtype=torch.float32, device=rows.device)
+    with torch.cuda.device(rows.device):
+        _capi.check(_lib.bitsmoe_quantize_tiles(rows.data_ptr(), k, dim, int(rows.stride(0)) if k > 1 else dim, int(bits),
+                                                int(iters), levels.data_ptr(), scale.data_ptr(), _stream_ptr(rows.device)))
+    return levels, scale
+
+
+def pack_slabs(levels: torch.Tensor, scale: torch.Tensor, dim: int, bits: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Levels / scales of one bit bucket (quantize_tiles) -> (payload uint32 words in runtime order for the
+    bucket's slabs of <= 64 rows, fp16 scales [slab][tile][row])."""
+    k = int(levels.shape[0])
+    n_tiles = (int(dim) + 127) // 128
+    _check(levels.is_cuda and levels.dtype == torch.int8 and levels.is_contiguous() and levels.shape[1] == n_tiles * 128,
+           "levels must be a contiguous CUDA int8 [k, ceil(dim/128)*128] tensor")
+    _check(scale.dtype == torch.float32 and scale.is_contiguous() and tuple(scale.shape) == (k, n_tiles),
+           "scale must be contiguous fp32 [k, ceil(dim/128)]")
+    payload = torch.empty((k * n_tiles * 4 * int(bits),), dtype=torch.uint32, device=levels.device)
+    scale16 = torch.empty((k * n_tiles,), dtype=torch.float16, device=levels.device)
+    with torch.cuda.device(levels.device):
+        _capi.check(_lib.bitsmoe_pack_slabs(levels.data_ptr(), scale.data_ptr(), k, int(dim), int(bits), payload.data_ptr(),
+                                            scale16.data_ptr(), _stream_ptr(levels.device)))
+    return payload, scale16
+
+
 def router_softmax_topk(router_logits: torch.Tensor, top_k: int, renormalize: bool = True,
                         round_dtype: Optional[torch.dtype] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """softmax (fp32) -> top-k -> optional renormalisation -> optional round trip through

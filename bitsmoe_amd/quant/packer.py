@@ -21,7 +21,7 @@ from typing import Dict, List, Sequence, Tuple
 import torch
 from torch import Tensor
 
-from .quantizer import pack_quantized, quantize_symmetric, unpack_quantized
+from .quantizer import pack_quantized, quantize_symmetric, quantize_tiles, unpack_quantized
 
 K_SLAB = 64
 N_TILE = 128
@@ -90,6 +90,22 @@ def _quantise_bucket(rows: Tensor, bits: int) -> Tuple[Tensor, Tensor]:
     return words, scale.to(torch.float16)
 
 
+def _pack_bucket(rows: Tensor, bits: int) -> Tuple[Tensor, Tensor]:
+    """rows [k, dim] of one bit bucket -> (payload words uint32 of its slabs in runtime order, scale fp16
+    [slab][tile][row]).  Low bit-widths: the quantiser and the slab packer are kernels; 16-bit slabs
+    (raw halves, all-ones scale) are laid out with tensor ops."""
+    if bits != 16 and rows.is_cuda:
+        from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
+
+        levels, scale = quantize_tiles(rows.to(torch.float32).contiguous(), bits)
+        return hip.pack_slabs(levels, scale, int(rows.shape[1]), bits)
+    words, scale = _quantise_bucket(rows, bits)
+    k_total = int(rows.shape[0])
+    pay = [_to_runtime_order(words[r0:r0 + K_SLAB]) for r0 in range(0, k_total, K_SLAB)]
+    sc = [scale[r0:r0 + K_SLAB].t().reshape(-1) for r0 in range(0, k_total, K_SLAB)]
+    return torch.cat(pay).to(torch.uint32), torch.cat(sc).to(torch.float16)
+
+
 def _bucket_segments(segments: Sequence[Tuple[int, Tuple[int, int]]], rank: int) -> Dict[int, List[Tuple[int, int]]]:
     seen = torch.zeros(rank, dtype=torch.bool)
     buckets: Dict[int, List[Tuple[int, int]]] = {}
@@ -145,7 +161,9 @@ def pack_rank_major(rank_major: Tensor, s_vec: Tensor,
         seg_rows.append([bits, cursor, cursor + k_total])
         cursor += k_total
         idx_dev = idx.to(device=device, dtype=torch.long)
-        words, scale = _quantise_bucket(rank_major.index_select(0, idx_dev), bits)
+        bucket_payload, bucket_scale = _pack_bucket(rank_major.index_select(0, idx_dev), bits)
+        payload_parts.append(bucket_payload)
+        scale_parts.append(bucket_scale)
         s_parts.append(s_vec.index_select(0, idx_dev).to(torch.float16))
         rank_idx_parts.append(idx)
         w = _words_per_row(bits)
@@ -156,8 +174,6 @@ def pack_rank_major(rank_major: Tensor, s_vec: Tensor,
             words_tile = k_slab * MICROS_PER_TILE * w
             for t in range(n_tiles):
                 tile_rows.append([pay_off + t * words_tile, scale_off + t * k_slab, min(N_TILE, dim - t * N_TILE)])
-            payload_parts.append(_to_runtime_order(words[r0:r0 + k_slab]))
-            scale_parts.append(scale[r0:r0 + k_slab].t().reshape(-1))       # [tile][row]
             pay_off += n_tiles * words_tile
             scale_off += n_tiles * k_slab
 
@@ -168,7 +184,7 @@ def pack_rank_major(rank_major: Tensor, s_vec: Tensor,
 
     rank_idx = cat(rank_idx_parts, torch.int32, "cpu")
     return {
-        "payload_buffer": cat(payload_parts, torch.int64, device).to(torch.uint32),
+        "payload_buffer": cat([p.view(torch.int32) for p in payload_parts], torch.int32, device).view(torch.uint32),
         "rank_idx_buffer": rank_idx.to(device),
         "tile_meta_buffer": torch.tensor(tile_rows, dtype=torch.int32, device=device).reshape(-1, 3),
         "slab_meta_buffer": torch.tensor(slab_rows, dtype=torch.int32, device=device).reshape(-1, 4),

@@ -50,6 +50,26 @@ def quantize_symmetric(x: Tensor, bits: int = 8, dim: int = 0, eps: float = 1e-8
     return levels, scale.squeeze(dim)
 
 
+def quantize_tiles(rows: Tensor, bits: int, iters: int = 50):
+    """quantize_symmetric per (row, 128-column tile) of a matrix [k, dim], the way the packer applies it
+    (reference: bitsmoe/quant/packer.py:226-246, 273): (levels int8 [k, ceil(dim/128)*128] with zero
+    padding, scale fp32 [k, ceil(dim/128)]).  One kernel on the GPU; tensor ops elsewhere."""
+    if rows.is_cuda:
+        from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
+
+        return hip.quantize_tiles(rows, bits, iters)
+    k, dim = (int(v) for v in rows.shape)
+    n_tiles = (dim + 127) // 128
+    levels = torch.zeros((k, n_tiles * 128), dtype=torch.int8)
+    scale = torch.empty((k, n_tiles), dtype=torch.float32)
+    for t in range(n_tiles):
+        c0, c1 = t * 128, min(dim, t * 128 + 128)
+        q, s = quantize_symmetric(rows[:, c0:c1].to(torch.float32), bits=bits, dim=1, iters=iters)
+        levels[:, c0:c1] = q
+        scale[:, t] = s
+    return levels, scale
+
+
 def dequantize_symmetric(x_quant: Tensor, scale: Tensor, dim: int = 0) -> Tensor:
     """levels * scale, computed in fp32 and returned as fp16 (reference: quantizer.py:116-128)."""
     return (x_quant.to(torch.float32) * scale.to(torch.float32).unsqueeze(dim)).to(torch.float16)

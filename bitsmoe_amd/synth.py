@@ -16,8 +16,7 @@ import torch
 import torch.nn as nn
 
 from bitsmoe_amd.models.dense import DenseSwiGLUMLP, SoftmaxGreedyGate
-from bitsmoe_amd.quant.packer import (K_SLAB, K_STAGE, MICROS_PER_TILE, N_TILE, _quantise_bucket, _words_per_row,
-                                      pack_rank_major)
+from bitsmoe_amd.quant.packer import K_SLAB, MICROS_PER_TILE, N_TILE, _pack_bucket, _words_per_row, pack_rank_major
 
 
 @dataclass
@@ -77,12 +76,11 @@ def pack_uniform_experts(weights: torch.Tensor, bits: int) -> Dict[str, object]:
     device = weights.device
     n_tiles = (dim + N_TILE - 1) // N_TILE
     w = _words_per_row(bits)
-    words, scale = _quantise_bucket(weights.reshape(n * k, dim), bits)       # [n*k, tiles, 4, w]
+    # K is a multiple of 64, so the slabs of the n * K rows taken as one bucket never straddle two matrices
+    payload, scale = _pack_bucket(weights.reshape(n * k, dim), bits)
+    payload = payload.view(n, -1)
+    scale = scale.view(n, -1)
     slabs = k // K_SLAB
-    stages = K_SLAB // K_STAGE
-    words = words.view(n, slabs, stages, K_STAGE, n_tiles, MICROS_PER_TILE, w)
-    payload = words.permute(0, 1, 4, 2, 5, 3, 6).reshape(n, -1).to(torch.uint32).contiguous()
-    scale = scale.view(n, slabs, K_SLAB, n_tiles).permute(0, 1, 3, 2).reshape(n, -1).contiguous()
     words_tile = K_SLAB * MICROS_PER_TILE * w
     slab_rows, tile_rows = [], []
     for s in range(slabs):

@@ -248,6 +248,25 @@ int bitsmoe_pack_bitplanes(const int8_t* levels, int64_t rows, int64_t cols, int
 int bitsmoe_unpack_bitplanes(const uint32_t* words, int64_t rows, int64_t groups,
                              int32_t bits, int8_t* levels_out, void* stream);
 
+/*
+ * The quantiser that defines the payload's contents, one wavefront per (row, 128-column tile).
+ * Replaces quantize_symmetric as the packer calls it (bitsmoe/quant/quantizer.py:30-84 through
+ * bitsmoe/quant/packer.py:226-246, 273): rows fp32 [k, dim] (row_stride elements apart) ->
+ * levels int8 [k, ceil(dim/128)*128] (padding columns 0), scale fp32 [k, ceil(dim/128)].
+ * bits 2/3/4: mean-abs start and `iters` least-squares refinements (the reference uses 50);
+ * 6/8: absmax; 1: sign and mean-abs.
+ */
+int bitsmoe_quantize_tiles(const float* rows, int64_t k, int64_t dim, int64_t row_stride, int32_t bits,
+                           int32_t iters, int8_t* levels_out, float* scale_out, void* stream);
+/*
+ * Slab packer for the rows of ONE bit bucket.  Replaces _pack_lowbit_slab_payload_and_scale +
+ * _reorder_packed_rows_to_runtime_layout (bitsmoe/quant/packer.py:169-306): levels as written by
+ * bitsmoe_quantize_tiles -> payload words [slab of <= 64 rows][tile][stage][micro][row][plane]
+ * (k * ceil(dim/128) * 4 * bits words) and fp16 scales [slab][tile][row] (k * ceil(dim/128)).
+ */
+int bitsmoe_pack_slabs(const int8_t* levels, const float* scale, int64_t k, int64_t dim, int32_t bits,
+                       uint32_t* payload_out, void* scale_out_f16, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

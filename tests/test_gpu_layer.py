@@ -43,6 +43,43 @@ def test_gpu_packer_matches_oracle_packer(cuda_device, rank, dim):
                             bufs["rank_idx_buffer"], bufs["payload_buffer"], bufs["scale_buffer"])
 
 
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 6, 8])
+@pytest.mark.parametrize("k,dim", [(70, 160), (64, 128), (1, 32), (150, 768)])
+def test_quantiser_and_slab_packer_kernels(cuda_device, bits, k, dim):
+    """bitsmoe_quantize_tiles: the levels are the CPU restatement's except where x / scale sits on a
+    rounding tie (the wavefront's summation order moves a scale by an ulp), scales agree to fp32 rounding.
+    bitsmoe_pack_slabs: the words built from the kernel's OWN levels are exactly the words the oracle's
+    bit-plane packer and runtime reorder give for those levels (ragged last slab, tail tile included)."""
+    import torch
+
+    from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
+
+    rng = np.random.default_rng(bits * 1000 + k + dim)
+    x = rng.normal(0, 0.02, size=(k, dim)).astype(np.float32)
+    n_tiles = (dim + 127) // 128
+    levels, scale = hip.quantize_tiles(torch.from_numpy(x).to(cuda_device), bits)
+    levels_n, scale_n = levels.cpu().numpy(), scale.cpu().numpy()
+    assert levels_n.shape == (k, n_tiles * 128) and scale_n.shape == (k, n_tiles)
+    mismatched = 0
+    for t in range(n_tiles):
+        c0, c1 = t * 128, min(dim, t * 128 + 128)
+        q_ref, s_ref = o.quantize_symmetric(x[:, c0:c1], bits)
+        assert np.allclose(scale_n[:, t], s_ref, rtol=2e-5, atol=0)
+        mismatched += int((levels_n[:, c0:c1] != q_ref).sum())
+        assert not levels_n[:, c1:t * 128 + 128].any()          # padding columns hold level 0
+    assert mismatched <= max(1, int(2e-4 * k * dim)), f"{mismatched} levels differ from the oracle"
+    payload, scale16 = hip.pack_slabs(levels, scale, dim, bits)
+    pay_ref, sc_ref = [], []
+    for r0 in range(0, k, 64):
+        k_slab = min(64, k - r0)
+        packed = o.pack_bitplanes(levels_n[r0:r0 + k_slab], bits)
+        rows = packed.reshape(k_slab, n_tiles, 4, bits).transpose(1, 0, 2, 3)
+        pay_ref.append(o._runtime_order(rows, k_slab).reshape(-1))
+        sc_ref.append(scale_n[r0:r0 + k_slab].T.reshape(-1).astype(np.float16))
+    assert np.array_equal(payload.cpu().view(torch.int32).numpy().view(np.uint32), np.concatenate(pay_ref))
+    assert np.array_equal(scale16.cpu().numpy(), np.concatenate(sc_ref))
+
+
 def test_batched_uniform_packer_equals_general_packer(cuda_device):
     import torch
 
