@@ -47,6 +47,8 @@ WORKLOADS = {
     "c2-t32": ("c2", 32, "hbm"),
     "c2-t64": ("c2", 64, "hbm"),
     "c3-t4096": ("c3", 4096, "mfma"),
+    "c2-ckpt-t64": ("c2", 64, "hbm"),
+    "c3-ckpt-t4096": ("c3", 4096, "mfma"),
     "c5-stack-t32": ("c5", 32, "hbm"),
     "c5-stack-t2048": ("c5", 2048, "mfma"),
 }
@@ -385,23 +387,28 @@ def main() -> int:
     use_graph = not args.no_graph
     built = {}       # spec key of the layer shape -> its distinct copies (c2 and c3 are one layer shape and seed)
 
-    def blocks_of(spec_key):
+    def blocks_of(spec_key, layout="uniform"):
         shape_key = "c2" if spec_key == "c3" else spec_key
+        if layout != "uniform":
+            shape_key += "/" + layout
         if shape_key not in built:
             spec = SPECS[spec_key]
             n = spec.n_layers if spec.n_layers > 1 else max(1, args.layers)
             t0 = time.perf_counter()
             # (the stack shares its three orthonormal bases between the layers: they are outside the operator
             # and factorising 78 matrices of 2048 x 2048 on the host would take longer than the benchmark)
-            built[shape_key] = [make_layer(SPECS[shape_key], device=dev, dtype=torch.bfloat16, seed=42, layer_idx=i,
-                                           basis_seed=(42 if spec.n_layers > 1 else None)) for i in range(n)]
+            built[shape_key] = [make_layer(SPECS[shape_key.split("/")[0]], device=dev, dtype=torch.bfloat16, seed=42, layer_idx=i,
+                                           basis_seed=(42 if spec.n_layers > 1 or layout != "uniform" else None),
+                                           layout=layout) for i in range(n)]
             torch.cuda.synchronize()
             built[shape_key + "/build_s"] = time.perf_counter() - t0
         return built[shape_key]
 
     def measure(name, steps, warmup):
         skey, toks, bnd = WORKLOADS[name]
-        blocks = blocks_of(skey)
+        # "-ckpt-": the same shape with checkpoint-shaped matrices (three widths per matrix, ragged slabs,
+        # dropped ranks) instead of one width per expert
+        blocks = blocks_of(skey, "checkpoint" if "-ckpt-" in name else "uniform")
         stack = SPECS[skey].n_layers > 1
         if stack:       # one step = one pass over the whole stack
             r, inp = run_workload(blocks, SPECS[skey], toks, max(2, steps // len(blocks)), max(1, warmup // len(blocks)),

@@ -27,6 +27,13 @@ from bitsmoe_amd.models.base_mlp import buffer_generation
 _BUFFER_NAMES = ("payload", "rank_idx", "tile_meta", "slab_meta", "scale", "s")
 
 
+def _dense_via_operator() -> bool:
+    """BITSMOE_DENSE_VIA_OPERATOR=1: shared and super experts run as 16-bit packed experts of the operator."""
+    import os
+
+    return os.environ.get("BITSMOE_DENSE_VIA_OPERATOR", "0") == "1"
+
+
 class BitsMoE_BaseSparseMoeBlock(nn.Module):
     _SHARED_BASIS_BUFFER_KEYS = ("shared_vh_gate_proj", "shared_vh_up_proj", "shared_u_down")
 
@@ -107,6 +114,7 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         self._cached_token_count = -1
         self._cached_flat_token_ids: Optional[torch.Tensor] = None
         self._matsets = None
+        self._dense_sets: Dict[str, object] = {}         # dense experts packed as 16-bit matrix sets (per kind)
         self._buffer_generation_seen = -1
         self._basis_cache: Dict[object, object] = {}      # per dtype: the three bases; ("stacked", dtype): gate over up
 
@@ -228,13 +236,80 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
 
     def _run_super_experts(self, hidden_states, final_hidden_states, flat_selected_experts, flat_token_ids,
                            flat_route_weights_hidden) -> None:
+        """Dense "super" experts (reference: bitsmoe/models/base_block.py:291-307) without the reference's
+        host synchronisation (`mask.any()` and boolean-mask indexing read the device per expert): the
+        block stays capturable into a HIP graph when a layer has super experts.
+          * default: each super expert runs on ALL tokens and its output is scaled by the token's routing
+            weight for that expert -- zero where the token did not select it (library GEMMs; a handful of
+            experts in a few layers, so the extra rows cost little at decode sizes);
+          * BITSMOE_DENSE_VIA_OPERATOR=1: the super experts are packed as 16-bit matrices once and go through
+            the routed-expert operator like any packed expert (device-built routing tables, work
+            proportional to the tokens that selected them)."""
+        if not self._super_expert_items:
+            return
+        top_k = self.top_k
+        sel = flat_selected_experts.reshape(-1, top_k)
+        w = flat_route_weights_hidden.reshape(-1, top_k)
+        if _dense_via_operator():
+            g2l = self._super_global_to_local(hidden_states.device)
+            tok, off, rw = mlp_forward_cuda.route(sel, w.to(torch.float32), g2l, len(self._super_expert_items))
+            out = self._dense_operator_forward("super", [layer for _, layer in self._super_expert_items],
+                                               hidden_states, tok, off, rw)
+            final_hidden_states.add_(out.to(hidden_states.dtype))
+            return
         for expert_idx, layer in self._super_expert_items:
-            mask = flat_selected_experts == expert_idx
-            if not bool(mask.any()):
-                continue
-            token_ids = flat_token_ids[mask]
-            out = layer(hidden_states.index_select(0, token_ids)) * flat_route_weights_hidden[mask].unsqueeze(-1)
-            final_hidden_states.index_add_(0, token_ids, out.to(hidden_states.dtype))
+            weight = (w * (sel == expert_idx).to(w.dtype)).sum(dim=1, keepdim=True)      # 0 where not selected
+            final_hidden_states.add_((layer(hidden_states) * weight).to(hidden_states.dtype))
+
+    # ---- dense experts through the routed-expert operator ----------------------------------
+    def _super_global_to_local(self, device: torch.device) -> torch.Tensor:
+        cached = self._basis_cache.get(("super_g2l", str(device)))
+        if cached is None:
+            g2l = torch.full((self.num_experts,), -1, dtype=torch.int32)
+            for local, (idx, _) in enumerate(self._super_expert_items):
+                g2l[idx] = local
+            cached = g2l.to(device)
+            self._basis_cache[("super_g2l", str(device))] = cached
+        return cached
+
+    def _dense_operator_forward(self, key: str, modules, hidden_states: torch.Tensor, token_indices: torch.Tensor,
+                                expert_offsets: torch.Tensor, route_flat: torch.Tensor) -> torch.Tensor:
+        """Dense SwiGLU experts as packed 16-bit matrices through moe_forward_sets: fp32 [tokens, hidden].
+        The packed copies are made once per block (a snapshot of the modules' weights; cleared with the
+        runtime cache)."""
+        from bitsmoe_amd.models.dense import pack_dense_mlps
+
+        packed = self._dense_sets.get(key)
+        if packed is None:
+            gate_l, up_l, down_l, inter = pack_dense_mlps(modules, hidden_states.device)
+            sets = tuple(mlp_forward_cuda.MatrixSet(*lists, intermediate_size=inter, name=f"{key}_{p}")
+                         for lists, p in ((gate_l, "gate"), (up_l, "up"), (down_l, "down")))
+            packed = (sets, inter)
+            self._dense_sets[key] = packed
+        (gate, up, down), inter = packed
+        hidden = int(hidden_states.shape[1])
+        x = hidden_states.contiguous()
+        return mlp_forward_cuda.moe_forward_sets(x, x, token_indices, expert_offsets, route_flat, gate, up, down,
+                                                 hidden, inter, self._act_type())
+
+    def _always_on_forward(self, key: str, module, hidden_states: torch.Tensor,
+                           token_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """A shared expert (every token, weight 1 or `token_weights` [tokens, 1]) -> [tokens, hidden] in the
+        activation dtype: the module itself (library GEMMs), or with BITSMOE_DENSE_VIA_OPERATOR=1 an
+        always-on 16-bit expert of the routed-expert operator."""
+        if not _dense_via_operator():
+            out = module(hidden_states)
+            return out if token_weights is None else token_weights.to(out.dtype) * out
+        t = int(hidden_states.shape[0])
+        dev = hidden_states.device
+        cached = self._basis_cache.get(("always_on", t, str(dev)))
+        if cached is None:
+            cached = (torch.arange(t, dtype=torch.int32, device=dev), torch.tensor([0, t], dtype=torch.int32, device=dev),
+                      torch.ones((t,), dtype=torch.float32, device=dev))
+            self._basis_cache[("always_on", t, str(dev))] = cached
+        tok, off, ones = cached
+        rw = ones if token_weights is None else token_weights.reshape(-1).to(torch.float32).contiguous()
+        return self._dense_operator_forward(key, [module], hidden_states, tok, off, rw).to(hidden_states.dtype)
 
     def prepare_runtime_fastpath(self, warmup: bool = True) -> None:
         device = self._runtime_device()

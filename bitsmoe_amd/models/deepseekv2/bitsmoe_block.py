@@ -41,5 +41,7 @@ class BitsMoE_DeepSeekSparseMoeBlock(BitsMoE_BaseSparseMoeBlock):
         weights = topk_weight.reshape(-1, topk_weight.shape[-1]).to(torch.float32)
         y = self._routed_forward(hidden_states, selected, weights).reshape(*orig_shape)
         if getattr(self.config, "n_shared_experts", None) is not None and hasattr(self, "shared_experts"):
-            y = y + self.shared_experts(identity)
+            # (reference: bitsmoe/models/deepseekv2/bitsmoe_block.py:123-124)
+            shared = self._always_on_forward("shared", self.shared_experts, identity.reshape(-1, orig_shape[-1]))
+            y = y + shared.reshape(*orig_shape)
         return y

@@ -46,3 +46,33 @@ class SoftmaxGreedyGate(nn.Module):
         else:
             weight = weight * self.routed_scaling_factor
         return idx, weight, None
+
+
+def pack_dense_mlps(modules, device=None):
+    """Dense SwiGLU experts (modules with bias-free gate_proj / up_proj / down_proj linears) as packed
+    16-bit matrices the routed-expert operator can run: the slab layout stores fp16 halves as they are
+    (bitsmoe/quant/packer.py:309-374), so a dense expert is a packed expert whose "basis" is the identity:
+        gate / up   rank-major [hidden, intermediate] = W.T   (row k multiplies x[:, k])
+        down        rank-major [hidden, intermediate] = W     (row r is output column r)
+    with rank_idx = arange(hidden) and s = 1.  The operator is then called with h_gate = h_up = x and
+    rank_out = hidden, and returns the experts' output in hidden space.
+    Returns (gate_lists, up_lists, down_lists, intermediate_size): the six buffer lists per projection."""
+    from bitsmoe_amd.quant.packer import pack_rank_major
+
+    names = ("payload_buffer", "rank_idx_buffer", "tile_meta_buffer", "slab_meta_buffer", "scale_buffer", "s_buffer")
+    lists = {p: tuple([] for _ in names) for p in ("gate", "up", "down")}
+    inter = None
+    for mod in modules:
+        wg, wu, wd = mod.gate_proj.weight, mod.up_proj.weight, mod.down_proj.weight
+        dev = wg.device if device is None else device
+        hidden = int(wg.shape[1])
+        inter = int(wg.shape[0]) if inter is None else inter
+        if int(wg.shape[0]) != inter or tuple(wu.shape) != tuple(wg.shape) or tuple(wd.shape) != (hidden, inter):
+            raise ValueError("dense experts of one set must share their shapes")
+        ones = torch.ones((hidden,), dtype=torch.float32, device=dev)
+        for proj, mat in (("gate", wg.detach().t()), ("up", wu.detach().t()), ("down", wd.detach())):
+            bufs = pack_rank_major(mat.to(device=dev, dtype=torch.float32).contiguous(), ones, [(16, (0, hidden))])
+            for lst, name in zip(lists[proj], names):
+                lst.append(bufs[name])
+    return (tuple(tuple(x) for x in lists["gate"]), tuple(tuple(x) for x in lists["up"]),
+            tuple(tuple(x) for x in lists["down"]), inter)

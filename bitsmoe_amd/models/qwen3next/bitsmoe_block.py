@@ -28,6 +28,7 @@ class BitsMoE_Qwen3NextSparseMoeBlock(BitsMoE_Qwen3MoeSparseMoeBlock):
         router_logits, selected, weights = self._route(hidden_states)
         final = self._routed_forward(hidden_states, selected, weights)
         if hasattr(self, "shared_expert") and hasattr(self, "shared_expert_gate"):
-            shared = self.shared_expert(hidden_states)
-            final = final + torch.sigmoid(self.shared_expert_gate(hidden_states)) * shared
+            # (reference: bitsmoe/models/qwen3next/bitsmoe_block.py:144-147)
+            gate = torch.sigmoid(self.shared_expert_gate(hidden_states))
+            final = final + self._always_on_forward("shared", self.shared_expert, hidden_states, gate)
         return final.reshape(batch_size, sequence_length, hidden_dim), router_logits

@@ -96,6 +96,41 @@ def pack_uniform_experts(weights: torch.Tensor, bits: int) -> Dict[str, object]:
     }
 
 
+def checkpoint_segments(rank: int, g: torch.Generator) -> List[Tuple[int, Tuple[int, int]]]:
+    """Bit allocation over the ranks of one matrix the way a compressed checkpoint has it
+    (bitsmoe/quant/packer.py:566-589): the leading ranks get 4 bits, the next 3, the bulk 2, the last
+    ones are dropped; the cut points are arbitrary (no multiples of 64: every bucket ends in a ragged slab).
+    About 4 % / 12 % / 79 % / 5 % of the ranks: 2.1 bits per kept-or-dropped rank on average."""
+    r = torch.rand(3, generator=g)
+    c1 = max(1, int(rank * (0.02 + 0.04 * float(r[0]))))
+    c2 = max(c1 + 1, int(rank * (0.12 + 0.08 * float(r[1]))))
+    keep = min(rank, max(c2 + 1, int(rank * (0.93 + 0.04 * float(r[2])))))
+    segs = [(4, (0, c1)), (3, (c1, c2)), (2, (c2, keep))]
+    if keep < rank:
+        segs.append((0, (keep, rank)))
+    return segs
+
+
+def make_checkpoint_shaped_experts(spec: LayerSpec, seed: int, device, mlp_cls, config) -> List[nn.Module]:
+    """E packed expert containers whose matrices mix three widths with ragged slabs and dropped ranks."""
+    k = int(spec.rank or spec.hidden_size)
+    dim = spec.intermediate_size
+    experts = [mlp_cls(config, intermediate_size=dim) for _ in range(spec.num_experts)]
+    g = torch.Generator(device=device).manual_seed(seed)
+    g_cpu = torch.Generator().manual_seed(seed)
+    ones = torch.ones((k,), dtype=torch.float32, device=device)
+    for mod in experts:
+        for tag in ("gate", "up", "down"):
+            w = torch.randn((k, dim), generator=g, device=device, dtype=torch.float32) * 0.02
+            bufs = pack_rank_major(w, ones, checkpoint_segments(k, g_cpu))
+            for name in ("payload_buffer", "rank_idx_buffer", "tile_meta_buffer", "slab_meta_buffer", "scale_buffer",
+                         "s_buffer", "segments", "original_indices", "original_rank", "groupsize"):
+                mod._bind(f"{tag}_{name}", bufs[name])
+        mod.is_bitsmoe_packed = True
+        mod.skip_expert = False
+    return experts
+
+
 def make_packed_experts(spec: LayerSpec, bits: Sequence[int], seed: int, device, mlp_cls, config,
                         s_mode: str = "ones") -> List[nn.Module]:
     """The E packed expert containers of one layer."""
@@ -151,10 +186,13 @@ _BASIS_CACHE: Dict[Tuple[int, int, str], torch.Tensor] = {}
 
 
 def make_layer(spec: LayerSpec, device="cuda", dtype=torch.bfloat16, seed: int = 42, layer_idx: int = 0,
-               s_mode: str = "ones", basis_seed: Optional[int] = None) -> nn.Module:
+               s_mode: str = "ones", basis_seed: Optional[int] = None, layout: str = "uniform",
+               super_experts: Sequence[int] = ()) -> nn.Module:
     """A ready-to-run sparse-MoE block of `spec`'s family on `device`.  `basis_seed`: take the three
     shared bases from this seed instead of the layer's own (layers of a stack may share them: the
-    host factorisation of three 2048 x 2048 matrices per layer dominates the build otherwise)."""
+    host factorisation of three 2048 x 2048 matrices per layer dominates the build otherwise).
+    layout "uniform": one bit-width per expert (the benchmark configurations); "checkpoint": three widths
+    per matrix with arbitrary cut points and dropped ranks (make_checkpoint_shaped_experts)."""
     from bitsmoe_amd.models.deepseekv2.bitsmoe_block import BitsMoE_DeepSeekSparseMoeBlock
     from bitsmoe_amd.models.deepseekv2.bitsmoe_mlp import BitsMoE_DeepSeekMLP
     from bitsmoe_amd.models.qwen3moe.bitsmoe_block import BitsMoE_Qwen3MoeSparseMoeBlock
@@ -188,11 +226,24 @@ def make_layer(spec: LayerSpec, device="cuda", dtype=torch.bfloat16, seed: int =
     with torch.no_grad():
         for p in src.parameters():
             p.copy_((torch.randn(p.shape, generator=g, device=device, dtype=torch.float32) * 0.02).to(p.dtype))
-    block = block_cls(config, layer_idx, source_block=src)
+    block = block_cls(config, layer_idx, source_block=src, super_experts=list(super_experts))
     bits = draw_bits(spec, seed)
-    experts = make_packed_experts(spec, bits, seed * 104729 + 3, device, mlp_cls, config, s_mode=s_mode)
+    if layout == "checkpoint":
+        experts = make_checkpoint_shaped_experts(spec, seed * 104729 + 3, device, mlp_cls, config)
+        bits = []
+        for mod in experts:      # mean bits per stored row, for the record
+            seg = mod.gate_segments.tolist()
+            bits.append(sum(b * (e - s) for b, s, e in seg) / max(1, sum(e - s for _, s, e in seg)))
+    else:
+        experts = make_packed_experts(spec, bits, seed * 104729 + 3, device, mlp_cls, config, s_mode=s_mode)
     for e, mod in enumerate(experts):
         block.set_expert(e, mod, packed=True)
+    for e in super_experts:       # dense routed experts that stay unquantised (bitsmoe/models/base_block.py:291-307)
+        dense = DenseSwiGLUMLP(h, spec.intermediate_size, dtype=dtype, device=device)
+        with torch.no_grad():
+            for p in dense.parameters():
+                p.copy_((torch.randn(p.shape, generator=g, device=device, dtype=torch.float32) * 0.02).to(p.dtype))
+        block.set_expert(int(e), dense, packed=False)
     r = int(spec.rank or h)
     bseed = seed if basis_seed is None else int(basis_seed)
 

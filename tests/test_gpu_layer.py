@@ -116,7 +116,7 @@ def _block_reference(block, x):
     spec = block.spec
     isz = spec.intermediate_size
     mats = [[helpers.from_torch_matrix(*[lst[e] for lst in block._static_lists(p)], isz)
-             for e in range(spec.num_experts)] for p in ("gate", "up", "down")]
+             for e in range(block._packed_expert_count)] for p in ("gate", "up", "down")]
     x64 = x.float().cpu().numpy().astype(np.float64)
     if spec.family == "deepseekv2":
         gw = block.gate.weight.detach().float().cpu().numpy()
@@ -130,12 +130,20 @@ def _block_reference(block, x):
         w = helpers.bf16_round(w)       # the weights take a round trip through the activation dtype
     y = o.block_forward(x64, block.shared_vh_gate_proj.float().cpu().numpy(),
                         block.shared_vh_up_proj.float().cpu().numpy(), block.shared_u_down.float().cpu().numpy(),
-                        idx, w, mats[0], mats[1], mats[2], isz)
+                        idx, w, mats[0], mats[1], mats[2], isz,
+                        global_to_local=block._packed_global_to_local.cpu().numpy())
 
     def dense_mlp(mod, inp):
         f = lambda lin: lin.weight.detach().float().cpu().numpy().astype(np.float64)
         g, u = inp @ f(mod.gate_proj).T, inp @ f(mod.up_proj).T
         return (g / (1 + np.exp(-g)) * u) @ f(mod.down_proj).T
+
+    # dense "super" experts: the tokens that selected them, weighted by the routing weight
+    # (bitsmoe/models/base_block.py:291-307)
+    for e_idx, layer in block._super_expert_items:
+        hit = (idx == e_idx)
+        weight = (np.asarray(w, np.float64) * hit).sum(axis=1, keepdims=True)
+        y = y + weight * dense_mlp(layer, x64)
 
     if spec.family == "qwen3next":
         gate_w = block.shared_expert_gate.weight.detach().float().cpu().numpy().astype(np.float64)
@@ -169,3 +177,46 @@ def test_block_forward_matches_oracle(cuda_device, family, kw, tokens):
     ref, idx = _block_reference(block, x.reshape(tokens, -1))
     err = helpers.norm_err(y.float().cpu().numpy().reshape(tokens, -1), ref)
     assert err <= 1e-2, f"{family}: normalised error {err:.3e}"
+
+
+@pytest.mark.parametrize("via_operator", [False, True])
+@pytest.mark.parametrize("family,kw", [("qwen3moe", {}), ("qwen3next", {"shared_intermediate": 128}),
+                                       ("deepseekv2", {"shared_intermediate": 256})])
+def test_block_with_super_and_shared_experts(cuda_device, family, kw, via_operator, monkeypatch):
+    """A layer with two dense "super" experts among the routed ones (and the family's shared expert): the
+    block against the float64 restatement, with the dense experts as library GEMMs and as 16-bit packed
+    experts of the operator (BITSMOE_DENSE_VIA_OPERATOR=1); the forward does not synchronise with the
+    host, so it is captured into a HIP graph and every replay must equal the eager result."""
+    import torch
+
+    from bitsmoe_amd.synth import make_layer
+
+    monkeypatch.setenv("BITSMOE_DENSE_VIA_OPERATOR", "1" if via_operator else "0")
+    spec = _small_spec(family, **kw)
+    block = make_layer(spec, device=cuda_device, dtype=torch.bfloat16, seed=9, s_mode="rand", super_experts=(1, 6))
+    block.prepare_runtime_fastpath(warmup=True)
+    assert [i for i, _ in block._super_expert_items] == [1, 6] and block._packed_expert_count == spec.num_experts - 2
+    tokens = 24
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn((1, tokens, spec.hidden_size), generator=g).to(torch.bfloat16).to(cuda_device)
+    first = lambda out: out[0] if isinstance(out, tuple) else out
+    with torch.no_grad():
+        y = first(block(x))
+    ref, idx = _block_reference(block, x.reshape(tokens, -1))
+    assert (idx == 1).any() and (idx == 6).any()           # the super experts are in use
+    err = helpers.norm_err(y.float().cpu().numpy().reshape(tokens, -1), ref)
+    assert err <= 1e-2, f"{family}: normalised error {err:.3e}"
+    # graph capture: impossible with a host synchronisation inside the forward
+    side = torch.cuda.Stream(device=cuda_device)
+    side.wait_stream(torch.cuda.current_stream(cuda_device))
+    with torch.cuda.stream(side), torch.no_grad():
+        first(block(x))
+    torch.cuda.current_stream(cuda_device).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.no_grad(), torch.cuda.graph(graph):
+        yg = first(block(x))
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert float((yg.float() - y.float()).abs().max()) <= 2e-2 * float(y.float().abs().max())
