@@ -108,10 +108,16 @@ struct bitsmoe_matset {
     // experts by decreasing payload size (prepared sets of at most EXPERT_ORDER_MAX experts): the
     // decode kernels start the expensive experts' workgroups first
     std::vector<uint8_t> expert_bits;   // prepared sets: the bit-width all slabs of an expert share, or 0
+    bool uniform_experts = false;       // prepared sets: no expert mixes widths
     bool has_cost_order = false;
     uint16_t cost_order[512] = {};
     uint32_t* d_prepared = nullptr;   // wave-native copy of every payload (see wave_layout.h), every slab padded to 64 rows
-    void* d_prepared_rows = nullptr;  // the prepared copy's row tables: rank_idx', s', scale' (padded the same way)
+    void* d_prepared_rows = nullptr;  // the prepared copy's row tables: rank_idx', source of each row, s', scale'
+    bitsmoe::SlabTask* d_prep_tasks = nullptr;       // (expert, slab) of every slab of the prepared copy
+    int32_t prep_max_slabs = 0;       // largest slab count of the prepared copy (row stride of d_fast_slabs)
+    int32_t pad_rank_plus1 = 0;       // 1 + largest rank the prepared rank table holds, padding rows included
+    std::vector<int64_t> prep_row_offsets;
+    const int32_t* d_row_src = nullptr;   // (inside d_prepared_rows)
     std::vector<bitsmoe::FastExpert> fast_experts_host;
     std::vector<std::vector<int32_t>> rank_idx_host;
     bitsmoe::FastExpert* d_fast_experts = nullptr;   // [n_experts]

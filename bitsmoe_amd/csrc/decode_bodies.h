@@ -326,6 +326,170 @@ __device__ __forceinline__ void gateup_walk_item(gptr<uint32_t> payload, gptr<__
     }
 }
 
+// ------------------------------------- the same walk for experts whose slab groups differ in width
+// An expert of a compressed checkpoint mixes widths (the leading ranks 4 bits, then 3, the bulk 2:
+// bitsmoe/quant/packer.py:566-589); the prepared copy stores every group of GU_SLABS slabs at ONE width, so
+// the walk only has to switch the decode between groups.  Everything but the payload is laid out alike
+// for all widths (row g*512 + 8*lane of the rank table, scale row (g*8 + q) * n_tiles * 64): only the
+// payload address and the field decode depend on the group's width.
+// `grp_tab[g]` (LDS) = (width, payload word offset of the group's first slab) for g < n_groups; the caller
+// fills it and puts a workgroup barrier behind it.
+constexpr int WALK_MAX_GROUPS = 32;      // 16384 contraction rows
+template <bool BF16, bool IDENT, bool SPLIT>
+__device__ __forceinline__ void gateup_walk_item_mixed(gptr<uint32_t> payload, gptr<__half> scale_s, gptr<int32_t> rank_idx,
+                                                       const int2* __restrict__ grp_tab, const uint16_t* __restrict__ h,
+                                                       int64_t ld, const int32_t* __restrict__ token_indices, int a0, int n_a,
+                                                       int A, int T, int I, int n_tiles, int t, int g_begin, int g_end,
+                                                       float* __restrict__ out, uint16_t* __restrict__ hs_all,
+                                                       float* __restrict__ cterm_lds, int tid) {
+    const int pair = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform
+    // (`lane` is given an opaque copy per group below: what a group's body derives from it -- block
+    // offsets, LDS addresses, masks -- is then computed inside that body instead of being hoisted out of
+    // the loop over groups for all nine bodies at once, which costs more registers than there are)
+    int lane = tid & 63;
+    int n = lane & 15, kg = lane >> 4;
+    uint32_t unit = (uint32_t)(pair * 64 + lane);
+    uint32_t hi_unit = (uint32_t)hi_index0(kg, n, 2 * pair);
+    int item_zero = 0;
+    asm volatile("" : "+s"(item_zero));   // keeps this item's address arithmetic out of the caller's loop
+    auto group_rec = [&](int g) {      // (width, payload word offset of slab 8 g's block of tile t)
+        const int2 v = grp_tab[g];
+        const int w = __builtin_amdgcn_readfirstlane(v.x);
+        return int2{w, __builtin_amdgcn_readfirstlane(v.y) + t * 256 * w + item_zero};
+    };
+
+    uint32_t pw[GU_SLABS][4];   // slab q's block of the current group; refilled for the next group right after use
+    // slab q of a group of width w whose first block starts at word pack0
+    auto issue_at = [&](auto q_c, int w, int pack0) {
+        constexpr int q = decltype(q_c)::value;
+        load_pair_role0(payload + (uint32_t)(pack0 + q * (n_tiles * 256 * w)), w, unit, hi_unit, pw[q]);
+    };
+    int tki[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) tki[i] = token_indices[min(a0 + pair + 4 * i, A - 1)];
+    auto rank_at = [&](int g) {
+        const int k = g * (GU_SLABS * SLAB_ROWS) + 8 * lane;
+        if constexpr (IDENT) return k;
+        else return (int)rank_idx[k];
+    };
+    auto scale_at = [&](int g) {
+        return *reinterpret_cast<gptr_u32x4>(
+            scale_s + (uint32_t)(((g * GU_SLABS + (lane >> 3)) * n_tiles + t) * SLAB_ROWS + 8 * (lane & 7)));
+    };
+    const uint16_t* trow[4];
+    auto act_at = [&](int i, int rank) { return *reinterpret_cast<const u32x4*>(trow[i] + rank); };
+    uint16_t* hs = hs_all;
+    float cterm[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    int rank_cur = rank_at(g_begin);
+    int rank_nxt = g_begin + 1 < g_end ? rank_at(g_begin + 1) : 0;
+    u32x4 sc_cur = scale_at(g_begin);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) trow[i] = h + (int64_t)min(max(__builtin_amdgcn_readfirstlane(tki[i]), 0), T - 1) * ld;
+    u32x4 raw0 = act_at(0, rank_cur);
+    u32x4 raw1 = act_at(1, rank_cur);
+    int2 rec = group_rec(g_begin);
+    f32x4 acc[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+    f32x4 corr = {0, 0, 0, 0};
+    // W: this group's width.  SAME: the next group exists and has this width (its payload is requested between
+    // this group's blocks); MORE: a next group exists (its ranks, scales and activations are requested).
+    auto group_step = [&](auto w_c, auto same_c, auto more_c, int g, int pack0) {
+        constexpr int W = decltype(w_c)::value;
+        constexpr bool same = decltype(same_c)::value, more = decltype(more_c)::value;
+        Masks3 m3;
+        if constexpr (W == 3) m3 = masks3_role0();
+        int rank_nxt2 = 0;
+        if (g + 2 < g_end) rank_nxt2 = rank_at(g + 2);
+        u32x4 sc_nxt = {0, 0, 0, 0};
+        if constexpr (more) sc_nxt = scale_at(g + 1);
+        hs = hs_all + (g & 1) * (MAX_A * GU_STRIDE);
+        auto stage = [&](auto i_c, u32x4 raw) {
+            constexpr int i = decltype(i_c)::value;
+            const u32x4 v = scaled_f16x8<BF16>(raw, sc_cur);
+            *reinterpret_cast<u32x4*>(&hs[(pair + 4 * i) * GU_STRIDE + 8 * lane]) = v;
+            cterm[i] += wave_sum_lane63(const_term_partial<W>(v));
+        };
+        if (pair < n_a) stage(I0{}, raw0);
+        if (pair + 4 < n_a) stage(I1{}, raw1);
+        if (pair + 8 < n_a) stage(I2{}, act_at(2, rank_cur));
+        if (pair + 12 < n_a) stage(I3{}, act_at(3, rank_cur));
+        __syncthreads();   // the operand is complete
+        if constexpr (more) {
+            raw0 = act_at(0, rank_nxt);
+            raw1 = act_at(1, rank_nxt);
+        }
+        const uint16_t* ap16 = &hs[n * GU_STRIDE + 16 * kg];
+        static_for([&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            const u32x4 a_lo = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS);
+            const u32x4 a_hi = *reinterpret_cast<const u32x4*>(ap16 + q * SLAB_ROWS + 8);
+            gateup_pair<W, false>(pw[q], a_lo, a_hi, n >> 3, acc, corr, W == 3 ? &m3 : nullptr);
+            if constexpr (same) issue_at(qc, W, pack0 + GU_SLABS * (n_tiles * 256 * W));
+        }, std::make_integer_sequence<int, GU_SLABS>{});
+        sc_cur = sc_nxt;
+        rank_cur = rank_nxt;
+        rank_nxt = rank_nxt2;
+    };
+    // Runs of groups of one width, each walked by a loop compiled for that width.  A run requests its own
+    // first payload (no block registers are live from one run to the next), behind the activations and
+    // scales of its first group, which were requested one group earlier.
+    for (int g = g_begin; g < g_end;) {
+        lane = tid & 63;
+        asm volatile("" : "+v"(lane));
+        n = lane & 15;
+        kg = lane >> 4;
+        unit = (uint32_t)(pair * 64 + lane);
+        hi_unit = (uint32_t)hi_index0(kg, n, 2 * pair);
+        int g1 = g + 1;
+        while (g1 < g_end && __builtin_amdgcn_readfirstlane(grp_tab[g1].x) == rec.x) ++g1;
+        const int2 next = g1 < g_end ? group_rec(g1) : int2{0, 0};
+        auto run = [&](auto w_c) {
+            constexpr int W = decltype(w_c)::value;
+            int pack0 = rec.y;
+            static_for([&](auto qc) { issue_at(qc, W, pack0); }, std::make_integer_sequence<int, GU_SLABS>{});
+            for (; g + 1 < g1; ++g, pack0 += GU_SLABS * (n_tiles * 256 * W))
+                group_step(w_c, std::true_type{}, std::true_type{}, g, pack0);
+            if (g1 < g_end)
+                group_step(w_c, std::false_type{}, std::true_type{}, g, pack0);
+            else
+                group_step(w_c, std::false_type{}, std::false_type{}, g, pack0);
+            ++g;
+        };
+        if (rec.x == 2)
+            run(std::integral_constant<int, 2>{});
+        else if (rec.x == 3)
+            run(std::integral_constant<int, 3>{});
+        else
+            run(std::integral_constant<int, 4>{});
+        rec = next;
+    }
+    // the constant terms of the chunk's assignments, from the wavefronts that staged them
+    if (lane == 63) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) cterm_lds[pair + 4 * i] = cterm[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) corr[j] = cterm_lds[4 * kg + j];
+#pragma unroll
+    for (int nbl = 0; nbl < 2; ++nbl) {
+        const int c = t * N_TILE + 32 * pair + 16 * nbl + n;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int a = 4 * kg + j;
+            if (a < n_a && c < I) {
+                if constexpr (SPLIT)
+                    atomicAdd(&out[(int64_t)(a0 + a) * I + c], acc[nbl][j] - corr[j]);
+                else
+                    out[(int64_t)(a0 + a) * I + c] = acc[nbl][j] - corr[j];
+            }
+        }
+    }
+}
+
 // ------------------------------------------------ gate AND up of one tile, z = silu(G) * U out
 // The same walk for BOTH projections of one expert, one after the other in one workgroup (first all
 // slab groups of the gate matrix, then all of the up matrix; the payload stream of a wavefront runs on

@@ -292,7 +292,9 @@ __global__ __launch_bounds__(256, 4) void k_gateup_decode(
 // (gate, up); 256 threads = 4 wavefronts.  An expert with more than 16 assignments is served in
 // 16-assignment chunks, one after the other (or one workgroup per chunk: GRID_CHUNKS).
 // The kernel also clears `zero_out` (the forward's accumulator, added into by the down kernel).
-template <bool BF16, int MODE, bool IDENT>
+// MIXED: experts whose slab groups differ in width (gateup_walk_item_mixed); a kernel of its own, so that
+// the one-width kernel keeps its registers to itself.
+template <bool BF16, int MODE, bool IDENT, bool MIXED>
 __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
     const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
@@ -333,8 +335,17 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const int max_slabs = mt ? up_max_slabs : gate_max_slabs;
     const FastExpert fe = fe_tab[e];
     const FastSlab first = load_fast_slab(fs_tab, e * max_slabs);
+    // the widths and payload offsets of the expert's slab groups (read by the mixed-width walk only, but
+    // requested here, together with the expert's record)
+    __shared__ int2 grp_tab[MIXED ? WALK_MAX_GROUPS : 1];
+    if constexpr (MIXED) {
+        if (tid < WALK_MAX_GROUPS && tid * GU_SLABS < max_slabs) {
+            const FastSlab gs = fs_tab[(int64_t)e * max_slabs + tid * GU_SLABS];
+            grp_tab[tid] = int2{gs.bits, gs.pack_off};
+        }
+    }
     if (a_end <= a_begin || first.bits == 0) return;
-    const int n_groups = max_slabs / GU_SLABS;
+    const int n_groups = fe.num_slabs / GU_SLABS;
 
     gptr<uint32_t> payload = as_global(fe.payload);
     gptr<__half> scale_s = as_global(fe.scale_s);
@@ -347,23 +358,28 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     __shared__ __attribute__((aligned(16))) uint16_t hs_all[2 * MAX_A * GU_STRIDE];
     __shared__ float cterm_lds[MAX_A];
 
+    if constexpr (MIXED) __syncthreads();        // grp_tab is complete
     for (int a0 = a_begin; a0 < a_end; a0 += MAX_A) {
         const int n_a = min(MAX_A, a_end - a0);
         if (a0 != a_begin) __syncthreads();      // the previous chunk's readers of the operand are done
-        auto run = [&](auto w_c) {
-            gateup_walk_item<BF16, IDENT, decltype(w_c)::value, false>(payload, scale_s, rank_idx, first, h, ld, token_indices,
-                                                                       a0, n_a, A, T, I, n_tiles, t, 0, n_groups, out, hs_all,
-                                                                       cterm_lds, tid);
-        };
-        if (first.bits == 2)
-            run(std::integral_constant<int, 2>{});
-        else if (first.bits == 3)
-            run(std::integral_constant<int, 3>{});
-        else if (first.bits == 4)
-            run(std::integral_constant<int, 4>{});
+        if constexpr (MIXED) {
+            gateup_walk_item_mixed<BF16, IDENT, false>(payload, scale_s, rank_idx, grp_tab, h, ld, token_indices, a0, n_a, A, T, I,
+                                                       n_tiles, t, 0, n_groups, out, hs_all, cterm_lds, tid);
+        } else {
+            auto run = [&](auto w_c) {
+                gateup_walk_item<BF16, IDENT, decltype(w_c)::value, false>(payload, scale_s, rank_idx, first, h, ld,
+                                                                           token_indices, a0, n_a, A, T, I, n_tiles, t, 0,
+                                                                           n_groups, out, hs_all, cterm_lds, tid);
+            };
+            if (first.bits == 2)
+                run(std::integral_constant<int, 2>{});
+            else if (first.bits == 3)
+                run(std::integral_constant<int, 3>{});
+            else if (first.bits == 4)
+                run(std::integral_constant<int, 4>{});
+        }
     }
 }
-
 
 // gateup_walk_z_item launched as a grid: grid.x = (expert coordinate) * n_tiles; 256 threads.  One
 // workgroup forms BOTH projections of its tile and writes Z / Zsum; it also clears `zero_out`.
@@ -546,14 +562,17 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     // walking gate/up kernel, which also clears rank_accum and needs no cleared G / U.
     // (its 16-byte activation loads also need rank_idx in runs of eight and aligned rows)
     auto rows16 = [](const void* p, int64_t ld) { return ((uintptr_t)p & 15) == 0 && ld % 8 == 0; };
-    const bool walk = gate->all_affine && up->all_affine && gate->rank_chunked8 && up->rank_chunked8 &&
-                   rows16(h_gate, ldg) && rows16(h_up, ldu);
+    // (the ranks that padding rows read, with zero scales, must be columns of the activations too)
+    const bool walk = gate->role == ROLE_GATE_UP && up->role == ROLE_GATE_UP && gate->rank_chunked8 && up->rank_chunked8 &&
+                   rows16(h_gate, ldg) && rows16(h_up, ldu) && gate->pad_rank_plus1 <= Rg && up->pad_rank_plus1 <= Ru &&
+                   std::max(gate->prep_max_slabs, up->prep_max_slabs) <= WALK_MAX_GROUPS * GU_SLABS;
     // Both projections in one workgroup, z = silu(G) * U handed to the down kernel ready-made: when the two
     // matrices of every expert share bit-width and slab count, and (expert, tile) pairs alone fill most of
     // the chip.  BITSMOE_DECODE_FUSED_Z=0 / 1 switches it off / on regardless of the size (experiments).
     const char* fused_var = getenv("BITSMOE_DECODE_FUSED_Z");      // (read per call: tests switch it)
     const int fused_env = fused_var && fused_var[0] ? atoi(fused_var) : -1;
-    const bool fused_possible = walk && gate->max_slabs == up->max_slabs && gate->expert_bits == up->expert_bits;
+    const bool fused_possible = walk && gate->all_affine && up->all_affine && gate->prep_max_slabs == up->prep_max_slabs &&
+                                gate->expert_bits == up->expert_bits;
     const bool fused_z = fused_possible && fused_env > 0;
     if (!walk) {
         // G and U are adjacent in the workspace: one range; rank_accum is the second
@@ -564,7 +583,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         BITSMOE_HIP_TRY(hipGetLastError());
     }
     record(prof, 1, st);
-    const int max_slabs = std::max(gate->max_slabs, up->max_slabs);
+    const int max_slabs = std::max(gate->prep_max_slabs, up->prep_max_slabs);
     const int gu_groups = (max_slabs + GU_SLABS - 1) / GU_SLABS;
     // Tiles per workgroup: long runs amortise the start-up round trips, but the grid must
     // still hold a few workgroups per CU (two rounds of three per CU measured best).
@@ -581,8 +600,8 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     };
     const ExpertOrder gate_order = order_of(gate), up_order = order_of(up);
     auto launch_gateup = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs, gate->max_slabs,
-                           up->d_fast_experts, up->d_fast_slabs, up->max_slabs, (const uint16_t*)h_gate,
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs, gate->prep_max_slabs,
+                           up->d_fast_experts, up->d_fast_slabs, up->prep_max_slabs, (const uint16_t*)h_gate,
                            (const uint16_t*)h_up, Rg, Ru, ldg, ldu, tok, off, (int)T, (int)A, I, E, n_tiles, gu_groups, n_tchunks,
                            tiles_per_wg, G, U, gate_order, up_order);
     };
@@ -603,11 +622,16 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
             fn(bf16_c, std::integral_constant<int, GRID_EXPERTS>{});
     };
     auto launch_walk_mode = [&](auto bf16_c, auto mode_c) {
-        auto kern = k_gateup_walk<decltype(bf16_c)::value, decltype(mode_c)::value, false>;
-        if (gate->rank_identity && up->rank_identity) kern = k_gateup_walk<decltype(bf16_c)::value, decltype(mode_c)::value, true>;
+        // (one width per expert in both sets: the kernel compiled for that; else the one that switches per slab group)
+        const bool ident = gate->rank_identity && up->rank_identity;
+        const bool mixed = !(gate->uniform_experts && up->uniform_experts);
+        constexpr bool B = decltype(bf16_c)::value;
+        constexpr int M = decltype(mode_c)::value;
+        auto kern = mixed ? (ident ? k_gateup_walk<B, M, true, true> : k_gateup_walk<B, M, false, true>)
+                          : (ident ? k_gateup_walk<B, M, true, false> : k_gateup_walk<B, M, false, false>);
         hipLaunchKernelGGL(kern, dim3((unsigned)(e_dim * n_tiles), 2),
-                           dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs, gate->max_slabs, up->d_fast_experts,
-                           up->d_fast_slabs, up->max_slabs, (const uint16_t*)h_gate, (const uint16_t*)h_up, ldg, ldu,
+                           dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs, gate->prep_max_slabs, up->d_fast_experts,
+                           up->d_fast_slabs, up->prep_max_slabs, (const uint16_t*)h_gate, (const uint16_t*)h_up, ldg, ldu,
                            tok, off, (int)T, (int)A, I, E, n_tiles, G, U, rank_accum, T * (int64_t)rank_out, gate_order,
                            up_order);
     };
@@ -616,7 +640,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         if (gate->rank_identity && up->rank_identity) kern = k_gateup_walk_z<decltype(bf16_c)::value, decltype(mode_c)::value, true>;
         // Z takes the place of G in the workspace, Zsum that of U
         hipLaunchKernelGGL(kern, dim3((unsigned)(e_dim * n_tiles)), dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs,
-                           up->d_fast_experts, up->d_fast_slabs, gate->max_slabs, (const uint16_t*)h_gate, (const uint16_t*)h_up,
+                           up->d_fast_experts, up->d_fast_slabs, gate->prep_max_slabs, (const uint16_t*)h_gate, (const uint16_t*)h_up,
                            ldg, ldu, tok, off, (int)T, (int)A, I, E, n_tiles, (uint16_t*)G, U, rank_accum,
                            T * (int64_t)rank_out, gate_order);
     };
@@ -638,7 +662,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 2, st);
     record(prof, 3, st);      // (SiLU happens inside the down kernel)
-    const int dn_groups = (down->max_slabs + DN_SLABS_PER_WG - 1) / DN_SLABS_PER_WG;
+    const int dn_groups = (down->prep_max_slabs + DN_SLABS_PER_WG - 1) / DN_SLABS_PER_WG;
     const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4 + DN_SLABS_PER_WG * SLAB_ROWS * 8 + MAX_A * 8;
     int dn_tiles_per_wg = n_tiles;
     while (dn_tiles_per_wg > 1 && units * dn_groups * ((n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg) < 600)
@@ -647,7 +671,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     auto launch_down = [&](auto kernel) {
         const int n_work = e_dim * dn_groups * dn_tchunks;
         hipLaunchKernelGGL(kernel, dim3((unsigned)((n_work + 7) / 8 * 8)), dim3(256), z_bytes, st, down->d_fast_experts,
-                           down->d_fast_slabs, down->max_slabs, G, U, rw, tok, off, (int)T, (int)A, I, E, n_tiles,
+                           down->d_fast_slabs, down->prep_max_slabs, G, U, rw, tok, off, (int)T, (int)A, I, E, n_tiles,
                            dn_groups, dn_tchunks, dn_tiles_per_wg, n_work, rank_out, rank_accum);
     };
     auto launch_down_mode = [&](auto zready_c, auto mode_c) {

@@ -1182,7 +1182,8 @@ bool mfma_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, c
 static bool direct_ok(const bitsmoe_matset* gate, const bitsmoe_matset* up) {
     return gate->rank_chunked8 && up->rank_chunked8 && gate->d_scale_s && up->d_scale_s;
 }
-static inline int direct_ld(const bitsmoe_matset* set) { return (set->max_rank_plus1 + 7) / 8 * 8; }
+// (columns of the f16 copy of bf16 activations: every rank the prepared rank table names, padding rows included)
+static inline int direct_ld(const bitsmoe_matset* set) { return (set->pad_rank_plus1 + 7) / 8 * 8; }
 
 // Carving of the workspace, shared by the size query and the launcher.
 struct MfmaWorkspace {
@@ -1192,7 +1193,7 @@ static MfmaWorkspace mfma_workspace(const bitsmoe_matset* gate, const bitsmoe_ma
                                     int64_t T, int64_t A, int I) {
     const int64_t max_mtiles = A / PF_M + gate->n_experts;
     const size_t direct = align256((size_t)T * direct_ld(gate) * 2) + align256((size_t)T * direct_ld(up) * 2);
-    const size_t gathered = align256((size_t)A * gate->max_slabs * SLAB_ROWS * 2) + align256((size_t)A * up->max_slabs * SLAB_ROWS * 2);
+    const size_t gathered = align256((size_t)A * gate->prep_max_slabs * SLAB_ROWS * 2) + align256((size_t)A * up->prep_max_slabs * SLAB_ROWS * 2);
     MfmaWorkspace w;
     size_t at = 0;
     auto take = [&](size_t bytes) { const size_t here = at; at += align256(bytes); return here; };
@@ -1207,7 +1208,7 @@ static MfmaWorkspace mfma_workspace(const bitsmoe_matset* gate, const bitsmoe_ma
     w.acts = take(std::max(direct_ok(gate, up) ? direct : 0, gathered));
     w.z = take((size_t)A * I * 2);
     w.u = take((size_t)A * I * 2);
-    w.y = take((size_t)(A + 1) * down->max_slabs * SLAB_ROWS * 2);
+    w.y = take((size_t)(A + 1) * down->prep_max_slabs * SLAB_ROWS * 2);
     w.total = at;
     return w;
 }
@@ -1225,11 +1226,14 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     const int n_tiles = gate->n_tiles;
     const int64_t max_mtiles = A / PF_M + E;
     // ldg_in / ldu_in: elements between the caller's activation rows (>= Rg / Ru)
+    // (padding rows have zero scales but their activations are still read and multiplied: every rank they
+    // name has to be a column of h)
     const bool direct = direct_ok(gate, up) && Rg % 8 == 0 && Ru % 8 == 0 && ldg_in % 8 == 0 && ldu_in % 8 == 0 &&
+                        gate->pad_rank_plus1 <= Rg && up->pad_rank_plus1 <= Ru &&
                         (((uintptr_t)h_gate | (uintptr_t)h_up) & 15) == 0 &&
                         T * std::max(ldg_in, ldu_in) < ((int64_t)1 << 31);
-    const int ldg = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(gate) : (int)ldg_in) : gate->max_slabs * SLAB_ROWS;
-    const int ldu = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(up) : (int)ldu_in) : up->max_slabs * SLAB_ROWS;
+    const int ldg = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(gate) : (int)ldg_in) : gate->prep_max_slabs * SLAB_ROWS;
+    const int ldu = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(up) : (int)ldu_in) : up->prep_max_slabs * SLAB_ROWS;
     const MfmaWorkspace w = mfma_workspace(gate, up, down, T, A, I);
     char* ws = (char*)workspace;
     MTile* mtiles = (MTile*)(ws + w.mtiles);
@@ -1243,7 +1247,7 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     uint16_t* z = (uint16_t*)(ws + w.z);     // gate output, then silu(gate) * up in place
     uint16_t* Ubuf = (uint16_t*)(ws + w.u);
     _Float16* y = (_Float16*)(ws + w.y);
-    const int ldy = down->max_slabs * SLAB_ROWS;
+    const int ldy = down->prep_max_slabs * SLAB_ROWS;
 
     record(prof, 0, st);
     const bool convert = direct && act_dtype == BITSMOE_DT_BF16;
@@ -1284,7 +1288,7 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
         const int64_t wgs = (max_mtiles + 31) / 32 * 32 * 2 * n_tp;
         auto launch = [&](auto kernel) -> hipError_t {
             hipLaunchKernelGGL(kernel, dim3((unsigned)wgs), dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs,
-                               gate->max_slabs, up->d_fast_experts, up->d_fast_slabs, up->max_slabs, Hs_g, Hs_u, ldg, ldu, tok,
+                               gate->prep_max_slabs, up->d_fast_experts, up->d_fast_slabs, up->prep_max_slabs, Hs_g, Hs_u, ldg, ldu, tok,
                                (int)T, mtiles, n_mtiles, I, n_tiles, z, Ubuf);
             return hipGetLastError();
         };
@@ -1297,18 +1301,18 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     }
     record(prof, 3, st);
     {
-        const int n_pairs = (down->max_slabs + DN_SLABS_MFMA - 1) / DN_SLABS_MFMA;
+        const int n_pairs = (down->prep_max_slabs + DN_SLABS_MFMA - 1) / DN_SLABS_MFMA;
         const int64_t wgs = (max_mtiles + 31) / 32 * 32 * n_pairs;
         hipLaunchKernelGGL(k_down_mfma, dim3((unsigned)wgs), dim3(256), 0, st, down->d_fast_experts, down->d_fast_slabs,
-                           down->max_slabs, z, mtiles, n_mtiles, tok, slot, token_start, token_list, (int)A, I, n_tiles,
+                           down->prep_max_slabs, z, mtiles, n_mtiles, tok, slot, token_start, token_list, (int)A, I, n_tiles,
                            n_pairs, y, ldy);
         record(prof, 4, st);
         if (down->rank_identity)
             hipLaunchKernelGGL(k_combine_tokens<true>, dim3((unsigned)T), dim3(256), 0, st, down->d_fast_experts,
-                               down->max_slabs, y, ldy, token_start, token_list, rw, rank_out, rank_accum);
+                               down->prep_max_slabs, y, ldy, token_start, token_list, rw, rank_out, rank_accum);
         else
             hipLaunchKernelGGL(k_combine_tokens<false>, dim3((unsigned)T), dim3(256), 0, st, down->d_fast_experts,
-                               down->max_slabs, y, ldy, token_start, token_list, rw, rank_out, rank_accum);
+                               down->prep_max_slabs, y, ldy, token_start, token_list, rw, rank_out, rank_accum);
         BITSMOE_HIP_TRY(hipGetLastError());
     }
     record(prof, 5, st);

@@ -231,6 +231,7 @@ extern "C" void bitsmoe_matset_destroy(bitsmoe_matset* set) {
     if (set->d_prepared) (void)hipFree(set->d_prepared);
     if (set->d_scale_s) (void)hipFree(set->d_scale_s);
     if (set->d_prepared_rows) (void)hipFree(set->d_prepared_rows);
+    if (set->d_prep_tasks) (void)hipFree(set->d_prep_tasks);
     if (set->d_fast_experts) (void)hipFree(set->d_fast_experts);
     if (set->d_fast_slabs) (void)hipFree(set->d_fast_slabs);
     delete set;

@@ -7,19 +7,6 @@
 
 namespace bitsmoe {
 
-// code (unsigned, before the level offset) of element (row, col) of a (slab, tile) block of `k_slab`
-// rows in the reference bit-plane layout; `blk` points at the block's first word.  Rows past
-// k_slab (a ragged slab is padded to 64 rows in the prepared copy) read as the code of level zero.
-__device__ inline uint32_t ref_code(const uint32_t* __restrict__ blk, int w, int k_slab, int row, int col) {
-    if (row >= k_slab) return (uint32_t)level_offset(w);
-    const int stage = row >> 4, r = row & 15, micro = col >> 5, lane = col & 31;
-    const int rows_cur = min(K_STAGE, k_slab - stage * K_STAGE);
-    const uint32_t* words = blk + stage * (K_STAGE * MICROS * w) + micro * (rows_cur * w) + r * w;
-    uint32_t u = 0;
-    for (int p = 0; p < w; ++p) u |= ((words[p] >> lane) & 1u) << p;
-    return u;
-}
-
 // (row, col) of contraction index x of the run owned by (nb, kg, n)
 __device__ inline void run_element(int role, int nb, int kg, int n, int x, int* row, int* col) {
     if (role == ROLE_GATE_UP) {          // 16 rows 16*kg + x, column 16*nb + n
@@ -31,22 +18,47 @@ __device__ inline void run_element(int role, int nb, int kg, int n, int x, int* 
     }
 }
 
-// grid: (slab tasks, tiles); every thread builds whole output words of one block.  Reads the caller's
-// reference layout (through its own tile_meta / slab_meta), writes the prepared copy at the offsets of
-// the FastSlab table.
+// Where a row of the prepared copy comes from: (source slab << 8) | row inside that slab, or -1 for a
+// padding row.  The prepared copy keeps the caller's local row order but cuts it into slabs of its own:
+// rows [64 p, 64 p + 64) whatever bucket they came from, stored at the widest width among them (a narrower
+// code is the same LEVEL at a wider width: level = code - 2^(w-1), and the scale stays per row), so that a
+// bucket whose row count is no multiple of 64 leaves no gap in the row numbering.
+struct PrepSource {
+    const int32_t* row_src;      // [rows of the prepared copy], all experts
+    const int32_t* rank_base;    // the prepared rank table's first element: an expert's rows start at fe.rank_idx - rank_base
+};
+
+// The level (signed) of prepared row `row` of prepared slab `ps`, column `col` of tile `t`.
+__device__ inline int source_level(const MatView& mv, const int32_t* __restrict__ row_src, int ps, int row, int t, int col) {
+    const int src = row_src[ps * SLAB_ROWS + row];
+    if (src < 0) return 0;
+    const int s = src >> 8, r = src & 255;
+    const int w = mv.slab_meta[s * 4 + 0], k_slab = mv.slab_meta[s * 4 + 1];
+    const uint32_t* __restrict__ blk = mv.payload + mv.tile_meta[(mv.slab_meta[s * 4 + 3] + t) * 3 + 0];
+    const int stage = r >> 4, rr = r & 15, micro = col >> 5, lane = col & 31;
+    const int rows_cur = min(K_STAGE, k_slab - stage * K_STAGE);
+    const uint32_t* words = blk + stage * (K_STAGE * MICROS * w) + micro * (rows_cur * w) + rr * w;
+    int u = 0;
+    for (int p = 0; p < w; ++p) u |= (int)((words[p] >> lane) & 1u) << p;
+    return u - level_offset(w);
+}
+
+// grid: (prepared slab tasks, tiles); every thread builds whole output words of one block.  Reads the
+// caller's reference layout (through its own tile_meta / slab_meta), writes the prepared copy at the
+// offsets of the FastSlab table.
 __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src, const FastExpert* __restrict__ fexp,
                                                  const FastSlab* __restrict__ fslabs, int max_slabs,
-                                                 const SlabTask* __restrict__ tasks, int role) {
+                                                 const SlabTask* __restrict__ tasks, PrepSource ps_tab, int role) {
     const SlabTask task = tasks[blockIdx.x];
     const MatView mv = src[task.expert];
-    const int si = task.slab;
-    const int w = mv.slab_meta[si * 4 + 0];
-    const int k_slab = mv.slab_meta[si * 4 + 1];
-    const int tile_off = mv.slab_meta[si * 4 + 3];
-    const int t = tile_off + blockIdx.y;
-    const uint32_t* __restrict__ in = mv.payload + mv.tile_meta[t * 3 + 0];
-    const FastSlab fs = fslabs[(int64_t)task.expert * max_slabs + si];
-    uint32_t* __restrict__ out = const_cast<uint32_t*>(fexp[task.expert].payload) + fs.pack_off + (int)blockIdx.y * 256 * w;
+    const FastExpert fe = fexp[task.expert];
+    const int ps = task.slab;
+    const int t = blockIdx.y;
+    const FastSlab fs = fslabs[(int64_t)task.expert * max_slabs + ps];
+    const int w = fs.bits;
+    const int32_t* __restrict__ row_src = ps_tab.row_src + (fe.rank_idx - ps_tab.rank_base);
+    uint32_t* __restrict__ out = const_cast<uint32_t*>(fe.payload) + fs.pack_off + t * 256 * w;
+    auto code_at = [&](int row, int col) { return (uint32_t)(source_level(mv, row_src, ps, row, t, col) + level_offset(w)); };
     const int nbs = (role == ROLE_GATE_UP) ? 8 : 4;        // output blocks per lane
     const int run = (role == ROLE_GATE_UP) ? 16 : 32;      // contraction indices per (lane, nb)
     const int n_words = 256 * w;
@@ -62,14 +74,14 @@ __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src
                     for (int x = 0; x < 16; ++x) {
                         int row, col;
                         run_element(role, nb, kg, n8 + 8 * upper, x, &row, &col);
-                        word |= ((ref_code(in, w, k_slab, row, col) >> 2) & 1u) << pos1s(x, upper);
+                        word |= ((code_at(row, col) >> 2) & 1u) << pos1s(x, upper);
                     }
             } else {                      // j = l*4 + nb
                 const int nb = j & 3, l = j >> 2, n = l & 15, kg = l >> 4;
                 for (int x = 0; x < 32; ++x) {
                     int row, col;
                     run_element(role, nb, kg, n, x, &row, &col);
-                    word |= ((ref_code(in, w, k_slab, row, col) >> 2) & 1u) << pos1(x);
+                    word |= ((code_at(row, col) >> 2) & 1u) << pos1(x);
                 }
             }
             out[idx] = word;
@@ -94,7 +106,7 @@ __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src
             const int x = sub * codes + i;
             int row, col;
             run_element(role, nb, kg, n, x, &row, &col);
-            const uint32_t u = ref_code(in, w, k_slab, row, col);
+            const uint32_t u = code_at(row, col);
             if (role == ROLE_GATE_UP)      // staggered fields; one may wrap around bit 31
                 word |= rotl32(fb == 4 ? (u & 15u) : (u & 3u), fb == 4 ? pos4s(i) : pos2s(w, i));
             else if (fb == 4)
@@ -106,43 +118,42 @@ __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src
     }
 }
 
-// The per-row tables of the prepared copy, every slab padded to 64 rows: s' (multiplier), scale'
-// [(slab, tile)][64] and, for gate/up sets, scale_s' = scale * s * stagger factor (a power of two: the
+// The per-row tables of the prepared copy: s' (multiplier), scale' [(slab, tile)][64] and, for gate/up
+// sets, scale_s' = scale * s * stagger factor of the row at the PREPARED slab's width (a power of two: the
 // decoded weight carries its inverse), each rounded once to fp16.  Padding rows get zeros, so whatever
-// the kernels read for them contributes nothing.  grid (slab tasks, tiles), 64 threads.
+// the kernels read for them contributes nothing.  grid (prepared slab tasks, tiles), 64 threads.
 __global__ __launch_bounds__(64) void k_prepare_rows(const MatView* __restrict__ views, const FastExpert* __restrict__ fexp,
                                                      const FastSlab* __restrict__ fslabs, int max_slabs,
-                                                     const SlabTask* __restrict__ tasks) {
+                                                     const SlabTask* __restrict__ tasks, PrepSource ps_tab) {
     const SlabTask task = tasks[blockIdx.x];
     const MatView mv = views[task.expert];
     const FastExpert fe = fexp[task.expert];
-    const int si = task.slab;
-    const int w = mv.slab_meta[si * 4 + 0];
-    const int k_slab = mv.slab_meta[si * 4 + 1];
-    const int rank_off = mv.slab_meta[si * 4 + 2];
-    const int t = mv.slab_meta[si * 4 + 3] + blockIdx.y;
-    const int scale_off = mv.tile_meta[t * 3 + 1];
-    const FastSlab fs = fslabs[(int64_t)task.expert * max_slabs + si];
+    const int ps = task.slab;
+    const int t = blockIdx.y;
+    const FastSlab fs = fslabs[(int64_t)task.expert * max_slabs + ps];
     const int row = threadIdx.x;
-    const bool valid = row < k_slab;
-    const float sv = valid ? __half2float(mv.s[rank_off + row]) : 0.0f;
-    const float sc = valid ? __half2float(mv.scale[scale_off + row]) : 0.0f;
-    const int out_sc = fs.scale_off + (int)blockIdx.y * SLAB_ROWS + row;
+    const int src = (ps_tab.row_src + (fe.rank_idx - ps_tab.rank_base))[ps * SLAB_ROWS + row];
+    float sv = 0.0f, sc = 0.0f;
+    if (src >= 0) {
+        const int s = src >> 8, r = src & 255;
+        sv = __half2float(mv.s[mv.slab_meta[s * 4 + 2] + r]);
+        sc = __half2float(mv.scale[mv.tile_meta[(mv.slab_meta[s * 4 + 3] + t) * 3 + 1] + r]);
+    }
+    const int out_sc = fs.scale_off + t * SLAB_ROWS + row;
     const_cast<__half*>(fe.scale)[out_sc] = __float2half(sc);
-    if (fe.scale_s) const_cast<__half*>(fe.scale_s)[out_sc] = __float2half(sc * sv * (float)stagger_factor(w, row));
-    if (blockIdx.y == 0) const_cast<__half*>(fe.s)[fs.rank_off + row] = __float2half(sv);
+    if (fe.scale_s) const_cast<__half*>(fe.scale_s)[out_sc] = __float2half(sc * sv * (float)stagger_factor(fs.bits, row));
+    if (t == 0) const_cast<__half*>(fe.s)[fs.rank_off + row] = __float2half(sv);
 }
 
 // Dense fp32 dequantisation FROM THE PREPARED COPY, written to mirror the decode of the hot kernels
 // (fields, not planes); rows in the caller's local row order, output identical to k_dequant_matrix.
+// grid (prepared slabs of the expert, tiles).
 __global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* the caller's tables */, FastExpert fe,
-                                                          const FastSlab* __restrict__ fs_row, int role, int I,
-                                                          float* __restrict__ out) {
-    const int si = blockIdx.x;
-    const int w = mv.slab_meta[si * 4 + 0];
-    const int k_slab = mv.slab_meta[si * 4 + 1];
-    const int rank_off = mv.slab_meta[si * 4 + 2];
-    const FastSlab fs = fs_row[si];
+                                                          const FastSlab* __restrict__ fs_row, const int32_t* __restrict__ row_src,
+                                                          int role, int I, float* __restrict__ out) {
+    const int ps = blockIdx.x;
+    const FastSlab fs = fs_row[ps];
+    const int w = fs.bits;
     const uint32_t* __restrict__ blk = fe.payload + fs.pack_off + (int)blockIdx.y * 256 * w;
     const int nbs = (role == ROLE_GATE_UP) ? 8 : 4;
     const int run = (role == ROLE_GATE_UP) ? 16 : 32;
@@ -178,9 +189,11 @@ __global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* the call
             }
         }
         const int c = blockIdx.y * N_TILE + col;
-        if (c < I && row < k_slab) {
+        const int src = row_src[ps * SLAB_ROWS + row];
+        if (c < I && src >= 0) {
+            const int local_row = mv.slab_meta[(src >> 8) * 4 + 2] + (src & 255);
             const float q = (float)((int)u - level_offset(w));
-            out[(int64_t)(rank_off + row) * I + c] = q * __half2float(fe.scale[fs.scale_off + (int)blockIdx.y * SLAB_ROWS + row]);
+            out[(int64_t)local_row * I + c] = q * __half2float(fe.scale[fs.scale_off + (int)blockIdx.y * SLAB_ROWS + row]);
         }
     }
 }
@@ -200,7 +213,7 @@ extern "C" int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* s
     if (rc != BITSMOE_OK) {
         // nothing of a failed attempt stays behind: the set remains usable by the generic kernels
         void** owned[] = {(void**)&set->d_prepared, (void**)&set->d_fast_experts, (void**)&set->d_fast_slabs,
-                          (void**)&set->d_scale_s, (void**)&set->d_prepared_rows};
+                          (void**)&set->d_scale_s, (void**)&set->d_prepared_rows, (void**)&set->d_prep_tasks};
         for (void** p : owned) {
             if (*p) (void)hipFree(*p);
             *p = nullptr;
@@ -218,52 +231,91 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
                   "only the generic kernels can run it");
         return BITSMOE_E_UNSUPPORTED;
     }
-    const int E = set->n_experts, n_tiles = set->n_tiles, max_slabs = set->max_slabs;
-    // Offsets of the prepared copy: every slab is a full 64-row slab there (a ragged slab of the caller's
-    // layout is padded), so slab si of an expert holds local rows [64 si, 64 si + 64), its tiles follow
-    // each other in payload' (256 w words each) and in scale' (64 each).
-    std::vector<FastSlab> fslabs((size_t)E * max_slabs, FastSlab{0, 0, 0, 0});
+    const int E = set->n_experts, n_tiles = set->n_tiles;
+    // The slabs of the prepared copy: the caller's local rows in their order, cut every 64 rows; gate/up
+    // sets in whole groups of GU_SLABS slabs (what one workgroup of the walking kernel contracts over
+    // between two barriers), a group stored at ONE width, the widest among its rows.
+    const int unit = role == ROLE_GATE_UP ? GU_SLABS : 1;
+    std::vector<int> n_ps(E);
+    int pms = 0;
+    for (int e = 0; e < E; ++e) {
+        int64_t rows = 0;
+        for (int si = 0; si < set->descs[e].num_slabs; ++si) rows += set->slab_meta_host[e][si * 4 + 1];
+        n_ps[e] = (int)round_up(std::max<int64_t>((rows + SLAB_ROWS - 1) / SLAB_ROWS, 1), unit);
+        pms = std::max(pms, n_ps[e]);
+    }
+    set->prep_max_slabs = pms;
+    std::vector<FastSlab> fslabs((size_t)E * pms, FastSlab{0, 0, 0, 0});
+    std::vector<SlabTask> tasks;
     std::vector<int64_t> pay_off(E), row_off(E), sc_off(E);
     int64_t pay_words = 0, rows_total = 0, scale_total = 0;
     for (int e = 0; e < E; ++e) {
-        pay_off[e] = pay_words;
         row_off[e] = rows_total;
         sc_off[e] = scale_total;
-        const auto& slab = set->slab_meta_host[e];
-        int64_t words = 0;
-        const int ns = set->descs[e].num_slabs;
-        for (int si = 0; si < ns; ++si) {
-            const int bits = slab[si * 4 + 0];
-            BITSMOE_REQUIRE(words < ((int64_t)1 << 31) - (int64_t)n_tiles * 256 * 4, "expert %d: prepared payload exceeds int32 word offsets", e);
-            fslabs[(size_t)e * max_slabs + si] = FastSlab{bits, (int32_t)words, si * n_tiles * SLAB_ROWS, si * SLAB_ROWS};
-            words += (int64_t)n_tiles * 256 * bits;
-        }
-        pay_words += round_up(words, 64);                               // keep every matrix 256-byte aligned
-        rows_total += round_up((int64_t)ns * SLAB_ROWS, 64);
-        scale_total += round_up((int64_t)ns * n_tiles * SLAB_ROWS, 128);
+        rows_total += (int64_t)n_ps[e] * SLAB_ROWS;
+        scale_total += round_up((int64_t)n_ps[e] * n_tiles * SLAB_ROWS, 128);
     }
-    // rank_idx' on the host (the kernels' eligibility flags are read off it): a padding row reads rank -1,
-    // which every kernel treats as "no such row" -- except whole padded runs of eight rows, which read the
-    // ranks 0..7 (their scale is zero) so that they do not break the runs-of-eight property below.
-    std::vector<int32_t> rank_rows((size_t)std::max<int64_t>(rows_total, 1), -1);
+    std::vector<int32_t> rank_rows((size_t)std::max<int64_t>(rows_total, 1), -1), row_src((size_t)std::max<int64_t>(rows_total, 1), -1);
+    int pad_rank_plus1 = set->max_rank_plus1;
     for (int e = 0; e < E; ++e) {
         const auto& slab = set->slab_meta_host[e];
         const auto& rk = set->rank_idx_host[e];
+        int32_t* rr = rank_rows.data() + row_off[e];
+        int32_t* rs = row_src.data() + row_off[e];
+        std::vector<int> width(n_ps[e], 0);
+        int64_t p = 0;
         for (int si = 0; si < set->descs[e].num_slabs; ++si) {
-            const int k_slab = slab[si * 4 + 1], rank_off = slab[si * 4 + 2];
-            int32_t* dst = rank_rows.data() + row_off[e] + (int64_t)si * SLAB_ROWS;
-            for (int r = 0; r < SLAB_ROWS; ++r) {
-                if (r < k_slab)
-                    dst[r] = rk[rank_off + r];
-                else if ((r & ~7) >= k_slab && set->max_rank_plus1 >= 8)
-                    dst[r] = r & 7;
+            const int bits = slab[si * 4 + 0], k_slab = slab[si * 4 + 1], rank_off = slab[si * 4 + 2];
+            for (int r = 0; r < k_slab; ++r, ++p) {
+                rr[p] = rk[rank_off + r];
+                rs[p] = (si << 8) | r;
+                width[p / SLAB_ROWS] = std::max(width[p / SLAB_ROWS], bits);
             }
         }
+        // Padding rows (zero scales) behind the last row.  When the real rows are the identity (row k holds
+        // rank k: what ascending bit buckets without gaps give) the padding rows continue it, so that the set
+        // keeps its identity and runs-of-eight properties; kernels skip ranks outside the activations / the
+        // output, and pad_rank_plus1 tells the launchers how far the padding reaches.  Otherwise a run of
+        // eight that is all padding reads the ranks 0..7, the rest of a run that the last rows begin
+        // continues that run, and any other padding row has rank -1 ("no such row" to every kernel).
+        const int64_t rows_e = p, rows_p = (int64_t)n_ps[e] * SLAB_ROWS;
+        bool ident_e = true;
+        for (int64_t j = 0; j < rows_e && ident_e; ++j) ident_e = rr[j] == (int32_t)j;
+        for (; p < rows_p; ++p) {
+            const int64_t run0 = p & ~(int64_t)7;
+            if (ident_e) {
+                rr[p] = (int32_t)p;
+                pad_rank_plus1 = std::max(pad_rank_plus1, rr[p] + 1);
+            } else if (run0 >= rows_e) {
+                if (set->max_rank_plus1 >= 8) rr[p] = (int32_t)(p & 7);
+            } else if (rr[run0] >= 0 && (rr[run0] & 7) == 0) {
+                rr[p] = rr[run0] + (int32_t)(p - run0);
+                pad_rank_plus1 = std::max(pad_rank_plus1, rr[p] + 1);
+            }
+        }
+        for (int ps = 0; ps < n_ps[e]; ++ps)
+            if (width[ps] == 0) width[ps] = ps > 0 ? width[ps - 1] : 2;      // (a slab of padding only)
+        if (role == ROLE_GATE_UP)
+            for (int g0 = 0; g0 < n_ps[e]; g0 += GU_SLABS) {
+                int w = 0;
+                for (int q = 0; q < GU_SLABS; ++q) w = std::max(w, width[g0 + q]);
+                for (int q = 0; q < GU_SLABS; ++q) width[g0 + q] = w;
+            }
+        pay_off[e] = pay_words;
+        int64_t words = 0;
+        for (int ps = 0; ps < n_ps[e]; ++ps) {
+            BITSMOE_REQUIRE(words < ((int64_t)1 << 31) - (int64_t)n_tiles * 256 * 4, "expert %d: prepared payload exceeds int32 word offsets", e);
+            fslabs[(size_t)e * pms + ps] = FastSlab{width[ps], (int32_t)words, ps * n_tiles * SLAB_ROWS, ps * SLAB_ROWS};
+            words += (int64_t)n_tiles * 256 * width[ps];
+            tasks.push_back(SlabTask{e, ps});
+        }
+        pay_words += round_up(words, 64);      // keep every matrix 256-byte aligned
     }
+    set->pad_rank_plus1 = pad_rank_plus1;
     // every aligned run of 8 rows = 8 consecutive logical ranks starting at a multiple of 8?  rank'[k] == k?
     bool chunked8 = E > 0, identity = E > 0;
     for (int e = 0; e < E && (chunked8 || identity); ++e) {
-        const int64_t n = (int64_t)set->descs[e].num_slabs * SLAB_ROWS;
+        const int64_t n = (int64_t)n_ps[e] * SLAB_ROWS;
         const int32_t* r = rank_rows.data() + row_off[e];
         for (int64_t k = 0; k < n; ++k) {
             if (r[k] != (int32_t)k) identity = false;
@@ -272,32 +324,33 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
     }
     set->rank_chunked8 = chunked8;
     set->rank_identity = identity;
-    // does every aligned group of GU_SLABS slabs have one width (the same test the split gate/up kernel
-    // applies per workgroup), and is every expert ONE run of equal-width slabs (what the walking kernel assumes)?
-    bool all_uniform = max_slabs % GU_SLABS == 0, all_affine = max_slabs % GU_SLABS == 0;
-    for (int e = 0; e < E && all_uniform; ++e) {
-        if (set->descs[e].num_slabs != max_slabs) all_uniform = all_affine = false;
-        for (int si = 0; si < set->descs[e].num_slabs && all_uniform; ++si) {
-            const int bits = fslabs[(size_t)e * max_slabs + si].bits;
-            if (bits != fslabs[(size_t)e * max_slabs + si / GU_SLABS * GU_SLABS].bits) all_uniform = false;
-            if (bits != fslabs[(size_t)e * max_slabs].bits) all_affine = false;
-        }
+    // one width per expert and the same slab count everywhere (what the kernel that forms both projections in one
+    // workgroup still assumes)?  The walking kernel itself only needs whole groups of one width: true by construction.
+    bool all_affine = role == ROLE_GATE_UP;
+    for (int e = 0; e < E && all_affine; ++e) {
+        if (n_ps[e] != pms) all_affine = false;
+        for (int ps = 1; ps < n_ps[e] && all_affine; ++ps)
+            if (fslabs[(size_t)e * pms + ps].bits != fslabs[(size_t)e * pms].bits) all_affine = false;
     }
-    set->all_uniform8 = all_uniform;
-    set->all_affine = all_uniform && all_affine;
+    set->all_uniform8 = role == ROLE_GATE_UP;
+    set->all_affine = all_affine;
     set->vector_aligned = true;       // (the prepared tables are the library's own, 256-byte aligned allocations)
 
     BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_prepared, (size_t)std::max<int64_t>(pay_words, 1) * 4));
-    // one allocation for the row tables: rank' (i32), s' (f16), scale' (f16)
-    const size_t rows_bytes = (size_t)round_up(rows_total * 4, 256) + (size_t)round_up(rows_total * 2, 256) +
+    // one allocation for the row tables: rank' (i32), source of every row (i32), s' (f16), scale' (f16)
+    const size_t rows_bytes = 2 * (size_t)round_up(rows_total * 4, 256) + (size_t)round_up(rows_total * 2, 256) +
                               (size_t)round_up(scale_total * 2, 256);
     BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_prepared_rows, std::max<size_t>(rows_bytes, 256)));
     int32_t* d_rank = (int32_t*)set->d_prepared_rows;
-    __half* d_s = (__half*)((char*)set->d_prepared_rows + round_up(rows_total * 4, 256));
+    int32_t* d_src = (int32_t*)((char*)d_rank + round_up(rows_total * 4, 256));
+    __half* d_s = (__half*)((char*)d_src + round_up(rows_total * 4, 256));
     __half* d_scale = (__half*)((char*)d_s + round_up(rows_total * 2, 256));
     if (role == ROLE_GATE_UP)
         BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_scale_s, (size_t)std::max<int64_t>(scale_total, 1) * 2));
     BITSMOE_HIP_TRY(hipMemcpyAsync(d_rank, rank_rows.data(), (size_t)rows_total * 4, hipMemcpyHostToDevice, st));
+    BITSMOE_HIP_TRY(hipMemcpyAsync(d_src, row_src.data(), (size_t)rows_total * 4, hipMemcpyHostToDevice, st));
+    BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_prep_tasks, sizeof(SlabTask) * std::max<size_t>(tasks.size(), 1)));
+    BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_prep_tasks, tasks.data(), sizeof(SlabTask) * tasks.size(), hipMemcpyHostToDevice, st));
 
     std::vector<FastExpert> fexp(E);
     set->expert_bits.assign(E, 0);
@@ -309,19 +362,22 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
         f.s = d_s + row_off[e];
         f.rank_idx = d_rank + row_off[e];
         f.scale_s = set->d_scale_s ? set->d_scale_s + sc_off[e] : nullptr;
-        f.num_slabs = set->descs[e].num_slabs;
-        f.uniform_bits = f.num_slabs > 0 ? set->slab_meta_host[e][0] : 0;
-        for (int si = 1; si < f.num_slabs; ++si)
-            if (set->slab_meta_host[e][si * 4] != f.uniform_bits) f.uniform_bits = 0;
+        f.num_slabs = n_ps[e];
+        f.uniform_bits = fslabs[(size_t)e * pms].bits;
+        for (int ps = 1; ps < n_ps[e]; ++ps)
+            if (fslabs[(size_t)e * pms + ps].bits != f.uniform_bits) f.uniform_bits = 0;
         set->expert_bits[e] = (uint8_t)f.uniform_bits;
     }
+    set->uniform_experts = true;
+    for (int e = 0; e < E; ++e)
+        if (set->expert_bits[e] == 0) set->uniform_experts = false;
     set->has_cost_order = E <= EXPERT_ORDER_MAX;
     if (set->has_cost_order) {
         std::vector<int> order(E);
         for (int e = 0; e < E; ++e) order[e] = e;
         auto words = [&](int e) {       // payload words per tile of expert e
             int64_t w = 0;
-            for (int si = 0; si < set->descs[e].num_slabs; ++si) w += set->slab_meta_host[e][si * 4];
+            for (int ps = 0; ps < n_ps[e]; ++ps) w += fslabs[(size_t)e * pms + ps].bits;
             return w;
         };
         std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return words(a) > words(b); });
@@ -331,14 +387,17 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
     BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_fast_experts, fexp.data(), sizeof(FastExpert) * fexp.size(), hipMemcpyHostToDevice, st));
     BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_fast_slabs, sizeof(FastSlab) * fslabs.size()));
     BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_fast_slabs, fslabs.data(), sizeof(FastSlab) * fslabs.size(), hipMemcpyHostToDevice, st));
-    hipLaunchKernelGGL(k_prepare_rows, dim3((unsigned)set->total_slabs, n_tiles), dim3(64), 0, st, set->d_views,
-                       set->d_fast_experts, set->d_fast_slabs, max_slabs, set->d_slab_tasks);
+    const PrepSource ps_tab{d_src, d_rank};
+    hipLaunchKernelGGL(k_prepare_rows, dim3((unsigned)tasks.size(), n_tiles), dim3(64), 0, st, set->d_views,
+                       set->d_fast_experts, set->d_fast_slabs, pms, set->d_prep_tasks, ps_tab);
     BITSMOE_HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(k_prepack, dim3((unsigned)set->total_slabs, n_tiles), dim3(256), 0, st, set->d_views,
-                       set->d_fast_experts, set->d_fast_slabs, max_slabs, set->d_slab_tasks, role);
+    hipLaunchKernelGGL(k_prepack, dim3((unsigned)tasks.size(), n_tiles), dim3(256), 0, st, set->d_views,
+                       set->d_fast_experts, set->d_fast_slabs, pms, set->d_prep_tasks, ps_tab, role);
     BITSMOE_HIP_TRY(hipGetLastError());
     BITSMOE_HIP_TRY(hipStreamSynchronize(st));      // (the host vectors above are read by the copies until here)
     set->fast_experts_host = fexp;
+    set->prep_row_offsets = row_off;
+    set->d_row_src = d_src;
     set->role = role;
     return BITSMOE_OK;
 }
@@ -361,9 +420,11 @@ extern "C" int bitsmoe_dequant_matrix_prepared(const bitsmoe_matset* set, int32_
     mv.num_tiles = d.num_tiles;
     mv.rank_len = d.rank_len;
     mv.flags = 1;
-    hipLaunchKernelGGL(k_dequant_prepared, dim3(d.num_slabs, set->n_tiles), dim3(256), 0, st, mv,
-                       set->fast_experts_host[expert], set->d_fast_slabs + (int64_t)expert * set->max_slabs, set->role,
-                       set->intermediate_size, out_device);
+    const FastExpert& fe = set->fast_experts_host[expert];
+    const int32_t* d_src = set->d_row_src + set->prep_row_offsets[expert];
+    hipLaunchKernelGGL(k_dequant_prepared, dim3(fe.num_slabs, set->n_tiles), dim3(256), 0, st, mv, fe,
+                       set->d_fast_slabs + (int64_t)expert * set->prep_max_slabs, d_src, set->role, set->intermediate_size,
+                       out_device);
     BITSMOE_HIP_TRY(hipGetLastError());
     return BITSMOE_OK;
 }

@@ -330,10 +330,11 @@ def test_forward_mfma_path_scattered_ranks(cuda_device, dtype_name):
     assert err < 3e-3
 
 
-def _checkpoint_shaped_experts(seed, n_experts, rank, dim):
+def _checkpoint_shaped_experts(seed, n_experts, rank, dim, permute=True):
     """Experts packed the way a checkpoint's are (bitsmoe/quant/packer.py:566-589, 615-643): per matrix three
     width buckets in descending order of width whose sizes are no multiples of 64 (ragged last slabs), about
-    5 % of the ranks dropped (0-bit segment), and the kept rows in a permuted order of ranks."""
+    5 % of the ranks dropped (0-bit segment), and the kept rows in a permuted order of ranks -- or, with
+    permute=False, in ascending order (row k holds rank k, the dropped ranks are the last ones)."""
     rng = np.random.default_rng(seed)
     mats = ([], [], [])
     for _ in range(n_experts):
@@ -345,24 +346,29 @@ def _checkpoint_shaped_experts(seed, n_experts, rank, dim):
             segs = [(4, (0, cut1)), (3, (cut1, cut2)), (2, (cut2, rank - n_drop)), (0, (rank - n_drop, rank))]
             m = helpers.make_matrix(rng, rank, dim, segs)
             # the packer keeps rows in segment order; give them a permuted set of logical ranks
-            m["rank_idx"] = perm[m["rank_idx"]].astype(np.int32)
+            if permute:
+                m["rank_idx"] = perm[m["rank_idx"]].astype(np.int32)
             lst.append(m)
     return mats
 
 
 @pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
 @pytest.mark.parametrize("path_name,tokens", [("decode", 9), ("decode", 70), ("mfma", 300), ("auto", 40)])
-def test_forward_checkpoint_shaped_layout_on_fast_paths(cuda_device, path_name, tokens, dtype_name):
+@pytest.mark.parametrize("rank,permute", [(300, True), (300, False), (512, False), (1088, False)])
+def test_forward_checkpoint_shaped_layout_on_fast_paths(cuda_device, path_name, tokens, dtype_name, rank, permute):
     """Several width buckets per expert with ragged slabs, dropped and permuted ranks: the matrix sets are
-    prepared (padded copy) and the decode / grouped-GEMM kernels run them -- not the generic fallback."""
+    prepared (padded copy) and the decode / grouped-GEMM kernels run them -- not the generic fallback.
+    Ascending ranks keep the identity through the padding rows (whose ranks may lie beyond the activations'
+    and the output's width: rank 300); with the rank a multiple of 512 the gate/up kernel that walks a tile
+    over slab groups of different widths runs, with 1088 over three groups and a padded tail."""
     import torch
 
     from bitsmoe_amd.algorithms import _capi
 
     hip = _hip()
     path = {"decode": _capi.PATH_DECODE, "mfma": _capi.PATH_MFMA, "auto": _capi.PATH_AUTO}[path_name]
-    e, k, rank, dim = 6, 2, 300, 256
-    gate, up, down = _checkpoint_shaped_experts(900 + tokens, e, rank, dim)
+    e, k, dim = 6, 2, 256
+    gate, up, down = _checkpoint_shaped_experts(900 + tokens, e, rank, dim, permute=permute)
     rng = np.random.default_rng(tokens)
     dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
     h_gate = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(dt)
