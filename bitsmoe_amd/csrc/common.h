@@ -71,8 +71,11 @@ bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up,
 int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
                           const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg,
                           int64_t ldu, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
-                          int I, float* rank_accum, float* G, float* U, int64_t inter_floats, bitsmoe_profile* prof,
-                          hipStream_t st);
+                          int I, float* rank_accum, float* G, float* U, int64_t inter_floats, int part_capacity,
+                          bitsmoe_profile* prof, hipStream_t st);
+// How many partial results of the two fp32 intermediates the decode path's workspace holds (the gate/up kernel
+// may split its contraction over workgroups when there are few assignments).
+inline int decode_part_capacity(int64_t n_assign) { return n_assign <= 1024 ? 4 : n_assign <= 4096 ? 2 : 1; }
 
 bool mfma_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I);
 size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int64_t T,

@@ -706,10 +706,12 @@ __device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4
 // assignments) waits in LDS, and z is built two assignment rows at a time.
 // ZREADY: `G` holds Z (16-bit operands, [A, I]) and `U` holds Zsum ([A, n_tiles] fp32) as written by
 // gateup_walk_z_item: the z phase is a copy into LDS instead of two fp32 reads and a SiLU per element.
+// Otherwise G and U are the first of `n_part` partial results, part_stride floats apart, that are added up.
 template <int W, bool ZREADY = false>
 __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gptr<__half> svec, gptr<int32_t> rank_idx,
-                                 const FastSlab fs, const float* __restrict__ G, const float* __restrict__ U,
-                                 const float* __restrict__ route_w, const int32_t* __restrict__ token_indices,
+                                 const FastSlab fs, const float* __restrict__ G, const float* __restrict__ U, int n_part,
+                                 int64_t part_stride, const float* __restrict__ route_w,
+                                 const int32_t* __restrict__ token_indices,
                                  int a_begin, int a_end, int T, int I, int tb, int nt, int rank_out,
                                  float* __restrict__ rank_accum, uint16_t* __restrict__ z, int z_stride, float* __restrict__ zsum,
                                  int2* __restrict__ rows, int2* __restrict__ assigns, int tid, int lane) {
@@ -798,6 +800,16 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                     const int64_t gi = (int64_t)(a0 + a) * I + c;
                     gv[j] = *reinterpret_cast<const f32x4*>(G + gi);
                     uv[j] = *reinterpret_cast<const f32x4*>(U + gi);
+                }
+                // (the gate/up kernel split the contraction: the sums are totals of partial results)
+                for (int p = 1; p < n_part; ++p) {
+#pragma unroll
+                    for (int j = 0; j < ZROWS; ++j) {
+                        const int a = min(ab + j, n_a - 1);
+                        const int64_t gi = (int64_t)(a0 + a) * I + c + p * part_stride;
+                        gv[j] += *reinterpret_cast<const f32x4*>(G + gi);
+                        uv[j] += *reinterpret_cast<const f32x4*>(U + gi);
+                    }
                 }
 #pragma unroll
                 for (int j = 0; j < ZROWS; ++j) {

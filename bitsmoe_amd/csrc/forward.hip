@@ -49,9 +49,9 @@ extern "C" size_t bitsmoe_forward_workspace_bytes(int64_t n_tokens, int64_t n_as
     (void)n_experts;
     (void)rank_out;
     if (n_assign < 0 || intermediate_size < 0) return 0;
-    // two fp32 [A, I] intermediates (gate and up outputs)
+    // two fp32 [A, I] intermediates (gate and up outputs), several partial results of them for small batches
     const size_t inter = align_up((size_t)n_assign * (size_t)intermediate_size * sizeof(float), 256);
-    return 2 * inter + 256;
+    return 2 * inter * (size_t)decode_part_capacity(n_assign) + 256;
 }
 
 // The path bitsmoe_moe_forward takes for these sets, sizes and `path` request
@@ -169,7 +169,8 @@ extern "C" int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bit
     if (chosen == BITSMOE_PATH_DECODE)
         return launch_forward_decode(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
                                      token_indices, expert_offsets, route_w, n_assign, rank_out, intermediate_size,
-                                     rank_accum, G, U, (int64_t)(inter / sizeof(float)), profile, st);
+                                     rank_accum, G, U, (int64_t)(inter / sizeof(float)), decode_part_capacity(n_assign), profile,
+                                     st);
     return launch_forward_generic(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
                                   token_indices, expert_offsets, route_w, n_assign, rank_out,
                                   intermediate_size, rank_accum, G, U, profile, st);

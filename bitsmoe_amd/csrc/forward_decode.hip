@@ -23,6 +23,7 @@
 // return in order, so a small request behind a large one waits for the large one.
 #include "decode_bodies.h"
 
+#include <atomic>
 #include <cstdlib>
 
 namespace bitsmoe {
@@ -288,9 +289,16 @@ __global__ __launch_bounds__(256, 4) void k_gateup_decode(
 }
 
 // ------------------------------------------------------- gate / up, one workgroup per tile
-// gateup_walk_item launched as a grid of its own: grid.x = (expert coordinate) * n_tiles, grid.y = 2
-// (gate, up); 256 threads = 4 wavefronts.  An expert with more than 16 assignments is served in
-// 16-assignment chunks, one after the other (or one workgroup per chunk: GRID_CHUNKS).
+// gateup_walk_item launched as a grid of its own; 256 threads = 4 wavefronts.  An item is (expert
+// coordinate, tile, projection), item = (coordinate * n_tiles + tile) * 2 + projection; an expert with
+// more than 16 assignments is served in 16-assignment chunks, one after the other (or one workgroup per
+// chunk: GRID_CHUNKS).
+// The first `n_unsplit` workgroups take one item each; behind them every item is shared by `split`
+// workgroups, each of which contracts over its share of the item's slab groups and stores its sums into
+// a partial result of its own: partial p of G / U lies p * part_stride floats behind G / U.  The down
+// kernel adds the `n_part` partials up (n_part = split when any item is split, else 1), so a workgroup
+// with a whole item stores zeros into the partials 1 .. n_part - 1 of its elements.  The launcher splits
+// the items when there are too few of them to fill the chip.
 // The kernel also clears `zero_out` (the forward's accumulator, added into by the down kernel).
 // MIXED: experts whose slab groups differ in width (gateup_walk_item_mixed); a kernel of its own, so that
 // the one-width kernel keeps its registers to itself.
@@ -300,15 +308,23 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
     const uint16_t* __restrict__ h_gate, const uint16_t* __restrict__ h_up, int64_t ldg, int64_t ldu,
     const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
-    int E, int n_tiles, float* __restrict__ G, float* __restrict__ U, float* __restrict__ zero_out,
-    int64_t zero_n, const ExpertOrder gate_order, const ExpertOrder up_order) {
-    const int mt = blockIdx.y;
-    const int bid = blockIdx.x;
+    int E, int n_tiles, float* __restrict__ G, float* __restrict__ U, int n_unsplit, int split, int n_part,
+    int64_t part_stride, float* __restrict__ zero_out, int64_t zero_n, const ExpertOrder gate_order,
+    const ExpertOrder up_order) {
     const int tid = threadIdx.x;
     {   // this workgroup's share of the accumulator (before any exit)
-        const int64_t total = (int64_t)gridDim.x * 2 * 256;
-        for (int64_t i = ((int64_t)mt * gridDim.x + bid) * 256 + tid; i < zero_n; i += total) zero_out[i] = 0.0f;
+        const int64_t total = (int64_t)gridDim.x * 256;
+        for (int64_t i = (int64_t)blockIdx.x * 256 + tid; i < zero_n; i += total) zero_out[i] = 0.0f;
     }
+    int item = blockIdx.x, part = 0, parts = 1;
+    if (item >= n_unsplit) {
+        const int r = item - n_unsplit;
+        item = n_unsplit + r / split;
+        part = r % split;
+        parts = split;
+    }
+    const int mt = item & 1;
+    const int bid = item >> 1;
     const int t = bid % n_tiles;
     int e = bid / n_tiles;
     int chunk = -1;
@@ -346,13 +362,29 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     }
     if (a_end <= a_begin || first.bits == 0) return;
     const int n_groups = fe.num_slabs / GU_SLABS;
+    // this workgroup's share of the slab groups, and the partial result it writes
+    const int g_begin = (int)((int64_t)part * n_groups / parts), g_end = (int)((int64_t)(part + 1) * n_groups / parts);
 
     gptr<uint32_t> payload = as_global(fe.payload);
     gptr<__half> scale_s = as_global(fe.scale_s);
     gptr<int32_t> rank_idx = as_global(fe.rank_idx);
     const uint16_t* __restrict__ h = mt ? h_up : h_gate;
     const int64_t ld = mt ? ldu : ldg;
-    float* __restrict__ out = mt ? U : G;
+    float* __restrict__ out = (mt ? U : G) + part * part_stride;
+    // partials nobody else writes for these elements: all but the own one of a share without slab groups,
+    // 1 .. n_part - 1 of a whole item
+    {
+        const int p_first = parts > 1 ? part : 1, p_end = parts > 1 ? (g_begin == g_end ? part + 1 : part) : n_part;
+        const int cols = min(N_TILE, I - t * N_TILE);
+        for (int p = p_first; p < p_end; ++p) {
+            float* __restrict__ zp = (mt ? U : G) + p * part_stride;
+            for (int i = tid; i < (a_end - a_begin) * N_TILE; i += 256) {
+                const int a = i / N_TILE, c = i - a * N_TILE;
+                if (c < cols) zp[(int64_t)(a_begin + a) * I + t * N_TILE + c] = 0.0f;
+            }
+        }
+    }
+    if (g_begin == g_end) return;
 
     // two copies of the operand, used in turn: one workgroup barrier per group instead of two
     __shared__ __attribute__((aligned(16))) uint16_t hs_all[2 * MAX_A * GU_STRIDE];
@@ -364,12 +396,12 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
         if (a0 != a_begin) __syncthreads();      // the previous chunk's readers of the operand are done
         if constexpr (MIXED) {
             gateup_walk_item_mixed<BF16, IDENT, false>(payload, scale_s, rank_idx, grp_tab, h, ld, token_indices, a0, n_a, A, T, I,
-                                                       n_tiles, t, 0, n_groups, out, hs_all, cterm_lds, tid);
+                                                       n_tiles, t, g_begin, g_end, out, hs_all, cterm_lds, tid);
         } else {
             auto run = [&](auto w_c) {
                 gateup_walk_item<BF16, IDENT, decltype(w_c)::value, false>(payload, scale_s, rank_idx, first, h, ld,
-                                                                           token_indices, a0, n_a, A, T, I, n_tiles, t, 0,
-                                                                           n_groups, out, hs_all, cterm_lds, tid);
+                                                                           token_indices, a0, n_a, A, T, I, n_tiles, t, g_begin,
+                                                                           g_end, out, hs_all, cterm_lds, tid);
             };
             if (first.bits == 2)
                 run(std::integral_constant<int, 2>{});
@@ -449,14 +481,15 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk_z(
 // per-tile sums of its rows, the epilogue's row and assignment records.
 // A workgroup takes four slabs of one expert and a run of tiles; with few active experts the
 // tiles are split over several workgroups (their partial sums meet in the atomics of the combine).
-// ZREADY: G / U hold Z / Zsum written by k_gateup_walk_z instead of the fp32 gate and up sums.
+// ZREADY: G / U hold Z / Zsum written by k_gateup_walk_z instead of the fp32 gate and up sums.  Otherwise the
+// sums are the totals of `n_part` partial results part_stride floats apart (k_gateup_walk).
 template <int MODE, bool ZREADY>
 __global__ __launch_bounds__(256, 4) void k_down_decode(
     const FastExpert* __restrict__ down_fe, const FastSlab* __restrict__ down_fs, int max_slabs,
-    const float* __restrict__ G, const float* __restrict__ U, const float* __restrict__ route_w,
-    const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
-    int E, int n_tiles, int n_groups, int n_tchunks, int tiles_per_wg, int n_work, int rank_out,
-    float* __restrict__ rank_accum) {
+    const float* __restrict__ G, const float* __restrict__ U, int n_part, int64_t part_stride,
+    const float* __restrict__ route_w, const int32_t* __restrict__ token_indices,
+    const int32_t* __restrict__ expert_offsets, int T, int A, int I, int E, int n_tiles, int n_groups, int n_tchunks,
+    int tiles_per_wg, int n_work, int rank_out, float* __restrict__ rank_accum) {
     // Workgroup b runs on XCD b % 8, and every XCD has its own L2: the workgroups of one expert
     // (which all read that expert's G / U rows) are given ids of one residue class, so that they
     // share one L2.  The grid is a multiple of 8; ids past the work exit.
@@ -507,17 +540,17 @@ __global__ __launch_bounds__(256, 4) void k_down_decode(
     // the four wavefronts may run four different instantiations; every one of them executes
     // the same two workgroup barriers per assignment chunk
     if (fs.bits == 2)
-        down_wave<2, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
-                           rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
+        down_wave<2, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, route_w, token_indices, a_begin,
+                           a_end, T, I, tb, nt, rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else if (fs.bits == 3)
-        down_wave<3, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
-                           rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
+        down_wave<3, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, route_w, token_indices, a_begin,
+                           a_end, T, I, tb, nt, rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else if (fs.bits == 4)
-        down_wave<4, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
-                           rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
+        down_wave<4, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, route_w, token_indices, a_begin,
+                           a_end, T, I, tb, nt, rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else
-        down_wave<0, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, route_w, token_indices, a_begin, a_end, T, I, tb, nt,
-                           rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
+        down_wave<0, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, route_w, token_indices, a_begin,
+                           a_end, T, I, tb, nt, rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
 }
 
 __global__ void k_fill_zero2(float* __restrict__ p1, int64_t n1, float* __restrict__ p2, int64_t n2) {
@@ -531,6 +564,19 @@ static inline void record(bitsmoe_profile* p, int i, hipStream_t st) {
     if (p) (void)hipEventRecord(p->ev[i], st);
 }
 
+// Compute units of the current device (asked once per device; 256 when the query fails).
+static int cu_count() {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
 bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I) {
     const int n_tiles = (I + N_TILE - 1) / N_TILE;
     const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4 + DN_SLABS_PER_WG * SLAB_ROWS * 8 + MAX_A * 8;
@@ -541,8 +587,8 @@ bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up,
 int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
                           const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg,
                           int64_t ldu, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
-                          int I, float* rank_accum, float* G, float* U, int64_t inter_floats, bitsmoe_profile* prof,
-                          hipStream_t st) {
+                          int I, float* rank_accum, float* G, float* U, int64_t inter_floats, int part_capacity,
+                          bitsmoe_profile* prof, hipStream_t st) {
     const int E = gate->n_experts;
     const int n_tiles = gate->n_tiles;
     record(prof, 0, st);
@@ -621,6 +667,22 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         else
             fn(bf16_c, std::integral_constant<int, GRID_EXPERTS>{});
     };
+    // The walking kernel's workgroups: one per item, unless the items fill less than half of the chip's
+    // `slots` (four resident workgroups per CU): then every item is split over `split` workgroups, each of
+    // which contracts over a share of the slab groups, and the down kernel adds the `n_part` partial results
+    // up.  (Halving only the cheapest items of a grid whose last round is partly empty -- 1536 items on 1024
+    // slots -- was measured too: the gate/up kernel gains nothing, the down kernel's SiLU pass reads twice as much.)
+    const int64_t n_items = (int64_t)e_dim * n_tiles * 2;
+    const int64_t slots = 4 * (int64_t)cu_count();
+    const int max_part = (int)std::min<int64_t>(part_capacity, 4);
+    int64_t n_unsplit = n_items;
+    int split = 1;
+    if (walk && !fused_z && n_items * 2 <= slots) {
+        while (split * 2 <= max_part && split * 2 <= gu_groups && n_items * split * 2 <= slots) split *= 2;
+        if (split > 1) n_unsplit = 0;
+    }
+    const int n_part = n_unsplit < n_items ? split : 1;
+    const int64_t part_stride = 2 * inter_floats;
     auto launch_walk_mode = [&](auto bf16_c, auto mode_c) {
         // (one width per expert in both sets: the kernel compiled for that; else the one that switches per slab group)
         const bool ident = gate->rank_identity && up->rank_identity;
@@ -629,11 +691,11 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         constexpr int M = decltype(mode_c)::value;
         auto kern = mixed ? (ident ? k_gateup_walk<B, M, true, true> : k_gateup_walk<B, M, false, true>)
                           : (ident ? k_gateup_walk<B, M, true, false> : k_gateup_walk<B, M, false, false>);
-        hipLaunchKernelGGL(kern, dim3((unsigned)(e_dim * n_tiles), 2),
-                           dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs, gate->prep_max_slabs, up->d_fast_experts,
+        hipLaunchKernelGGL(kern, dim3((unsigned)(n_unsplit + (n_items - n_unsplit) * split)), dim3(256), 0, st,
+                           gate->d_fast_experts, gate->d_fast_slabs, gate->prep_max_slabs, up->d_fast_experts,
                            up->d_fast_slabs, up->prep_max_slabs, (const uint16_t*)h_gate, (const uint16_t*)h_up, ldg, ldu,
-                           tok, off, (int)T, (int)A, I, E, n_tiles, G, U, rank_accum, T * (int64_t)rank_out, gate_order,
-                           up_order);
+                           tok, off, (int)T, (int)A, I, E, n_tiles, G, U, (int)n_unsplit, split, n_part, part_stride, rank_accum,
+                           T * (int64_t)rank_out, gate_order, up_order);
     };
     auto launch_walk_z_mode = [&](auto bf16_c, auto mode_c) {
         auto kern = k_gateup_walk_z<decltype(bf16_c)::value, decltype(mode_c)::value, false>;
@@ -671,8 +733,8 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     auto launch_down = [&](auto kernel) {
         const int n_work = e_dim * dn_groups * dn_tchunks;
         hipLaunchKernelGGL(kernel, dim3((unsigned)((n_work + 7) / 8 * 8)), dim3(256), z_bytes, st, down->d_fast_experts,
-                           down->d_fast_slabs, down->prep_max_slabs, G, U, rw, tok, off, (int)T, (int)A, I, E, n_tiles,
-                           dn_groups, dn_tchunks, dn_tiles_per_wg, n_work, rank_out, rank_accum);
+                           down->d_fast_slabs, down->prep_max_slabs, G, U, walk && !fused_z ? n_part : 1, part_stride, rw, tok, off,
+                           (int)T, (int)A, I, E, n_tiles, dn_groups, dn_tchunks, dn_tiles_per_wg, n_work, rank_out, rank_accum);
     };
     auto launch_down_mode = [&](auto zready_c, auto mode_c) {
         launch_down(k_down_decode<decltype(mode_c)::value, decltype(zready_c)::value>);
@@ -690,3 +752,4 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
 }
 
 }  // namespace bitsmoe
+
