@@ -137,3 +137,42 @@ def test_block_sees_an_expert_reloaded_in_place(cuda_device):
     scale = float(y2.abs().max())
     assert float((y1 - y2).abs().max()) <= 1e-3 * scale
     assert float((y0 - y2).abs().max()) > 5e-2 * scale
+
+
+def test_block_state_dict_round_trip_through_a_checkpoint(cuda_device):
+    """state_dict() of a packed block, saved and loaded back the way a checkpoint is (tensors only, on the CPU),
+    restores the block on the GPU: the packed buffers are bound again (bitsmoe/models/base_mlp.py:319-383)
+    and the matrix sets of the next forward are built from the loaded bytes."""
+    import io
+
+    import torch
+
+    from bitsmoe_amd.synth import LayerSpec, make_layer
+
+    spec = LayerSpec("tiny", "qwen3next", 6, 2, 128, 256, (0.5, 0.3, 0.2), "normal", True, 128, rank=128)
+    source = make_layer(spec, device=cuda_device, dtype=torch.bfloat16, seed=5)
+    target = make_layer(spec, device=cuda_device, dtype=torch.bfloat16, seed=5)      # same shapes ...
+    x = torch.randn((1, 11, 128), generator=torch.Generator().manual_seed(3)).to(torch.bfloat16).to(cuda_device)
+
+    def run(block):
+        y = block(x)
+        return (y[0] if isinstance(y, tuple) else y).float().clone()
+
+    with torch.no_grad():
+        want = run(source)
+        for name, buf in target.named_buffers():      # ... other contents
+            if name.endswith("scale_buffer"):
+                buf.mul_(2.0)
+        for p in target.parameters():
+            p.mul_(0.5)
+        spoiled = run(target)
+        blob = io.BytesIO()
+        torch.save({k: v.cpu() for k, v in source.state_dict().items()}, blob)
+        blob.seek(0)
+        state = torch.load(blob, map_location="cpu", weights_only=True)
+        missing, unexpected = target.load_state_dict(state, strict=False)
+        assert not unexpected, unexpected
+        got = run(target)
+    scale = float(want.abs().max())
+    assert float((spoiled - want).abs().max()) > 5e-2 * scale
+    assert float((got - want).abs().max()) <= 1e-3 * scale
