@@ -4,8 +4,10 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2-t64] [--no-extras] [--no-cpu]
 
 A "step" is one pass of the hot path over one batch that is already resident in HBM:
-routing/permute kernel -> gate & up -> SiLU*mul -> down -> top-k weighted combine
-(operator scope: from the router's top-k ids to rank_accum [T, rank_out]).  The layer is
+routing/permute -> gate & up -> SiLU*mul -> down -> top-k weighted combine
+(operator scope: from the router's top-k ids to rank_accum [T, rank_out]; one call of
+bitsmoe_moe_forward_routed, which runs small batches without a routing kernel -- the forward's kernels find
+their assignments themselves -- and builds routing tables first otherwise; `config.routing` says which).  The layer is
 synthetic (random-init factors of the named shape, quantised and packed on the GPU).
 
 Cold weights.  A model streams a different layer's weights on every step, so a benchmark that
@@ -106,12 +108,14 @@ class _LayerState:
         self.rank_out = int(block.shared_u_down.shape[1])
         self.isz = int(block._packed_intermediate_size)
         self.g2l = block._packed_global_to_local
+        self.l2g = block._packed_local_to_global
         self.n_packed = block._packed_expert_count
 
 
 def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, layers_per_step=1, block_scope=True):
-    """Times `steps` steps; a step is `layers_per_step` consecutive layer-steps (routing kernel + operator)
-    of the rotation blocks[0], blocks[1], ... (one block: the same layer replayed, warm caches)."""
+    """Times `steps` steps; a step is `layers_per_step` consecutive layer-steps (routing + operator, from the
+    router's top-k output to rank_accum: one call, bitsmoe_moe_forward_routed) of the rotation blocks[0],
+    blocks[1], ... (one block: the same layer replayed, warm caches)."""
     import torch
 
     from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
@@ -122,10 +126,13 @@ def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, l
 
     def layer_step(i, profile=None):
         st = layers[i % n_layers]
-        tok, off, rw = hip.route(st.selected, st.weights, st.g2l, st.n_packed)
         gate, up, down = st.sets
-        out = hip.moe_forward_sets(st.h_gate, st.h_up, tok, off, rw, gate, up, down, st.rank_out, st.isz, 0, profile=profile)
-        return tok, off, rw, out
+        return hip.moe_forward_routed(st.h_gate, st.h_up, st.selected, st.weights, st.g2l, st.l2g, gate, up, down,
+                                      st.rank_out, st.isz, 0, profile=profile)
+
+    def layer_tables(i):      # (the routing tables, for the accounting and the CPU check only)
+        st = layers[i % n_layers]
+        return hip.route(st.selected, st.weights, st.g2l, st.n_packed)
 
     n_layer_steps = steps * layers_per_step
     for i in range(max(warmup * layers_per_step, n_layers)):
@@ -157,13 +164,13 @@ def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, l
             torch.cuda.current_stream(dev).wait_stream(side)
             torch.cuda.synchronize(dev)
             with torch.cuda.graph(graph):
-                g_outs = [layer_step(i)[3] for i in range(n_layers)]
+                g_outs = [layer_step(i) for i in range(n_layers)]
             # every replay must reproduce the eager result (fp32 atomics: summation order may differ)
             for _ in range(3):
                 graph.replay()
                 torch.cuda.synchronize(dev)
                 for i in (0, n_layers - 1):
-                    ref_out = layer_step(i)[3]
+                    ref_out = layer_step(i)
                     torch.cuda.synchronize(dev)
                     if not torch.allclose(g_outs[i], ref_out, rtol=1e-4, atol=1e-5 * float(ref_out.abs().max())):
                         raise RuntimeError("graph replay differs from the eager result")
@@ -207,7 +214,8 @@ def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, l
     # algorithmic work of one layer-step: the mean over the layers of the rotation
     works, last = [], None
     for i in range(n_layers):
-        tok, off, rw, out = layer_step(i)
+        out = layer_step(i)
+        tok, off, rw = layer_tables(i)
         torch.cuda.synchronize(dev)
         counts = (off[1:] - off[:-1]).cpu().tolist()
         works.append(algorithmic_work(layers[i].block, counts, tokens, int(tok.numel())))
@@ -219,6 +227,8 @@ def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, l
         "tokens": tokens, "layers_in_rotation": n_layers, "layers_per_step": layers_per_step,
         "ms_per_step": elapsed / steps * 1e3, "ms_per_layer": ms_layer, "tokens_per_s": tokens * steps / elapsed,
         "launch": launch, "eager_ms_per_step": eager / steps * 1e3, "hipgraph_ms_per_step": graph_ms,
+        "routing": "inside the gate/up and down kernels" if hip.routed_is_inline(
+            layers[0].h_gate, layers[0].h_up, int(layers[0].selected.shape[1]), *layers[0].sets) else "routing kernel(s) first",
         "kernel_ms": {"prepare": ms_fill, "gate_up": ms_gateup, "silu_mul": ms_silu, "down": ms_down,
                       "combine": ms_combine},
         "kernel_ms_events_raw": dict(zip(("prepare", "gate_up", "silu_mul", "down", "combine"), raw)),
@@ -474,12 +484,12 @@ def main() -> int:
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": res["ms_per_step"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"{args.workload}: {WORKLOAD_DESC[spec_key]}, {tokens} tokens, operator scope "
-                               "(routing kernel + gate/up + SiLU*mul + down + combine), inputs resident in HBM, "
+                               "(routing + gate/up + SiLU*mul + down + combine), inputs resident in HBM, "
                                f"{res['layers_in_rotation']} distinct layers in rotation "
                                f"({'cold' if res['layers_in_rotation'] > 1 else 'warm'} weights)",
                    "tokens": tokens, "mean_bits": sum(bits) / len(bits), "active_experts": res["active_experts"],
                    "device": get_cuda_device_name(), "layer_build_s": round(built[shape_key + "/build_s"], 2),
-                   "launch": res["launch"], "activation_dtype": "bf16",
+                   "launch": res["launch"], "routing": res["routing"], "activation_dtype": "bf16",
                    "arithmetic": "bf16 activations in, f16 MFMA operands, fp32 accumulation"},
         "eager_ms_per_step": res["eager_ms_per_step"], "hipgraph_ms_per_step": res["hipgraph_ms_per_step"],
         "block_scope": res.get("block_scope"), "warm": res.get("warm"),

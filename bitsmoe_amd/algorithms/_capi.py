@@ -38,6 +38,9 @@ EXPORTED_SYMBOLS = (
     "bitsmoe_moe_forward_strided",
     "bitsmoe_static_scratch_bytes",
     "bitsmoe_moe_forward_static",
+    "bitsmoe_forward_routed_workspace_bytes",
+    "bitsmoe_moe_forward_routed",
+    "bitsmoe_forward_routed_is_inline",
     "bitsmoe_profile_create",
     "bitsmoe_profile_destroy",
     "bitsmoe_profile_read",
@@ -126,6 +129,17 @@ def load() -> ctypes.CDLL:
     lib.bitsmoe_moe_forward_static.argtypes = [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_int64, c_int64,
         c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p,
+    ]
+    lib.bitsmoe_forward_routed_workspace_bytes.restype = c_size_t
+    lib.bitsmoe_forward_routed_workspace_bytes.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32]
+    lib.bitsmoe_forward_routed_is_inline.restype = c_int32
+    lib.bitsmoe_forward_routed_is_inline.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
+                                                     c_int64, c_int64, c_int64, c_int32, c_int32]
+    lib.bitsmoe_moe_forward_routed.restype = c_int32
+    lib.bitsmoe_moe_forward_routed.argtypes = [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_int64, c_int64,
+        c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_int32, c_int32, c_int32, c_int32,
+        c_void_p, c_void_p, c_size_t, c_void_p, c_void_p,
     ]
     lib.bitsmoe_profile_create.restype = c_int32
     lib.bitsmoe_profile_create.argtypes = [POINTER(c_void_p)]

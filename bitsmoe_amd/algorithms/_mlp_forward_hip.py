@@ -268,6 +268,59 @@ def moe_forward_sets(h_gate: torch.Tensor, h_up: torch.Tensor, token_indices: to
     return out
 
 
+def routed_is_inline(h_gate: torch.Tensor, h_up: torch.Tensor, top_k: int, gate: MatrixSet, up: MatrixSet, down: MatrixSet,
+                     path: int = _capi.PATH_AUTO) -> bool:
+    """Would moe_forward_routed run these activations without a routing kernel?"""
+    n_tokens = int(h_gate.shape[0])
+    return bool(_lib.bitsmoe_forward_routed_is_inline(
+        gate.handle, up.handle, down.handle, h_gate.data_ptr(), h_up.data_ptr(), int(h_gate.shape[1]), int(h_up.shape[1]),
+        int(h_gate.stride(0)) if n_tokens > 1 else int(h_gate.shape[1]),
+        int(h_up.stride(0)) if n_tokens > 1 else int(h_up.shape[1]), n_tokens, int(top_k), int(path)))
+
+
+def moe_forward_routed(h_gate: torch.Tensor, h_up: torch.Tensor, selected: torch.Tensor, weights: torch.Tensor,
+                       global_to_local: torch.Tensor, local_to_global: torch.Tensor, gate: MatrixSet, up: MatrixSet,
+                       down: MatrixSet, rank_out: int, intermediate_size: int, act_type: int = 0,
+                       path: int = _capi.PATH_AUTO, profile: Optional[Profile] = None,
+                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Routing and forward in one call, from the router's output: selected [T, k] expert ids (int32 / int64) and
+    weights fp32 [T, k]; global_to_local int32 [n_global] (-1: not a packed expert) and its inverse
+    local_to_global int32 [n_experts].  Small batches run without any routing kernel (the forward's kernels find
+    their assignments themselves); otherwise the routing tables are built first.  Returns rank_accum fp32
+    [tokens, rank_out], equal to moe_forward_sets(*route(...)) up to the order of fp32 atomics."""
+    _check(h_gate.dim() == 2 and h_up.dim() == 2 and h_gate.stride(1) == 1 and h_up.stride(1) == 1,
+           "h_gate/h_up must be 2D with unit column stride")
+    _check(selected.dim() == 2 and selected.shape == weights.shape and selected.shape[0] == h_gate.shape[0],
+           "selected and weights must be [tokens, top_k]")
+    _check(selected.dtype in (torch.int32, torch.int64), "selected must be int32 or int64")
+    _check(weights.dtype == torch.float32 and global_to_local.dtype == torch.int32 and local_to_global.dtype == torch.int32,
+           "weights must be float32, the id maps int32")
+    dev = h_gate.device
+    selected = selected.contiguous()
+    weights = weights.contiguous()
+    n_tokens, top_k = int(selected.shape[0]), int(selected.shape[1])
+    dt = _capi.DT_F16 if h_gate.dtype == torch.float16 else _capi.DT_BF16
+    if path != _capi.PATH_GENERIC and _AUTO_PREPARE and gate.role < 0 and up.role < 0 and down.role < 0:
+        if gate.fast_capable and up.fast_capable and down.fast_capable:
+            gate.prepare(0)
+            up.prepare(0)
+            down.prepare(1)
+    if out is None:
+        out = torch.empty((n_tokens, int(rank_out)), dtype=torch.float32, device=dev)
+    nbytes = int(_lib.bitsmoe_forward_routed_workspace_bytes(gate.handle, up.handle, down.handle, n_tokens, top_k, int(path)))
+    ws = _workspace(dev, nbytes)
+    with torch.cuda.device(dev):
+        _capi.check(_lib.bitsmoe_moe_forward_routed(
+            gate.handle, up.handle, down.handle, h_gate.data_ptr(), h_up.data_ptr(), dt, n_tokens,
+            int(h_gate.shape[1]), int(h_up.shape[1]), int(h_gate.stride(0)) if n_tokens > 1 else int(h_gate.shape[1]),
+            int(h_up.stride(0)) if n_tokens > 1 else int(h_up.shape[1]),
+            selected.data_ptr(), 1 if selected.dtype == torch.int64 else 0, weights.data_ptr(), top_k,
+            global_to_local.data_ptr(), int(global_to_local.numel()), local_to_global.data_ptr(),
+            int(rank_out), int(intermediate_size), int(act_type), int(path), out.data_ptr(), ws.data_ptr(), ws.numel(),
+            profile._handle if profile is not None else None, _stream_ptr(dev)))
+    return out
+
+
 def _check_cuda_contig(t: torch.Tensor, name: str) -> None:
     _check(t.is_cuda, f"{name} must be CUDA tensor")
     _check(t.is_contiguous(), f"{name} must be contiguous")

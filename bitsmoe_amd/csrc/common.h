@@ -68,11 +68,23 @@ struct SlabTask {              // one (expert, slab) unit of the down projection
 };
 
 bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I);
+// The routed ids and weights of a forward whose kernels find their assignments themselves (no routing tables).
+struct DecodeRouted {
+    const void* selected;             // [T, top_k] expert ids as the router numbers them
+    int ids_are_i64;
+    const float* weights;             // [T, top_k]
+    int top_k;
+    const int32_t* local_to_global;   // [n_experts]: the router's id of every expert of the matrix sets
+    const int32_t* global_to_local;   // [n_global]: its inverse, -1 for ids that belong to no expert of the sets
+    int n_global;
+};
+bool decode_inline_route_ok(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, const void* h_gate,
+                            const void* h_up, int Rg, int Ru, int64_t ldg, int64_t ldu, int64_t T, int top_k, int I);
 int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
                           const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg,
                           int64_t ldu, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
                           int I, float* rank_accum, float* G, float* U, int64_t inter_floats, int part_capacity,
-                          bitsmoe_profile* prof, hipStream_t st);
+                          const DecodeRouted* routed, bitsmoe_profile* prof, hipStream_t st);
 // How many partial results of the two fp32 intermediates the decode path's workspace holds (the gate/up kernel
 // may split its contraction over workgroups when there are few assignments).
 inline int decode_part_capacity(int64_t n_assign) { return n_assign <= 1024 ? 4 : n_assign <= 4096 ? 2 : 1; }

@@ -83,6 +83,86 @@ __device__ inline ChunkRef nth_chunk(const int32_t* __restrict__ expert_offsets,
     return ChunkRef{__builtin_amdgcn_readfirstlane(found_e), __builtin_amdgcn_readfirstlane(found_c)};
 }
 
+// ------------------------------------------------------------------------- where assignments come from
+// The kernels see an expert's assignments through one of two sources.  Tables: the routing tables the
+// operator is given (token_indices / route_w in expert-sorted order, an expert's range from expert_offsets);
+// assignment a is row a of the [A, I] intermediates.  Inline: the workgroup has found its expert's entries
+// among the T * k routed (token, slot) pairs itself (inline_route); assignment j is then flat entry ent[j]
+// = token * k + slot, which is also its row of the intermediates -- no routing kernel runs before the
+// forward, and gate/up and down workgroups agree on the rows without any table in memory.
+struct AssignTables {
+    const int32_t* __restrict__ token_indices;
+    const float* __restrict__ route_w;
+    int A;
+    __device__ __forceinline__ int token(int a) const { return token_indices[min(a, A - 1)]; }
+    __device__ __forceinline__ int token_if(int a, bool ok) const { return ok ? token_indices[a] : -1; }
+    __device__ __forceinline__ float weight_if(int a, bool ok) const { return ok ? route_w[a] : 0.0f; }
+    __device__ __forceinline__ int row(int a) const { return a; }
+};
+constexpr int ROUTE_INLINE_MAX_FLAT = 1024;      // routed entries (tokens x top-k) a workgroup scans itself
+constexpr int ROUTE_INLINE_MAX_ROWS = 256;       // assignments of one expert (at most one per token)
+struct InlineRouteLds {
+    uint16_t tok[ROUTE_INLINE_MAX_ROWS];
+    uint16_t ent[ROUTE_INLINE_MAX_ROWS];
+    int wave_sum[4];
+};
+struct AssignInline {
+    const uint16_t* tok;       // LDS
+    const uint16_t* ent;       // LDS
+    const float* __restrict__ weights;      // [T * k] routing weights in entry order
+    int n;
+    __device__ __forceinline__ int token(int a) const { return tok[min(a, n - 1)]; }
+    __device__ __forceinline__ int token_if(int a, bool ok) const { return ok ? (int)tok[a] : -1; }
+    __device__ __forceinline__ float weight_if(int a, bool ok) const { return ok ? weights[ent[a]] : 0.0f; }
+    __device__ __forceinline__ int row(int a) const { return ent[a]; }
+};
+__device__ __forceinline__ int routed_id(const void* __restrict__ selected, int ids_are_i64, int i) {
+    return ids_are_i64 ? (int)reinterpret_cast<const int64_t*>(selected)[i] : reinterpret_cast<const int32_t*>(selected)[i];
+}
+// The entries of the expert with global id `gid` among selected[0 .. n_flat) (n_flat <= ROUTE_INLINE_MAX_FLAT,
+// ids 32 or 64 bits wide), in entry order -- the order the routing kernel's stable sort gives
+// (bitsmoe/models/base_block.py:258-289) -- written to `r`; returns their number (wave-uniform).  All 256
+// threads call it; it contains two workgroup barriers.  Ids that belong to no packed expert match nothing.
+__device__ inline int inline_route(const void* __restrict__ selected, int ids_are_i64, int n_flat, int top_k, int gid,
+                                   InlineRouteLds& r, int tid) {
+    const int lane = tid & 63, wave = tid >> 6;
+    const int base = 4 * tid;
+    int ids[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int i = min(base + k, n_flat - 1);
+        ids[k] = ids_are_i64 ? (int)reinterpret_cast<const int64_t*>(selected)[i] : reinterpret_cast<const int32_t*>(selected)[i];
+    }
+    int count = 0;
+    bool hit[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        hit[k] = base + k < n_flat && ids[k] == gid;
+        count += hit[k] ? 1 : 0;
+    }
+    const int incl = wave_inclusive_scan(count);
+    if (lane == 63) r.wave_sum[wave] = incl;
+    __syncthreads();
+    int before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const int s = r.wave_sum[w];
+        before += w < wave ? s : 0;
+        total += s;
+    }
+    int pos = before + incl - count;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        if (hit[k] && pos < ROUTE_INLINE_MAX_ROWS) {
+            r.tok[pos] = (uint16_t)((base + k) / top_k);
+            r.ent[pos] = (uint16_t)(base + k);
+        }
+        pos += hit[k] ? 1 : 0;
+    }
+    __syncthreads();
+    return __builtin_amdgcn_readfirstlane(min(total, ROUTE_INLINE_MAX_ROWS));
+}
+
 constexpr int GRID_EXPERTS = 0;   // the expert coordinate of the grid is the expert
 constexpr int GRID_ACTIVE = 1;    // ... counts active experts (nth_active_expert)
 constexpr int GRID_CHUNKS = 2;    // ... counts 16-assignment chunks (nth_chunk)
@@ -193,10 +273,10 @@ __device__ __forceinline__ u32x4 scaled_f16x8(u32x4 raw, u32x4 sc) {
 // assignment, whatever its G / U rows hold.
 // `hs_all`: LDS, 2 * MAX_A * GU_STRIDE 16-bit elements; `cterm_lds`: LDS, MAX_A floats.  The caller
 // guarantees that no wavefront still reads either when the item begins (a workgroup barrier).
-template <bool BF16, bool IDENT, int W, bool SPLIT>
+template <bool BF16, bool IDENT, int W, bool SPLIT, class AS>
 __device__ __forceinline__ void gateup_walk_item(gptr<uint32_t> payload, gptr<__half> scale_s, gptr<int32_t> rank_idx,
                                                  const FastSlab first, const uint16_t* __restrict__ h, int64_t ld,
-                                                 const int32_t* __restrict__ token_indices, int a0, int n_a, int A, int T,
+                                                 const AS& as, int a0, int n_a, int T,
                                                  int I, int n_tiles, int t, int g_begin, int g_end, float* __restrict__ out,
                                                  uint16_t* __restrict__ hs_all, float* __restrict__ cterm_lds, int tid) {
     const int pair = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform
@@ -221,7 +301,7 @@ __device__ __forceinline__ void gateup_walk_item(gptr<uint32_t> payload, gptr<__
     // scalar loads in flight together)
     int tki[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) tki[i] = token_indices[min(a0 + pair + 4 * i, A - 1)];
+    for (int i = 0; i < 4; ++i) tki[i] = as.token(a0 + pair + 4 * i);
     // rows 8*lane .. 8*lane + 7 of group g: first logical rank, the f16 bits of their eight
     // scale * s * stagger factor (folded once when the set was prepared), the activations
     auto rank_at = [&](int g) {
@@ -317,10 +397,11 @@ __device__ __forceinline__ void gateup_walk_item(gptr<uint32_t> payload, gptr<__
         for (int j = 0; j < 4; ++j) {
             const int a = 4 * kg + j;
             if (a < n_a && c < I) {
+                const int64_t row = as.row(a0 + a);
                 if constexpr (SPLIT)
-                    atomicAdd(&out[(int64_t)(a0 + a) * I + c], acc[nbl][j] - corr[j]);
+                    atomicAdd(&out[row * I + c], acc[nbl][j] - corr[j]);
                 else
-                    out[(int64_t)(a0 + a) * I + c] = acc[nbl][j] - corr[j];
+                    out[row * I + c] = acc[nbl][j] - corr[j];
             }
         }
     }
@@ -335,11 +416,11 @@ __device__ __forceinline__ void gateup_walk_item(gptr<uint32_t> payload, gptr<__
 // `grp_tab[g]` (LDS) = (width, payload word offset of the group's first slab) for g < n_groups; the caller
 // fills it and puts a workgroup barrier behind it.
 constexpr int WALK_MAX_GROUPS = 32;      // 16384 contraction rows
-template <bool BF16, bool IDENT, bool SPLIT>
+template <bool BF16, bool IDENT, bool SPLIT, class AS>
 __device__ __forceinline__ void gateup_walk_item_mixed(gptr<uint32_t> payload, gptr<__half> scale_s, gptr<int32_t> rank_idx,
                                                        const int2* __restrict__ grp_tab, const uint16_t* __restrict__ h,
-                                                       int64_t ld, const int32_t* __restrict__ token_indices, int a0, int n_a,
-                                                       int A, int T, int I, int n_tiles, int t, int g_begin, int g_end,
+                                                       int64_t ld, const AS& as, int a0, int n_a,
+                                                       int T, int I, int n_tiles, int t, int g_begin, int g_end,
                                                        float* __restrict__ out, uint16_t* __restrict__ hs_all,
                                                        float* __restrict__ cterm_lds, int tid) {
     const int pair = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform
@@ -366,7 +447,7 @@ __device__ __forceinline__ void gateup_walk_item_mixed(gptr<uint32_t> payload, g
     };
     int tki[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) tki[i] = token_indices[min(a0 + pair + 4 * i, A - 1)];
+    for (int i = 0; i < 4; ++i) tki[i] = as.token(a0 + pair + 4 * i);
     auto rank_at = [&](int g) {
         const int k = g * (GU_SLABS * SLAB_ROWS) + 8 * lane;
         if constexpr (IDENT) return k;
@@ -481,10 +562,11 @@ __device__ __forceinline__ void gateup_walk_item_mixed(gptr<uint32_t> payload, g
         for (int j = 0; j < 4; ++j) {
             const int a = 4 * kg + j;
             if (a < n_a && c < I) {
+                const int64_t row = as.row(a0 + a);
                 if constexpr (SPLIT)
-                    atomicAdd(&out[(int64_t)(a0 + a) * I + c], acc[nbl][j] - corr[j]);
+                    atomicAdd(&out[row * I + c], acc[nbl][j] - corr[j]);
                 else
-                    out[(int64_t)(a0 + a) * I + c] = acc[nbl][j] - corr[j];
+                    out[row * I + c] = acc[nbl][j] - corr[j];
             }
         }
     }
@@ -707,11 +789,10 @@ __device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4
 // ZREADY: `G` holds Z (16-bit operands, [A, I]) and `U` holds Zsum ([A, n_tiles] fp32) as written by
 // gateup_walk_z_item: the z phase is a copy into LDS instead of two fp32 reads and a SiLU per element.
 // Otherwise G and U are the first of `n_part` partial results, part_stride floats apart, that are added up.
-template <int W, bool ZREADY = false>
+template <int W, bool ZREADY, class AS>
 __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gptr<__half> svec, gptr<int32_t> rank_idx,
                                  const FastSlab fs, const float* __restrict__ G, const float* __restrict__ U, int n_part,
-                                 int64_t part_stride, const float* __restrict__ route_w,
-                                 const int32_t* __restrict__ token_indices,
+                                 int64_t part_stride, const AS& as,
                                  int a_begin, int a_end, int T, int I, int tb, int nt, int rank_out,
                                  float* __restrict__ rank_accum, uint16_t* __restrict__ z, int z_stride, float* __restrict__ zsum,
                                  int2* __restrict__ rows, int2* __restrict__ assigns, int tid, int lane) {
@@ -761,8 +842,8 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
         }
         // token ids and routing weights of the chunk (lane a holds assignment a): for the epilogue,
         // kept in LDS until then (every wavefront writes the same sixteen entries)
-        const int tok_lane = (lane < n_a) ? token_indices[a0 + lane] : -1;
-        const float rw_lane = (lane < n_a) ? route_w[a0 + lane] : 0.0f;
+        const int tok_lane = as.token_if(a0 + lane, lane < n_a);
+        const float rw_lane = as.weight_if(a0 + lane, lane < n_a);
         __syncthreads();   // the previous chunk is done with z
         if constexpr (ZREADY) {
             const uint16_t* __restrict__ Zg = reinterpret_cast<const uint16_t*>(G);
@@ -797,7 +878,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
 #pragma unroll
                 for (int j = 0; j < ZROWS; ++j) {
                     const int a = min(ab + j, n_a - 1);
-                    const int64_t gi = (int64_t)(a0 + a) * I + c;
+                    const int64_t gi = (int64_t)as.row(a0 + a) * I + c;
                     gv[j] = *reinterpret_cast<const f32x4*>(G + gi);
                     uv[j] = *reinterpret_cast<const f32x4*>(U + gi);
                 }
@@ -806,7 +887,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
 #pragma unroll
                     for (int j = 0; j < ZROWS; ++j) {
                         const int a = min(ab + j, n_a - 1);
-                        const int64_t gi = (int64_t)(a0 + a) * I + c + p * part_stride;
+                        const int64_t gi = (int64_t)as.row(a0 + a) * I + c + p * part_stride;
                         gv[j] += *reinterpret_cast<const f32x4*>(G + gi);
                         uv[j] += *reinterpret_cast<const f32x4*>(U + gi);
                     }

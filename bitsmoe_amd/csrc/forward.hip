@@ -169,11 +169,97 @@ extern "C" int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bit
     if (chosen == BITSMOE_PATH_DECODE)
         return launch_forward_decode(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
                                      token_indices, expert_offsets, route_w, n_assign, rank_out, intermediate_size,
-                                     rank_accum, G, U, (int64_t)(inter / sizeof(float)), decode_part_capacity(n_assign), profile,
-                                     st);
+                                     rank_accum, G, U, (int64_t)(inter / sizeof(float)), decode_part_capacity(n_assign), nullptr,
+                                     profile, st);
     return launch_forward_generic(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
                                   token_indices, expert_offsets, route_w, n_assign, rank_out,
                                   intermediate_size, rank_accum, G, U, profile, st);
+}
+
+// ---- the forward from the router's output: routing inside the kernels where they can, else the routing kernel first
+static size_t routing_tables_bytes(int64_t n_flat, int32_t n_experts) {
+    return 2 * align_up((size_t)n_flat * 4, 256) + align_up((size_t)(n_experts + 1) * 4, 256) +
+           align_up(bitsmoe_route_workspace_bytes(n_flat, n_experts), 256);
+}
+
+extern "C" size_t bitsmoe_forward_routed_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                                                         const bitsmoe_matset* down, int64_t n_tokens, int32_t top_k,
+                                                         int32_t path) {
+    if (!gate || !up || !down || n_tokens < 0 || top_k <= 0) return 0;
+    const int64_t n_flat = n_tokens * top_k;
+    return bitsmoe_forward_workspace_bytes_sets(gate, up, down, n_tokens, n_flat, path) + routing_tables_bytes(n_flat, gate->n_experts);
+}
+
+extern "C" int bitsmoe_forward_routed_is_inline(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                                               const bitsmoe_matset* down, const void* h_gate, const void* h_up,
+                                               int32_t rank_gate, int32_t rank_up, int64_t ld_gate, int64_t ld_up,
+                                               int64_t n_tokens, int32_t top_k, int32_t path) {
+    if (!gate || !up || !down || n_tokens <= 0 || top_k <= 0) return 0;
+    const int I = gate->intermediate_size;
+    if (path != BITSMOE_PATH_AUTO && path != BITSMOE_PATH_DECODE) return 0;
+    if (resolve_path(gate, up, down, n_tokens * top_k, I, path) != BITSMOE_PATH_DECODE) return 0;
+    return decode_inline_route_ok(gate, up, down, h_gate, h_up, rank_gate, rank_up, ld_gate, ld_up, n_tokens, top_k, I) ? 1 : 0;
+}
+
+extern "C" int bitsmoe_moe_forward_routed(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                                          const void* h_gate, const void* h_up, int32_t act_dtype, int64_t n_tokens,
+                                          int32_t rank_gate, int32_t rank_up, int64_t ld_gate, int64_t ld_up,
+                                          const void* selected, int32_t ids_are_i64, const float* weights, int32_t top_k,
+                                          const int32_t* global_to_local, int32_t n_global,
+                                          const int32_t* local_to_global, int32_t rank_out, int32_t intermediate_size,
+                                          int32_t act_type, int32_t path, float* rank_accum, void* workspace,
+                                          size_t workspace_bytes, bitsmoe_profile* profile, void* stream) {
+    hipStream_t st = (hipStream_t)stream;
+    BITSMOE_REQUIRE(gate && up && down, "matrix sets must not be null");
+    BITSMOE_REQUIRE(top_k > 0 && n_tokens >= 0, "n_tokens must be >= 0 and top_k > 0");
+    BITSMOE_REQUIRE(n_tokens * top_k < ((int64_t)1 << 31), "too many assignments");
+    BITSMOE_REQUIRE(act_type == 0, "only SiLU act_type=0 is currently supported");
+    BITSMOE_REQUIRE(act_dtype == BITSMOE_DT_F16 || act_dtype == BITSMOE_DT_BF16, "act_dtype must be f16 (0) or bf16 (1)");
+    const int64_t n_flat = n_tokens * top_k;
+    const int E = gate->n_experts;
+    if (n_tokens == 0) return BITSMOE_OK;
+    const size_t need = bitsmoe_forward_routed_workspace_bytes(gate, up, down, n_tokens, top_k, path);
+    if (workspace == nullptr || workspace_bytes < need) {
+        set_error("workspace too small: need %zu bytes, got %zu", need, workspace_bytes);
+        return BITSMOE_E_WORKSPACE;
+    }
+    BITSMOE_REQUIRE(((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
+    // Routing inside the kernels: the same checks as the table form, then the decode launcher without tables.
+    const bool shapes_ok = E > 0 && E == up->n_experts && E == down->n_experts && intermediate_size > 0 && rank_out > 0 &&
+                           gate->intermediate_size == intermediate_size && up->intermediate_size == intermediate_size &&
+                           down->intermediate_size == intermediate_size && h_gate && h_up && selected && weights &&
+                           local_to_global && global_to_local && n_global > 0 && rank_accum && rank_gate > 0 && rank_up > 0 && ld_gate >= rank_gate &&
+                           ld_up >= rank_up && gate->max_rank_plus1 <= rank_gate && gate->min_rank >= 0 &&
+                           up->max_rank_plus1 <= rank_up && up->min_rank >= 0 &&
+                           (down->total_slabs == 0 || (down->min_rank < rank_out && down->max_rank_plus1 > 0)) &&
+                           path >= BITSMOE_PATH_AUTO && path <= BITSMOE_PATH_MFMA;
+    if (shapes_ok && (path == BITSMOE_PATH_AUTO || path == BITSMOE_PATH_DECODE) &&
+        resolve_path(gate, up, down, n_flat, intermediate_size, path) == BITSMOE_PATH_DECODE &&
+        decode_inline_route_ok(gate, up, down, h_gate, h_up, rank_gate, rank_up, ld_gate, ld_up, n_tokens, top_k,
+                               intermediate_size)) {
+        const size_t inter = align_up((size_t)n_flat * (size_t)intermediate_size * sizeof(float), 256);
+        float* G = (float*)workspace;
+        float* U = (float*)((char*)workspace + inter);
+        const DecodeRouted routed = {selected, ids_are_i64, weights, top_k, local_to_global, global_to_local, n_global};
+        return launch_forward_decode(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
+                                     nullptr, nullptr, nullptr, n_flat, rank_out, intermediate_size, rank_accum, G, U,
+                                     (int64_t)(inter / sizeof(float)), decode_part_capacity(n_flat), &routed, profile, st);
+    }
+    // Otherwise: routing tables at the end of the workspace, then the table form (which reports what is wrong
+    // with the arguments, if anything is).
+    BITSMOE_REQUIRE(global_to_local != nullptr, "global_to_local must not be null");
+    const size_t fwd = bitsmoe_forward_workspace_bytes_sets(gate, up, down, n_tokens, n_flat, path);
+    char* tail = (char*)workspace + align_up(fwd, 256);
+    int32_t* tok = (int32_t*)tail;
+    float* rw = (float*)(tail + align_up((size_t)n_flat * 4, 256));
+    int32_t* off = (int32_t*)(tail + 2 * align_up((size_t)n_flat * 4, 256));
+    void* route_ws = tail + 2 * align_up((size_t)n_flat * 4, 256) + align_up((size_t)(E + 1) * 4, 256);
+    const int rc = bitsmoe_route(selected, ids_are_i64, weights, global_to_local, n_global, n_tokens, top_k, E, tok, off, rw,
+                                 route_ws, bitsmoe_route_workspace_bytes(n_flat, E), st);
+    if (rc != BITSMOE_OK) return rc;
+    return bitsmoe_moe_forward_strided(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
+                                       tok, off, rw, n_flat, rank_out, intermediate_size, act_type, path, rank_accum, workspace,
+                                       align_up(fwd, 256), profile, st);
 }
 
 extern "C" size_t bitsmoe_static_scratch_bytes(void) { return (size_t)BITSMOE_STATIC_SCRATCH_BYTES; }

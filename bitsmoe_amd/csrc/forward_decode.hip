@@ -302,7 +302,11 @@ __global__ __launch_bounds__(256, 4) void k_gateup_decode(
 // The kernel also clears `zero_out` (the forward's accumulator, added into by the down kernel).
 // MIXED: experts whose slab groups differ in width (gateup_walk_item_mixed); a kernel of its own, so that
 // the one-width kernel keeps its registers to itself.
-template <bool BF16, int MODE, bool IDENT, bool MIXED>
+// ROUTED (GRID_EXPERTS or GRID_ACTIVE): there are no routing tables; the workgroup finds its expert's entries among the
+// n_flat = T * top_k routed ids itself (inline_route) and row = flat entry index of the intermediates.  With
+// GRID_ACTIVE the expert coordinate counts routed ENTRIES: the workgroup of entry s serves the expert that entry
+// names if s is that expert's first entry, and exits otherwise -- every active expert is served exactly once.
+template <bool BF16, int MODE, bool IDENT, bool MIXED, bool ROUTED>
 __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const FastExpert* __restrict__ gate_fe, const FastSlab* __restrict__ gate_fs, int gate_max_slabs,
     const FastExpert* __restrict__ up_fe, const FastSlab* __restrict__ up_fs, int up_max_slabs,
@@ -310,7 +314,9 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const int32_t* __restrict__ token_indices, const int32_t* __restrict__ expert_offsets, int T, int A, int I,
     int E, int n_tiles, float* __restrict__ G, float* __restrict__ U, int n_unsplit, int split, int n_part,
     int64_t part_stride, float* __restrict__ zero_out, int64_t zero_n, const ExpertOrder gate_order,
-    const ExpertOrder up_order) {
+    const ExpertOrder up_order, const void* __restrict__ selected, int ids_are_i64, int n_flat, int top_k,
+    const int32_t* __restrict__ local_to_global, const int32_t* __restrict__ global_to_local, int n_global) {
+    static_assert(!ROUTED || MODE != GRID_CHUNKS, "inline routing serves whole experts");
     const int tid = threadIdx.x;
     {   // this workgroup's share of the accumulator (before any exit)
         const int64_t total = (int64_t)gridDim.x * 256;
@@ -330,7 +336,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     int chunk = -1;
     if constexpr (MODE == GRID_EXPERTS) {      // expensive experts first (the identity when there is no order)
         if (E <= EXPERT_ORDER_MAX) e = mt ? up_order.e[e] : gate_order.e[e];
-    } else if constexpr (MODE == GRID_ACTIVE) {
+    } else if constexpr (MODE == GRID_ACTIVE && !ROUTED) {
         e = nth_active_expert(expert_offsets, E, A, e, tid & 63);
         if (e < 0) return;
     } else if constexpr (MODE == GRID_CHUNKS) {
@@ -339,12 +345,28 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
         chunk = ref.chunk;
         if (e < 0) return;
     }
-    // one round trip: assignment range, expert record, the record of the expert's first slab
-    int a_begin = max(expert_offsets[e], 0);
-    int a_end = min(expert_offsets[e + 1], A);
-    if (chunk >= 0) {
-        a_begin += MAX_A * chunk;
-        a_end = min(a_end, a_begin + MAX_A);
+    // one round trip: assignment range (or the routed ids), expert record, the record of the expert's first slab
+    int a_begin = 0, a_end = 0;
+    int gid = -1;
+    __shared__ std::conditional_t<ROUTED, InlineRouteLds, int> route_lds;
+    if constexpr (ROUTED && MODE == GRID_ACTIVE) {
+        // `e` is an entry index: serve the expert it names if this is the expert's first entry
+        const int slot = e;
+        if (slot >= n_flat) return;
+        gid = routed_id(selected, ids_are_i64, slot);
+        a_end = inline_route(selected, ids_are_i64, n_flat, top_k, gid, route_lds, tid);
+        if (a_end == 0 || route_lds.ent[0] != slot || gid < 0 || gid >= n_global) return;
+        e = global_to_local[gid];
+        if (e < 0 || e >= E) return;
+    } else if constexpr (ROUTED) {
+        gid = local_to_global[e];
+    } else {
+        a_begin = max(expert_offsets[e], 0);
+        a_end = min(expert_offsets[e + 1], A);
+        if (chunk >= 0) {
+            a_begin += MAX_A * chunk;
+            a_end = min(a_end, a_begin + MAX_A);
+        }
     }
     const FastExpert* __restrict__ fe_tab = mt ? up_fe : gate_fe;
     const FastSlab* __restrict__ fs_tab = mt ? up_fs : gate_fs;
@@ -360,6 +382,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
             grp_tab[tid] = int2{gs.bits, gs.pack_off};
         }
     }
+    if constexpr (ROUTED && MODE == GRID_EXPERTS) a_end = inline_route(selected, ids_are_i64, n_flat, top_k, gid, route_lds, tid);
     if (a_end <= a_begin || first.bits == 0) return;
     const int n_groups = fe.num_slabs / GU_SLABS;
     // this workgroup's share of the slab groups, and the partial result it writes
@@ -371,6 +394,13 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const uint16_t* __restrict__ h = mt ? h_up : h_gate;
     const int64_t ld = mt ? ldu : ldg;
     float* __restrict__ out = (mt ? U : G) + part * part_stride;
+    auto assignments = [&]() {
+        if constexpr (ROUTED)
+            return AssignInline{route_lds.tok, route_lds.ent, nullptr, a_end};
+        else
+            return AssignTables{token_indices, nullptr, A};
+    };
+    const auto as = assignments();
     // partials nobody else writes for these elements: all but the own one of a share without slab groups,
     // 1 .. n_part - 1 of a whole item
     {
@@ -380,7 +410,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
             float* __restrict__ zp = (mt ? U : G) + p * part_stride;
             for (int i = tid; i < (a_end - a_begin) * N_TILE; i += 256) {
                 const int a = i / N_TILE, c = i - a * N_TILE;
-                if (c < cols) zp[(int64_t)(a_begin + a) * I + t * N_TILE + c] = 0.0f;
+                if (c < cols) zp[(int64_t)as.row(a_begin + a) * I + t * N_TILE + c] = 0.0f;
             }
         }
     }
@@ -395,13 +425,13 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
         const int n_a = min(MAX_A, a_end - a0);
         if (a0 != a_begin) __syncthreads();      // the previous chunk's readers of the operand are done
         if constexpr (MIXED) {
-            gateup_walk_item_mixed<BF16, IDENT, false>(payload, scale_s, rank_idx, grp_tab, h, ld, token_indices, a0, n_a, A, T, I,
-                                                       n_tiles, t, g_begin, g_end, out, hs_all, cterm_lds, tid);
+            gateup_walk_item_mixed<BF16, IDENT, false>(payload, scale_s, rank_idx, grp_tab, h, ld, as, a0, n_a, T, I, n_tiles, t,
+                                                       g_begin, g_end, out, hs_all, cterm_lds, tid);
         } else {
             auto run = [&](auto w_c) {
-                gateup_walk_item<BF16, IDENT, decltype(w_c)::value, false>(payload, scale_s, rank_idx, first, h, ld,
-                                                                           token_indices, a0, n_a, A, T, I, n_tiles, t, g_begin,
-                                                                           g_end, out, hs_all, cterm_lds, tid);
+                gateup_walk_item<BF16, IDENT, decltype(w_c)::value, false>(payload, scale_s, rank_idx, first, h, ld, as, a0,
+                                                                           n_a, T, I, n_tiles, t, g_begin, g_end, out, hs_all,
+                                                                           cterm_lds, tid);
             };
             if (first.bits == 2)
                 run(std::integral_constant<int, 2>{});
@@ -483,13 +513,19 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk_z(
 // tiles are split over several workgroups (their partial sums meet in the atomics of the combine).
 // ZREADY: G / U hold Z / Zsum written by k_gateup_walk_z instead of the fp32 gate and up sums.  Otherwise the
 // sums are the totals of `n_part` partial results part_stride floats apart (k_gateup_walk).
-template <int MODE, bool ZREADY>
+// ROUTED (GRID_EXPERTS or GRID_ACTIVE): no routing tables; the workgroup finds its expert's entries among the routed
+// ids itself, as the gate/up kernel did (same rows of the intermediates), and takes the routing weights
+// from `sel_weights` in entry order.
+template <int MODE, bool ZREADY, bool ROUTED>
 __global__ __launch_bounds__(256, 4) void k_down_decode(
     const FastExpert* __restrict__ down_fe, const FastSlab* __restrict__ down_fs, int max_slabs,
     const float* __restrict__ G, const float* __restrict__ U, int n_part, int64_t part_stride,
     const float* __restrict__ route_w, const int32_t* __restrict__ token_indices,
     const int32_t* __restrict__ expert_offsets, int T, int A, int I, int E, int n_tiles, int n_groups, int n_tchunks,
-    int tiles_per_wg, int n_work, int rank_out, float* __restrict__ rank_accum) {
+    int tiles_per_wg, int n_work, int rank_out, float* __restrict__ rank_accum, const void* __restrict__ selected,
+    int ids_are_i64, int n_flat, int top_k, const int32_t* __restrict__ local_to_global,
+    const float* __restrict__ sel_weights, const int32_t* __restrict__ global_to_local, int n_global) {
+    static_assert(!ROUTED || (MODE != GRID_CHUNKS && !ZREADY), "inline routing serves whole experts");
     // Workgroup b runs on XCD b % 8, and every XCD has its own L2: the workgroups of one expert
     // (which all read that expert's G / U rows) are given ids of one residue class, so that they
     // share one L2.  The grid is a multiple of 8; ids past the work exit.
@@ -501,7 +537,7 @@ __global__ __launch_bounds__(256, 4) void k_down_decode(
     const int e_slot = bid / (n_tchunks * n_groups);
     const int tid = threadIdx.x;
     int e = e_slot, chunk = -1;
-    if constexpr (MODE == GRID_ACTIVE) {
+    if constexpr (MODE == GRID_ACTIVE && !ROUTED) {
         e = nth_active_expert(expert_offsets, E, A, e_slot, tid & 63);
     } else if constexpr (MODE == GRID_CHUNKS) {
         const ChunkRef ref = nth_chunk(expert_offsets, E, A, e_slot, tid & 63);
@@ -515,16 +551,39 @@ __global__ __launch_bounds__(256, 4) void k_down_decode(
     const int lane = tid & 63;
     const int si = grp * DN_SLABS_PER_WG + wave;
 
-    int a_begin = max(expert_offsets[e], 0);
-    int a_end = min(expert_offsets[e + 1], A);
-    if (chunk >= 0) {      // this workgroup's chunk only
-        a_begin += MAX_A * chunk;
-        a_end = min(a_end, a_begin + MAX_A);
+    int a_begin = 0, a_end = 0, gid = -1;
+    __shared__ std::conditional_t<ROUTED, InlineRouteLds, int> route_lds;
+    if constexpr (ROUTED && MODE == GRID_ACTIVE) {
+        // `e` is an entry index: serve the expert it names if this is the expert's first entry
+        const int slot = e;
+        if (slot >= n_flat) return;
+        gid = routed_id(selected, ids_are_i64, slot);
+        a_end = inline_route(selected, ids_are_i64, n_flat, top_k, gid, route_lds, tid);
+        if (a_end == 0 || route_lds.ent[0] != slot || gid < 0 || gid >= n_global) return;
+        e = global_to_local[gid];
+        if (e < 0 || e >= E) return;
+    } else if constexpr (ROUTED) {
+        gid = local_to_global[e];
+    } else {
+        a_begin = max(expert_offsets[e], 0);
+        a_end = min(expert_offsets[e + 1], A);
+        if (chunk >= 0) {      // this workgroup's chunk only
+            a_begin += MAX_A * chunk;
+            a_end = min(a_end, a_begin + MAX_A);
+        }
     }
     const FastExpert fe = down_fe[e];
     FastSlab fs = FastSlab{0, 0, 0, 0};
     if (si < max_slabs) fs = load_fast_slab(down_fs, e * max_slabs + si);
+    if constexpr (ROUTED && MODE == GRID_EXPERTS) a_end = inline_route(selected, ids_are_i64, n_flat, top_k, gid, route_lds, tid);
     if (a_end <= a_begin || grp * DN_SLABS_PER_WG >= fe.num_slabs) return;
+    auto assignments = [&]() {
+        if constexpr (ROUTED)
+            return AssignInline{route_lds.tok, route_lds.ent, sel_weights, a_end};
+        else
+            return AssignTables{token_indices, route_w, A};
+    };
+    const auto as = assignments();
 
     gptr<uint32_t> payload = as_global(fe.payload);
     gptr<__half> scale = as_global(fe.scale);
@@ -540,17 +599,17 @@ __global__ __launch_bounds__(256, 4) void k_down_decode(
     // the four wavefronts may run four different instantiations; every one of them executes
     // the same two workgroup barriers per assignment chunk
     if (fs.bits == 2)
-        down_wave<2, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, route_w, token_indices, a_begin,
-                           a_end, T, I, tb, nt, rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
+        down_wave<2, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
+                           rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else if (fs.bits == 3)
-        down_wave<3, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, route_w, token_indices, a_begin,
-                           a_end, T, I, tb, nt, rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
+        down_wave<3, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
+                           rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else if (fs.bits == 4)
-        down_wave<4, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, route_w, token_indices, a_begin,
-                           a_end, T, I, tb, nt, rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
+        down_wave<4, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
+                           rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else
-        down_wave<0, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, route_w, token_indices, a_begin,
-                           a_end, T, I, tb, nt, rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
+        down_wave<0, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
+                           rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
 }
 
 __global__ void k_fill_zero2(float* __restrict__ p1, int64_t n1, float* __restrict__ p2, int64_t n2) {
@@ -584,11 +643,34 @@ bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up,
            I % N_TILE == 0;
 }
 
+static int decode_grid_mode(int64_t A, int E) {
+    const int64_t active_max = std::min<int64_t>(E, A);
+    return (A >= (int64_t)16 * E || (E <= 64 && A >= (int64_t)3 * E)) ? GRID_CHUNKS : active_max * 2 <= E ? GRID_ACTIVE : GRID_EXPERTS;
+}
+static bool walk_possible(const bitsmoe_matset* gate, const bitsmoe_matset* up, const void* h_gate, const void* h_up, int Rg,
+                          int Ru, int64_t ldg, int64_t ldu) {
+    // (its 16-byte activation loads need rank_idx in runs of eight and aligned rows; the ranks that padding rows
+    // read, with zero scales, must be columns of the activations too)
+    auto rows16 = [](const void* p, int64_t ld) { return ((uintptr_t)p & 15) == 0 && ld % 8 == 0; };
+    return gate->role == ROLE_GATE_UP && up->role == ROLE_GATE_UP && gate->rank_chunked8 && up->rank_chunked8 &&
+           rows16(h_gate, ldg) && rows16(h_up, ldu) && gate->pad_rank_plus1 <= Rg && up->pad_rank_plus1 <= Ru &&
+           std::max(gate->prep_max_slabs, up->prep_max_slabs) <= WALK_MAX_GROUPS * GU_SLABS;
+}
+// Can the decode kernels find their assignments among the routed ids themselves (no routing tables)?
+bool decode_inline_route_ok(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, const void* h_gate,
+                            const void* h_up, int Rg, int Ru, int64_t ldg, int64_t ldu, int64_t T, int top_k, int I) {
+    const int64_t n_flat = T * top_k;
+    const char* fused_var = getenv("BITSMOE_DECODE_FUSED_Z");
+    return decode_path_supported(gate, up, down, I) && walk_possible(gate, up, h_gate, h_up, Rg, Ru, ldg, ldu) &&
+           !(fused_var && fused_var[0] && atoi(fused_var) > 0) && n_flat > 0 && n_flat <= ROUTE_INLINE_MAX_FLAT &&
+           T <= ROUTE_INLINE_MAX_ROWS && decode_grid_mode(n_flat, gate->n_experts) != GRID_CHUNKS;
+}
+
 int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
                           const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg,
                           int64_t ldu, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
                           int I, float* rank_accum, float* G, float* U, int64_t inter_floats, int part_capacity,
-                          bitsmoe_profile* prof, hipStream_t st) {
+                          const DecodeRouted* routed, bitsmoe_profile* prof, hipStream_t st) {
     const int E = gate->n_experts;
     const int n_tiles = gate->n_tiles;
     record(prof, 0, st);
@@ -600,18 +682,14 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     // search step) the chunk grid is already used from three assignments per expert on average.
     // At most min(E, A) experts can be active.
     const int64_t active_max = std::min<int64_t>(E, A);
-    const int mode = (A >= (int64_t)16 * E || (E <= 64 && A >= (int64_t)3 * E)) ? GRID_CHUNKS : active_max * 2 <= E ? GRID_ACTIVE : GRID_EXPERTS;
+    const int mode = decode_grid_mode(A, E);
     const int e_dim = mode == GRID_CHUNKS ? (int)(active_max + A / MAX_A) : mode == GRID_ACTIVE ? (int)active_max : E;
     // (expert, chunk) pairs expected to have work (e_dim is their upper bound in chunk mode)
     const int64_t units = mode == GRID_CHUNKS ? A / MAX_A + active_max / 2 : active_max;
     // Sets of affine single-width experts, enough (expert, tile) pairs to fill the chip: the
     // walking gate/up kernel, which also clears rank_accum and needs no cleared G / U.
     // (its 16-byte activation loads also need rank_idx in runs of eight and aligned rows)
-    auto rows16 = [](const void* p, int64_t ld) { return ((uintptr_t)p & 15) == 0 && ld % 8 == 0; };
-    // (the ranks that padding rows read, with zero scales, must be columns of the activations too)
-    const bool walk = gate->role == ROLE_GATE_UP && up->role == ROLE_GATE_UP && gate->rank_chunked8 && up->rank_chunked8 &&
-                   rows16(h_gate, ldg) && rows16(h_up, ldu) && gate->pad_rank_plus1 <= Rg && up->pad_rank_plus1 <= Ru &&
-                   std::max(gate->prep_max_slabs, up->prep_max_slabs) <= WALK_MAX_GROUPS * GU_SLABS;
+    const bool walk = walk_possible(gate, up, h_gate, h_up, Rg, Ru, ldg, ldu);
     // Both projections in one workgroup, z = silu(G) * U handed to the down kernel ready-made: when the two
     // matrices of every expert share bit-width and slab count, and (expert, tile) pairs alone fill most of
     // the chip.  BITSMOE_DECODE_FUSED_Z=0 / 1 switches it off / on regardless of the size (experiments).
@@ -689,13 +767,21 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         const bool mixed = !(gate->uniform_experts && up->uniform_experts);
         constexpr bool B = decltype(bf16_c)::value;
         constexpr int M = decltype(mode_c)::value;
-        auto kern = mixed ? (ident ? k_gateup_walk<B, M, true, true> : k_gateup_walk<B, M, false, true>)
-                          : (ident ? k_gateup_walk<B, M, true, false> : k_gateup_walk<B, M, false, false>);
+        auto kern = mixed ? (ident ? k_gateup_walk<B, M, true, true, false> : k_gateup_walk<B, M, false, true, false>)
+                          : (ident ? k_gateup_walk<B, M, true, false, false> : k_gateup_walk<B, M, false, false, false>);
+        if constexpr (M != GRID_CHUNKS) {
+            if (routed)
+                kern = mixed ? (ident ? k_gateup_walk<B, M, true, true, true> : k_gateup_walk<B, M, false, true, true>)
+                             : (ident ? k_gateup_walk<B, M, true, false, true> : k_gateup_walk<B, M, false, false, true>);
+        }
         hipLaunchKernelGGL(kern, dim3((unsigned)(n_unsplit + (n_items - n_unsplit) * split)), dim3(256), 0, st,
                            gate->d_fast_experts, gate->d_fast_slabs, gate->prep_max_slabs, up->d_fast_experts,
                            up->d_fast_slabs, up->prep_max_slabs, (const uint16_t*)h_gate, (const uint16_t*)h_up, ldg, ldu,
                            tok, off, (int)T, (int)A, I, E, n_tiles, G, U, (int)n_unsplit, split, n_part, part_stride, rank_accum,
-                           T * (int64_t)rank_out, gate_order, up_order);
+                           T * (int64_t)rank_out, gate_order, up_order, routed ? routed->selected : nullptr,
+                           routed ? routed->ids_are_i64 : 0, routed ? (int)A : 0, routed ? routed->top_k : 1,
+                           routed ? routed->local_to_global : nullptr, routed ? routed->global_to_local : nullptr,
+                           routed ? routed->n_global : 0);
     };
     auto launch_walk_z_mode = [&](auto bf16_c, auto mode_c) {
         auto kern = k_gateup_walk_z<decltype(bf16_c)::value, decltype(mode_c)::value, false>;
@@ -734,10 +820,22 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         const int n_work = e_dim * dn_groups * dn_tchunks;
         hipLaunchKernelGGL(kernel, dim3((unsigned)((n_work + 7) / 8 * 8)), dim3(256), z_bytes, st, down->d_fast_experts,
                            down->d_fast_slabs, down->prep_max_slabs, G, U, walk && !fused_z ? n_part : 1, part_stride, rw, tok, off,
-                           (int)T, (int)A, I, E, n_tiles, dn_groups, dn_tchunks, dn_tiles_per_wg, n_work, rank_out, rank_accum);
+                           (int)T, (int)A, I, E, n_tiles, dn_groups, dn_tchunks, dn_tiles_per_wg, n_work, rank_out, rank_accum,
+                           routed ? routed->selected : nullptr, routed ? routed->ids_are_i64 : 0, routed ? (int)A : 0,
+                           routed ? routed->top_k : 1, routed ? routed->local_to_global : nullptr,
+                           routed ? routed->weights : nullptr, routed ? routed->global_to_local : nullptr,
+                           routed ? routed->n_global : 0);
     };
     auto launch_down_mode = [&](auto zready_c, auto mode_c) {
-        launch_down(k_down_decode<decltype(mode_c)::value, decltype(zready_c)::value>);
+        constexpr int M = decltype(mode_c)::value;
+        constexpr bool Z = decltype(zready_c)::value;
+        if constexpr (M != GRID_CHUNKS && !Z) {
+            if (routed) {
+                launch_down(k_down_decode<M, Z, true>);
+                return;
+            }
+        }
+        launch_down(k_down_decode<M, Z, false>);
     };
     // (G and U are fp32 and the operands f16 whatever the activation type was)
     if (fused_z)

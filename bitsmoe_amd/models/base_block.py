@@ -51,6 +51,7 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         self._packed_expert_count = 0
         self._packed_intermediate_size = 0
         self._packed_global_to_local: Optional[torch.Tensor] = None
+        self._packed_local_to_global: Optional[torch.Tensor] = None
         for proj in ("gate", "up", "down"):
             for name in _BUFFER_NAMES:
                 setattr(self, f"_{proj}_{name}_static", ())
@@ -168,6 +169,7 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
             g2l[torch.tensor([idx for idx, _ in packed_items], dtype=torch.long)] = torch.arange(
                 len(experts), dtype=torch.int32)
         self._packed_global_to_local = g2l.to(device)
+        self._packed_local_to_global = torch.tensor([idx for idx, _ in packed_items], dtype=torch.int32, device=device)
         for proj in ("gate", "up", "down"):
             for name in _BUFFER_NAMES:
                 attr = f"{proj}_{name}_buffer" if name != "s" else f"{proj}_s_buffer"
@@ -363,6 +365,26 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         u_down = self._shared_basis(h_gate_proj.dtype)[2]
         return torch.matmul(rank_accum.to(u_down.dtype), u_down.T)
 
+    def _packed_forward_routed(self, h_gate_proj, h_up_proj, selected_experts, routing_weights_fp32,
+                               token_count: int) -> torch.Tensor:
+        if self.shared_u_down.numel() == 0:
+            raise RuntimeError(f"Layer {self.layer_idx} missing shared_u_down for packed routed experts.")
+        if not (_HAS_MLP_FORWARD_CUDA and mlp_forward_cuda is not None and h_gate_proj.is_cuda and h_up_proj.is_cuda):
+            raise RuntimeError(
+                "Packed routed experts require CUDA mlp_forward extension; python fallback is intentionally disabled.")
+        rank_out = int(self.shared_u_down.shape[1])
+        intermediate_size = int(self._packed_intermediate_size)
+        if intermediate_size <= 0:
+            raise RuntimeError(f"Layer {self.layer_idx} has no packed experts for CUDA path.")
+        gate, up, down = self._ensure_matsets()
+        sel = selected_experts.reshape(token_count, self.top_k)
+        w = routing_weights_fp32.reshape(token_count, self.top_k)
+        rank_accum = mlp_forward_cuda.moe_forward_routed(h_gate_proj, h_up_proj, sel, w, self._packed_global_to_local,
+                                                         self._packed_local_to_global, gate, up, down, rank_out,
+                                                         intermediate_size, self._act_type())
+        u_down = self._shared_basis(h_gate_proj.dtype)[2]
+        return torch.matmul(rank_accum.to(u_down.dtype), u_down.T)
+
     def _packed_forward_grouped(self, h_gate_proj, h_up_proj, token_indices, expert_offsets_t, route_flat,
                                 token_count: int) -> torch.Tensor:
         if self.shared_u_down.numel() == 0:
@@ -395,11 +417,11 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
             self._run_super_experts(hidden_states, final, flat_selected,
                                     self._get_flat_token_ids(token_count, hidden_states.device),
                                     flat_w32.to(hidden_states.dtype))
-        routing = self._build_packed_routing(flat_selected, None, flat_w32)
-        if routing is not None:
-            token_indices, expert_offsets_t, route_flat = routing
-            packed = self._packed_forward_grouped(h_gate_proj, h_up_proj, token_indices, expert_offsets_t,
-                                                  route_flat, token_count).to(hidden_states.dtype)
+        if self._packed_expert_count > 0 and self._packed_global_to_local is not None:
+            # routing tables (bitsmoe/models/base_block.py:258-289) and operator (:381-408) as one call: small
+            # batches run without a routing kernel, the forward's kernels find their assignments themselves
+            packed = self._packed_forward_routed(h_gate_proj, h_up_proj, selected_experts, routing_weights_fp32,
+                                                 token_count).to(hidden_states.dtype)
             # without dense experts the sum "zeros + packed" of the reference is `packed` itself
             final = packed if final is None else final + packed
         if final is None:

@@ -202,6 +202,35 @@ int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bitsmoe_matset
                                 bitsmoe_profile* profile, void* stream);
 
 /*
+ * The forward from the router's output: what the block does between its router and its output
+ * projection (bitsmoe/models/base_block.py:258-289 builds the routing tables with framework ops and
+ * :381-408 calls the operator) as one call.  selected / weights: [n_tokens, top_k] expert ids (32- or
+ * 64-bit, as the router numbers them) and routing weights; global_to_local [n_global] maps a router id
+ * to the expert's index in the matrix sets or -1 (ids that belong to no packed expert are dropped),
+ * local_to_global [n_experts] is its inverse.  For batches of at most 1024 routed entries and 256
+ * tokens whose grid walks the experts themselves, on matrix sets the decode kernels take, no routing
+ * kernel runs at all: every workgroup finds its expert's entries among the routed ids itself, and
+ * row t * top_k + j of the intermediates belongs to entry (t, j).  Otherwise bitsmoe_route fills tables at the end of the workspace and
+ * bitsmoe_moe_forward_strided runs on them.  Results equal those of the two-call form (the order
+ * of an expert's assignments is the same; fp32 atomics aside).
+ */
+size_t bitsmoe_forward_routed_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                                              const bitsmoe_matset* down, int64_t n_tokens, int32_t top_k,
+                                              int32_t path);
+/* 1 if bitsmoe_moe_forward_routed would run these arguments without a routing kernel, else 0. */
+int bitsmoe_forward_routed_is_inline(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                                     const void* h_gate, const void* h_up, int32_t rank_gate, int32_t rank_up,
+                                     int64_t ld_gate, int64_t ld_up, int64_t n_tokens, int32_t top_k, int32_t path);
+int bitsmoe_moe_forward_routed(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                               const void* h_gate, const void* h_up, int32_t act_dtype, int64_t n_tokens,
+                               int32_t rank_gate, int32_t rank_up, int64_t ld_gate, int64_t ld_up,
+                               const void* selected, int32_t ids_are_i64, const float* weights, int32_t top_k,
+                               const int32_t* global_to_local, int32_t n_global,
+                               const int32_t* local_to_global, int32_t rank_out, int32_t intermediate_size,
+                               int32_t act_type, int32_t path, float* rank_accum, void* workspace,
+                               size_t workspace_bytes, bitsmoe_profile* profile, void* stream);
+
+/*
  * The forward for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc): bitsmoe_moe_forward_strided without the
  * workspace argument.  No counterpart in the reference, whose operator allocates its

@@ -1,0 +1,83 @@
+"""The forward from the router's output (bitsmoe_moe_forward_routed): with and without routing tables."""
+import numpy as np
+import pytest
+
+import helpers
+from oracle import ref_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+
+def _hip():
+    from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
+
+    return hip
+
+
+def _case(cuda_device, seed, n_global, n_super, tokens, top_k, rank, dim, i64, dtype_name, experts="uniform", path=None):
+    import torch
+
+    from bitsmoe_amd.algorithms import _capi
+
+    hip = _hip()
+    rng = np.random.default_rng(seed)
+    # some router ids belong to no packed expert (super experts served elsewhere): their entries are dropped
+    keep = np.ones(n_global, bool)
+    if n_super:
+        keep[rng.choice(n_global, size=n_super, replace=False)] = False
+    g2l = np.full(n_global, -1, np.int32)
+    g2l[keep] = np.arange(keep.sum(), dtype=np.int32)
+    l2g = np.nonzero(keep)[0].astype(np.int32)
+    e = int(keep.sum())
+    if experts == "uniform":
+        gate, up, down = helpers.make_experts(seed, e, rank, rank, dim, choices=(2, 3, 4), uniform_bits=True)
+    elif experts == "mixed":
+        gate, up, down = helpers.make_experts(seed, e, rank, rank, dim, choices=(2, 3, 4), slab_multiple=64)
+    else:       # slabs of other widths: the generic kernels, routing tables
+        gate, up, down = helpers.make_experts(seed, e, rank, rank, dim, choices=(2, 8), slab_multiple=64)
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    h_gate = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(dt)
+    h_up = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(dt)
+    idx, w = o.router_qwen(rng.normal(size=(tokens, n_global)).astype(np.float32), top_k)
+    tok, off, rw = o.build_routing(idx, w, g2l, e)
+    ref = o.moe_forward(h_gate.float().numpy(), h_up.float().numpy(), tok, off, rw, gate, up, down, rank, dim)
+    sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=dim) for m in (gate, up, down)]
+    sel = torch.from_numpy(idx.astype(np.int64 if i64 else np.int32)).to(cuda_device)
+    wt = torch.from_numpy(w).to(cuda_device)
+    g2l_t, l2g_t = torch.from_numpy(g2l).to(cuda_device), torch.from_numpy(l2g).to(cuda_device)
+    kwargs = {} if path is None else {"path": path}
+    got = hip.moe_forward_routed(h_gate.to(cuda_device), h_up.to(cuda_device), sel, wt, g2l_t, l2g_t, *sets, rank, dim, 0,
+                                 **kwargs)
+    tok_d, off_d, rw_d = hip.route(sel, wt, g2l_t, e)
+    two_calls = hip.moe_forward_sets(h_gate.to(cuda_device), h_up.to(cuda_device), tok_d, off_d, rw_d, *sets, rank, dim, 0,
+                                     **kwargs)
+    scale = float(two_calls.abs().max())
+    assert float((got - two_calls).abs().max()) <= 1e-5 * scale        # same sums, fp32 atomics in another order
+    err = helpers.norm_err(got.cpu().numpy(), ref)
+    assert err <= 3e-3, f"normalised error {err:.3e}"
+    inline = hip.routed_is_inline(h_gate.to(cuda_device), h_up.to(cuda_device), top_k, *sets, **kwargs)
+    return sets, inline
+
+
+# (router ids, of them not packed, tokens, top_k, 64-bit ids, no routing kernel expected): 8 experts with 9 tokens and
+# 128 experts with 40 or 128 tokens walk the experts themselves; 1 to 8 tokens walk the routed entries (few active
+# experts; several entries of one expert, ids that belong to no packed expert); 300 tokens (grouped GEMM) and a
+# grid over 16-assignment chunks take the table form
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+@pytest.mark.parametrize("n_global,n_super,tokens,top_k,i64,expect_inline", [
+    (8, 0, 9, 2, True, True), (10, 2, 9, 2, False, True), (128, 0, 40, 8, True, True), (130, 2, 128, 8, True, True),
+    (8, 0, 1, 2, True, True), (32, 0, 4, 2, True, True), (40, 8, 6, 2, False, True), (128, 0, 8, 8, True, True),
+    (8, 0, 300, 2, True, False), (64, 0, 64, 6, False, False),
+])
+def test_forward_from_router_output(cuda_device, n_global, n_super, tokens, top_k, i64, expect_inline, dtype_name):
+    sets, inline = _case(cuda_device, 500 + tokens, n_global, n_super, tokens, top_k, 512, 256, i64, dtype_name)
+    assert sets[0].role == 0 and sets[2].role == 1
+    assert inline == expect_inline
+
+
+@pytest.mark.parametrize("experts", ["mixed", "generic"])
+def test_forward_from_router_output_other_layouts(cuda_device, experts):
+    """Experts of mixed widths (the walking kernel's mixed form, rank 512: whole groups) and sets the fast
+    kernels cannot take (8-bit slabs: routing tables, generic kernels)."""
+    _, inline = _case(cuda_device, 77, 12, 1, 11, 2, 512, 256, True, "bf16", experts=experts)
+    assert inline == (experts == "mixed")
