@@ -661,6 +661,8 @@ bool decode_inline_route_ok(const bitsmoe_matset* gate, const bitsmoe_matset* up
                             const void* h_up, int Rg, int Ru, int64_t ldg, int64_t ldu, int64_t T, int top_k, int I) {
     const int64_t n_flat = T * top_k;
     const char* fused_var = getenv("BITSMOE_DECODE_FUSED_Z");
+    const char* inline_var = getenv("BITSMOE_ROUTE_INLINE");       // 0: always build routing tables first (experiments)
+    if (inline_var && inline_var[0] == '0') return false;
     return decode_path_supported(gate, up, down, I) && walk_possible(gate, up, h_gate, h_up, Rg, Ru, ldg, ldu) &&
            !(fused_var && fused_var[0] && atoi(fused_var) > 0) && n_flat > 0 && n_flat <= ROUTE_INLINE_MAX_FLAT &&
            T <= ROUTE_INLINE_MAX_ROWS && decode_grid_mode(n_flat, gate->n_experts) != GRID_CHUNKS;
