@@ -14,6 +14,7 @@ constexpr int GU_STRIDE = GU_SLABS * SLAB_ROWS + 8;  // 16-bit elements; +8 stag
 constexpr int DN_SLABS_PER_WG = 4;                 // one slab per wavefront
 constexpr int MAX_A = 16;                          // assignments per MFMA pass
 constexpr int ZROWS = 2;                           // assignment rows of G / U the down kernel's z build fetches together
+constexpr int ZROWS_WIDE = 6;                      // ... where z is so large that only three workgroups fit a CU anyway
 constexpr int ZSUM_STRIDE = 16;                    // tiles per assignment row of the down kernel's z sums (I <= 1920)
 
 // With few assignments most experts are idle; launching a workgroup per (expert, ...) then
@@ -789,7 +790,9 @@ __device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4
 // ZREADY: `G` holds Z (16-bit operands, [A, I]) and `U` holds Zsum ([A, n_tiles] fp32) as written by
 // gateup_walk_z_item: the z phase is a copy into LDS instead of two fp32 reads and a SiLU per element.
 // Otherwise G and U are the first of `n_part` partial results, part_stride floats apart, that are added up.
-template <int W, bool ZREADY, class AS>
+// ZR: assignment rows whose G / U loads are in flight together while z is built (one memory round trip per ZR
+// rows: the pass is latency-bound; more rows need more registers).
+template <int W, bool ZREADY, int ZR, class AS>
 __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gptr<__half> svec, gptr<int32_t> rank_idx,
                                  const FastSlab fs, const float* __restrict__ G, const float* __restrict__ U, int n_part,
                                  int64_t part_stride, const AS& as,
@@ -871,12 +874,12 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
         } else
         // z[a][c] = silu(G) * U as 16-bit operands for the rows a < n_a (other rows feed
         // output rows that are never stored).  Each thread owns four neighbouring columns
-        // and walks the assignments ZROWS at a time, their vector loads issued together.
+        // and walks the assignments ZR at a time, their vector loads issued together.
         for (int c = tb * N_TILE + tid * 4; c < min((tb + nt) * N_TILE, I); c += 1024) {
-            for (int ab = 0; ab < n_a; ab += ZROWS) {
-                f32x4 gv[ZROWS], uv[ZROWS];
+            for (int ab = 0; ab < n_a; ab += ZR) {
+                f32x4 gv[ZR], uv[ZR];
 #pragma unroll
-                for (int j = 0; j < ZROWS; ++j) {
+                for (int j = 0; j < ZR; ++j) {
                     const int a = min(ab + j, n_a - 1);
                     const int64_t gi = (int64_t)as.row(a0 + a) * I + c;
                     gv[j] = *reinterpret_cast<const f32x4*>(G + gi);
@@ -885,7 +888,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                 // (the gate/up kernel split the contraction: the sums are totals of partial results)
                 for (int p = 1; p < n_part; ++p) {
 #pragma unroll
-                    for (int j = 0; j < ZROWS; ++j) {
+                    for (int j = 0; j < ZR; ++j) {
                         const int a = min(ab + j, n_a - 1);
                         const int64_t gi = (int64_t)as.row(a0 + a) * I + c + p * part_stride;
                         gv[j] += *reinterpret_cast<const f32x4*>(G + gi);
@@ -893,7 +896,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                     }
                 }
 #pragma unroll
-                for (int j = 0; j < ZROWS; ++j) {
+                for (int j = 0; j < ZR; ++j) {
                     if (ab + j < n_a) {
                         uint16_t zb[4];
                         float part = 0.0f;      // sum of the four operands as rounded

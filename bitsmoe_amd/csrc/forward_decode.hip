@@ -516,8 +516,10 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk_z(
 // ROUTED (GRID_EXPERTS or GRID_ACTIVE): no routing tables; the workgroup finds its expert's entries among the routed
 // ids itself, as the gate/up kernel did (same rows of the intermediates), and takes the routing weights
 // from `sel_weights` in entry order.
-template <int MODE, bool ZREADY, bool ROUTED>
-__global__ __launch_bounds__(256, 4) void k_down_decode(
+// ZR: rows of G / U in flight while z is built; more than the usual two only where z is so large that three
+// workgroups fit a CU, which leaves each of them more registers (launch bounds follow).
+template <int MODE, bool ZREADY, bool ROUTED, int ZR>
+__global__ __launch_bounds__(256, ZR > ZROWS ? 3 : 4) void k_down_decode(
     const FastExpert* __restrict__ down_fe, const FastSlab* __restrict__ down_fs, int max_slabs,
     const float* __restrict__ G, const float* __restrict__ U, int n_part, int64_t part_stride,
     const float* __restrict__ route_w, const int32_t* __restrict__ token_indices,
@@ -599,16 +601,16 @@ __global__ __launch_bounds__(256, 4) void k_down_decode(
     // the four wavefronts may run four different instantiations; every one of them executes
     // the same two workgroup barriers per assignment chunk
     if (fs.bits == 2)
-        down_wave<2, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
+        down_wave<2, ZREADY, ZR>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else if (fs.bits == 3)
-        down_wave<3, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
+        down_wave<3, ZREADY, ZR>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else if (fs.bits == 4)
-        down_wave<4, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
+        down_wave<4, ZREADY, ZR>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else
-        down_wave<0, ZREADY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
+        down_wave<0, ZREADY, ZR>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
 }
 
@@ -831,13 +833,25 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     auto launch_down_mode = [&](auto zready_c, auto mode_c) {
         constexpr int M = decltype(mode_c)::value;
         constexpr bool Z = decltype(zready_c)::value;
+        // (z beyond 40 KB: at most three workgroups per CU fit the LDS, the kernel compiled for three takes more
+        // rows of G / U per round trip)
+        const bool wide = !Z && z_bytes > 40 * 1024;
         if constexpr (M != GRID_CHUNKS && !Z) {
             if (routed) {
-                launch_down(k_down_decode<M, Z, true>);
+                if (wide)
+                    launch_down(k_down_decode<M, Z, true, ZROWS_WIDE>);
+                else
+                    launch_down(k_down_decode<M, Z, true, ZROWS>);
                 return;
             }
         }
-        launch_down(k_down_decode<M, Z, false>);
+        if constexpr (!Z) {
+            if (wide) {
+                launch_down(k_down_decode<M, Z, false, ZROWS_WIDE>);
+                return;
+            }
+        }
+        launch_down(k_down_decode<M, Z, false, ZROWS>);
     };
     // (G and U are fp32 and the operands f16 whatever the activation type was)
     if (fused_z)
