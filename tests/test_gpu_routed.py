@@ -81,3 +81,46 @@ def test_forward_from_router_output_other_layouts(cuda_device, experts):
     kernels cannot take (8-bit slabs: routing tables, generic kernels)."""
     _, inline = _case(cuda_device, 77, 12, 1, 11, 2, 512, 256, True, "bf16", experts=experts)
     assert inline == (experts == "mixed")
+
+
+def test_forward_from_router_output_under_graph_replay(cuda_device):
+    """The one-call forward neither allocates nor synchronises: captured into a HIP graph, every replay -- with
+    eager work and synchronisations in between -- reproduces the eager result."""
+    import torch
+
+    hip = _hip()
+    rng = np.random.default_rng(5)
+    e, tokens, top_k, rank, dim = 16, 8, 4, 512, 256
+    gate, up, down = helpers.make_experts(5, e, rank, rank, dim, choices=(2, 3, 4), uniform_bits=True)
+    sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=dim) for m in (gate, up, down)]
+    h_gate = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(torch.bfloat16).to(cuda_device)
+    h_up = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(torch.bfloat16).to(cuda_device)
+    idx, w = o.router_qwen(rng.normal(size=(tokens, e)).astype(np.float32), top_k)
+    sel, wt = torch.from_numpy(idx).to(cuda_device), torch.from_numpy(w).to(cuda_device)
+    ids = torch.arange(e, dtype=torch.int32, device=cuda_device)
+    out = torch.empty((tokens, rank), dtype=torch.float32, device=cuda_device)
+
+    def run():
+        return hip.moe_forward_routed(h_gate, h_up, sel, wt, ids, ids, *sets, rank, dim, 0, out=out)
+
+    eager = run().clone()          # (prepares the sets on first use)
+    torch.cuda.synchronize()
+    assert hip.routed_is_inline(h_gate, h_up, top_k, *sets)
+    side = torch.cuda.Stream(device=cuda_device)
+    side.wait_stream(torch.cuda.current_stream(cuda_device))
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream(cuda_device).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run()
+    scale = float(eager.abs().max())
+    for _ in range(3):
+        out.fill_(7.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert float((out - eager).abs().max()) <= 1e-5 * scale
+        again = run().clone()          # eager work between the replays
+        torch.cuda.synchronize()
+        assert float((again - eager).abs().max()) <= 1e-5 * scale
