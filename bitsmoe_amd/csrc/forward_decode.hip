@@ -665,9 +665,18 @@ bool decode_inline_route_ok(const bitsmoe_matset* gate, const bitsmoe_matset* up
     const char* fused_var = getenv("BITSMOE_DECODE_FUSED_Z");
     const char* inline_var = getenv("BITSMOE_ROUTE_INLINE");       // 0: always build routing tables first (experiments)
     if (inline_var && inline_var[0] == '0') return false;
-    return decode_path_supported(gate, up, down, I) && walk_possible(gate, up, h_gate, h_up, Rg, Ru, ldg, ldu) &&
-           !(fused_var && fused_var[0] && atoi(fused_var) > 0) && n_flat > 0 && n_flat <= ROUTE_INLINE_MAX_FLAT &&
-           T <= ROUTE_INLINE_MAX_ROWS && decode_grid_mode(n_flat, gate->n_experts) != GRID_CHUNKS;
+    if (!(decode_path_supported(gate, up, down, I) && walk_possible(gate, up, h_gate, h_up, Rg, Ru, ldg, ldu) &&
+          !(fused_var && fused_var[0] && atoi(fused_var) > 0) && n_flat > 0 && n_flat <= ROUTE_INLINE_MAX_FLAT &&
+          T <= ROUTE_INLINE_MAX_ROWS))
+        return false;
+    // Where it pays (graph replays, same box, against the routing kernel first).  On the active-expert grid
+    // always: 3 to 5 us less per layer.  On the expert grid every expert's workgroups scan the ids, also those of
+    // experts nobody chose, which with tables exit after one load: a gain of 1 to 3 us from two entries per
+    // expert on average on a 128-expert layer of six tiles, a loss of 1 to 5 us below that, on layers of eleven
+    // tiles (more workgroups per expert) and on a 512-expert layer.  The chunk grid keeps its tables.
+    const int mode = decode_grid_mode(n_flat, gate->n_experts);
+    if (mode == GRID_ACTIVE) return true;
+    return mode == GRID_EXPERTS && n_flat >= 2 * (int64_t)gate->n_experts && gate->n_experts <= 256 && gate->n_tiles <= 8;
 }
 
 int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,

@@ -208,9 +208,11 @@ int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bitsmoe_matset
  * 64-bit, as the router numbers them) and routing weights; global_to_local [n_global] maps a router id
  * to the expert's index in the matrix sets or -1 (ids that belong to no packed expert are dropped),
  * local_to_global [n_experts] is its inverse.  For batches of at most 1024 routed entries and 256
- * tokens whose grid walks the experts themselves, on matrix sets the decode kernels take, no routing
- * kernel runs at all: every workgroup finds its expert's entries among the routed ids itself, and
- * row t * top_k + j of the intermediates belongs to entry (t, j).  Otherwise bitsmoe_route fills tables at the end of the workspace and
+ * tokens, on matrix sets the decode kernels take, no routing kernel runs where that was measured to be
+ * faster (few active experts, or at least two entries per expert on layers of up to 256 experts and 8
+ * column tiles; bitsmoe_forward_routed_is_inline tells): every workgroup finds its expert's entries among
+ * the routed ids itself, and row t * top_k + j of the intermediates belongs to entry (t, j).  Otherwise
+ * bitsmoe_route fills tables at the end of the workspace and
  * bitsmoe_moe_forward_strided runs on them.  Results equal those of the two-call form (the order
  * of an expert's assignments is the same; fp32 atomics aside).
  */
