@@ -16,7 +16,7 @@ cache instead of HBM.  The decode workloads therefore build `--layers` distinct 
 layer (different seeds: different weights and bit draws) and cycle through them inside the timed
 loop; with 4 copies 555 MB of other weights pass between two visits of a layer.  The headline
 `value`, `ms_per_step` and `roofline` are the COLD figures; the one-layer replay is reported
-beside them as `warm`.  `c5-stack-*` runs BASELINE configs[4]: the 26-layer DeepSeek-V2-Lite-
+beside them as `warm`.  `c5-stack-*` runs the stack configuration of the benchmark set: the 26-layer DeepSeek-V2-Lite-
 shaped stack, one step = one pass over all 26 layers (per-layer figures reported).
 
 Prints ONE JSON line.  `value` is tokens/s of the primary workload (default: the

@@ -761,7 +761,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     // The walking kernel's workgroups: one per item, unless the items fill less than half of the chip's
     // `slots` (four resident workgroups per CU): then every item is split over `split` workgroups, each of
     // which contracts over a share of the slab groups, and the down kernel adds the `n_part` partial results
-    // up.  (Halving only the cheapest items of a grid whose last round is partly empty -- 1536 items on 1024
+    // up.  (Halving only the cheapest items of a grid whose final batch of workgroups is partly empty -- 1536 items on 1024
     // slots -- was measured too: the gate/up kernel gains nothing, the down kernel's SiLU pass reads twice as much.)
     const int64_t n_items = (int64_t)e_dim * n_tiles * 2;
     const int64_t slots = 4 * (int64_t)cu_count();
