@@ -36,6 +36,9 @@ def _dense_via_operator() -> bool:
 
 class BitsMoE_BaseSparseMoeBlock(nn.Module):
     _SHARED_BASIS_BUFFER_KEYS = ("shared_vh_gate_proj", "shared_vh_up_proj", "shared_u_down")
+    # Decoder layers written for per-expert MoE modules take (hidden, router_logits) from the Qwen blocks, as the
+    # reference returns them; those written for fused expert parameters take the hidden states alone.
+    host_expects_tensor = False
 
     def _init_bitsmoe_common_state(self, super_experts: Optional[List[int]] = None,
                                    track_super_projected_weights: bool = False) -> None:

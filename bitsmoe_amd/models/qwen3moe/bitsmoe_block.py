@@ -49,4 +49,5 @@ class BitsMoE_Qwen3MoeSparseMoeBlock(BitsMoE_BaseSparseMoeBlock):
         self._ensure_runtime_cache(hidden_states.device)
         router_logits, selected, weights = self._route(hidden_states)
         final = self._routed_forward(hidden_states, selected, weights)
-        return final.reshape(batch_size, sequence_length, hidden_dim), router_logits
+        final = final.reshape(batch_size, sequence_length, hidden_dim)
+        return final if self.host_expects_tensor else (final, router_logits)

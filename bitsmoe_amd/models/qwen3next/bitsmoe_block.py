@@ -31,4 +31,5 @@ class BitsMoE_Qwen3NextSparseMoeBlock(BitsMoE_Qwen3MoeSparseMoeBlock):
             # (reference: bitsmoe/models/qwen3next/bitsmoe_block.py:144-147)
             gate = torch.sigmoid(self.shared_expert_gate(hidden_states))
             final = final + self._always_on_forward("shared", self.shared_expert, hidden_states, gate)
-        return final.reshape(batch_size, sequence_length, hidden_dim), router_logits
+        final = final.reshape(batch_size, sequence_length, hidden_dim)
+        return final if self.host_expects_tensor else (final, router_logits)
