@@ -92,10 +92,63 @@ inline int decode_part_capacity(int64_t n_assign) { return n_assign <= 1024 ? 4 
 bool mfma_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I);
 size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int64_t T,
                             int64_t A, int I);
+// Work of the grouped-GEMM path's front end that the routing launches can carry, so that a forward from the
+// router's output needs fewer launches: the f16 copy of bf16 activations rides in extra workgroups of the
+// counting launch, the scan also builds the tile list (it has the expert offsets at hand) and the scatter also
+// writes every assignment's slot within its token and the per-token counts.  The per-token lists then have a
+// fixed stride: token t's list starts at t * top_k (token_start), its length is token_count[t].
+struct MTile;
+struct RouteSideJobs {
+    const uint16_t* src_g = nullptr;     // bf16 activations (rows sg / su elements apart); null: no copy
+    const uint16_t* src_u = nullptr;
+    int64_t T = 0, sg = 0, su = 0;
+    int ldg = 0, ldu = 0;                // columns of the copies (multiples of 8)
+    uint16_t* dst_g = nullptr;
+    uint16_t* dst_u = nullptr;
+    int32_t* slot = nullptr;             // [n_flat], by position in the routing tables; null: not wanted
+    int32_t* token_count = nullptr;      // [T]
+    int32_t* token_start = nullptr;      // [T + 1]
+    MTile* mtiles = nullptr;             // [max_mtiles]; null: not wanted
+    int32_t* n_mtiles = nullptr;
+    int max_mtiles = 0;
+    const FastExpert* gate_fe = nullptr;
+    const FastExpert* up_fe = nullptr;
+};
+constexpr int MFMA_FRONT_CONVERTED = 1;        // the f16 copies are made
+constexpr int MFMA_FRONT_TOKEN_COUNTED = 2;    // slot, token_count and token_start (stride top_k) are written
+constexpr int MFMA_FRONT_MTILES = 4;           // the tile list is built
+// Fills `jobs` for a call of launch_forward_mfma with the same arguments; false: that call needs none of them.
+bool mfma_front_jobs(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                     const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg_in,
+                     int64_t ldu_in, int64_t A, int I, void* workspace, RouteSideJobs* jobs);
+// bitsmoe_route with side jobs; *jobs_done: which of them the launches carried (MFMA_FRONT_* bits).
+int route_with_jobs(const void* selected, int32_t ids_are_i64, const float* weights, const int32_t* global_to_local,
+                    int32_t n_global, int64_t n_tokens, int32_t top_k, int32_t n_packed, int32_t* token_indices,
+                    int32_t* expert_offsets, float* route_flat, void* workspace, size_t workspace_bytes,
+                    const RouteSideJobs* jobs, int* jobs_done, hipStream_t st);
+// front_done: MFMA_FRONT_* bits of what an earlier launch on the stream has already produced in `workspace`.
 int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
                         const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg_in,
                         int64_t ldu_in, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
-                        int I, float* rank_accum, void* workspace, bitsmoe_profile* prof, hipStream_t st);
+                        int I, float* rank_accum, void* workspace, int front_done, bitsmoe_profile* prof, hipStream_t st);
+
+// bf16 -> f16, eight elements at a time: group `i` of `total = T * (ld / 8)` groups of one projection.
+__device__ inline void convert_bf16_group(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst, int64_t stride,
+                                          int ld, int64_t i) {
+    typedef uint32_t v4 __attribute__((ext_vector_type(4)));
+    const int per_row = ld >> 3;
+    const int64_t row = i / per_row;
+    const int c = (int)(i - row * per_row) * 8;
+    const v4 v = *reinterpret_cast<const v4*>(src + row * stride + c);
+    v4 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t lo = __builtin_bit_cast(uint16_t, (_Float16)__uint_as_float(v[k] << 16));
+        const uint32_t hi = __builtin_bit_cast(uint16_t, (_Float16)__uint_as_float(v[k] & 0xFFFF0000u));
+        o[k] = lo | (hi << 16);
+    }
+    *reinterpret_cast<v4*>(dst + row * ld + c) = o;
+}
 
 }  // namespace bitsmoe
 

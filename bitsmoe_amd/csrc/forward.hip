@@ -103,6 +103,16 @@ extern "C" int bitsmoe_moe_forward(const bitsmoe_matset* gate, const bitsmoe_mat
                                        stream);
 }
 
+// front_done: what an earlier launch on the stream already left in the workspace for the grouped-GEMM path
+// (MFMA_FRONT_* bits; 0 for callers that bring nothing).
+static int forward_strided_impl(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                                const void* h_gate, const void* h_up, int32_t act_dtype, int64_t n_tokens,
+                                int32_t rank_gate, int32_t rank_up, int64_t ld_gate, int64_t ld_up,
+                                const int32_t* token_indices, const int32_t* expert_offsets, const float* route_w,
+                                int64_t n_assign, int32_t rank_out, int32_t intermediate_size, int32_t act_type,
+                                int32_t path, float* rank_accum, void* workspace, size_t workspace_bytes, int front_done,
+                                bitsmoe_profile* profile, hipStream_t st);
+
 extern "C" int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bitsmoe_matset* up,
                                            const bitsmoe_matset* down, const void* h_gate, const void* h_up,
                                            int32_t act_dtype, int64_t n_tokens, int32_t rank_gate,
@@ -112,7 +122,18 @@ extern "C" int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bit
                                            int32_t intermediate_size, int32_t act_type, int32_t path,
                                            float* rank_accum, void* workspace, size_t workspace_bytes,
                                            bitsmoe_profile* profile, void* stream) {
-    hipStream_t st = (hipStream_t)stream;
+    return forward_strided_impl(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
+                                token_indices, expert_offsets, route_w, n_assign, rank_out, intermediate_size, act_type, path,
+                                rank_accum, workspace, workspace_bytes, 0, profile, (hipStream_t)stream);
+}
+
+static int forward_strided_impl(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                                const void* h_gate, const void* h_up, int32_t act_dtype, int64_t n_tokens,
+                                int32_t rank_gate, int32_t rank_up, int64_t ld_gate, int64_t ld_up,
+                                const int32_t* token_indices, const int32_t* expert_offsets, const float* route_w,
+                                int64_t n_assign, int32_t rank_out, int32_t intermediate_size, int32_t act_type,
+                                int32_t path, float* rank_accum, void* workspace, size_t workspace_bytes, int front_done,
+                                bitsmoe_profile* profile, hipStream_t st) {
     BITSMOE_REQUIRE(gate && up && down, "matrix sets must not be null");
     BITSMOE_REQUIRE(act_type == 0, "only SiLU act_type=0 is currently supported");
     BITSMOE_REQUIRE(act_dtype == BITSMOE_DT_F16 || act_dtype == BITSMOE_DT_BF16, "act_dtype must be f16 (0) or bf16 (1)");
@@ -162,7 +183,7 @@ extern "C" int bitsmoe_moe_forward_strided(const bitsmoe_matset* gate, const bit
     if (chosen == BITSMOE_PATH_MFMA)
         return launch_forward_mfma(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
                                    token_indices, expert_offsets, route_w, n_assign, rank_out, intermediate_size, rank_accum,
-                                   workspace, profile, st);
+                                   workspace, front_done, profile, st);
     const size_t inter = align_up((size_t)n_assign * (size_t)intermediate_size * sizeof(float), 256);
     float* G = (float*)workspace;
     float* U = (float*)((char*)workspace + inter);
@@ -254,12 +275,19 @@ extern "C" int bitsmoe_moe_forward_routed(const bitsmoe_matset* gate, const bits
     float* rw = (float*)(tail + align_up((size_t)n_flat * 4, 256));
     int32_t* off = (int32_t*)(tail + 2 * align_up((size_t)n_flat * 4, 256));
     void* route_ws = tail + 2 * align_up((size_t)n_flat * 4, 256) + align_up((size_t)(E + 1) * 4, 256);
-    const int rc = bitsmoe_route(selected, ids_are_i64, weights, global_to_local, n_global, n_tokens, top_k, E, tok, off, rw,
-                                 route_ws, bitsmoe_route_workspace_bytes(n_flat, E), st);
+    // The grouped-GEMM path's f16 copy of the activations and its per-token tables ride in the routing launches.
+    RouteSideJobs jobs;
+    const char* jobs_var = getenv("BITSMOE_ROUTE_JOBS");      // 0: the grouped-GEMM path makes them itself (experiments)
+    const bool carry = !(jobs_var && jobs_var[0] == '0') && shapes_ok && resolve_path(gate, up, down, n_flat, intermediate_size, path) == BITSMOE_PATH_MFMA &&
+                       mfma_front_jobs(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
+                                       n_flat, intermediate_size, workspace, &jobs);
+    int front_done = 0;
+    const int rc = route_with_jobs(selected, ids_are_i64, weights, global_to_local, n_global, n_tokens, top_k, E, tok, off, rw,
+                                   route_ws, bitsmoe_route_workspace_bytes(n_flat, E), carry ? &jobs : nullptr, &front_done, st);
     if (rc != BITSMOE_OK) return rc;
-    return bitsmoe_moe_forward_strided(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
-                                       tok, off, rw, n_flat, rank_out, intermediate_size, act_type, path, rank_accum, workspace,
-                                       align_up(fwd, 256), profile, st);
+    return forward_strided_impl(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up, tok, off,
+                                rw, n_flat, rank_out, intermediate_size, act_type, path, rank_accum, workspace,
+                                align_up(fwd, 256), front_done, profile, st);
 }
 
 extern "C" size_t bitsmoe_static_scratch_bytes(void) { return (size_t)BITSMOE_STATIC_SCRATCH_BYTES; }

@@ -26,17 +26,9 @@
 #include <type_traits>
 
 #include "fast_helpers.h"
+#include "mtiles.h"
 
 namespace bitsmoe {
-
-constexpr int PF_M = 128;        // assignments per workgroup tile
-
-struct MTile {
-    int32_t expert;   // -1: unused slot
-    int32_t a_begin;
-    int32_t rows;
-    int32_t pad;
-};
 
 // -(1.5 * 2^W) as a packed f16 pair: times the scale it is the constant that turns
 // (2^W + code) * scale into (code - 2^(W-1)) * scale.
@@ -62,17 +54,7 @@ __global__ __launch_bounds__(256) void k_token_count(const int32_t* __restrict__
 }
 
 // One workgroup: the list of (expert, first assignment, rows <= 128) tiles from
-// expert_offsets, then token_start = exclusive scan of token_count (T + 1 entries).
-// The list is ordered by decreasing cost (a counting sort over a few cost classes: the body the
-// tile runs -- full to quarter height -- then the bit-widths of the expert's gate and up
-// matrices): workgroups start in list order, so the long ones run first and the short ones fill
-// the end of the launch.  Which of two tiles of one class comes first is left to the LDS atomics:
-// no result depends on the order.
-constexpr int MT_KEYS = 32;
-__device__ inline int mtile_key(int rows, int wsum) {      // 0 = most expensive
-    const int c = rows > 96 ? 0 : rows > 64 ? 1 : rows > 32 ? 2 : 3;
-    return c * 8 + (7 - min(max(wsum - 1, 0), 7));           // wsum: 4 .. 8, or 0 (mixed widths: taken as the most expensive)
-}
+// expert_offsets (build_mtile_list), then token_start = exclusive scan of token_count (T + 1 entries).
 __global__ __launch_bounds__(256) void k_build_mtiles(const int32_t* __restrict__ expert_offsets, int E, int A,
                                                       int max_tiles, MTile* __restrict__ tiles,
                                                       int32_t* __restrict__ n_tiles_out,
@@ -81,64 +63,9 @@ __global__ __launch_bounds__(256) void k_build_mtiles(const int32_t* __restrict_
                                                       const FastExpert* __restrict__ gate_fe,
                                                       const FastExpert* __restrict__ up_fe) {
     __shared__ int scan[256];
-    __shared__ int hist[MT_KEYS], cursor[MT_KEYS];
-    __shared__ int base_s;
+    __shared__ MTileLds mt_lds;
     const int tid = threadIdx.x;
-    if (tid < MT_KEYS) hist[tid] = 0;
-    __syncthreads();
-    auto expert_tiles = [&](int e, int* begin, int* cnt, int* k_full, int* k_last) {
-        *begin = 0;
-        *cnt = 0;
-        *k_full = 0;
-        *k_last = 0;
-        if (e >= E) return;
-        *begin = min(max(expert_offsets[e], 0), A);
-        const int end = min(max(expert_offsets[e + 1], 0), A);
-        *cnt = max(end - *begin, 0);
-        if (*cnt == 0) return;
-        const int wg = gate_fe ? gate_fe[e].uniform_bits : 2, wu = up_fe ? up_fe[e].uniform_bits : 2;
-        const int wsum = (wg == 0 || wu == 0) ? 8 : wg + wu;
-        *k_full = mtile_key(PF_M, wsum);
-        *k_last = mtile_key(*cnt - (*cnt - 1) / PF_M * PF_M, wsum);
-    };
-    // pass 1: tiles per cost class
-    for (int e0 = 0; e0 < E; e0 += 256) {
-        int begin, cnt, k_full, k_last;
-        expert_tiles(e0 + tid, &begin, &cnt, &k_full, &k_last);
-        const int nt = (cnt + PF_M - 1) / PF_M;
-        if (nt > 1) atomicAdd(&hist[k_full], nt - 1);
-        if (nt > 0) atomicAdd(&hist[k_last], 1);
-    }
-    __syncthreads();
-    if (tid == 0) {
-        int run = 0;
-        for (int k = 0; k < MT_KEYS; ++k) {
-            cursor[k] = run;
-            run += hist[k];
-        }
-        base_s = run;
-    }
-    __syncthreads();
-    // pass 2: every expert claims places for its tiles
-    for (int e0 = 0; e0 < E; e0 += 256) {
-        const int e = e0 + tid;
-        int begin, cnt, k_full, k_last;
-        expert_tiles(e, &begin, &cnt, &k_full, &k_last);
-        const int nt = (cnt + PF_M - 1) / PF_M;
-        if (nt > 1) {
-            const int at = atomicAdd(&cursor[k_full], nt - 1);
-            for (int j = 0; j < nt - 1; ++j)
-                if (at + j < max_tiles) tiles[at + j] = MTile{e, begin + j * PF_M, PF_M, 0};
-        }
-        if (nt > 0) {
-            const int at = atomicAdd(&cursor[k_last], 1);
-            if (at < max_tiles) tiles[at] = MTile{e, begin + (nt - 1) * PF_M, cnt - (nt - 1) * PF_M, 0};
-        }
-    }
-    __syncthreads();
-    const int total = min(base_s, max_tiles);
-    for (int i = total + tid; i < max_tiles; i += 256) tiles[i] = MTile{-1, 0, 0, 0};
-    if (tid == 0) *n_tiles_out = total;
+    build_mtile_list(expert_offsets, E, A, max_tiles, tiles, n_tiles_out, gate_fe, up_fe, mt_lds);
 
     if (token_count == nullptr) return;
     // every thread scans one contiguous run of tokens (a multiple of four: 16-byte loads)
@@ -1071,6 +998,7 @@ template <bool IDENTITY>
 __global__ __launch_bounds__(256) void k_combine_tokens(const FastExpert* __restrict__ down_fe, int max_slabs,
                                                         const _Float16* __restrict__ y, int ldy,
                                                         const int32_t* __restrict__ token_start,
+                                                        const int32_t* __restrict__ token_count,
                                                         const int2* __restrict__ token_list,
                                                         const float* __restrict__ route_w, int rank_out,
                                                         float* __restrict__ rank_accum) {
@@ -1082,7 +1010,8 @@ __global__ __launch_bounds__(256) void k_combine_tokens(const FastExpert* __rest
     __shared__ float rw_s[CB_SORT];
     const int t = blockIdx.x;
     const int tid = threadIdx.x;
-    const int begin = token_start[t], count = token_start[t + 1] - begin;
+    // (token_count given: lists of a fixed stride, only partly filled)
+    const int begin = token_start[t], count = token_count ? token_count[t] : token_start[t + 1] - begin;
     float* out_row = rank_accum + (int64_t)t * rank_out;
     constexpr int STEP = IDENTITY ? 256 * 8 : CB_COLS;
     for (int c0 = 0; c0 < rank_out; c0 += STEP) {
@@ -1108,14 +1037,15 @@ __global__ __launch_bounds__(256) void k_combine_tokens(const FastExpert* __rest
             __syncthreads();
             if (IDENTITY) {
                 const int r0 = c0 + tid * 8;
-                // four entries at a time: their eight loads are in flight together (an entry past
+                // eight entries at a time: their loads are in flight together (an entry past
                 // the list or past its expert's rows loads from a valid address and is not added)
-                for (int i0 = 0; i0 < nl; i0 += 4) {
-                    u32x4 yv[4];
-                    float rw[4];
-                    bool ok[4];
+                constexpr int CB_FLIGHT = 8;
+                for (int i0 = 0; i0 < nl; i0 += CB_FLIGHT) {
+                    u32x4 yv[CB_FLIGHT];
+                    float rw[CB_FLIGHT];
+                    bool ok[CB_FLIGHT];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
+                    for (int u = 0; u < CB_FLIGHT; ++u) {
                         const int i = min(i0 + u, nl - 1);
                         ok[u] = i0 + u < nl && r0 < nrow_s[i];
                         const int rr = ok[u] ? r0 : 0;
@@ -1123,7 +1053,7 @@ __global__ __launch_bounds__(256) void k_combine_tokens(const FastExpert* __rest
                         rw[u] = rw_s[i];
                     }
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
+                    for (int u = 0; u < CB_FLIGHT; ++u) {
                         if (!ok[u]) continue;
 #pragma unroll
                         for (int k = 0; k < 8; ++k) {
@@ -1218,22 +1148,70 @@ size_t mfma_workspace_bytes(const bitsmoe_matset* gate, const bitsmoe_matset* up
     return mfma_workspace(gate, up, down, T, A, I).total;
 }
 
-int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
-                        const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg_in,
-                        int64_t ldu_in, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
-                        int I, float* rank_accum, void* workspace, bitsmoe_profile* prof, hipStream_t st) {
-    const int E = gate->n_experts;
-    const int n_tiles = gate->n_tiles;
-    const int64_t max_mtiles = A / PF_M + E;
+// How the gate/up kernel gets its activations: `direct`: rows read through the token index (from the caller's f16
+// rows, or from an f16 copy of bf16 rows: `convert`), else gathered per assignment; ldg / ldu: elements per row of
+// what the kernel reads.
+struct ActsPlan {
+    bool direct, convert;
+    int ldg, ldu;
+};
+static ActsPlan acts_plan(const bitsmoe_matset* gate, const bitsmoe_matset* up, const void* h_gate, const void* h_up,
+                          int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg_in, int64_t ldu_in) {
     // ldg_in / ldu_in: elements between the caller's activation rows (>= Rg / Ru)
     // (padding rows have zero scales but their activations are still read and multiplied: every rank they
     // name has to be a column of h)
-    const bool direct = direct_ok(gate, up) && Rg % 8 == 0 && Ru % 8 == 0 && ldg_in % 8 == 0 && ldu_in % 8 == 0 &&
-                        gate->pad_rank_plus1 <= Rg && up->pad_rank_plus1 <= Ru &&
-                        (((uintptr_t)h_gate | (uintptr_t)h_up) & 15) == 0 &&
-                        T * std::max(ldg_in, ldu_in) < ((int64_t)1 << 31);
-    const int ldg = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(gate) : (int)ldg_in) : gate->prep_max_slabs * SLAB_ROWS;
-    const int ldu = direct ? (act_dtype == BITSMOE_DT_BF16 ? direct_ld(up) : (int)ldu_in) : up->prep_max_slabs * SLAB_ROWS;
+    ActsPlan p;
+    p.direct = direct_ok(gate, up) && Rg % 8 == 0 && Ru % 8 == 0 && ldg_in % 8 == 0 && ldu_in % 8 == 0 &&
+               gate->pad_rank_plus1 <= Rg && up->pad_rank_plus1 <= Ru && (((uintptr_t)h_gate | (uintptr_t)h_up) & 15) == 0 &&
+               T * std::max(ldg_in, ldu_in) < ((int64_t)1 << 31);
+    p.convert = p.direct && act_dtype == BITSMOE_DT_BF16;
+    p.ldg = p.direct ? (p.convert ? direct_ld(gate) : (int)ldg_in) : gate->prep_max_slabs * SLAB_ROWS;
+    p.ldu = p.direct ? (p.convert ? direct_ld(up) : (int)ldu_in) : up->prep_max_slabs * SLAB_ROWS;
+    return p;
+}
+static inline size_t acts_up_offset(const bitsmoe_matset* gate, const ActsPlan& p, int64_t T, int64_t A) {
+    return p.direct ? align256((size_t)T * direct_ld(gate) * 2) : align256((size_t)A * p.ldg * 2);
+}
+
+bool mfma_front_jobs(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                     const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg_in,
+                     int64_t ldu_in, int64_t A, int I, void* workspace, RouteSideJobs* jobs) {
+    const ActsPlan p = acts_plan(gate, up, h_gate, h_up, act_dtype, T, Rg, Ru, ldg_in, ldu_in);
+    const MfmaWorkspace w = mfma_workspace(gate, up, down, T, A, I);
+    char* ws = (char*)workspace;
+    *jobs = RouteSideJobs{};
+    jobs->T = T;
+    if (p.convert) {
+        jobs->src_g = (const uint16_t*)h_gate;
+        jobs->src_u = (const uint16_t*)h_up;
+        jobs->sg = ldg_in;
+        jobs->su = ldu_in;
+        jobs->ldg = p.ldg;
+        jobs->ldu = p.ldu;
+        jobs->dst_g = (uint16_t*)(ws + w.acts);
+        jobs->dst_u = (uint16_t*)(ws + w.acts + acts_up_offset(gate, p, T, A));
+    }
+    jobs->slot = (int32_t*)(ws + w.slot);
+    jobs->token_count = (int32_t*)(ws + w.token_count);
+    jobs->token_start = (int32_t*)(ws + w.token_start);
+    jobs->mtiles = (MTile*)(ws + w.mtiles);
+    jobs->n_mtiles = (int32_t*)(ws + w.n_mtiles);
+    jobs->max_mtiles = (int)(A / PF_M + gate->n_experts);
+    jobs->gate_fe = gate->d_fast_experts;
+    jobs->up_fe = up->d_fast_experts;
+    return true;
+}
+
+int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                        const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg_in,
+                        int64_t ldu_in, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
+                        int I, float* rank_accum, void* workspace, int front_done, bitsmoe_profile* prof, hipStream_t st) {
+    const int E = gate->n_experts;
+    const int n_tiles = gate->n_tiles;
+    const int64_t max_mtiles = A / PF_M + E;
+    const ActsPlan plan = acts_plan(gate, up, h_gate, h_up, act_dtype, T, Rg, Ru, ldg_in, ldu_in);
+    const bool direct = plan.direct;
+    const int ldg = plan.ldg, ldu = plan.ldu;
     const MfmaWorkspace w = mfma_workspace(gate, up, down, T, A, I);
     char* ws = (char*)workspace;
     MTile* mtiles = (MTile*)(ws + w.mtiles);
@@ -1243,27 +1221,32 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     int32_t* slot = (int32_t*)(ws + w.slot);
     int2* token_list = (int2*)(ws + w.token_list);
     const uint16_t* Hs_g = (const uint16_t*)(ws + w.acts);
-    const uint16_t* Hs_u = (const uint16_t*)(ws + w.acts + (direct ? align256((size_t)T * direct_ld(gate) * 2) : align256((size_t)A * ldg * 2)));
+    const uint16_t* Hs_u = (const uint16_t*)(ws + w.acts + acts_up_offset(gate, plan, T, A));
     uint16_t* z = (uint16_t*)(ws + w.z);     // gate output, then silu(gate) * up in place
     uint16_t* Ubuf = (uint16_t*)(ws + w.u);
     _Float16* y = (_Float16*)(ws + w.y);
     const int ldy = down->prep_max_slabs * SLAB_ROWS;
 
     record(prof, 0, st);
-    const bool convert = direct && act_dtype == BITSMOE_DT_BF16;
-    if (convert) {      // the conversion pass clears the per-token counters on its way
+    const bool convert = plan.convert;
+    // slot, token_count, token_start (fixed stride: the lists' lengths come from token_count) and the tile list are
+    // there already
+    const bool counted = (front_done & MFMA_FRONT_TOKEN_COUNTED) != 0 && (front_done & MFMA_FRONT_MTILES) != 0;
+    if (convert && !(front_done & MFMA_FRONT_CONVERTED)) {      // the conversion pass clears the per-token counters on its way
         const int64_t groups = T * (std::max(ldg, ldu) / 8);
         hipLaunchKernelGGL(k_bf16_to_f16, dim3((unsigned)std::min<int64_t>((groups + 255) / 256, 2048), 2), dim3(256), 0, st,
                            (const uint16_t*)h_gate, (const uint16_t*)h_up, T, ldg_in, ldu_in, ldg, ldu, (uint16_t*)Hs_g,
-                           (uint16_t*)Hs_u, token_count, (int)(T + 1));
+                           (uint16_t*)Hs_u, token_count, counted ? 0 : (int)(T + 1));
         BITSMOE_HIP_TRY(hipGetLastError());
-    } else {
+    } else if (!counted) {
         BITSMOE_REQUIRE(launch_fill_zero((float*)token_count, T + 1, st) == BITSMOE_OK, "zero fill failed");
     }
-    hipLaunchKernelGGL(k_token_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, st, tok, off, E, (int)A, (int)T,
-                       token_count, slot);
-    hipLaunchKernelGGL(k_build_mtiles, dim3(1), dim3(256), 0, st, off, E, (int)A, (int)max_mtiles, mtiles, n_mtiles,
-                       token_count, (int)T, token_start, gate->d_fast_experts, up->d_fast_experts);
+    if (!counted)
+        hipLaunchKernelGGL(k_token_count, dim3((unsigned)((A + 255) / 256)), dim3(256), 0, st, tok, off, E, (int)A, (int)T,
+                           token_count, slot);
+    if (!counted)
+        hipLaunchKernelGGL(k_build_mtiles, dim3(1), dim3(256), 0, st, off, E, (int)A, (int)max_mtiles, mtiles, n_mtiles,
+                           token_count, (int)T, token_start, gate->d_fast_experts, up->d_fast_experts);
     BITSMOE_HIP_TRY(hipGetLastError());
     if (direct) {
         if (!convert) {
@@ -1309,10 +1292,12 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
         record(prof, 4, st);
         if (down->rank_identity)
             hipLaunchKernelGGL(k_combine_tokens<true>, dim3((unsigned)T), dim3(256), 0, st, down->d_fast_experts,
-                               down->prep_max_slabs, y, ldy, token_start, token_list, rw, rank_out, rank_accum);
+                               down->prep_max_slabs, y, ldy, token_start, counted ? token_count : nullptr, token_list, rw,
+                               rank_out, rank_accum);
         else
             hipLaunchKernelGGL(k_combine_tokens<false>, dim3((unsigned)T), dim3(256), 0, st, down->d_fast_experts,
-                               down->prep_max_slabs, y, ldy, token_start, token_list, rw, rank_out, rank_accum);
+                               down->prep_max_slabs, y, ldy, token_start, counted ? token_count : nullptr, token_list, rw,
+                               rank_out, rank_accum);
         BITSMOE_HIP_TRY(hipGetLastError());
     }
     record(prof, 5, st);

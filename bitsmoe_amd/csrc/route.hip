@@ -1,7 +1,10 @@
 // Routing / permute: token-to-expert histogram, exclusive scan and STABLE scatter built
 // on wave64 ballots.  No host synchronisation; the number of kept assignments stays on
 // the device as expert_offsets[n_packed].
+#include <algorithm>
+
 #include "common.h"
+#include "mtiles.h"
 
 namespace bitsmoe {
 
@@ -208,8 +211,21 @@ __global__ __launch_bounds__(ROUTE_THREADS) void k_route_fused(
 template <typename IdT>
 __global__ __launch_bounds__(ROUTE_THREADS) void k_route_count(
     const IdT* __restrict__ selected, const int32_t* __restrict__ g2l, int n_global, int64_t n_flat,
-    int n_packed, int id_bits, int32_t* __restrict__ entry_rank, int32_t* __restrict__ chunk_hist) {
+    int n_packed, int id_bits, int32_t* __restrict__ entry_rank, int32_t* __restrict__ chunk_hist, int n_chunks,
+    const RouteSideJobs jobs) {
     extern __shared__ int lds[];
+    if ((int)blockIdx.x >= n_chunks) {
+        // workgroups past the routing chunks: the f16 copy of the activations, grid-stride over groups of eight
+        const int64_t n_g = jobs.T * (jobs.ldg >> 3), n_u = jobs.T * (jobs.ldu >> 3);
+        const int64_t step = (int64_t)(gridDim.x - n_chunks) * ROUTE_THREADS;
+        for (int64_t i = (int64_t)(blockIdx.x - n_chunks) * ROUTE_THREADS + threadIdx.x; i < n_g + n_u; i += step) {
+            if (i < n_g)
+                convert_bf16_group(jobs.src_g, jobs.dst_g, jobs.sg, jobs.ldg, i);
+            else
+                convert_bf16_group(jobs.src_u, jobs.dst_u, jobs.su, jobs.ldu, i - n_g);
+        }
+        return;
+    }
     int* hist = lds;
     int local[ROUTE_ROUNDS], rank[ROUTE_ROUNDS];
     const int64_t chunk_base = (int64_t)blockIdx.x * ROUTE_CHUNK;
@@ -231,12 +247,17 @@ __global__ __launch_bounds__(ROUTE_THREADS) void k_route_count(
 // One workgroup.  chunk_hist[b][e] (entries of expert e in chunk b) becomes the number of entries of
 // e in earlier chunks; expert_offsets the exclusive scan of the per-expert totals.  The chunks of an
 // expert are split over `parts` threads (parts * n_packed <= 1024) that first add up their runs.
+// With side jobs: the tile list of the grouped-GEMM path from the offsets just made, and token_start[t] = t * top_k.
 __global__ __launch_bounds__(1024) void k_route_scan(int32_t* __restrict__ chunk_hist, int n_chunks,
-                                                      int n_packed, int32_t* __restrict__ expert_offsets) {
+                                                      int n_packed, int32_t* __restrict__ expert_offsets,
+                                                      const RouteSideJobs jobs, int n_flat, int top_k) {
     extern __shared__ int lds[];
-    int* totals = lds;                       // [n_packed]
-    int* wave_sums = lds + n_packed;         // [32]
-    int* partial = lds + n_packed + 32;      // [parts][n_packed] when parts > 1
+    __shared__ MTileLds mt_lds;
+    int* totals = lds;                       // [n_packed + 1]
+    int* wave_sums = lds + n_packed + 1;     // [32]
+    int* partial = lds + n_packed + 33;      // [parts][n_packed] when parts > 1
+    if (jobs.token_start != nullptr)
+        for (int64_t t = threadIdx.x; t <= jobs.T; t += blockDim.x) jobs.token_start[t] = (int32_t)(t * top_k);
     const int tid = threadIdx.x;
     const int parts = n_packed <= 512 ? min(1024 / n_packed, 16) : 1;
     if (parts > 1) {
@@ -276,7 +297,15 @@ __global__ __launch_bounds__(1024) void k_route_scan(int32_t* __restrict__ chunk
     __syncthreads();
     const int total = block_exclusive_scan(totals, n_packed, wave_sums);
     for (int e = threadIdx.x; e < n_packed; e += blockDim.x) expert_offsets[e] = totals[e];
-    if (threadIdx.x == 0) expert_offsets[n_packed] = total;
+    if (threadIdx.x == 0) {
+        expert_offsets[n_packed] = total;
+        totals[n_packed] = total;
+    }
+    if (jobs.mtiles != nullptr) {
+        __syncthreads();
+        build_mtile_list(totals, n_packed, n_flat, jobs.max_mtiles, jobs.mtiles, jobs.n_mtiles, jobs.gate_fe, jobs.up_fe,
+                         mt_lds);
+    }
 }
 
 template <typename IdT>
@@ -284,25 +313,35 @@ __global__ __launch_bounds__(ROUTE_THREADS) void k_route_scatter(
     const IdT* __restrict__ selected, const float* __restrict__ weights, const int32_t* __restrict__ g2l,
     int n_global, int64_t n_flat, int top_k, int n_packed, const int32_t* __restrict__ entry_rank,
     const int32_t* __restrict__ chunk_hist, const int32_t* __restrict__ expert_offsets,
-    int32_t* __restrict__ token_indices, float* __restrict__ route_flat) {
+    int32_t* __restrict__ token_indices, float* __restrict__ route_flat, int32_t* __restrict__ slot,
+    int32_t* __restrict__ token_count) {
     const int64_t idx = (int64_t)blockIdx.x * ROUTE_THREADS + threadIdx.x;
     if (idx >= n_flat) return;
     const int r = entry_rank[idx];
+    const int64_t token = idx / top_k;
+    int before = 0;      // kept entries of the same token in front of this one (they are neighbours in the flat order)
+    if (slot != nullptr) {
+        for (int64_t i = token * top_k; i < idx; ++i) before += entry_rank[i] >= 0;
+        if (idx == token * top_k + top_k - 1) token_count[token] = before + (r >= 0);
+    }
     if (r < 0) return;
     const int id = load_local_id<IdT>(selected, g2l, n_global, n_packed, idx, n_flat);
     const int64_t chunk = idx / ROUTE_CHUNK;
     const int pos = expert_offsets[id] + chunk_hist[chunk * n_packed + id] + r;
-    token_indices[pos] = (int32_t)(idx / top_k);
+    token_indices[pos] = (int32_t)token;
     route_flat[pos] = weights[idx];
+    if (slot != nullptr) slot[pos] = before;
 }
 
 template <typename IdT>
 static int route_impl(const IdT* selected, const float* weights, const int32_t* g2l, int n_global,
                       int64_t n_flat, int top_k, int n_packed, int32_t* token_indices,
-                      int32_t* expert_offsets, float* route_flat, void* workspace, hipStream_t st) {
+                      int32_t* expert_offsets, float* route_flat, void* workspace, const RouteSideJobs* jobs,
+                      int* jobs_done, hipStream_t st) {
+    if (jobs_done) *jobs_done = 0;
     int id_bits = 0;
     while ((1 << id_bits) < n_packed) ++id_bits;
-    const size_t lds_bytes = (size_t)(n_packed + 32) * sizeof(int);
+    const size_t lds_bytes = (size_t)(n_packed + 33) * sizeof(int);
     // histogram + wave sums, and the per-(round, wavefront) tables of the low-barrier variant
     const size_t lds_rank_bytes = lds_bytes + (n_packed <= ROUTE_TABLE_MAX_EXPERTS
                                                    ? ((size_t)ROUTE_ROUNDS * (ROUTE_THREADS / 64) * n_packed +
@@ -318,16 +357,30 @@ static int route_impl(const IdT* selected, const float* weights, const int32_t* 
     const int64_t n_chunks = (n_flat + ROUTE_CHUNK - 1) / ROUTE_CHUNK;
     int32_t* entry_rank = (int32_t*)workspace;
     int32_t* chunk_hist = entry_rank + ((n_flat + 63) / 64) * 64;
-    hipLaunchKernelGGL(k_route_count<IdT>, dim3((unsigned)n_chunks), dim3(ROUTE_THREADS), lds_rank_bytes, st,
-                       selected, g2l, n_global, n_flat, n_packed, id_bits, entry_rank, chunk_hist);
+    // side jobs: extra workgroups of the counting launch copy the activations, the scatter writes slots and counts
+    RouteSideJobs carried;
+    int64_t copy_blocks = 0;
+    if (jobs != nullptr) {
+        carried = *jobs;
+        if (carried.src_g != nullptr) {
+            const int64_t groups = carried.T * ((carried.ldg >> 3) + (carried.ldu >> 3));
+            copy_blocks = std::min<int64_t>((groups + ROUTE_THREADS * 4 - 1) / (ROUTE_THREADS * 4), 4096);
+        }
+    }
+    hipLaunchKernelGGL(k_route_count<IdT>, dim3((unsigned)(n_chunks + copy_blocks)), dim3(ROUTE_THREADS), lds_rank_bytes, st,
+                       selected, g2l, n_global, n_flat, n_packed, id_bits, entry_rank, chunk_hist, (int)n_chunks, carried);
     BITSMOE_HIP_TRY(hipGetLastError());
     hipLaunchKernelGGL(k_route_scan, dim3(1), dim3(1024), lds_bytes + (n_packed <= 512 ? (size_t)16 * n_packed * sizeof(int) : 0),
-                       st, chunk_hist, (int)n_chunks, n_packed, expert_offsets);
+                       st, chunk_hist, (int)n_chunks, n_packed, expert_offsets, carried, (int)n_flat, top_k);
     BITSMOE_HIP_TRY(hipGetLastError());
     hipLaunchKernelGGL(k_route_scatter<IdT>, dim3((unsigned)((n_flat + ROUTE_THREADS - 1) / ROUTE_THREADS)),
                        dim3(ROUTE_THREADS), 0, st, selected, weights, g2l, n_global, n_flat, top_k, n_packed,
-                       entry_rank, chunk_hist, expert_offsets, token_indices, route_flat);
+                       entry_rank, chunk_hist, expert_offsets, token_indices, route_flat, carried.slot,
+                       carried.slot ? carried.token_count : nullptr);
     BITSMOE_HIP_TRY(hipGetLastError());
+    if (jobs_done)
+        *jobs_done = (copy_blocks > 0 ? MFMA_FRONT_CONVERTED : 0) |
+                     (carried.slot && carried.token_start ? MFMA_FRONT_TOKEN_COUNTED : 0) | (carried.mtiles ? MFMA_FRONT_MTILES : 0);
     return BITSMOE_OK;
 }
 
@@ -346,7 +399,17 @@ extern "C" int bitsmoe_route(const void* selected, int32_t ids_are_i64, const fl
                              int32_t top_k, int32_t n_packed, int32_t* token_indices,
                              int32_t* expert_offsets, float* route_flat, void* workspace,
                              size_t workspace_bytes, void* stream) {
-    hipStream_t st = (hipStream_t)stream;
+    return route_with_jobs(selected, ids_are_i64, weights, global_to_local, n_global, n_tokens, top_k, n_packed,
+                           token_indices, expert_offsets, route_flat, workspace, workspace_bytes, nullptr, nullptr,
+                           (hipStream_t)stream);
+}
+
+int bitsmoe::route_with_jobs(const void* selected, int32_t ids_are_i64, const float* weights,
+                             const int32_t* global_to_local, int32_t n_global, int64_t n_tokens, int32_t top_k,
+                             int32_t n_packed, int32_t* token_indices, int32_t* expert_offsets, float* route_flat,
+                             void* workspace, size_t workspace_bytes, const RouteSideJobs* jobs, int* jobs_done,
+                             hipStream_t st) {
+    if (jobs_done) *jobs_done = 0;
     BITSMOE_REQUIRE(n_tokens >= 0 && top_k > 0, "n_tokens must be >= 0 and top_k > 0");
     BITSMOE_REQUIRE(n_packed >= 0 && n_packed <= ROUTE_MAX_EXPERTS, "n_packed=%d outside [0,%d]", n_packed, ROUTE_MAX_EXPERTS);
     BITSMOE_REQUIRE(n_global >= 0, "n_global must be >= 0");
@@ -365,7 +428,7 @@ extern "C" int bitsmoe_route(const void* selected, int32_t ids_are_i64, const fl
     }
     if (ids_are_i64)
         return route_impl<int64_t>((const int64_t*)selected, weights, global_to_local, n_global, n_flat, top_k,
-                                   n_packed, token_indices, expert_offsets, route_flat, workspace, st);
+                                   n_packed, token_indices, expert_offsets, route_flat, workspace, jobs, jobs_done, st);
     return route_impl<int32_t>((const int32_t*)selected, weights, global_to_local, n_global, n_flat, top_k,
-                               n_packed, token_indices, expert_offsets, route_flat, workspace, st);
+                               n_packed, token_indices, expert_offsets, route_flat, workspace, jobs, jobs_done, st);
 }

@@ -68,6 +68,9 @@ def _case(cuda_device, seed, n_global, n_super, tokens, top_k, rank, dim, i64, d
     (8, 0, 9, 2, True, True), (10, 2, 9, 2, False, True), (128, 0, 40, 8, True, True), (130, 2, 128, 8, True, True),
     (8, 0, 1, 2, True, True), (32, 0, 4, 2, True, True), (40, 8, 6, 2, False, True), (128, 0, 8, 8, True, True),
     (8, 0, 300, 2, True, False), (64, 0, 64, 6, False, False),
+    # grouped GEMM behind the routing kernel's several-workgroup form: the f16 copy of the activations and the
+    # per-token tables are made by the routing launches (with and without dropped entries)
+    (10, 2, 700, 2, False, False), (8, 0, 600, 3, True, False),
 ])
 def test_forward_from_router_output(cuda_device, n_global, n_super, tokens, top_k, i64, expect_inline, dtype_name):
     sets, inline = _case(cuda_device, 500 + tokens, n_global, n_super, tokens, top_k, 512, 256, i64, dtype_name)
