@@ -825,7 +825,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
         auto compute = [&](auto b_c, int i) {
             constexpr int B = decltype(b_c)::value;
             u32x4 az[4];
-            const uint16_t* zp = z + n * z_stride + (tb + i) * N_TILE + 8 * kg;
+            const uint16_t* zp = z + n * z_stride + i * N_TILE + 8 * kg;      // (z holds this workgroup's tiles only)
 #pragma unroll
             for (int m = 0; m < 4; ++m) az[m] = *reinterpret_cast<const u32x4*>(zp + 32 * m);
             f32x4 corr;
@@ -861,7 +861,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                     const int a = idx / pieces, p = idx - a * pieces;
                     const int c = tb * N_TILE + 8 * p;
                     v[k] = *reinterpret_cast<const u32x4*>(Zg + (int64_t)(a0 + a) * I + c);
-                    dst[k] = a * z_stride + c;
+                    dst[k] = a * z_stride + 8 * p;
                 }
 #pragma unroll
                 for (int k = 0; k < 3; ++k)
@@ -908,7 +908,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                         u32x2 packed;
                         packed[0] = (uint32_t)zb[0] | ((uint32_t)zb[1] << 16);
                         packed[1] = (uint32_t)zb[2] | ((uint32_t)zb[3] << 16);
-                        *reinterpret_cast<u32x2*>(z + (ab + j) * z_stride + c) = packed;
+                        *reinterpret_cast<u32x2*>(z + (ab + j) * z_stride + c - tb * N_TILE) = packed;
                         // the 32 lanes of a half wavefront hold one tile's 128 columns: their sum
                         // arrives in lanes 31 and 63 (whole rows of 16 lanes are active or not)
                         part = dpp_add_f32<0x111>(part);

@@ -511,6 +511,46 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk_z(
 // per-tile sums of its rows, the epilogue's row and assignment records.
 // A workgroup takes four slabs of one expert and a run of tiles; with few active experts the
 // tiles are split over several workgroups (their partial sums meet in the atomics of the combine).
+// z = silu(G) * U as 16-bit operands [A, I] and the per-tile sums of the rounded operands [A, n_tiles], from the fp32
+// gate and up sums (the totals of `n_part` partial results): what the down kernel's workgroups otherwise each form
+// for themselves, two rows per memory round trip.  Worth a launch of its own where those workgroups hold full
+// 16-assignment chunks and many of them share a chunk.  A thread owns four columns, 32 lanes one tile of one row.
+__global__ __launch_bounds__(256) void k_decode_silu(const float* __restrict__ G, const float* __restrict__ U, int n_part,
+                                                     int64_t part_stride, int A, int I, int n_tiles,
+                                                     uint16_t* __restrict__ Z, float* __restrict__ Zsum) {
+    const int64_t unit = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 5;      // (row, tile)
+    const int lane32 = threadIdx.x & 31;
+    const int a = (int)(unit / n_tiles), t = (int)(unit - (int64_t)a * n_tiles);
+    if (a >= A) return;                  // (whole half-wavefronts leave)
+    const int c = t * N_TILE + 4 * lane32;
+    const bool in = c < I;
+    const int64_t gi = (int64_t)a * I + (in ? c : 0);
+    f32x4 gv = *reinterpret_cast<const f32x4*>(G + gi), uv = *reinterpret_cast<const f32x4*>(U + gi);
+    for (int p = 1; p < n_part; ++p) {
+        gv += *reinterpret_cast<const f32x4*>(G + gi + p * part_stride);
+        uv += *reinterpret_cast<const f32x4*>(U + gi + p * part_stride);
+    }
+    uint16_t zb[4];
+    float part = 0.0f;      // sum of the four operands as rounded
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        zb[x] = in ? to_operand<false>(silu_f32(gv[x]) * uv[x]) : (uint16_t)0;
+        part += __half2float(__ushort_as_half(zb[x]));
+    }
+    if (in) {
+        u32x2 packed;
+        packed[0] = (uint32_t)zb[0] | ((uint32_t)zb[1] << 16);
+        packed[1] = (uint32_t)zb[2] | ((uint32_t)zb[3] << 16);
+        *reinterpret_cast<u32x2*>(Z + (int64_t)a * I + c) = packed;
+    }
+    part = dpp_add_f32<0x111>(part);
+    part = dpp_add_f32<0x112>(part);
+    part = dpp_add_f32<0x114>(part);
+    part = dpp_add_f32<0x118>(part);
+    part = dpp_add_f32<0x142, 0xa>(part);
+    if (lane32 == 31) Zsum[(int64_t)a * n_tiles + t] = part;
+}
+
 // ZREADY: G / U hold Z / Zsum written by k_gateup_walk_z instead of the fp32 gate and up sums.  Otherwise the
 // sums are the totals of `n_part` partial results part_stride floats apart (k_gateup_walk).
 // ROUTED (GRID_EXPERTS or GRID_ACTIVE): no routing tables; the workgroup finds its expert's entries among the routed
@@ -593,7 +633,7 @@ __global__ __launch_bounds__(256, ZR > ZROWS ? 3 : 4) void k_down_decode(
     gptr<int32_t> rank_idx = as_global(fe.rank_idx);
     extern __shared__ __attribute__((aligned(16))) unsigned char dsmem[];
     uint16_t* z = reinterpret_cast<uint16_t*>(dsmem);
-    const int z_stride = n_tiles * N_TILE + 8;
+    const int z_stride = tiles_per_wg * N_TILE + 8;      // (the workgroup's own tiles)
     float* zsum = reinterpret_cast<float*>(dsmem + (size_t)MAX_A * z_stride * 2);      // [assignment][tile]
     int2* rows = reinterpret_cast<int2*>(zsum + MAX_A * ZSUM_STRIDE) + wave * SLAB_ROWS;     // this wavefront's (rank, multiplier) per row
     int2* assigns = reinterpret_cast<int2*>(zsum + MAX_A * ZSUM_STRIDE) + DN_SLABS_PER_WG * SLAB_ROWS;    // (token, routing weight) per assignment
@@ -822,17 +862,40 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     }
     BITSMOE_HIP_TRY(hipGetLastError());
     record(prof, 2, st);
-    record(prof, 3, st);      // (SiLU happens inside the down kernel)
+    // z formed once by a small launch of its own instead of by every down workgroup: on the chunk grid (full
+    // 16-assignment chunks: eight dependent round trips of two rows each in every one of the workgroups that share
+    // a chunk), when the workspace has a free slot behind the partial results.  BITSMOE_DECODE_SPLIT_Z=0 / 1
+    // switches it off / on wherever it is possible (experiments).
+    const char* split_z_var = getenv("BITSMOE_DECODE_SPLIT_Z");
+    const int split_z_env = split_z_var && split_z_var[0] ? atoi(split_z_var) : -1;
+    const bool split_z_possible = !fused_z && !routed && (walk ? n_part : 1) < part_capacity && I % 4 == 0;
+    const bool split_z = split_z_possible && (split_z_env >= 0 ? split_z_env > 0 : mode == GRID_CHUNKS);
+    const int parts_in = walk && !fused_z ? n_part : 1;
+    float* down_g = G;
+    float* down_u = U;
+    if (split_z) {
+        uint16_t* Z = reinterpret_cast<uint16_t*>(G + parts_in * part_stride);
+        float* Zsum = U + parts_in * part_stride;
+        const int64_t threads = A * (int64_t)n_tiles * 32;
+        hipLaunchKernelGGL(k_decode_silu, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, G, U, parts_in, part_stride,
+                           (int)A, I, n_tiles, Z, Zsum);
+        BITSMOE_HIP_TRY(hipGetLastError());
+        down_g = reinterpret_cast<float*>(Z);
+        down_u = Zsum;
+    }
+    record(prof, 3, st);      // (otherwise SiLU happens inside the down kernel)
     const int dn_groups = (down->prep_max_slabs + DN_SLABS_PER_WG - 1) / DN_SLABS_PER_WG;
-    const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4 + DN_SLABS_PER_WG * SLAB_ROWS * 8 + MAX_A * 8;
     int dn_tiles_per_wg = n_tiles;
+    // (600 measured best on the 26-layer stack at 32 tokens against 300, 1200 and 2400: the kernel is bound by the
+    // instructions a workgroup issues, and more, shorter workgroups add their fixed part)
     while (dn_tiles_per_wg > 1 && units * dn_groups * ((n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg) < 600)
         dn_tiles_per_wg = (dn_tiles_per_wg + 1) / 2;
+    const size_t z_bytes = (size_t)MAX_A * (dn_tiles_per_wg * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4 + DN_SLABS_PER_WG * SLAB_ROWS * 8 + MAX_A * 8;
     const int dn_tchunks = (n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg;
     auto launch_down = [&](auto kernel) {
         const int n_work = e_dim * dn_groups * dn_tchunks;
         hipLaunchKernelGGL(kernel, dim3((unsigned)((n_work + 7) / 8 * 8)), dim3(256), z_bytes, st, down->d_fast_experts,
-                           down->d_fast_slabs, down->prep_max_slabs, G, U, walk && !fused_z ? n_part : 1, part_stride, rw, tok, off,
+                           down->d_fast_slabs, down->prep_max_slabs, down_g, down_u, split_z ? 1 : parts_in, part_stride, rw, tok, off,
                            (int)T, (int)A, I, E, n_tiles, dn_groups, dn_tchunks, dn_tiles_per_wg, n_work, rank_out, rank_accum,
                            routed ? routed->selected : nullptr, routed ? routed->ids_are_i64 : 0, routed ? (int)A : 0,
                            routed ? routed->top_k : 1, routed ? routed->local_to_global : nullptr,
@@ -863,7 +926,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         launch_down(k_down_decode<M, Z, false, ZROWS>);
     };
     // (G and U are fp32 and the operands f16 whatever the activation type was)
-    if (fused_z)
+    if (fused_z || split_z)
         with_mode(launch_down_mode, std::true_type{});
     else
         with_mode(launch_down_mode, std::false_type{});
