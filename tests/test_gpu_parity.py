@@ -320,6 +320,23 @@ def test_forward_decode_path_both_projections_in_one_workgroup(cuda_device, bits
     assert err < 3e-3
 
 
+@pytest.mark.parametrize("split_z", ["0", "1", None])
+@pytest.mark.parametrize("bits", [(2,), (2, 3, 4)])
+def test_forward_decode_path_z_by_its_own_launch(cuda_device, bits, split_z, monkeypatch):
+    """The chunk grid (3 experts, 40 tokens x 2: chunks of 16 assignments and ragged last chunks): z = silu(G) * U
+    formed once by a small launch and copied by the down workgroups (BITSMOE_DECODE_SPLIT_Z=1, the default on this
+    grid) and formed by every down workgroup itself (=0) -- both against the oracle."""
+    from bitsmoe_amd.algorithms import _capi
+
+    if split_z is None:
+        monkeypatch.delenv("BITSMOE_DECODE_SPLIT_Z", raising=False)
+    else:
+        monkeypatch.setenv("BITSMOE_DECODE_SPLIT_Z", split_z)
+    err = _forward_case(cuda_device, 740 + len(bits), 3, 40, 2, 1024, 256, 384, "bf16", bits, path=_capi.PATH_DECODE,
+                        tol=1e-2, uniform_bits=True)
+    assert err < 3e-3
+
+
 @pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
 def test_forward_mfma_path_scattered_ranks(cuda_device, dtype_name):
     """rank_idx without runs of eight consecutive ranks: the activations are gathered first."""
