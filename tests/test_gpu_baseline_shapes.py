@@ -93,6 +93,28 @@ def test_full_size_matches_oracle(cuda_device, key, tokens):
     print(f"{key} T={tokens}: err {err:.2e}")
 
 
+@pytest.mark.parametrize("key,tokens", [("c2", 1), ("c2", 8), ("c2", 32), ("c2", 64), ("c3", 4096), ("c4", 256), ("c5", 32)])
+def test_full_size_from_router_output(cuda_device, key, tokens):
+    """The one-call forward from the router's ids and weights (routing inside the decode kernels; at prefill size
+    the routing launches carry the grouped GEMM's front end) against the oracle, and against the two-call form."""
+    from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
+    from bitsmoe_amd.synth import SPECS
+
+    spec = SPECS[key]
+    block = _layer("c2" if key == "c3" else key, cuda_device)
+    h_gate, h_up, selected, weights = _inputs(block, spec, tokens, 17 + tokens, cuda_device)
+    tok, off, rw, two_calls = _run(block, h_gate, h_up, selected, weights)
+    gate, up, down = block._ensure_matsets()
+    got = hip.moe_forward_routed(h_gate, h_up, selected, weights, block._packed_global_to_local,
+                                 block._packed_local_to_global, gate, up, down, int(block.shared_u_down.shape[1]),
+                                 int(block._packed_intermediate_size), 0)
+    ref = _oracle(block, h_gate, h_up, *(t.cpu().numpy() for t in (tok, off, rw)))
+    scale = float(np.abs(ref).max())
+    err = float(np.abs(got.cpu().numpy() - ref).max()) / scale
+    assert err <= 1e-2, f"{spec.name} T={tokens}: normalised error {err:.3e}"
+    assert float((got - two_calls).abs().max()) <= 2e-3 * scale       # (fp32 atomics in another order; f16 intermediates)
+
+
 @pytest.mark.parametrize("key,tokens", [("c2", 64), ("c1", 16), ("c5", 32)])
 def test_full_size_both_projections_in_one_workgroup(cuda_device, key, tokens, monkeypatch):
     """The decode path that forms z in the gate/up kernel (BITSMOE_DECODE_FUSED_Z=1) at full size."""

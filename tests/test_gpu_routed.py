@@ -78,6 +78,36 @@ def test_forward_from_router_output(cuda_device, n_global, n_super, tokens, top_
     assert inline == expect_inline
 
 
+@pytest.mark.parametrize("dtype_name,choices", [("bf16", (2,)), ("f16", (2, 2, 2, 3, 4))])
+def test_forward_from_router_output_more_items_than_workgroup_slots(cuda_device, dtype_name, choices):
+    """More (expert, tile, projection) items than the chip holds workgroups at once (128 experts x 5 tiles x 2);
+    64 tokens, top-8 with skewed logits: experts with no entry, with one, and with more than one chunk of 16."""
+    import torch
+
+    hip = _hip()
+    rng = np.random.default_rng(41)
+    e, tokens, top_k, rank, dim = 128, 64, 8, 512, 640
+    gate, up, down = helpers.make_experts(41, e, rank, rank, dim, choices=choices, uniform_bits=True)
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    h_gate = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(dt)
+    h_up = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(dt)
+    logits = rng.normal(size=(tokens, e)).astype(np.float32)
+    logits[:, :3] += 4.0
+    idx, w = o.router_qwen(logits, top_k)
+    ids = np.arange(e, dtype=np.int32)
+    tok, off, rw = o.build_routing(idx, w, ids, e)
+    counts = np.diff(off)
+    assert counts.max() > 16 and counts.min() == 0
+    ref = o.moe_forward(h_gate.float().numpy(), h_up.float().numpy(), tok, off, rw, gate, up, down, rank, dim)
+    sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=dim) for m in (gate, up, down)]
+    sel, wt = torch.from_numpy(idx.astype(np.int64)).to(cuda_device), torch.from_numpy(w).to(cuda_device)
+    ids_t = torch.from_numpy(ids).to(cuda_device)
+    got = hip.moe_forward_routed(h_gate.to(cuda_device), h_up.to(cuda_device), sel, wt, ids_t, ids_t, *sets, rank, dim, 0)
+    assert hip.routed_is_inline(h_gate.to(cuda_device), h_up.to(cuda_device), top_k, *sets)
+    err = helpers.norm_err(got.cpu().numpy(), ref)
+    assert err <= 3e-3, f"normalised error {err:.3e}"
+
+
 @pytest.mark.parametrize("experts", ["mixed", "generic"])
 def test_forward_from_router_output_other_layouts(cuda_device, experts):
     """Experts of mixed widths (the walking kernel's mixed form, rank 512: whole groups) and sets the fast
