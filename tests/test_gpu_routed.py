@@ -157,3 +157,59 @@ def test_forward_from_router_output_under_graph_replay(cuda_device):
         again = run().clone()          # eager work between the replays
         torch.cuda.synchronize()
         assert float((again - eager).abs().max()) <= 1e-5 * scale
+
+
+def test_grouped_gemm_from_router_output_under_graph_replay(cuda_device):
+    """The prefill-sized one-call forward (three routing launches that also make the activation copy, the tile
+    list and the per-token tables, then the grouped GEMM): captured into a HIP graph, every replay -- with eager
+    work and synchronisations in between, and with other routings run through the same workspace-free entry in
+    between -- reproduces the eager result bit for bit (no atomics on this path)."""
+    import torch
+
+    hip = _hip()
+    rng = np.random.default_rng(9)
+    n_global, tokens, top_k, rank, dim = 10, 700, 2, 512, 256
+    keep = np.ones(n_global, bool)
+    keep[[3, 7]] = False                      # two router ids belong to no packed expert: their entries are dropped
+    g2l = np.full(n_global, -1, np.int32)
+    g2l[keep] = np.arange(keep.sum(), dtype=np.int32)
+    l2g = np.nonzero(keep)[0].astype(np.int32)
+    e = int(keep.sum())
+    gate, up, down = helpers.make_experts(9, e, rank, rank, dim, choices=(2, 3, 4), uniform_bits=True)
+    sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=dim) for m in (gate, up, down)]
+    h_gate = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(torch.bfloat16).to(cuda_device)
+    h_up = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(torch.bfloat16).to(cuda_device)
+    idx, w = o.router_qwen(rng.normal(size=(tokens, n_global)).astype(np.float32), top_k)
+    idx2, w2 = o.router_qwen(rng.normal(size=(tokens, n_global)).astype(np.float32), top_k)
+    sel, wt = torch.from_numpy(idx).to(cuda_device), torch.from_numpy(w).to(cuda_device)
+    sel2, wt2 = torch.from_numpy(idx2).to(cuda_device), torch.from_numpy(w2).to(cuda_device)
+    g2l_t, l2g_t = torch.from_numpy(g2l).to(cuda_device), torch.from_numpy(l2g).to(cuda_device)
+    out = torch.empty((tokens, rank), dtype=torch.float32, device=cuda_device)
+
+    def run(s=sel, ww=wt, dst=out):
+        return hip.moe_forward_routed(h_gate, h_up, s, ww, g2l_t, l2g_t, *sets, rank, dim, 0, out=dst)
+
+    eager = run().clone()
+    torch.cuda.synchronize()
+    assert not hip.routed_is_inline(h_gate, h_up, top_k, *sets)
+    tok, off, rw = o.build_routing(idx, w, g2l, e)
+    ref = o.moe_forward(h_gate.float().cpu().numpy(), h_up.float().cpu().numpy(), tok, off, rw, gate, up, down, rank, dim)
+    assert helpers.norm_err(eager.cpu().numpy(), ref) <= 3e-3
+    side = torch.cuda.Stream(device=cuda_device)
+    side.wait_stream(torch.cuda.current_stream(cuda_device))
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream(cuda_device).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run()
+    other = torch.empty_like(out)
+    for _ in range(3):
+        out.fill_(7.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        run(sel2, wt2, other)          # another routing between the replays
+        torch.cuda.synchronize()
+        assert not torch.equal(other, eager)
