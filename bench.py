@@ -21,7 +21,8 @@ shaped stack, one step = one pass over all 26 layers (per-layer figures reported
 
 Prints ONE JSON line.  `value` is tokens/s of the primary workload (default: the
 Qwen3-30B-A3B-shaped layer at decode, 64 tokens); `extras` holds the other decode batch
-sizes, the 4096-token prefill and the stack; `roofline` is the dominant kernel of the primary workload
+sizes, the 4096-token prefill, the other layer shapes of the benchmark set (c1, c4), checkpoint-shaped experts and the
+stack; `roofline` is the dominant kernel of the primary workload
 (algorithmic bytes / HIP-event duration against 8 TB/s, or algorithmic FLOP/s against the
 2.5 PFLOP/s dense bf16 MFMA peak); `cpu_baseline` is the CPU restatement of the reference
 algorithm (oracle/oracle.c, OpenMP) timed on this host's cores on the same workload — the
@@ -51,12 +52,17 @@ WORKLOADS = {
     "c3-t4096": ("c3", 4096, "mfma"),
     "c2-ckpt-t64": ("c2", 64, "hbm"),
     "c3-ckpt-t4096": ("c3", 4096, "mfma"),
+    "c1-t16": ("c1", 16, "hbm"),
+    "c4-t256": ("c4", 256, "hbm"),
     "c5-stack-t32": ("c5", 32, "hbm"),
     "c5-stack-t2048": ("c5", 2048, "mfma"),
 }
 WORKLOAD_DESC = {
     "c2": "Qwen3-30B-A3B-shaped MoE layer (128 experts, top-8, hidden 2048, intermediate 768, mixed 2/3/4-bit, group 128)",
     "c3": "Qwen3-30B-A3B-shaped MoE layer (128 experts, top-8, hidden 2048, intermediate 768, mixed 2/3/4-bit, group 128)",
+    "c1": "DeepSeek-V2-Lite-shaped MoE layer (64 experts, top-6, hidden 2048, intermediate 1408, mixed 2/3/4-bit, group 128)",
+    "c4": "Qwen3-Next-80B-A3B-shaped MoE layer (512 experts, top-10, one shared expert outside the operator, hidden 2048, "
+          "intermediate 512, mixed 2/3/4-bit, group 128)",
     "c5": "DeepSeek-V2-Lite-shaped stack of 26 MoE layers (64 routed + 2 shared experts, top-6, hidden 2048, "
           "intermediate 1408, mixed 2/3/4-bit, group 128, Zipf(1.2)-skewed routing)",
 }
