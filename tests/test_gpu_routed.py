@@ -14,7 +14,8 @@ def _hip():
     return hip
 
 
-def _case(cuda_device, seed, n_global, n_super, tokens, top_k, rank, dim, i64, dtype_name, experts="uniform", path=None):
+def _case(cuda_device, seed, n_global, n_super, tokens, top_k, rank, dim, i64, dtype_name, experts="uniform", path=None,
+          scramble_ranks=False):
     import torch
 
     from bitsmoe_amd.algorithms import _capi
@@ -35,6 +36,9 @@ def _case(cuda_device, seed, n_global, n_super, tokens, top_k, rank, dim, i64, d
         gate, up, down = helpers.make_experts(seed, e, rank, rank, dim, choices=(2, 3, 4), slab_multiple=64)
     else:       # slabs of other widths: the generic kernels, routing tables
         gate, up, down = helpers.make_experts(seed, e, rank, rank, dim, choices=(2, 8), slab_multiple=64)
+    if scramble_ranks:       # rows of gate / up read arbitrary columns of h instead of runs of eight
+        for m in gate + up:
+            m["rank_idx"] = rng.permutation(rank).astype(np.int32)[m["rank_idx"]]
     dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
     h_gate = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(dt)
     h_up = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(dt)
@@ -106,6 +110,15 @@ def test_forward_from_router_output_more_items_than_workgroup_slots(cuda_device,
     assert hip.routed_is_inline(h_gate.to(cuda_device), h_up.to(cuda_device), top_k, *sets)
     err = helpers.norm_err(got.cpu().numpy(), ref)
     assert err <= 3e-3, f"normalised error {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+def test_grouped_gemm_from_router_output_with_scattered_ranks(cuda_device, dtype_name):
+    """Prefill size with rank tables the gate/up kernel cannot read activations through (no runs of eight
+    consecutive ranks): the routing launches still build the tile list and the per-token tables, the activations
+    are gathered per assignment by the grouped-GEMM launcher."""
+    _, inline = _case(cuda_device, 93, 10, 2, 700, 2, 256, 256, False, dtype_name, scramble_ranks=True)
+    assert not inline
 
 
 @pytest.mark.parametrize("experts", ["mixed", "generic"])
