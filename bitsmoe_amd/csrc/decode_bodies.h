@@ -771,7 +771,7 @@ __device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4
             else if constexpr (W == 4)
                 bw = decode_fields4<false>(b.w[nb * 4 + m]);
             else
-                bw = decode_fields3<false>(b.w[nb * 2 + (m >> 1)], 8 * (m & 1), b.w[8 + nb], 4 * m);
+                bw = decode_r1w3<false>(b.w, nb, m);
             t = mfma16<false>(az[m], bw, t);
         }
         acc[nb] += (t - corr) * sc[nb];
@@ -817,7 +817,8 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
         auto issue = [&](auto b_c, int i) {
             constexpr int B = decltype(b_c)::value;
             const int t = tb + i;
-            load_block_role1<WL>(payload + (uint32_t)(fs.pack_off + (t + chunk_zero) * 256 * WL), lane, buf[B]);
+            load_block_role1<WL>(payload + (uint32_t)(fs.pack_off + (t + chunk_zero) * (WL == 3 ? R1W3_BLOCK_WORDS : 256 * WL)), lane,
+                                 buf[B]);
             gptr<__half> sp = scale + (uint32_t)(fs.scale_off + t * SLAB_ROWS + n);
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) sc[B][nb] = gload_half(sp + 16 * nb);

@@ -54,16 +54,21 @@ struct Block16 {   // up to 16 payload words of one lane for one (slab, tile) bl
     uint32_t w[16];
 };
 
-// role 1 loads: 2-bit 8 words [nb][h], 4-bit 16 words [nb][m], 3-bit 8 low words + 4 high words [nb]
+// role 1 loads: 2-bit 8 words [nb][h], 4-bit 16 words [nb][m], 3-bit 13 words (five code pairs each)
 template <int W>
 __device__ __forceinline__ void load_block_role1(gptr<uint32_t> blk, int lane, Block16& b) {
-    gptr_u32x4 p = reinterpret_cast<gptr_u32x4>(blk + (W == 4 ? lane * 16 : lane * 8));
-    u32x4 v0 = p[0], v1 = p[1], v2 = {0, 0, 0, 0}, v3 = {0, 0, 0, 0};
+    gptr_u32x4 p = reinterpret_cast<gptr_u32x4>(blk + (W == 4 ? lane * 16 : W == 3 ? lane * 4 : lane * 8));
+    u32x4 v0 = p[0], v1, v2 = {0, 0, 0, 0}, v3 = {0, 0, 0, 0};
+    if constexpr (W == 3) {
+        v1 = p[64];       // (+256 words)
+        v2 = p[128];
+        v3[0] = blk[768 + lane];
+    } else {
+        v1 = p[1];
+    }
     if constexpr (W == 4) {
         v2 = p[2];
         v3 = p[3];
-    } else if constexpr (W == 3) {
-        v2 = *reinterpret_cast<gptr_u32x4>(blk + 512 + lane * 4);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {

@@ -772,7 +772,7 @@ __device__ __forceinline__ void down_half_mfma(int bits, const uint16_t* stage, 
                 b = decode_fields4<false>(blk.w[nb * 4 + m]);
                 off = neg_offset_pair<4>();
             } else {
-                b = decode_fields3<false>(blk.w[nb * 2 + HH], 8 * km, blk.w[8 + nb], 4 * m);
+                b = decode_r1w3<false>(blk.w, nb, m);
                 off = neg_offset_pair<3>();
             }
             for (int i = 0; i < 4; ++i) b[i] = pk_mul_f16(pk_add_f16(b[i], off), scp[nb]);
@@ -819,15 +819,16 @@ __device__ __forceinline__ void down_tile_loop(const uint32_t* __restrict__ payl
         for (int j = 0; j < NJ; ++j)
             load_to_lds16(z + (rowbase[j] + (uint32_t)(64 * h)), st + j * 2048 + wave * 512);
     };
-    // role 1 block: 2-bit 8 words per lane, 4-bit 16, 3-bit 8 low words + 4 high words
-    // (fast_helpers.h); load i fills words 4i .. 4i+3 of every lane's sixteen
-    const uint32_t lane_words = (uint32_t)lane * (W == 4 ? 16u : W != 0 ? 8u : 4u);
+    // role 1 block: 2-bit 8 words per lane, 4-bit 16, 3-bit 13 (three regions of four words per lane, the
+    // thirteenth in a region of its own: four lanes fetch the same 16 bytes and each keeps its word)
+    // (fast_helpers.h, wave_layout.h); load i fills words 4i .. 4i+3 of every lane's sixteen
+    const uint32_t lane_words = (uint32_t)lane * (W == 4 ? 16u : W == 2 ? 8u : 4u);
     auto request_b = [&](int t) {
-        const uint32_t base = W != 0 ? (uint32_t)(fs.pack_off + t * 256 * W) : 0u;
+        const uint32_t base = W != 0 ? (uint32_t)(fs.pack_off + t * block_words(ROLE_DOWN, W)) : 0u;
         const uint32_t o0 = base + lane_words;
-        const uint32_t o1 = W != 0 ? o0 + 4u : o0;
-        const uint32_t o2 = W == 4 ? o0 + 8u : W == 3 ? base + 512u + (uint32_t)lane * 4u : o0;
-        const uint32_t o3 = W == 4 ? o0 + 12u : o0;
+        const uint32_t o1 = W == 3 ? o0 + 256u : W != 0 ? o0 + 4u : o0;
+        const uint32_t o2 = W == 4 ? o0 + 8u : W == 3 ? o0 + 512u : o0;
+        const uint32_t o3 = W == 4 ? o0 + 12u : W == 3 ? base + 768u + (uint32_t)(lane & ~3) : o0;
         load_to_lds16(payload + o0, wbuf);
         load_to_lds16(payload + o1, wbuf + 256);
         load_to_lds16(payload + o2, wbuf + 512);
@@ -845,6 +846,10 @@ __device__ __forceinline__ void down_tile_loop(const uint32_t* __restrict__ payl
             blk.w[4 * i + 1] = v[1];
             blk.w[4 * i + 2] = v[2];
             blk.w[4 * i + 3] = v[3];
+        }
+        if (W == 3) {      // the thirteenth word: this lane's of the four its load brought
+            const int k = lane & 3;
+            blk.w[12] = k == 0 ? blk.w[12] : k == 1 ? blk.w[13] : k == 2 ? blk.w[14] : blk.w[15];
         }
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) scp[nb] = (uint32_t)sbuf[16 * nb + n] * 0x10001u;

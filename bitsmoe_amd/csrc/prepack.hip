@@ -57,13 +57,31 @@ __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src
     const FastSlab fs = fslabs[(int64_t)task.expert * max_slabs + ps];
     const int w = fs.bits;
     const int32_t* __restrict__ row_src = ps_tab.row_src + (fe.rank_idx - ps_tab.rank_base);
-    uint32_t* __restrict__ out = const_cast<uint32_t*>(fe.payload) + fs.pack_off + t * 256 * w;
+    uint32_t* __restrict__ out = const_cast<uint32_t*>(fe.payload) + fs.pack_off + t * block_words(role, w);
     auto code_at = [&](int row, int col) { return (uint32_t)(source_level(mv, row_src, ps, row, t, col) + level_offset(w)); };
     const int nbs = (role == ROLE_GATE_UP) ? 8 : 4;        // output blocks per lane
     const int run = (role == ROLE_GATE_UP) ? 16 : 32;      // contraction indices per (lane, nb)
-    const int n_words = 256 * w;
+    const int n_words = block_words(role, w);
     for (int idx = threadIdx.x; idx < n_words; idx += blockDim.x) {
         uint32_t word = 0;
+        if (w == 3 && role == ROLE_DOWN) {
+            // whole 3-bit fields, five pairs of neighbouring codes per word (wave_layout.h)
+            const int l = idx < 768 ? (idx & 255) >> 2 : idx - 768;
+            const int j = idx < 768 ? (idx >> 8) * 4 + (idx & 3) : 12;
+            const int n = l & 15, kg = l >> 4;
+            for (int sl = 0; sl < 5; ++sl) {
+                const int P = 5 * j + sl;
+                if (P >= 64) break;
+                const int nb = P >> 4, m = (P >> 2) & 3, i = P & 3;
+                for (int odd = 0; odd < 2; ++odd) {
+                    int row, col;
+                    run_element(role, nb, kg, n, 8 * m + 2 * i + odd, &row, &col);
+                    word |= (code_at(row, col) & 7u) << (r1w3_slot_pos(sl) + 16 * odd);
+                }
+            }
+            out[idx] = word;
+            continue;
+        }
         if (w == 3 && idx >= 512) {
             // third bit of the 3-bit codes
             const int j = idx - 512;
@@ -76,13 +94,6 @@ __global__ __launch_bounds__(256) void k_prepack(const MatView* __restrict__ src
                         run_element(role, nb, kg, n8 + 8 * upper, x, &row, &col);
                         word |= ((code_at(row, col) >> 2) & 1u) << pos1s(x, upper);
                     }
-            } else {                      // j = l*4 + nb
-                const int nb = j & 3, l = j >> 2, n = l & 15, kg = l >> 4;
-                for (int x = 0; x < 32; ++x) {
-                    int row, col;
-                    run_element(role, nb, kg, n, x, &row, &col);
-                    word |= ((code_at(row, col) >> 2) & 1u) << pos1(x);
-                }
             }
             out[idx] = word;
             continue;
@@ -154,7 +165,7 @@ __global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* the call
     const int ps = blockIdx.x;
     const FastSlab fs = fs_row[ps];
     const int w = fs.bits;
-    const uint32_t* __restrict__ blk = fe.payload + fs.pack_off + (int)blockIdx.y * 256 * w;
+    const uint32_t* __restrict__ blk = fe.payload + fs.pack_off + (int)blockIdx.y * block_words(role, w);
     const int nbs = (role == ROLE_GATE_UP) ? 8 : 4;
     const int run = (role == ROLE_GATE_UP) ? 16 : 32;
     for (int idx = threadIdx.x; idx < SLAB_ROWS * N_TILE; idx += blockDim.x) {
@@ -167,7 +178,10 @@ __global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* the call
         run_element(role, nb, kg, n, x, &row, &col);
         uint32_t u;
         const int unit = (role == ROLE_GATE_UP) ? idx2_role0(nb, l) : (l * nbs + nb);
-        if (w == 4) {
+        if (w == 3 && role == ROLE_DOWN) {
+            const int P = 16 * nb + 4 * (x >> 3) + ((x & 7) >> 1);
+            u = (blk[r1w3_word_index(l, P / 5)] >> (r1w3_slot_pos(P % 5) + 16 * (x & 1))) & 7u;
+        } else if (w == 4) {
             const int per = run / 8;
             const uint32_t word = blk[unit * per + (x >> 3)];
             u = (role == ROLE_GATE_UP ? rotr32(word, pos4s(x & 7)) : word >> pos4(x & 7)) & 15u;
@@ -178,13 +192,8 @@ __global__ __launch_bounds__(256) void k_dequant_prepared(MatView mv /* the call
             if (w == 3) {
                 uint32_t hi;
                 int p;
-                if (role == ROLE_GATE_UP) {
-                    hi = blk[512 + hi_index0(kg, n, nb)];
-                    p = pos1s(x, n >> 3);
-                } else {
-                    hi = blk[512 + l * 4 + nb];
-                    p = pos1(x);
-                }
+                hi = blk[512 + hi_index0(kg, n, nb)];      // (role 0: role 1 took the branch above)
+                p = pos1s(x, n >> 3);
                 u |= ((hi >> p) & 1u) << 2;
             }
         }
@@ -306,7 +315,7 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
         for (int ps = 0; ps < n_ps[e]; ++ps) {
             BITSMOE_REQUIRE(words < ((int64_t)1 << 31) - (int64_t)n_tiles * 256 * 4, "expert %d: prepared payload exceeds int32 word offsets", e);
             fslabs[(size_t)e * pms + ps] = FastSlab{width[ps], (int32_t)words, ps * n_tiles * SLAB_ROWS, ps * SLAB_ROWS};
-            words += (int64_t)n_tiles * 256 * width[ps];
+            words += (int64_t)n_tiles * block_words(role, width[ps]);
             tasks.push_back(SlabTask{e, ps});
         }
         pay_words += round_up(words, 64);      // keep every matrix 256-byte aligned

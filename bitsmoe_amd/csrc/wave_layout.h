@@ -18,8 +18,9 @@
 //   Role 1: a run of 16 codes with index x = 0..15 sits in a word, precisely:
 //     2-bit fields:  field LSB at  (x & ~1) + 16*(x & 1)
 //     4-bit fields:  8 codes per word, field LSB at 4*(x'/2) + 16*(x' & 1), x' = x % 8
-//     3-bit codes :  low two bits as 2-bit fields, bit 2 as single bits at
-//                    (y/2) + 16*(y & 1) of a separate word (y = index in a run of 32)
+//     3-bit codes :  whole 3-bit fields, five PAIRS of neighbouring codes per word: pair P = 16*nb + 4*m + e'/2
+//                    of the lane (0..63) sits in word P/5 of the lane's thirteen, its two fields at bits
+//                    1 + 3*(P%5) and 17 + 3*(P%5) (832 words per block instead of 768)
 //   so that ONE rotate and ONE and-or turn a word into a packed pair of 16-bit floats
 //   (2^w + code) for two neighbouring contraction indices: the pair lives 16 bits apart.
 //
@@ -44,7 +45,7 @@
 //           w=4: word[idx2(nb, l)*2 + j]
 //           w=3: low word[idx2(nb, l)], high word[512 + hi_index0(kg, n, nb)]
 //   role 1: w=2: word[(l*4 + nb)*2 + h]           w=4: word[(l*4 + nb)*4 + m]
-//           w=3: low  word[(l*4 + nb)*2 + h]      high word[512 + l*4 + nb]
+//           w=3: word j of lane l at (j/4)*256 + l*4 + j%4 for j < 12 (three 16-byte loads per lane), word 12 at 768 + l
 //
 // Decoded operand value is (2^w + code); the true level is code - 2^(w-1), so every dot
 // product carries the constant 1.5 * 2^w times the sum of the other operand, which the
@@ -73,6 +74,13 @@ __host__ __device__ inline int pos2(int x) { return (x & ~1) + 16 * (x & 1); }
 __host__ __device__ inline int pos4(int x) { return 4 * (x >> 1) + 16 * (x & 1); }
 // index y (0..31) of a run of 32 single bits (role 1) / (0..15) + 8*upper (role 0)
 __host__ __device__ inline int pos1(int y) { return (y >> 1) + 16 * (y & 1); }
+
+// role 1, 3-bit: words of one (slab, tile) block, the place of word j (0..12) of lane l, the low-half bit offset of
+// slot sl (0..4) of a word, and the words of a block of either role and width
+constexpr int R1W3_BLOCK_WORDS = 13 * 64;
+__host__ __device__ inline int r1w3_word_index(int l, int j) { return j < 12 ? (j >> 2) * 256 + l * 4 + (j & 3) : 768 + l; }
+__host__ __device__ inline int r1w3_slot_pos(int sl) { return 1 + 3 * sl; }
+__host__ __device__ inline int block_words(int role, int w) { return (role == 1 && w == 3) ? R1W3_BLOCK_WORDS : 256 * w; }
 
 // role 0 (staggered): field LSB of code x (0..15) of a run in a two-bit field word, w = 2 or 3
 __host__ __device__ inline int pos2s(int w, int x) {
@@ -171,6 +179,21 @@ __device__ inline u32x4 decode_fields3(uint32_t z, int first, uint32_t hi, int h
     for (int i = 0; i < 4; ++i) {
         const uint32_t lo = (rotr32(z, first + 2 * i - C::POS) & m) | C::MAGIC;
         r[i] = (rotr32(hi, hi_first + i - (C::POS + 2)) & mh) | lo;
+    }
+    return r;
+}
+
+// role 1, 3-bit: the four registers of k-step m of row block nb from the lane's thirteen words (indices fold to
+// constants where nb and m are unrolled).  One rotate (none for the slot that already sits in place) and one and-or each.
+template <bool BF16>
+__device__ __forceinline__ u32x4 decode_r1w3(const uint32_t (&w)[16], int nb, int m) {
+    using C = Codec<3, BF16>;
+    const uint32_t mask = vreg((7u << C::POS) * 0x10001u);
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int P = 16 * nb + 4 * m + i;
+        r[i] = (rotr32(w[P / 5], r1w3_slot_pos(P % 5) - C::POS) & mask) | C::MAGIC;
     }
     return r;
 }
