@@ -19,7 +19,9 @@ loop; with 4 copies 555 MB of other weights pass between two visits of a layer. 
 beside them as `warm`.  `c5-stack-*` runs the stack configuration of the benchmark set: the 26-layer DeepSeek-V2-Lite-
 shaped stack, one step = one pass over all 26 layers (per-layer figures reported).
 
-Prints ONE JSON line.  `value` is tokens/s of the primary workload (default: the
+The LAST stdout line is one compact JSON record (< 4 KB); the full record with every field of every workload
+is written to gpurun_out/bench_full.json (--full-json PATH; --print-full also prints it as an earlier line).
+`value` is tokens/s of the primary workload (default: the
 Qwen3-30B-A3B-shaped layer at decode, 64 tokens); `extras` holds the other decode batch
 sizes, the 4096-token prefill, the other layer shapes of the benchmark set (c1, c4), checkpoint-shaped experts and the
 stack; `roofline` is the dominant kernel of the primary workload
@@ -390,6 +392,50 @@ def cpu_baseline(block, inputs, tokens, budget_s=12.0):
          "output_ok": bool(err <= 1e-2)}
 
 
+COMPACT_LIMIT = 4096     # bytes: the last stdout line must stay below this
+
+
+def _r(v, digits=4):
+    return round(v, digits) if isinstance(v, float) else v
+
+
+def compact_line(full):
+    """The last stdout line: the contract's fields, the roofline and CPU baseline of the primary workload, and
+    per extra workload only {ms_per_step, launch, operator_frac, gateup_frac, down_frac, block_ms}."""
+    roof = full.get("roofline") or {}
+    keep_roof = ("bound", "kernel", "achieved", "peak", "unit", "frac", "traffic", "launch_ms", "weights",
+                 "down_kernel_frac", "operator_frac")
+    cpu = full.get("cpu_baseline")
+    if cpu:
+        cpu = {k: _r(cpu[k], 2) for k in ("value", "unit", "cores", "kind", "sample") if k in cpu}
+    extras = {}
+    for name, r in (full.get("extras") or {}).items():
+        rf = r.get("roofline") or {}
+        extras[name] = {"ms_per_step": _r(r.get("ms_per_step"), 5), "launch": r.get("launch"),
+                        "operator_frac": _r(rf.get("operator_frac")), "gateup_frac": _r(rf.get("frac")),
+                        "down_frac": _r(rf.get("down_kernel_frac")),
+                        "block_ms": _r((r.get("block_scope") or {}).get("ms_per_step"), 5)}
+    cfg = dict(full.get("config") or {})
+    out = {k: full.get(k) for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+                                    "higher_is_better", "scaling", "vs_baseline", "dtype", "data")}
+    out["value"] = _r(out["value"], 1)
+    out["ms_per_step"] = _r(out["ms_per_step"], 6)
+    out["config"] = cfg
+    out["roofline"] = {k: _r(roof[k], 5) for k in keep_roof if k in roof}
+    out["cpu_baseline"] = cpu
+    out["parity"] = full.get("parity")
+    out["block_ms"] = _r((full.get("block_scope") or {}).get("ms_per_step"), 5)
+    out["warm_ms_per_step"] = _r((full.get("warm") or {}).get("ms_per_step"), 6)
+    out["extras"] = extras
+    text = json.dumps(out)
+    if len(text) >= COMPACT_LIMIT:       # never let the tail grow past what is kept: drop the least needed first
+        for victim in ("extras", "parity", "warm_ms_per_step", "block_ms"):
+            out.pop(victim, None)
+            if len(json.dumps(out)) < COMPACT_LIMIT:
+                break
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -403,6 +449,11 @@ def main() -> int:
     ap.add_argument("--no-stack", action="store_true", help="leave the 26-layer c5 stack out of the extras")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only (no HIP graph replay)")
+    ap.add_argument("--full-json", default=None,
+                    help="where the full record is written (default gpurun_out/bench_full.json)")
+    ap.add_argument("--print-full", action="store_true", help="also print the full record as an earlier stdout line")
+    ap.add_argument("--no-warm", action="store_true", help="skip the one-layer (warm) replay of the same workload")
+    ap.add_argument("--no-block", action="store_true", help="skip the block-scope timing")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run 5 plain fp32 copies (torch.mul(src, 1, out=dst)) of this many MiB: the known-size "
                          "kernel that hardware byte counters are scaled by")
@@ -449,11 +500,12 @@ def main() -> int:
         stack = SPECS[skey].n_layers > 1
         if stack:       # one step = one pass over the whole stack
             r, inp = run_workload(blocks, SPECS[skey], toks, max(2, steps // len(blocks)), max(1, warmup // len(blocks)),
-                                  use_graph=use_graph, layers_per_step=len(blocks))
+                                  use_graph=use_graph, layers_per_step=len(blocks), block_scope=not args.no_block)
         else:
-            r, inp = run_workload(blocks, SPECS[skey], toks, steps, warmup, use_graph=use_graph)
+            r, inp = run_workload(blocks, SPECS[skey], toks, steps, warmup, use_graph=use_graph,
+                                  block_scope=not args.no_block)
         r["roofline"] = roofline_of(r, inp, bnd, name)
-        if len(blocks) > 1 and not stack:
+        if len(blocks) > 1 and not stack and not args.no_warm:
             # the same workload replaying ONE layer: weights may stay in the memory-side cache
             w, winp = run_workload(blocks[:1], SPECS[skey], toks, steps, warmup, use_graph=use_graph, block_scope=False)
             r["warm"] = {k: w[k] for k in ("ms_per_step", "tokens_per_s", "launch", "kernel_ms", "gateup_GBps", "down_GBps",
@@ -503,7 +555,18 @@ def main() -> int:
         "algorithmic_flops": res["algorithmic_flops"],
         "roofline": roof, "cpu_baseline": cpu, "parity": parity, "extras": extras,
     }
-    print(json.dumps(line))
+    # The full record (every workload with all its fields) goes to a file and to an EARLIER stdout line; the
+    # LAST line is the compact one, small enough for any harness that keeps only the tail of stdout.
+    full_path = args.full_json or os.path.join(ROOT, "gpurun_out", "bench_full.json")
+    try:
+        os.makedirs(os.path.dirname(full_path), exist_ok=True)
+        with open(full_path, "w") as f:
+            json.dump(line, f, indent=1)
+    except OSError as exc:
+        print(f"bench.py: full record not written ({exc})", file=sys.stderr)
+    if args.print_full:
+        print(json.dumps(line))
+    print(json.dumps(compact_line(line)))
     return 0
 
 

@@ -177,3 +177,52 @@ def test_operators_are_registered_with_the_dispatcher():
     with pytest.raises(NotImplementedError):
         torch.ops.bitsmoe.route(torch.zeros((2, 2), dtype=torch.int64), torch.zeros((2, 2)),
                                 torch.zeros((4,), dtype=torch.int32), 4)
+
+
+def test_bench_last_line_is_compact():
+    """bench.py's LAST stdout line must survive a harness that keeps only a few KB of tail: built here from
+    stub results for the primary workload and ten verbose extras."""
+    import json
+
+    import bench
+
+    verbose = {"ms_per_step": 0.0587123456, "launch": "hipgraph", "tokens_per_s": 1.09e6,
+               "kernel_ms": {k: 0.0123456789 for k in ("prepare", "gate_up", "silu_mul", "down", "combine")},
+               "kernel_ms_events_raw": {k: 0.0123456789 for k in ("prepare", "gate_up", "silu_mul", "down", "combine")},
+               "block_scope": {"ms_per_step": 0.103123, "note": "x" * 200},
+               "warm": {"ms_per_step": 0.048, "kernel_ms": {"gate_up": 0.02}},
+               "roofline": {"bound": "hbm", "kernel": "gate_up", "achieved": 4314.92, "peak": 8000.0, "unit": "GB/s",
+                            "frac": 0.539, "traffic": 124240548, "launch_ms": 0.0282, "weights": "cold",
+                            "down_kernel_frac": 0.33, "operator_frac": 0.389, "all_kernels_GBps": 3400.0,
+                            "algorithmic_bytes_per_launch": 121.7e6, "launch_ms_events_raw": 0.0326}}
+    full = {"metric": "MoE-layer tokens/s", "value": 1090533.7123, "unit": "tokens/s", "n_gpus": 1, "steps": 400,
+            "warmup": 20, "ms_per_step": 0.0586871234, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": "c2-t64: " + bench.WORKLOAD_DESC["c2"] + ", 64 tokens, operator scope "
+                                   "(routing + gate/up + SiLU*mul + down + combine), inputs resident in HBM, "
+                                   "4 distinct layers in rotation (cold weights)",
+                       "tokens": 64, "mean_bits": 2.21875, "active_experts": 125.75, "device": "AMD Instinct MI355X",
+                       "layer_build_s": 1.67, "launch": "eager", "routing": "inside the gate/up and down kernels",
+                       "activation_dtype": "bf16", "arithmetic": "bf16 activations in, f16 MFMA operands, fp32 accumulation"},
+            "roofline": verbose["roofline"],
+            "cpu_baseline": {"value": 474.48, "unit": "tokens/s", "cores": 16, "kind": "port",
+                             "sample": "20 full forwards of the same workload (64 tokens), best of 20, 134.9 ms each; "
+                                       "host has 16 logical CPUs", "note": "y" * 100},
+            "parity": {"routing_bit_exact": True, "output_max_norm_err": 3.5e-4, "output_tolerance": 1e-2, "output_ok": True},
+            "block_scope": verbose["block_scope"], "warm": verbose["warm"],
+            "extras": {name: dict(verbose) for name in bench.WORKLOADS if name != "c2-t64"}}
+    line = bench.compact_line(full)
+    text = json.dumps(line)
+    assert len(text) < bench.COMPACT_LIMIT
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline", "parity", "extras"):
+        assert key in line
+    for key in ("bound", "achieved", "peak", "unit", "frac", "traffic"):
+        assert key in line["roofline"]
+    for key in ("value", "unit", "cores", "kind", "sample"):
+        assert key in line["cpu_baseline"]
+    assert set(line["extras"]) == set(bench.WORKLOADS) - {"c2-t64"}
+    assert set(line["extras"]["c3-t4096"]) == {"ms_per_step", "launch", "operator_frac", "gateup_frac", "down_frac", "block_ms"}
+    # an oversized record still yields a last line under the limit
+    full["extras"] = {f"w{i}": dict(verbose) for i in range(80)}
+    assert len(json.dumps(bench.compact_line(full))) < bench.COMPACT_LIMIT
