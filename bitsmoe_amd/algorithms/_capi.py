@@ -23,6 +23,7 @@ PROFILE_PHASES = 5
 EXPORTED_SYMBOLS = (
     "bitsmoe_last_error",
     "bitsmoe_version",
+    "bitsmoe_set_option",
     "bitsmoe_matset_create",
     "bitsmoe_matset_destroy",
     "bitsmoe_matset_info",
@@ -85,6 +86,8 @@ def load() -> ctypes.CDLL:
     lib.bitsmoe_last_error.argtypes = []
     lib.bitsmoe_version.restype = c_char_p
     lib.bitsmoe_version.argtypes = []
+    lib.bitsmoe_set_option.restype = c_int32
+    lib.bitsmoe_set_option.argtypes = [c_char_p, c_int32]
     lib.bitsmoe_matset_create.restype = c_int32
     lib.bitsmoe_matset_create.argtypes = [POINTER(MatrixDesc), c_int32, c_int32, c_void_p, POINTER(c_void_p)]
     lib.bitsmoe_matset_destroy.restype = None

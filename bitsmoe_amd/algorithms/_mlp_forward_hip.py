@@ -13,6 +13,8 @@ bitsmoe/algorithms/cpp/mlp_forward.cu:2464-2503), `route`, `dequant_matrix`.
 from __future__ import annotations
 
 import ctypes
+import operator
+import os
 from collections import OrderedDict
 from typing import List, Optional, Sequence, Tuple
 
@@ -20,11 +22,16 @@ import torch
 
 from . import _capi
 
-import os
-
 _lib = _capi.load()
 # BITSMOE_NO_PREPARE=1 keeps every matrix set on the generic kernels (no wave-native copy)
 _AUTO_PREPARE = os.environ.get("BITSMOE_NO_PREPARE", "0") != "1"
+
+
+def set_option(name: str, value: int = -1) -> None:
+    """One of the launchers' experiment switches for the whole process ("route_inline", "route_jobs",
+    "decode_fused_z", "decode_split_z", "decode_fused"): 0 / 1, or -1 for the library's own choice.  The
+    library reads the BITSMOE_* environment forms of these once, when it is loaded."""
+    _capi.check(_lib.bitsmoe_set_option(name.encode(), int(value)))
 
 
 def _stream_ptr(device: torch.device) -> int:
@@ -111,6 +118,10 @@ class MatrixSet:
         is a snapshot: validated metadata, prepared payload copy, folded scales)."""
         return self._fingerprint == fingerprint(self._keep)
 
+    def payload_current(self) -> bool:
+        """The cheap form of is_current(): only the payload tensors' version counters are compared."""
+        return self._fingerprint[:self.n_experts] == fingerprint(self._keep[:1])
+
     def refresh(self) -> None:
         """Rebuild the snapshot from the buffers' current contents (same tensors, same role)."""
         role = self.role
@@ -179,43 +190,87 @@ class Profile:
 # prepare() makes a re-laid-out copy of the payload and a folded scale table.  The reference keeps
 # only meta tables per raw pointer and reads the payload live
 # (bitsmoe/algorithms/cpp/mlp_forward.cu:2464-2503, 2608-2619), so a caller of the list signature
-# may overwrite or swap buffers between calls.  The cache key therefore holds the address, size and
-# version counter of EVERY tensor of EVERY expert: a swapped middle expert or an in-place write
-# (`copy_`, `load_state_dict` on a child module) misses the cache and builds a fresh set.
+# may overwrite or swap buffers between calls.  Two levels:
+#   1. the six container objects of a projection are looked up by identity (the block's runtime cache holds
+#      stable tuples, bitsmoe/models/base_block.py:195-214); a hit is confirmed by a cheap staleness token --
+#      mutable containers: every element still the same tensor object; all containers: the version counters
+#      of the PAYLOAD tensors (any reload or re-quantisation writes them) -- about 35 us per call for 3 x 128
+#      experts instead of milliseconds for
+#   2. the full fingerprint: address, size and version counter of EVERY tensor of EVERY expert, taken on a
+#      level-1 miss (new containers, a swapped expert, a payload written in place) and on every call with
+#      BITSMOE_LIST_CACHE_CHECK=full; a fingerprint miss builds a fresh set.
+# BITSMOE_LIST_CACHE_CHECK=identity trusts the containers alone.  Inference tensors carry no version
+# counter: they are keyed by address and size only, and an in-place write to them needs
+# clear_matset_cache() (or MatrixSet.refresh()).
 _SET_CACHE: "OrderedDict[tuple, MatrixSet]" = OrderedDict()
 _SET_CACHE_LIMIT = int(os.environ.get("BITSMOE_SET_CACHE_LIMIT", "384"))     # sets kept (each pins its GPU copy)
+_LIST_CACHE_CHECK = os.environ.get("BITSMOE_LIST_CACHE_CHECK", "payload")
+if _LIST_CACHE_CHECK not in ("payload", "full", "identity"):
+    raise RuntimeError(f"BITSMOE_LIST_CACHE_CHECK={_LIST_CACHE_CHECK!r}: expected payload, full or identity")
+_IDENT_CACHE: "dict[tuple, tuple]" = {}     # ids of the six containers -> (containers, element snapshots, token, set)
+_is = operator.is_
 
 
 def clear_matset_cache() -> None:
     for ms in _SET_CACHE.values():
         ms.close()
     _SET_CACHE.clear()
+    _IDENT_CACHE.clear()
+
+
+def _version(t: torch.Tensor) -> int:
+    """Version counter of a tensor; inference tensors have none (reading it raises)."""
+    return -1 if t.is_inference() else t._version
 
 
 def fingerprint(lists: Sequence[Sequence[torch.Tensor]]) -> tuple:
     """(address, element count, version counter) of every tensor of the six buffer lists."""
-    return tuple((t.data_ptr(), t.numel(), t._version) for seq in lists for t in seq)
+    return tuple((t.data_ptr(), t.numel(), _version(t)) for seq in lists for t in seq)
+
+
+def _payload_token(payload: Sequence[torch.Tensor]) -> tuple:
+    try:
+        return tuple(map(_get_version, payload))
+    except RuntimeError:       # an inference tensor among them
+        return tuple(map(_version, payload))
+
+
+_get_version = operator.attrgetter("_version")
 
 
 def _lookup_set(lists: tuple, intermediate_size: int, name: str) -> MatrixSet:
+    ident = (int(intermediate_size),) + tuple(map(id, lists))
+    hit = _IDENT_CACHE.get(ident) if _LIST_CACHE_CHECK != "full" else None
+    if hit is not None:
+        containers, snaps, token, ms = hit
+        if ms._handle and all(map(_is, containers, lists)) and all(
+                isinstance(cur, tuple) or (len(cur) == len(snap) and all(map(_is, snap, cur)))
+                for snap, cur in zip(snaps, lists)) and (
+                _LIST_CACHE_CHECK == "identity" or token == _payload_token(lists[0])):
+            return ms
+        del _IDENT_CACHE[ident]
     key = (len(lists[0]), int(intermediate_size), fingerprint(lists))
     ms = _SET_CACHE.get(key)
     if ms is not None:
         _SET_CACHE.move_to_end(key)
-        return ms
-    # a set built from the same list objects or the same first payload address whose key no longer
-    # matches is stale (its buffers were overwritten or swapped): release its GPU copy now
-    for old_key, old in list(_SET_CACHE.items()):
-        if all(a is b for a, b in zip(old._keep_lists, lists)) or (
-                len(lists[0]) and old.n_experts and old._keep[0][0].data_ptr() == lists[0][0].data_ptr()):
-            old.close()
-            del _SET_CACHE[old_key]
-    ms = MatrixSet(*lists, intermediate_size=intermediate_size, name=name)
-    ms._keep_lists = lists
-    while len(_SET_CACHE) >= max(_SET_CACHE_LIMIT, 1):
-        _SET_CACHE.popitem(last=False)[1].close()
-    # the set holds the tensors themselves, so no address of the key can be recycled while it lives
-    _SET_CACHE[key] = ms
+    else:
+        # a set built from the same list objects or the same first payload address whose key no longer
+        # matches is stale (its buffers were overwritten or swapped): release its GPU copy now
+        for old_key, old in list(_SET_CACHE.items()):
+            if all(a is b for a, b in zip(old._keep_lists, lists)) or (
+                    len(lists[0]) and old.n_experts and old._keep[0][0].data_ptr() == lists[0][0].data_ptr()):
+                old.close()
+                del _SET_CACHE[old_key]
+        ms = MatrixSet(*lists, intermediate_size=intermediate_size, name=name)
+        ms._keep_lists = lists
+        while len(_SET_CACHE) >= max(_SET_CACHE_LIMIT, 1):
+            _SET_CACHE.popitem(last=False)[1].close()
+        # the set holds the tensors themselves, so no address of the key can be recycled while it lives
+        _SET_CACHE[key] = ms
+    if len(_IDENT_CACHE) >= 4 * max(_SET_CACHE_LIMIT, 1):
+        _IDENT_CACHE.clear()
+    # (the entry holds the containers, so their ids cannot be recycled while it lives)
+    _IDENT_CACHE[ident] = (lists, tuple(tuple(seq) for seq in lists), _payload_token(lists[0]), ms)
     return ms
 
 

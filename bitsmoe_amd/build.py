@@ -1,6 +1,7 @@
 """Builds libbitsmoe_hip.so in-tree with hipcc for gfx950.
 
-    python -m bitsmoe_amd.build            # compile every .hip source and link
+    python -m bitsmoe_amd.build                      # compile every .hip source and link
+    python -m bitsmoe_amd.build forward_decode.hip   # recompile only the named sources, link with the other objects
 
 hipcc cross-compiles without a GPU, so this runs on a CPU-only host.
 """
@@ -40,11 +41,13 @@ def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
 
-def build_library(verbose: bool = True, jobs: int = 8) -> Path:
+def build_library(verbose: bool = True, jobs: int = 8, only: list[str] | None = None) -> Path:
     hipcc = _hipcc()
     objdir = CSRC / "build"
     objdir.mkdir(exist_ok=True)
     srcs = sources()
+    stale = [s for s in srcs if only and s.name not in only and not (objdir / (s.stem + ".o")).exists()]
+    todo = [s for s in srcs if not only or s.name in only or s in stale]
 
     def compile_one(src: Path) -> Path:
         obj = objdir / (src.stem + ".o")
@@ -63,8 +66,9 @@ def build_library(verbose: bool = True, jobs: int = 8) -> Path:
             print(out, flush=True)
         return obj
 
-    with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(srcs)))) as pool:
-        objs = list(pool.map(compile_one, srcs))
+    with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo)))) as pool:
+        list(pool.map(compile_one, todo))
+    objs = [objdir / (s.stem + ".o") for s in srcs]
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *map(str, objs)]
     if verbose:
         print("[bitsmoe build]", " ".join(cmd), flush=True)
@@ -75,6 +79,6 @@ def build_library(verbose: bool = True, jobs: int = 8) -> Path:
 
 
 if __name__ == "__main__":
-    path = build_library()
+    path = build_library(only=sys.argv[1:] or None)
     print(f"built {path}")
     sys.exit(0)

@@ -15,8 +15,9 @@ static constexpr int MAX_DEVICES = 64;
 static void* g_scratch_ptr[MAX_DEVICES] = {};
 static std::mutex g_scratch_mutex;
 
-// The current device's copy of `scratch` (device address), or nullptr with the error set.
-static void* scratch_of_current_device() {
+// The current device's copy of `scratch` (device address), or nullptr with the error set.  Every matrix set
+// creation calls this, so by the time a forward runs the address of its device is cached.
+void* bitsmoe::static_scratch_of_current_device() {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) {
@@ -277,8 +278,7 @@ extern "C" int bitsmoe_moe_forward_routed(const bitsmoe_matset* gate, const bits
     void* route_ws = tail + 2 * align_up((size_t)n_flat * 4, 256) + align_up((size_t)(E + 1) * 4, 256);
     // The grouped-GEMM path's f16 copy of the activations and its per-token tables ride in the routing launches.
     RouteSideJobs jobs;
-    const char* jobs_var = getenv("BITSMOE_ROUTE_JOBS");      // 0: the grouped-GEMM path makes them itself (experiments)
-    const bool carry = !(jobs_var && jobs_var[0] == '0') && shapes_ok && resolve_path(gate, up, down, n_flat, intermediate_size, path) == BITSMOE_PATH_MFMA &&
+    const bool carry = options().route_jobs != 0 && shapes_ok && resolve_path(gate, up, down, n_flat, intermediate_size, path) == BITSMOE_PATH_MFMA &&
                        mfma_front_jobs(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
                                        n_flat, intermediate_size, workspace, &jobs);
     int front_done = 0;
@@ -311,7 +311,7 @@ extern "C" int bitsmoe_moe_forward_static(const bitsmoe_matset* gate, const bits
                   "(use bitsmoe_moe_forward with a caller-owned workspace)", need, (size_t)BITSMOE_STATIC_SCRATCH_BYTES);
         return BITSMOE_E_WORKSPACE;
     }
-    void* ptr = scratch_of_current_device();
+    void* ptr = static_scratch_of_current_device();
     if (!ptr) return BITSMOE_E_HIP;
     // Every path clears what it needs cleared with its own kernels (the array keeps the previous
     // call's contents), so the shared entry point can run on it as on any workspace.

@@ -707,11 +707,9 @@ static bool walk_possible(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
 bool decode_inline_route_ok(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, const void* h_gate,
                             const void* h_up, int Rg, int Ru, int64_t ldg, int64_t ldu, int64_t T, int top_k, int I) {
     const int64_t n_flat = T * top_k;
-    const char* fused_var = getenv("BITSMOE_DECODE_FUSED_Z");
-    const char* inline_var = getenv("BITSMOE_ROUTE_INLINE");       // 0: always build routing tables first (experiments)
-    if (inline_var && inline_var[0] == '0') return false;
+    if (options().route_inline == 0) return false;       // always build routing tables first (experiments)
     if (!(decode_path_supported(gate, up, down, I) && walk_possible(gate, up, h_gate, h_up, Rg, Ru, ldg, ldu) &&
-          !(fused_var && fused_var[0] && atoi(fused_var) > 0) && n_flat > 0 && n_flat <= ROUTE_INLINE_MAX_FLAT &&
+          options().decode_fused_z <= 0 && n_flat > 0 && n_flat <= ROUTE_INLINE_MAX_FLAT &&
           T <= ROUTE_INLINE_MAX_ROWS))
         return false;
     // Where it pays (graph replays, same box, against the routing kernel first).  On the active-expert grid
@@ -751,8 +749,7 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     // Both projections in one workgroup, z = silu(G) * U handed to the down kernel ready-made: when the two
     // matrices of every expert share bit-width and slab count, and (expert, tile) pairs alone fill most of
     // the chip.  BITSMOE_DECODE_FUSED_Z=0 / 1 switches it off / on regardless of the size (experiments).
-    const char* fused_var = getenv("BITSMOE_DECODE_FUSED_Z");      // (read per call: tests switch it)
-    const int fused_env = fused_var && fused_var[0] ? atoi(fused_var) : -1;
+    const int fused_env = options().decode_fused_z;
     const bool fused_possible = walk && gate->all_affine && up->all_affine && gate->prep_max_slabs == up->prep_max_slabs &&
                                 gate->expert_bits == up->expert_bits;
     const bool fused_z = fused_possible && fused_env > 0;
@@ -869,10 +866,9 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     record(prof, 2, st);
     // z formed once by a small launch of its own instead of by every down workgroup: on the chunk grid (full
     // 16-assignment chunks: eight dependent round trips of two rows each in every one of the workgroups that share
-    // a chunk), when the workspace has a free slot behind the partial results.  BITSMOE_DECODE_SPLIT_Z=0 / 1
+    // a chunk), when the workspace has a free slot behind the partial results.  option decode_split_z = 0 / 1
     // switches it off / on wherever it is possible (experiments).
-    const char* split_z_var = getenv("BITSMOE_DECODE_SPLIT_Z");
-    const int split_z_env = split_z_var && split_z_var[0] ? atoi(split_z_var) : -1;
+    const int split_z_env = options().decode_split_z;
     const bool split_z_possible = !fused_z && !routed && (walk ? n_part : 1) < part_capacity && I % 4 == 0;
     const bool split_z = split_z_possible && (split_z_env >= 0 ? split_z_env > 0 : mode == GRID_CHUNKS);
     const int parts_in = walk && !fused_z ? n_part : 1;

@@ -2,6 +2,7 @@
 #include "common.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 
 namespace bitsmoe {
@@ -74,6 +75,37 @@ int launch_fill_zero(float* p, int64_t n, hipStream_t st) {
 using namespace bitsmoe;
 
 extern "C" const char* bitsmoe_last_error(void) { return g_last_error.c_str(); }
+
+namespace bitsmoe {
+static int env_switch(const char* name) {
+    const char* v = getenv(name);
+    return v && v[0] ? atoi(v) : -1;
+}
+Options& options() {
+    static Options o = [] {
+        Options x;
+        x.route_inline = env_switch("BITSMOE_ROUTE_INLINE");
+        x.route_jobs = env_switch("BITSMOE_ROUTE_JOBS");
+        x.decode_fused_z = env_switch("BITSMOE_DECODE_FUSED_Z");
+        x.decode_split_z = env_switch("BITSMOE_DECODE_SPLIT_Z");
+        x.decode_fused = env_switch("BITSMOE_DECODE_FUSED");
+        return x;
+    }();
+    return o;
+}
+}  // namespace bitsmoe
+
+extern "C" int bitsmoe_set_option(const char* name, int32_t value) {
+    BITSMOE_REQUIRE(name != nullptr, "option name must not be null");
+    Options& o = options();
+    const std::string n(name);
+    int* slot = n == "route_inline" ? &o.route_inline : n == "route_jobs" ? &o.route_jobs
+                : n == "decode_fused_z" ? &o.decode_fused_z : n == "decode_split_z" ? &o.decode_split_z
+                : n == "decode_fused" ? &o.decode_fused : nullptr;
+    BITSMOE_REQUIRE(slot != nullptr, "unknown option '%s'", name);
+    *slot = value < 0 ? -1 : (int)value;
+    return BITSMOE_OK;
+}
 extern "C" const char* bitsmoe_version(void) { return "bitsmoe_hip 0.1 (gfx950)"; }
 
 static int validate_matrix(const bitsmoe_matrix_desc& d, int e, int I,
@@ -137,6 +169,9 @@ extern "C" int bitsmoe_matset_create(const bitsmoe_matrix_desc* descs, int32_t n
     set->intermediate_size = intermediate_size;
     set->n_tiles = (intermediate_size + N_TILE - 1) / N_TILE;
     BITSMOE_HIP_TRY(hipGetDevice(&set->device));
+    // the static scratch of this device is located now (a symbol query), so that bitsmoe_moe_forward_static
+    // never has to make one -- its first call may come under stream capture
+    if (static_scratch_of_current_device() == nullptr) return BITSMOE_E_HIP;
     set->descs.assign(descs, descs + n_experts);
     set->slab_meta_host.resize(n_experts);
     set->tile_meta_host.resize(n_experts);

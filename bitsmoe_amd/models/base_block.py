@@ -27,6 +27,11 @@ from bitsmoe_amd.models.base_mlp import buffer_generation
 _BUFFER_NAMES = ("payload", "rank_idx", "tile_meta", "slab_meta", "scale", "s")
 
 
+import os as _os
+
+_CHECK_VERSIONS = _os.environ.get("BITSMOE_BLOCK_CHECK_VERSIONS", "0") == "1"
+
+
 def _dense_via_operator() -> bool:
     """BITSMOE_DENSE_VIA_OPERATOR=1: shared and super experts run as 16-bit packed experts of the operator."""
     import os
@@ -92,7 +97,15 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
                 if current.shape != tensor.shape or current.dtype != tensor.dtype:
                     setattr(self, key, torch.empty_like(tensor))
         super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs)
+        # (the children -- packed containers, dense super / shared experts -- load after this returns; the cache,
+        # the matrix sets and the packed copies of dense experts are rebuilt on the next forward)
         self._invalidate_runtime_cache()
+
+    def _apply(self, fn, *args, **kwargs):
+        # .to() / .half() / .cuda() rebind or rewrite every parameter and buffer below this block
+        out = super()._apply(fn, *args, **kwargs)
+        self._invalidate_runtime_cache()
+        return out
 
     def set_super_expert_projected_weights(self, expert_idx: int, gate_us: torch.Tensor, up_us: torch.Tensor,
                                            down_svh: torch.Tensor) -> None:
@@ -125,7 +138,14 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
     def _ensure_runtime_cache(self, device: torch.device) -> None:
         if self._runtime_cache_ready and self._runtime_cache_device == device:
             if self._buffer_generation_seen == buffer_generation():
-                return
+                # BITSMOE_BLOCK_CHECK_VERSIONS=1: also compare the payload tensors' version counters on every
+                # forward, which catches `expert.gate_payload_buffer.copy_(...)` written past the containers
+                # (about 10 us per 100 experts on the host; off by default -- refresh_packed_weights() is the
+                # explicit form)
+                if not _CHECK_VERSIONS or self._matsets is None or all(ms.payload_current() for ms in self._matsets):
+                    return
+                self._invalidate_runtime_cache()
+                return self._ensure_runtime_cache(device)
             # Some expert container (of this block or another) rebound or reloaded a buffer since the
             # tuples and matrix sets were built.  The sets are snapshots: keep them only if every
             # tensor they were built from is still the bound one and unwritten.
@@ -263,8 +283,12 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
             final_hidden_states.add_(out.to(hidden_states.dtype))
             return
         for expert_idx, layer in self._super_expert_items:
-            weight = (w * (sel == expert_idx).to(w.dtype)).sum(dim=1, keepdim=True)      # 0 where not selected
-            final_hidden_states.add_((layer(hidden_states) * weight).to(hidden_states.dtype))
+            picked = sel == expert_idx
+            weight = (w * picked.to(w.dtype)).sum(dim=1, keepdim=True)      # 0 where not selected
+            # (where, not a bare product: an inf / NaN the expert produces for a token that did NOT select it must
+            # not reach that token's output -- the reference never runs the expert on such a token)
+            out = torch.where(picked.any(dim=1, keepdim=True), layer(hidden_states) * weight, 0)
+            final_hidden_states.add_(out.to(hidden_states.dtype))
 
     # ---- dense experts through the routed-expert operator ----------------------------------
     def _super_global_to_local(self, device: torch.device) -> torch.Tensor:

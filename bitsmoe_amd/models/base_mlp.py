@@ -164,6 +164,11 @@ class BitsMoE_BaseMoeMLP(nn.Module):
         )
         self.skip_expert = not self.is_bitsmoe_packed
 
+    def _apply(self, fn, *args, **kwargs):
+        out = super()._apply(fn, *args, **kwargs)      # (.to() / .cuda(): every buffer is a new tensor afterwards)
+        _BUFFER_GENERATION[0] += 1
+        return out
+
     def forward(self, x: torch.Tensor, h_gate_proj: Optional[torch.Tensor] = None,
                 h_up_proj: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError(

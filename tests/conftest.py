@@ -19,3 +19,19 @@ def cuda_device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def lib_option():
+    """Sets experiment switches of the library for one test and restores the library's own choice afterwards."""
+    from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
+
+    touched = []
+
+    def setter(name, value):
+        hip.set_option(name, value)
+        touched.append(name)
+
+    yield setter
+    for name in touched:
+        hip.set_option(name, -1)

@@ -116,11 +116,11 @@ def test_full_size_from_router_output(cuda_device, key, tokens):
 
 
 @pytest.mark.parametrize("key,tokens", [("c2", 64), ("c1", 16), ("c5", 32)])
-def test_full_size_both_projections_in_one_workgroup(cuda_device, key, tokens, monkeypatch):
-    """The decode path that forms z in the gate/up kernel (BITSMOE_DECODE_FUSED_Z=1) at full size."""
+def test_full_size_both_projections_in_one_workgroup(cuda_device, key, tokens, lib_option):
+    """The decode path that forms z in the gate/up kernel (option decode_fused_z = 1) at full size."""
     from bitsmoe_amd.synth import SPECS
 
-    monkeypatch.setenv("BITSMOE_DECODE_FUSED_Z", "1")
+    lib_option("decode_fused_z", 1)
     err = _check_against_oracle(_layer(key, cuda_device), SPECS[key], tokens, cuda_device, seed=11 + tokens)
     print(f"{key} T={tokens} (z formed by the gate/up kernel): err {err:.2e}")
 

@@ -308,13 +308,13 @@ def test_forward_decode_path_one_width_per_expert(cuda_device, bits):
 
 @pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
 @pytest.mark.parametrize("bits", [2, 3, 4])
-def test_forward_decode_path_both_projections_in_one_workgroup(cuda_device, bits, dtype_name, monkeypatch):
-    """BITSMOE_DECODE_FUSED_Z=1: one workgroup forms gate AND up of a tile and hands z = silu(G) * U to the
+def test_forward_decode_path_both_projections_in_one_workgroup(cuda_device, bits, dtype_name, lib_option):
+    """Option decode_fused_z = 1: one workgroup forms gate AND up of a tile and hands z = silu(G) * U to the
     down kernel as 16-bit operands (plus the row sums of its decode's constant term); 40 tokens over 3
     experts: chunks of 16 assignments and a ragged last chunk."""
     from bitsmoe_amd.algorithms import _capi
 
-    monkeypatch.setenv("BITSMOE_DECODE_FUSED_Z", "1")
+    lib_option("decode_fused_z", 1)
     err = _forward_case(cuda_device, 700 + bits, 3, 40, 2, 1024, 256, 384, dtype_name, (bits,), path=_capi.PATH_DECODE,
                         tol=1e-2, uniform_bits=True)
     assert err < 3e-3
@@ -322,16 +322,13 @@ def test_forward_decode_path_both_projections_in_one_workgroup(cuda_device, bits
 
 @pytest.mark.parametrize("split_z", ["0", "1", None])
 @pytest.mark.parametrize("bits", [(2,), (2, 3, 4)])
-def test_forward_decode_path_z_by_its_own_launch(cuda_device, bits, split_z, monkeypatch):
+def test_forward_decode_path_z_by_its_own_launch(cuda_device, bits, split_z, lib_option):
     """The chunk grid (3 experts, 40 tokens x 2: chunks of 16 assignments and ragged last chunks): z = silu(G) * U
-    formed once by a small launch and copied by the down workgroups (BITSMOE_DECODE_SPLIT_Z=1, the default on this
+    formed once by a small launch and copied by the down workgroups (option decode_split_z = 1, the default on this
     grid) and formed by every down workgroup itself (=0) -- both against the oracle."""
     from bitsmoe_amd.algorithms import _capi
 
-    if split_z is None:
-        monkeypatch.delenv("BITSMOE_DECODE_SPLIT_Z", raising=False)
-    else:
-        monkeypatch.setenv("BITSMOE_DECODE_SPLIT_Z", split_z)
+    lib_option("decode_split_z", -1 if split_z is None else int(split_z))
     err = _forward_case(cuda_device, 740 + len(bits), 3, 40, 2, 1024, 256, 384, "bf16", bits, path=_capi.PATH_DECODE,
                         tol=1e-2, uniform_bits=True)
     assert err < 3e-3

@@ -176,3 +176,46 @@ def test_block_state_dict_round_trip_through_a_checkpoint(cuda_device):
     scale = float(want.abs().max())
     assert float((spoiled - want).abs().max()) > 5e-2 * scale
     assert float((got - want).abs().max()) <= 1e-3 * scale
+
+
+def test_list_signature_identity_fast_path_and_inference_tensors(cuda_device):
+    """Repeated calls with the same containers find their sets by identity (no per-tensor fingerprint), a payload
+    written in place is still seen, and buffers made under inference_mode (no version counter) are accepted."""
+    import torch
+
+    from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
+
+    c = _case(cuda_device, 24)
+    lists = [helpers.to_device_lists(m, cuda_device) for m in (c["gate"], c["up"], c["down"])]
+    flat = [tuple(seq) for six in lists for seq in six]
+    hip.clear_matset_cache()
+    first = hip.moe_packed_forward(*c["dev_in"], *flat, c["rank"], c["dim"], 0).cpu().numpy()
+    assert len(hip._IDENT_CACHE) == 3
+    calls = []
+    real = hip.fingerprint
+    hip.fingerprint = lambda lists_: (calls.append(1), real(lists_))[1]
+    try:
+        again = hip.moe_packed_forward(*c["dev_in"], *flat, c["rank"], c["dim"], 0).cpu().numpy()
+        assert not calls                       # level 1 hit: containers by identity + payload versions
+        rng = np.random.default_rng(96)
+        bits = int(c["down"][1]["slab_meta"][0][0])
+        c["down"][1] = helpers.make_matrix(rng, c["rank"], c["dim"], [(bits, (0, c["rank"]))])
+        fresh = helpers.to_device_lists([c["down"][1]], cuda_device)
+        lists[2][0][1].copy_(fresh[0][0])
+        lists[2][4][1].copy_(fresh[4][0])
+        lists[2][5][1].copy_(fresh[5][0])
+        after = hip.moe_packed_forward(*c["dev_in"], *flat, c["rank"], c["dim"], 0).cpu().numpy()
+        assert calls                           # the down set's token no longer matched
+    finally:
+        hip.fingerprint = real
+    assert helpers.norm_err(again, first) <= 1e-5
+    assert helpers.norm_err(after, _oracle(c)) <= 1e-2
+    with torch.inference_mode():
+        inf = [tuple(tuple(t.clone() for t in seq) for seq in six) for six in lists]
+        flat_inf = [seq for six in inf for seq in six]
+        assert flat_inf[0][0].is_inference()
+        got = hip.moe_packed_forward(*c["dev_in"], *flat_inf, c["rank"], c["dim"], 0).cpu().numpy()
+        got2 = hip.moe_packed_forward(*c["dev_in"], *flat_inf, c["rank"], c["dim"], 0).cpu().numpy()
+    assert helpers.norm_err(got, _oracle(c)) <= 1e-2 and helpers.norm_err(got2, got) <= 1e-5
+    sets = [hip.MatrixSet(*six, intermediate_size=c["dim"]) for six in inf]
+    assert all(s.is_current() for s in sets)

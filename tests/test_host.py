@@ -226,3 +226,13 @@ def test_bench_last_line_is_compact():
     # an oversized record still yields a last line under the limit
     full["extras"] = {f"w{i}": dict(verbose) for i in range(80)}
     assert len(json.dumps(bench.compact_line(full))) < bench.COMPACT_LIMIT
+
+
+def test_set_option_names():
+    from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
+
+    for name in ("route_inline", "route_jobs", "decode_fused_z", "decode_split_z", "decode_fused"):
+        hip.set_option(name, 1)
+        hip.set_option(name, -1)
+    with pytest.raises(RuntimeError, match="unknown option"):
+        hip.set_option("no_such_switch", 1)

@@ -84,3 +84,59 @@ def test_static_scratch_forward_rejects_oversized_call(cuda_device):
     msg = lib.bitsmoe_last_error().decode()
     assert "static scratch" in msg and str(32 << 20) in msg
     torch.cuda.synchronize()
+
+
+def test_static_scratch_forward_under_graph_capture(cuda_device):
+    """The static entry point captured into a HIP graph (its scratch address was located when the matrix sets
+    were created, so nothing but launches happens during capture): two sizes in one graph, the second smaller,
+    replayed three times with eager work between the replays; every replay equals the eager result."""
+    import torch
+
+    from bitsmoe_amd.algorithms import _capi as capi, mlp_forward_cuda as hip
+
+    lib = capi.load()
+    n_experts, top_k, rank, dim = 8, 2, 512, 256
+    gate, up, down = helpers.make_experts(17, n_experts, rank, rank, dim, uniform_bits=True)
+    sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=dim) for m in (gate, up, down)]
+    assert sets[0].prepare(0) and sets[1].prepare(0) and sets[2].prepare(1)
+    handles = [s.handle for s in sets]
+    rng = np.random.default_rng(19)
+    g2l = np.arange(n_experts, dtype=np.int32)
+    cases = []
+    for tokens in (40, 3):
+        h_gate = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(torch.bfloat16).to(cuda_device)
+        h_up = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(torch.bfloat16).to(cuda_device)
+        idx, w = o.router_qwen(rng.normal(size=(tokens, n_experts)).astype(np.float32), top_k)
+        tok, off, rw = (torch.from_numpy(a).to(cuda_device) for a in o.build_routing(idx, w, g2l, n_experts))
+        out = torch.zeros((tokens, rank), dtype=torch.float32, device=cuda_device)
+        cases.append((h_gate, h_up, tok, off, rw, out))
+
+    def run(case, out, stream):
+        h_gate, h_up, tok, off, rw, _ = case
+        capi.check(lib.bitsmoe_moe_forward_static(
+            *handles, h_gate.data_ptr(), h_up.data_ptr(), capi.DT_BF16, int(h_gate.shape[0]), rank, rank,
+            int(h_gate.stride(0)), int(h_up.stride(0)), tok.data_ptr(), off.data_ptr(), rw.data_ptr(), int(tok.numel()),
+            rank, dim, 0, capi.PATH_DECODE, out.data_ptr(), stream))
+
+    eager = []
+    for case in cases:
+        ref = torch.zeros_like(case[5])
+        run(case, ref, int(torch.cuda.current_stream(cuda_device).cuda_stream))
+        eager.append(ref)
+    torch.cuda.synchronize(cuda_device)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        stream = int(torch.cuda.current_stream(cuda_device).cuda_stream)
+        for case in cases:
+            run(case, case[5], stream)
+    for _ in range(3):
+        for case in cases:
+            case[5].fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize(cuda_device)
+        for case, ref in zip(cases, eager):
+            assert helpers.norm_err(case[5].cpu().numpy(), ref.cpu().numpy()) <= 1e-5
+        # eager work of the program's own between the replays, on the same scratch
+        scratch_user = torch.zeros_like(cases[0][5])
+        run(cases[0], scratch_user, int(torch.cuda.current_stream(cuda_device).cuda_stream))
+        torch.cuda.synchronize(cuda_device)
