@@ -235,8 +235,10 @@ def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, l
         "tokens": tokens, "layers_in_rotation": n_layers, "layers_per_step": layers_per_step,
         "ms_per_step": elapsed / steps * 1e3, "ms_per_layer": ms_layer, "tokens_per_s": tokens * steps / elapsed,
         "launch": launch, "eager_ms_per_step": eager / steps * 1e3, "hipgraph_ms_per_step": graph_ms,
-        "routing": "inside the gate/up and down kernels" if hip.routed_is_inline(
+        "routing": "inside the forward's kernels" if hip.routed_is_inline(
             layers[0].h_gate, layers[0].h_up, int(layers[0].selected.shape[1]), *layers[0].sets) else "routing kernel(s) first",
+        # one kernel per (expert, tile) from the activations to the atomic combine (its time is the `gate_up` phase)
+        "fused": hip.decode_is_fused(layers[0].h_gate, layers[0].h_up, int(layers[0].selected.numel()), *layers[0].sets),
         "kernel_ms": {"prepare": ms_fill, "gate_up": ms_gateup, "silu_mul": ms_silu, "down": ms_down,
                       "combine": ms_combine},
         "kernel_ms_events_raw": dict(zip(("prepare", "gate_up", "silu_mul", "down", "combine"), raw)),
@@ -331,6 +333,17 @@ def roofline_of(res, inputs, bound, workload=None):
     roofline, HIP-event duration; `operator_*`: ALL algorithmic bytes / flops of a layer-step against the
     wall clock per layer-step of the timed loop (the figure the 70 % / 40 % layer targets are about)."""
     work = inputs["work"]
+    if bound == "hbm" and res.get("fused"):
+        # the one-kernel forward: ALL the algorithmic bytes of a layer-step move in that kernel
+        ms = res["kernel_ms"]["gate_up"]
+        achieved = work["bytes_total"] / (ms * 1e-3) / 1e9
+        return {"bound": "hbm", "kernel": "fused", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBS, "traffic": counter_traffic(workload, "fused"),
+                "algorithmic_bytes_per_launch": work["bytes_total"], "launch_ms": ms,
+                "launch_ms_events_raw": res["kernel_ms_events_raw"]["gate_up"], "event_gap_ms": res["event_gap_ms"],
+                "weights": "cold" if res["layers_in_rotation"] > 1 else "warm", "down_kernel_frac": None,
+                "all_kernels_GBps": res["kernels_GBps"], "all_kernels_frac": res["kernels_GBps"] / HBM_PEAK_GBS,
+                "operator_GBps": res["operator_GBps"], "operator_frac": res["operator_GBps"] / HBM_PEAK_GBS}
     if bound == "hbm":
         achieved = res["gateup_GBps"]
         return {"bound": "hbm", "kernel": "gate_up", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -454,6 +467,9 @@ def main() -> int:
     ap.add_argument("--print-full", action="store_true", help="also print the full record as an earlier stdout line")
     ap.add_argument("--no-warm", action="store_true", help="skip the one-layer (warm) replay of the same workload")
     ap.add_argument("--no-block", action="store_true", help="skip the block-scope timing")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="a library experiment switch for this run, e.g. decode_fused=0 (bitsmoe_set_option)")
+    ap.add_argument("--only", default=None, help="comma-separated extras to measure (default: all)")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run 5 plain fp32 copies (torch.mul(src, 1, out=dst)) of this many MiB: the known-size "
                          "kernel that hardware byte counters are scaled by")
@@ -472,6 +488,10 @@ def main() -> int:
     if not torch.cuda.is_available():
         raise RuntimeError("bench.py needs a GPU")
     dev = torch.device("cuda:0")
+    from bitsmoe_amd.algorithms import mlp_forward_cuda as _hip
+    for opt in args.option:
+        name, _, value = opt.partition("=")
+        _hip.set_option(name, int(value))
     use_graph = not args.no_graph
     built = {}       # spec key of the layer shape -> its distinct copies (c2 and c3 are one layer shape and seed)
 
@@ -533,6 +553,8 @@ def main() -> int:
         for name, (skey, toks, bnd) in WORKLOADS.items():
             if name == args.workload or (args.no_stack and SPECS[skey].n_layers > 1):
                 continue
+            if args.only is not None and name not in args.only.split(","):
+                continue
             r, _, _ = measure(name, max(5, args.steps // 2), max(2, args.warmup // 2))
             extras[name] = r
     bits = block.expert_bits
@@ -547,7 +569,8 @@ def main() -> int:
                                f"({'cold' if res['layers_in_rotation'] > 1 else 'warm'} weights)",
                    "tokens": tokens, "mean_bits": sum(bits) / len(bits), "active_experts": res["active_experts"],
                    "device": get_cuda_device_name(), "layer_build_s": round(built[shape_key + "/build_s"], 2),
-                   "launch": res["launch"], "routing": res["routing"], "activation_dtype": "bf16",
+                   "launch": res["launch"], "routing": res["routing"], "fused_kernel": bool(res.get("fused")),
+                   "activation_dtype": "bf16",
                    "arithmetic": "bf16 activations in, f16 MFMA operands, fp32 accumulation"},
         "eager_ms_per_step": res["eager_ms_per_step"], "hipgraph_ms_per_step": res["hipgraph_ms_per_step"],
         "block_scope": res.get("block_scope"), "warm": res.get("warm"),

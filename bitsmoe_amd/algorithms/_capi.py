@@ -9,7 +9,12 @@ import ctypes
 from ctypes import POINTER, Structure, c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent.parent / "csrc" / "libbitsmoe_hip.so"
+import os
+
+# BITSMOE_LIB_VARIANT=timeline loads the build with in-kernel time stamps (python -m bitsmoe_amd.build --timeline)
+_VARIANT = os.environ.get("BITSMOE_LIB_VARIANT", "")
+LIB_PATH = Path(__file__).resolve().parent.parent / "csrc" / (
+    f"libbitsmoe_hip_{_VARIANT}.so" if _VARIANT else "libbitsmoe_hip.so")
 
 DT_F16 = 0
 DT_BF16 = 1
@@ -42,6 +47,7 @@ EXPORTED_SYMBOLS = (
     "bitsmoe_forward_routed_workspace_bytes",
     "bitsmoe_moe_forward_routed",
     "bitsmoe_forward_routed_is_inline",
+    "bitsmoe_forward_decode_is_fused",
     "bitsmoe_profile_create",
     "bitsmoe_profile_destroy",
     "bitsmoe_profile_read",
@@ -138,6 +144,9 @@ def load() -> ctypes.CDLL:
     lib.bitsmoe_forward_routed_is_inline.restype = c_int32
     lib.bitsmoe_forward_routed_is_inline.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
                                                      c_int64, c_int64, c_int64, c_int32, c_int32]
+    lib.bitsmoe_forward_decode_is_fused.restype = c_int32
+    lib.bitsmoe_forward_decode_is_fused.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
+                                                    c_int64, c_int64, c_int64, c_int32]
     lib.bitsmoe_moe_forward_routed.restype = c_int32
     lib.bitsmoe_moe_forward_routed.argtypes = [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_int64, c_int64,

@@ -333,6 +333,16 @@ def routed_is_inline(h_gate: torch.Tensor, h_up: torch.Tensor, top_k: int, gate:
         int(h_up.stride(0)) if n_tokens > 1 else int(h_up.shape[1]), n_tokens, int(top_k), int(path)))
 
 
+def decode_is_fused(h_gate: torch.Tensor, h_up: torch.Tensor, n_assign: int, gate: MatrixSet, up: MatrixSet, down: MatrixSet,
+                    path: int = _capi.PATH_AUTO) -> bool:
+    """Would a forward over n_assign assignments run as one kernel per (expert, tile) (no gate/up and down launches)?"""
+    n_tokens = int(h_gate.shape[0])
+    return bool(_lib.bitsmoe_forward_decode_is_fused(
+        gate.handle, up.handle, down.handle, h_gate.data_ptr(), h_up.data_ptr(), int(h_gate.shape[1]), int(h_up.shape[1]),
+        int(h_gate.stride(0)) if n_tokens > 1 else int(h_gate.shape[1]),
+        int(h_up.stride(0)) if n_tokens > 1 else int(h_up.shape[1]), int(n_assign), int(path)))
+
+
 def moe_forward_routed(h_gate: torch.Tensor, h_up: torch.Tensor, selected: torch.Tensor, weights: torch.Tensor,
                        global_to_local: torch.Tensor, local_to_global: torch.Tensor, gate: MatrixSet, up: MatrixSet,
                        down: MatrixSet, rank_out: int, intermediate_size: int, act_type: int = 0,

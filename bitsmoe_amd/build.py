@@ -2,6 +2,8 @@
 
     python -m bitsmoe_amd.build                      # compile every .hip source and link
     python -m bitsmoe_amd.build forward_decode.hip   # recompile only the named sources, link with the other objects
+    python -m bitsmoe_amd.build --timeline           # libbitsmoe_hip_timeline.so: the same library with in-kernel time
+                                                     # stamps (python -m bitsmoe_amd.timeline reads them)
 
 hipcc cross-compiles without a GPU, so this runs on a CPU-only host.
 """
@@ -41,9 +43,11 @@ def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
 
-def build_library(verbose: bool = True, jobs: int = 8, only: list[str] | None = None) -> Path:
+def build_library(verbose: bool = True, jobs: int = 8, only: list[str] | None = None, timeline: bool = False) -> Path:
+    """timeline=True: the variant with in-kernel time stamps (-DBITSMOE_TIMELINE), as libbitsmoe_hip_timeline.so."""
     hipcc = _hipcc()
-    objdir = CSRC / "build"
+    objdir = CSRC / ("build_timeline" if timeline else "build")
+    lib_path = CSRC / ("libbitsmoe_hip_timeline.so" if timeline else LIB_NAME)
     objdir.mkdir(exist_ok=True)
     srcs = sources()
     stale = [s for s in srcs if only and s.name not in only and not (objdir / (s.stem + ".o")).exists()]
@@ -52,6 +56,8 @@ def build_library(verbose: bool = True, jobs: int = 8, only: list[str] | None = 
     def compile_one(src: Path) -> Path:
         obj = objdir / (src.stem + ".o")
         extra = os.environ.get("BITSMOE_HIPCC_EXTRA", "").split()   # e.g. -DNAME for kernel experiments
+        if timeline:
+            extra.append("-DBITSMOE_TIMELINE")
         cmd = [hipcc, *HIPCC_FLAGS, *extra, "-c", str(src), "-o", str(obj)]
         if verbose:
             print("[bitsmoe build]", " ".join(cmd), flush=True)
@@ -69,16 +75,17 @@ def build_library(verbose: bool = True, jobs: int = 8, only: list[str] | None = 
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo)))) as pool:
         list(pool.map(compile_one, todo))
     objs = [objdir / (s.stem + ".o") for s in srcs]
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *map(str, objs)]
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(lib_path), *map(str, objs)]
     if verbose:
         print("[bitsmoe build]", " ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stdout}{res.stderr}")
-    return LIB_PATH
+    return lib_path
 
 
 if __name__ == "__main__":
-    path = build_library(only=sys.argv[1:] or None)
+    args = [a for a in sys.argv[1:] if a != "--timeline"]
+    path = build_library(only=args or None, timeline="--timeline" in sys.argv[1:])
     print(f"built {path}")
     sys.exit(0)

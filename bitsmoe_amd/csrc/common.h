@@ -85,6 +85,17 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
                           int64_t ldu, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
                           int I, float* rank_accum, float* G, float* U, int64_t inter_floats, int part_capacity,
                           const DecodeRouted* routed, bitsmoe_profile* prof, hipStream_t st);
+// The one-kernel decode forward (forward_fused.hip): can it run these sets and activations, and does the
+// launcher choose it for this batch?  launch_forward_decode_fused runs it (rank_accum cleared by a small launch
+// of its own first, then ONE kernel from the activations to the atomics of the combine).
+bool decode_fused_possible(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                           const void* h_gate, const void* h_up, int Rg, int Ru, int64_t ldg, int64_t ldu, int I);
+bool decode_fused_chosen(const bitsmoe_matset* gate, int64_t A, int I);
+int launch_forward_decode_fused(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                                const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg,
+                                int64_t ldu, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
+                                int I, float* rank_accum, const DecodeRouted* routed, bitsmoe_profile* prof, hipStream_t st);
+
 // How many partial results of the two fp32 intermediates the decode path's workspace holds (the gate/up kernel
 // may split its contraction over workgroups when there are few assignments).
 inline int decode_part_capacity(int64_t n_assign) { return n_assign <= 1024 ? 4 : n_assign <= 4096 ? 2 : 1; }

@@ -9,6 +9,10 @@
 
 #include "fast_helpers.h"
 
+#ifndef BITSMOE_TL_DOWN_STAMP
+#define BITSMOE_TL_DOWN_STAMP(i) do {} while (0)      // (time stamps of the timeline build, forward_decode.hip)
+#endif
+
 namespace bitsmoe {
 constexpr int GU_STRIDE = GU_SLABS * SLAB_ROWS + 8;  // 16-bit elements; +8 staggers LDS banks
 constexpr int DN_SLABS_PER_WG = 4;                 // one slab per wavefront
@@ -274,12 +278,15 @@ __device__ __forceinline__ u32x4 scaled_f16x8(u32x4 raw, u32x4 sc) {
 // assignment, whatever its G / U rows hold.
 // `hs_all`: LDS, 2 * MAX_A * GU_STRIDE 16-bit elements; `cterm_lds`: LDS, MAX_A floats.  The caller
 // guarantees that no wavefront still reads either when the item begins (a workgroup barrier).
-template <bool BF16, bool IDENT, int W, bool SPLIT, class AS>
+// KEEP: the tile's sums are not stored; `keep[nbl]` receives them (the lane's rows a = 4*kg + j of column
+// 32*pair + 16*nbl + n), for a caller that goes on with them in registers.
+template <bool BF16, bool IDENT, int W, bool SPLIT, class AS, bool KEEP = false>
 __device__ __forceinline__ void gateup_walk_item(gptr<uint32_t> payload, gptr<__half> scale_s, gptr<int32_t> rank_idx,
                                                  const FastSlab first, const uint16_t* __restrict__ h, int64_t ld,
                                                  const AS& as, int a0, int n_a, int T,
                                                  int I, int n_tiles, int t, int g_begin, int g_end, float* __restrict__ out,
-                                                 uint16_t* __restrict__ hs_all, float* __restrict__ cterm_lds, int tid) {
+                                                 uint16_t* __restrict__ hs_all, float* __restrict__ cterm_lds, int tid,
+                                                 f32x4* __restrict__ keep = nullptr) {
     const int pair = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform
     const int lane = tid & 63;
     const int n = lane & 15, kg = lane >> 4;
@@ -368,6 +375,9 @@ __device__ __forceinline__ void gateup_walk_item(gptr<uint32_t> payload, gptr<__
             raw0 = act_at(0, rank_nxt);
             raw1 = act_at(1, rank_nxt);
         }
+        // (inside the one-kernel forward the scheduler otherwise sinks these two requests behind the payload
+        // requests below -- loads return in order, the next operand would wait for the next group's payload)
+        if constexpr (KEEP) __builtin_amdgcn_sched_barrier(0);
         const uint16_t* ap16 = &hs[n * GU_STRIDE + 16 * kg];
         static_for([&](auto qc) {
             constexpr int q = decltype(qc)::value;
@@ -391,6 +401,11 @@ __device__ __forceinline__ void gateup_walk_item(gptr<uint32_t> payload, gptr<__
 #pragma unroll
     for (int j = 0; j < 4; ++j) corr[j] = cterm_lds[4 * kg + j];
     // remove the constant term; lane holds rows a = 4*kg + j of column 32*pair + 16*nbl + n
+    if constexpr (KEEP) {
+        keep[0] = acc[0] - corr;
+        keep[1] = acc[1] - corr;
+        return;
+    }
 #pragma unroll
     for (int nbl = 0; nbl < 2; ++nbl) {
         const int c = t * N_TILE + 32 * pair + 16 * nbl + n;
@@ -925,6 +940,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
         if constexpr (W != 0) rows[lane] = int2{row_rank, __float_as_int(row_s)};
         if (lane < MAX_A) assigns[lane] = int2{tok_lane, __float_as_int(rw_lane)};
         __syncthreads();
+        if (a0 == a_begin) BITSMOE_TL_DOWN_STAMP(2);
         if constexpr (W == 4) {
             // (16 payload registers per tile: two buffers, one tile ahead)
             for (int i = 0; i < nt; i += 2) {
@@ -949,6 +965,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                 }
             }
         }
+        if (a0 == a_begin) BITSMOE_TL_DOWN_STAMP(3);
         if constexpr (W != 0) {
             // combine: rows of this slab are distinct output ranks; lane holds assignments 4*kg + j
 #pragma unroll
@@ -967,6 +984,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                 }
             }
         }
+        if (a0 == a_begin) BITSMOE_TL_DOWN_STAMP(4);
     }
 }
 

@@ -223,6 +223,20 @@ extern "C" int bitsmoe_forward_routed_is_inline(const bitsmoe_matset* gate, cons
     return decode_inline_route_ok(gate, up, down, h_gate, h_up, rank_gate, rank_up, ld_gate, ld_up, n_tokens, top_k, I) ? 1 : 0;
 }
 
+extern "C" int bitsmoe_forward_decode_is_fused(const bitsmoe_matset* gate, const bitsmoe_matset* up,
+                                              const bitsmoe_matset* down, const void* h_gate, const void* h_up,
+                                              int32_t rank_gate, int32_t rank_up, int64_t ld_gate, int64_t ld_up,
+                                              int64_t n_assign, int32_t path) {
+    if (!gate || !up || !down || n_assign <= 0) return 0;
+    const int I = gate->intermediate_size;
+    if (path != BITSMOE_PATH_AUTO && path != BITSMOE_PATH_DECODE) return 0;
+    if (resolve_path(gate, up, down, n_assign, I, path) != BITSMOE_PATH_DECODE) return 0;
+    return options().decode_fused != 0 && options().decode_fused_z <= 0 &&
+                   decode_fused_possible(gate, up, down, h_gate, h_up, rank_gate, rank_up, ld_gate, ld_up, I) &&
+                   (options().decode_fused > 0 || decode_fused_chosen(gate, n_assign, I))
+               ? 1 : 0;
+}
+
 extern "C" int bitsmoe_moe_forward_routed(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
                                           const void* h_gate, const void* h_up, int32_t act_dtype, int64_t n_tokens,
                                           int32_t rank_gate, int32_t rank_up, int64_t ld_gate, int64_t ld_up,

@@ -21,9 +21,31 @@
 // chain of five), (2) every workgroup keeps the payload of its next step in flight while it
 // computes the current one, (3) requests are ordered by when their data is needed: loads
 // return in order, so a small request behind a large one waits for the large one.
+// ---- optional in-kernel time stamps (builds with -DBITSMOE_TIMELINE only: `python -m bitsmoe_amd.build --timeline`)
+// Thread 0 of every workgroup of k_gateup_walk / k_down_decode writes the 100 MHz wall clock at its phase boundaries
+// (first assignment chunk) into a device array that bitsmoe_timeline_read_decode copies out.
+// gate/up: 0 entry, 1 tables and routed entries at hand, 2 first chunk's tile stored, 6 exit.
+// down:    0 entry, 1 tables and routed entries at hand, 2 z built (barrier passed), 3 tiles multiplied, 4 atomics issued, 6 exit.
+#ifdef BITSMOE_TIMELINE
+#include <hip/hip_runtime.h>
+namespace bitsmoe {
+constexpr int TL_STAMPS = 8;
+constexpr int TL_MAX_WG = 8192;
+__device__ unsigned long long g_tl_walk[TL_MAX_WG * TL_STAMPS];
+__device__ unsigned long long g_tl_down[TL_MAX_WG * TL_STAMPS];
+}  // namespace bitsmoe
+#define BITSMOE_TL(arr, i)                                                          \
+    do {                                                                            \
+        if (threadIdx.x == 0 && blockIdx.x < ::bitsmoe::TL_MAX_WG)                  \
+            ::bitsmoe::arr[blockIdx.x * ::bitsmoe::TL_STAMPS + (i)] = wall_clock64(); \
+    } while (0)
+#define BITSMOE_TL_DOWN_STAMP(i) BITSMOE_TL(g_tl_down, i)
+#else
+#define BITSMOE_TL(arr, i) do {} while (0)
+#endif
 #include "decode_bodies.h"
+#include "decode_launch.h"
 
-#include <atomic>
 #include <cstdlib>
 
 namespace bitsmoe {
@@ -317,6 +339,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const ExpertOrder up_order, const void* __restrict__ selected, int ids_are_i64, int n_flat, int top_k,
     const int32_t* __restrict__ local_to_global, const int32_t* __restrict__ global_to_local, int n_global) {
     static_assert(!ROUTED || MODE != GRID_CHUNKS, "inline routing serves whole experts");
+    BITSMOE_TL(g_tl_walk, 0);
     const int tid = threadIdx.x;
     {   // this workgroup's share of the accumulator (before any exit)
         const int64_t total = (int64_t)gridDim.x * 256;
@@ -384,6 +407,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     }
     if constexpr (ROUTED && MODE == GRID_EXPERTS) a_end = inline_route(selected, ids_are_i64, n_flat, top_k, gid, route_lds, tid);
     if (a_end <= a_begin || first.bits == 0) return;
+    BITSMOE_TL(g_tl_walk, 1);
     const int n_groups = fe.num_slabs / GU_SLABS;
     // this workgroup's share of the slab groups, and the partial result it writes
     const int g_begin = (int)((int64_t)part * n_groups / parts), g_end = (int)((int64_t)(part + 1) * n_groups / parts);
@@ -440,7 +464,9 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
             else if (first.bits == 4)
                 run(std::integral_constant<int, 4>{});
         }
+        if (a0 == a_begin) BITSMOE_TL(g_tl_walk, 2);
     }
+    BITSMOE_TL(g_tl_walk, 6);
 }
 
 // gateup_walk_z_item launched as a grid: grid.x = (expert coordinate) * n_tiles; 256 threads.  One
@@ -568,6 +594,7 @@ __global__ __launch_bounds__(256, ZR > ZROWS ? 3 : 4) void k_down_decode(
     int ids_are_i64, int n_flat, int top_k, const int32_t* __restrict__ local_to_global,
     const float* __restrict__ sel_weights, const int32_t* __restrict__ global_to_local, int n_global) {
     static_assert(!ROUTED || (MODE != GRID_CHUNKS && !ZREADY), "inline routing serves whole experts");
+    BITSMOE_TL(g_tl_down, 0);
     // Workgroup b runs on XCD b % 8, and every XCD has its own L2: the workgroups of one expert coordinate
     // (which all read the same G / U rows) are given ids of one residue class, so that they share one L2;
     // on the active-expert and the chunk grid coordinate c goes to XCD c % 8, so that the coordinates that have
@@ -624,6 +651,7 @@ __global__ __launch_bounds__(256, ZR > ZROWS ? 3 : 4) void k_down_decode(
     if (si < max_slabs) fs = load_fast_slab(down_fs, e * max_slabs + si);
     if constexpr (ROUTED && MODE == GRID_EXPERTS) a_end = inline_route(selected, ids_are_i64, n_flat, top_k, gid, route_lds, tid);
     if (a_end <= a_begin || grp * DN_SLABS_PER_WG >= fe.num_slabs) return;
+    BITSMOE_TL(g_tl_down, 1);
     auto assignments = [&]() {
         if constexpr (ROUTED)
             return AssignInline{route_lds.tok, route_lds.ent, sel_weights, a_end};
@@ -657,6 +685,7 @@ __global__ __launch_bounds__(256, ZR > ZROWS ? 3 : 4) void k_down_decode(
     else
         down_wave<0, ZREADY, ZR>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
+    BITSMOE_TL(g_tl_down, 6);
 }
 
 __global__ void k_fill_zero2(float* __restrict__ p1, int64_t n1, float* __restrict__ p2, int64_t n2) {
@@ -670,19 +699,6 @@ static inline void record(bitsmoe_profile* p, int i, hipStream_t st) {
     if (p) (void)hipEventRecord(p->ev[i], st);
 }
 
-// Compute units of the current device (asked once per device; 256 when the query fails).
-static int cu_count() {
-    static std::atomic<int> cached[64];
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    int n = cached[dev].load(std::memory_order_relaxed);
-    if (n == 0) {
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev].store(n, std::memory_order_relaxed);
-    }
-    return n;
-}
-
 bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I) {
     const int n_tiles = (I + N_TILE - 1) / N_TILE;
     const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4 + DN_SLABS_PER_WG * SLAB_ROWS * 8 + MAX_A * 8;
@@ -690,19 +706,6 @@ bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up,
            I % N_TILE == 0;
 }
 
-static int decode_grid_mode(int64_t A, int E) {
-    const int64_t active_max = std::min<int64_t>(E, A);
-    return (A >= (int64_t)16 * E || (E <= 64 && A >= (int64_t)3 * E)) ? GRID_CHUNKS : active_max * 2 <= E ? GRID_ACTIVE : GRID_EXPERTS;
-}
-static bool walk_possible(const bitsmoe_matset* gate, const bitsmoe_matset* up, const void* h_gate, const void* h_up, int Rg,
-                          int Ru, int64_t ldg, int64_t ldu) {
-    // (its 16-byte activation loads need rank_idx in runs of eight and aligned rows; the ranks that padding rows
-    // read, with zero scales, must be columns of the activations too)
-    auto rows16 = [](const void* p, int64_t ld) { return ((uintptr_t)p & 15) == 0 && ld % 8 == 0; };
-    return gate->role == ROLE_GATE_UP && up->role == ROLE_GATE_UP && gate->rank_chunked8 && up->rank_chunked8 &&
-           rows16(h_gate, ldg) && rows16(h_up, ldu) && gate->pad_rank_plus1 <= Rg && up->pad_rank_plus1 <= Ru &&
-           std::max(gate->prep_max_slabs, up->prep_max_slabs) <= WALK_MAX_GROUPS * GU_SLABS;
-}
 // Can the decode kernels find their assignments among the routed ids themselves (no routing tables)?
 bool decode_inline_route_ok(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, const void* h_gate,
                             const void* h_up, int Rg, int Ru, int64_t ldg, int64_t ldu, int64_t T, int top_k, int I) {
@@ -729,6 +732,13 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
                           const DecodeRouted* routed, bitsmoe_profile* prof, hipStream_t st) {
     const int E = gate->n_experts;
     const int n_tiles = gate->n_tiles;
+    // The whole chain in one kernel per (expert, tile) where the sets allow it (option decode_fused = 0 / 1: never /
+    // wherever possible).
+    if (options().decode_fused != 0 && options().decode_fused_z <= 0 &&
+        decode_fused_possible(gate, up, down, h_gate, h_up, Rg, Ru, ldg, ldu, I) &&
+        (options().decode_fused > 0 || decode_fused_chosen(gate, A, I)))
+        return launch_forward_decode_fused(gate, up, down, h_gate, h_up, act_dtype, T, Rg, Ru, ldg, ldu, tok, off, rw, A, rank_out,
+                                           I, rank_accum, routed, prof, st);
     record(prof, 0, st);
     // What the expert coordinate of the grids counts.  Few assignments: the experts that can be
     // active at most, not all of them.  Sixteen or more assignments per expert on average: most
@@ -940,3 +950,26 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
 
 }  // namespace bitsmoe
 
+#ifdef BITSMOE_TIMELINE
+// which: 0 = k_gateup_walk, 1 = k_down_decode
+extern "C" int bitsmoe_timeline_read_decode(int which, unsigned long long* host, int n_workgroups) {
+    using namespace bitsmoe;
+    if (!host || n_workgroups <= 0 || n_workgroups > TL_MAX_WG || which < 0 || which > 1) return BITSMOE_E_INVALID;
+    BITSMOE_HIP_TRY(hipDeviceSynchronize());
+    const size_t bytes = sizeof(unsigned long long) * TL_STAMPS * n_workgroups;
+    if (which == 0)
+        BITSMOE_HIP_TRY(hipMemcpyFromSymbol(host, HIP_SYMBOL(g_tl_walk), bytes));
+    else
+        BITSMOE_HIP_TRY(hipMemcpyFromSymbol(host, HIP_SYMBOL(g_tl_down), bytes));
+    return BITSMOE_OK;
+}
+extern "C" int bitsmoe_timeline_clear_decode(void) {
+    using namespace bitsmoe;
+    void* p = nullptr;
+    BITSMOE_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_tl_walk)));
+    BITSMOE_HIP_TRY(hipMemset(p, 0, sizeof(unsigned long long) * TL_STAMPS * TL_MAX_WG));
+    BITSMOE_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_tl_down)));
+    BITSMOE_HIP_TRY(hipMemset(p, 0, sizeof(unsigned long long) * TL_STAMPS * TL_MAX_WG));
+    return BITSMOE_OK;
+}
+#endif

@@ -223,6 +223,16 @@ size_t bitsmoe_forward_routed_workspace_bytes(const bitsmoe_matset* gate, const 
 int bitsmoe_forward_routed_is_inline(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
                                      const void* h_gate, const void* h_up, int32_t rank_gate, int32_t rank_up,
                                      int64_t ld_gate, int64_t ld_up, int64_t n_tokens, int32_t top_k, int32_t path);
+
+/*
+ * 1 when a forward of these sets over n_assign assignments would run as ONE kernel per (expert, tile) -- gate, up,
+ * SiLU, down and the atomic combine without intermediates in memory (forward_fused.hip) -- instead of a gate/up
+ * and a down launch; 0 otherwise.  No reference counterpart (the reference always launches both:
+ * bitsmoe/algorithms/cpp/mlp_forward.cu:2967-2991).  For callers that attribute time to kernels.
+ */
+int bitsmoe_forward_decode_is_fused(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                                    const void* h_gate, const void* h_up, int32_t rank_gate, int32_t rank_up,
+                                    int64_t ld_gate, int64_t ld_up, int64_t n_assign, int32_t path);
 int bitsmoe_moe_forward_routed(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
                                const void* h_gate, const void* h_up, int32_t act_dtype, int64_t n_tokens,
                                int32_t rank_gate, int32_t rank_up, int64_t ld_gate, int64_t ld_up,

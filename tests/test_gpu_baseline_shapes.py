@@ -125,6 +125,30 @@ def test_full_size_both_projections_in_one_workgroup(cuda_device, key, tokens, l
     print(f"{key} T={tokens} (z formed by the gate/up kernel): err {err:.2e}")
 
 
+@pytest.mark.parametrize("key,tokens", [("c2", 64), ("c2", 8), ("c1", 16), ("c4", 256), ("c5", 32)])
+def test_full_size_one_kernel_forward(cuda_device, key, tokens, lib_option):
+    """The one-kernel decode forward (option decode_fused = 1) at full size against the C oracle."""
+    from bitsmoe_amd.synth import SPECS
+
+    from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
+
+    lib_option("decode_fused", 1)
+    block, spec = _layer(key, cuda_device), SPECS[key]
+    err = _check_against_oracle(block, spec, tokens, cuda_device, seed=13 + tokens)
+    # ... and from the router's output (routing inside the kernel where the launcher chooses that)
+    h_gate, h_up, selected, weights = _inputs(block, spec, tokens, 19 + tokens, cuda_device)
+    tok, off, rw, _ = _run(block, h_gate, h_up, selected, weights)
+    gate, up, down = block._ensure_matsets()
+    assert hip.decode_is_fused(h_gate, h_up, int(selected.numel()), gate, up, down)
+    got = hip.moe_forward_routed(h_gate, h_up, selected, weights, block._packed_global_to_local,
+                                 block._packed_local_to_global, gate, up, down, int(block.shared_u_down.shape[1]),
+                                 int(block._packed_intermediate_size), 0).cpu().numpy()
+    ref = _oracle(block, h_gate, h_up, *(t.cpu().numpy() for t in (tok, off, rw)))
+    err_routed = float(np.abs(got - ref).max()) / float(np.abs(ref).max())
+    assert err_routed <= 1e-2
+    print(f"{key} T={tokens} (one kernel per expert and tile): err {err:.2e}, from the router's output {err_routed:.2e}")
+
+
 def test_full_size_paths_agree(cuda_device):
     """Generic (fp32), decode and grouped-GEMM kernels on one C2 batch: same result within the
     operand rounding of the fast paths."""

@@ -70,7 +70,7 @@ def test_routing_tables_bit_exact(cuda_device, tokens, top_k, n_global, n_super,
 
 
 def _forward_case(cuda_device, seed, n_experts, tokens, top_k, rank_in, rank_out, dim, dtype_name, choices,
-                  path=None, tol=1e-2, uniform_bits=False, slab_multiple=None, scramble_ranks=False):
+                  path=None, tol=1e-2, uniform_bits=False, slab_multiple=None, scramble_ranks=False, expect_fused=None):
     import torch
 
     hip = _hip()
@@ -95,6 +95,8 @@ def _forward_case(cuda_device, seed, n_experts, tokens, top_k, rank_in, rank_out
     got = out.cpu().numpy()
     err = helpers.norm_err(got, ref)
     assert err <= tol, f"normalised error {err:.3e} > {tol}"
+    if expect_fused is not None:      # (asked after the forward: the sets are prepared by then)
+        assert hip.decode_is_fused(h_gate.to(cuda_device), h_up.to(cuda_device), int(tok.size), *sets, **kwargs) == expect_fused
     return err
 
 
@@ -317,6 +319,23 @@ def test_forward_decode_path_both_projections_in_one_workgroup(cuda_device, bits
     lib_option("decode_fused_z", 1)
     err = _forward_case(cuda_device, 700 + bits, 3, 40, 2, 1024, 256, 384, dtype_name, (bits,), path=_capi.PATH_DECODE,
                         tol=1e-2, uniform_bits=True)
+    assert err < 3e-3
+
+
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+@pytest.mark.parametrize("choices", [(2,), (3,), (4,), (2, 3, 4)])
+@pytest.mark.parametrize("grid", ["experts", "active", "chunks"])
+def test_forward_decode_path_one_kernel(cuda_device, grid, choices, dtype_name, lib_option):
+    """Option decode_fused = 1: gate, up, SiLU, down and the combine of one (expert, tile) in ONE workgroup, no
+    intermediates in memory.  One width for all three matrices of an expert (the single walk with the down blocks
+    requested from its tail) and three independently drawn widths (the projections walked one after the other);
+    the three meanings of the grid's expert coordinate; chunks of 16 assignments with a ragged last one."""
+    from bitsmoe_amd.algorithms import _capi
+
+    lib_option("decode_fused", 1)
+    n_experts, tokens, top_k = {"experts": (8, 6, 2), "active": (16, 3, 2), "chunks": (3, 40, 2)}[grid]
+    err = _forward_case(cuda_device, 800 + 10 * len(choices) + choices[0], n_experts, tokens, top_k, 1024, 320, 384, dtype_name,
+                        choices, path=_capi.PATH_DECODE, tol=1e-2, uniform_bits=True, expect_fused=True)
     assert err < 3e-3
 
 
