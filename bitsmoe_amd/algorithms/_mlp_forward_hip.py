@@ -29,7 +29,7 @@ _AUTO_PREPARE = os.environ.get("BITSMOE_NO_PREPARE", "0") != "1"
 
 def set_option(name: str, value: int = -1) -> None:
     """One of the launchers' experiment switches for the whole process ("route_inline", "route_jobs",
-    "decode_fused_z", "decode_split_z", "decode_fused"): 0 / 1, or -1 for the library's own choice.  The
+    "decode_fused_z", "decode_split_z", "decode_fused", "prefill_split"): 0 / 1, or -1 for the library's own choice.  The
     library reads the BITSMOE_* environment forms of these once, when it is loaded."""
     _capi.check(_lib.bitsmoe_set_option(name.encode(), int(value)))
 

@@ -221,13 +221,14 @@ int hip_fail(hipError_t e, const char* what);
 
 // Experiment switches of the launchers (-1: the library's own choice).  Read from the environment ONCE, when
 // the library is loaded (BITSMOE_ROUTE_INLINE, BITSMOE_ROUTE_JOBS, BITSMOE_DECODE_FUSED_Z, BITSMOE_DECODE_SPLIT_Z,
-// BITSMOE_DECODE_FUSED); afterwards only bitsmoe_set_option changes them.  No launch path reads the environment.
+// BITSMOE_DECODE_FUSED, BITSMOE_PREFILL_SPLIT); afterwards only bitsmoe_set_option changes them.  No launch path reads the environment.
 struct Options {
     int route_inline = -1;      // 0: routing kernel first even where the decode kernels could route themselves
     int route_jobs = -1;        // 0: the grouped-GEMM front end by launches of its own
     int decode_fused_z = -1;    // 1: the decode gate/up kernel forms z itself
     int decode_split_z = -1;    // 0 / 1: z by the down workgroups / by a launch of its own wherever possible
     int decode_fused = -1;      // 0 / 1: never / wherever possible the one-kernel decode forward
+    int prefill_split = -1;     // 1: gate and up as two launches, SiLU in the second's epilogue (default: one launch and a SiLU pass)
 };
 Options& options();
 

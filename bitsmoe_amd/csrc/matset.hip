@@ -89,6 +89,7 @@ Options& options() {
         x.decode_fused_z = env_switch("BITSMOE_DECODE_FUSED_Z");
         x.decode_split_z = env_switch("BITSMOE_DECODE_SPLIT_Z");
         x.decode_fused = env_switch("BITSMOE_DECODE_FUSED");
+        x.prefill_split = env_switch("BITSMOE_PREFILL_SPLIT");
         return x;
     }();
     return o;
@@ -101,7 +102,7 @@ extern "C" int bitsmoe_set_option(const char* name, int32_t value) {
     const std::string n(name);
     int* slot = n == "route_inline" ? &o.route_inline : n == "route_jobs" ? &o.route_jobs
                 : n == "decode_fused_z" ? &o.decode_fused_z : n == "decode_split_z" ? &o.decode_split_z
-                : n == "decode_fused" ? &o.decode_fused : nullptr;
+                : n == "decode_fused" ? &o.decode_fused : n == "prefill_split" ? &o.prefill_split : nullptr;
     BITSMOE_REQUIRE(slot != nullptr, "unknown option '%s'", name);
     *slot = value < 0 ? -1 : (int)value;
     return BITSMOE_OK;

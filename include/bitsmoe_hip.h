@@ -266,9 +266,9 @@ int bitsmoe_moe_forward_static(const bitsmoe_matset* gate, const bitsmoe_matset*
 /*
  * Experiment switches of the launchers (no reference counterpart).  Each is read from the environment once,
  * when the library is loaded (BITSMOE_ROUTE_INLINE, BITSMOE_ROUTE_JOBS, BITSMOE_DECODE_FUSED_Z,
- * BITSMOE_DECODE_SPLIT_Z, BITSMOE_DECODE_FUSED); no launch path reads the environment.  bitsmoe_set_option changes
- * one for the whole process: name = "route_inline" | "route_jobs" | "decode_fused_z" | "decode_split_z" |
- * "decode_fused", value 0 / 1, or -1 for the library's own choice.  Not synchronised with forwards that run on
+ * BITSMOE_DECODE_SPLIT_Z, BITSMOE_DECODE_FUSED, BITSMOE_PREFILL_SPLIT); no launch path reads the environment.
+ * bitsmoe_set_option changes one for the whole process: name = "route_inline" | "route_jobs" | "decode_fused_z" |
+ * "decode_split_z" | "decode_fused" | "prefill_split", value 0 / 1, or -1 for the library's own choice.  Not synchronised with forwards that run on
  * other threads at the same time.
  */
 int bitsmoe_set_option(const char* name, int32_t value);

@@ -289,6 +289,20 @@ def test_forward_mfma_path_one_width_per_expert(cuda_device, bits, slabs, tokens
         assert err < 3e-3
 
 
+@pytest.mark.parametrize("split", [0, 1])
+def test_forward_mfma_path_silu_pass_or_up_epilogue(cuda_device, split, lib_option):
+    """Option prefill_split: 0 (default) one launch for both projections and a SiLU pass behind it; 1 gate and up as two
+    launches, z = silu(gate) * up stored by the up launch's epilogue over the gate sums.  Ragged tiles, two
+    widths-per-expert layouts (LDS-direct bodies and the register-staged one)."""
+    from bitsmoe_amd.algorithms import _capi
+
+    lib_option("prefill_split", split)
+    for uniform in (True, False):
+        err = _forward_case(cuda_device, 900 + split, 4, 300, 2, 256, 128, 384, "bf16", (2, 3, 4), path=_capi.PATH_MFMA,
+                            tol=1e-2, uniform_bits=uniform, slab_multiple=None if uniform else 64)
+        assert err < 3e-3
+
+
 def test_forward_mfma_path_more_slabs_than_the_slab_tables_hold(cuda_device):
     """65 slabs of one width: past the per-slab tables of the LDS-direct body, the register-staged body runs."""
     from bitsmoe_amd.algorithms import _capi
