@@ -5,6 +5,7 @@
 #include <atomic>
 
 #include "decode_bodies.h"
+#include "launch_policy.h"
 
 namespace bitsmoe {
 
@@ -23,7 +24,10 @@ inline int cu_count() {
 
 inline int decode_grid_mode(int64_t A, int E) {
     const int64_t active_max = std::min<int64_t>(E, A);
-    return (A >= (int64_t)16 * E || (E <= 64 && A >= (int64_t)3 * E)) ? GRID_CHUNKS : active_max * 2 <= E ? GRID_ACTIVE : GRID_EXPERTS;
+    return (A >= (int64_t)policy::CHUNK_GRID_MIN_ASSIGN_PER_EXPERT * E ||
+            (E <= policy::CHUNK_GRID_SMALL_LAYER && A >= (int64_t)policy::CHUNK_GRID_SMALL_LAYER_MIN_ASSIGN_PER_EXPERT * E))
+               ? GRID_CHUNKS
+               : active_max * 2 <= E ? GRID_ACTIVE : GRID_EXPERTS;
 }
 inline bool walk_possible(const bitsmoe_matset* gate, const bitsmoe_matset* up, const void* h_gate, const void* h_up, int Rg,
                           int Ru, int64_t ldg, int64_t ldu) {

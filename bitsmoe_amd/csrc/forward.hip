@@ -1,6 +1,7 @@
 // C-ABI entry point of the routed-expert forward: argument checks, workspace carving and
 // kernel-path selection.
 #include "common.h"
+#include "launch_policy.h"
 
 using namespace bitsmoe;
 
@@ -74,7 +75,7 @@ static int resolve_path(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     // grouped GEMM from 14 assignments per expert on average (measured crossovers on layers of 64,
     // 128 and 512 experts: 12 to 16; the decode kernels re-stream the payload for every 16
     // assignments, the grouped GEMM pays for a longer launch chain)
-    if (mfma_ok && n_assign >= (int64_t)14 * gate->n_experts) return BITSMOE_PATH_MFMA;
+    if (mfma_ok && n_assign >= (int64_t)policy::MFMA_MIN_ASSIGN_PER_EXPERT * gate->n_experts) return BITSMOE_PATH_MFMA;
     if (decode_ok) return BITSMOE_PATH_DECODE;
     if (mfma_ok) return BITSMOE_PATH_MFMA;      // (an intermediate size beyond the decode kernels' LDS budget)
     return BITSMOE_PATH_GENERIC;

@@ -722,7 +722,8 @@ bool decode_inline_route_ok(const bitsmoe_matset* gate, const bitsmoe_matset* up
     // tiles (more workgroups per expert) and on a 512-expert layer.  The chunk grid keeps its tables.
     const int mode = decode_grid_mode(n_flat, gate->n_experts);
     if (mode == GRID_ACTIVE) return true;
-    return mode == GRID_EXPERTS && n_flat >= 2 * (int64_t)gate->n_experts && gate->n_experts <= 256 && gate->n_tiles <= 8;
+    return mode == GRID_EXPERTS && n_flat >= policy::INLINE_ROUTE_MIN_ENTRIES_PER_EXPERT * (int64_t)gate->n_experts &&
+           gate->n_experts <= policy::INLINE_ROUTE_MAX_EXPERTS && gate->n_tiles <= policy::INLINE_ROUTE_MAX_TILES;
 }
 
 int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
@@ -777,7 +778,8 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     // Tiles per workgroup: long runs amortise the start-up round trips, but the grid must
     // still hold a few workgroups per CU (two rounds of three per CU measured best).
     int tiles_per_wg = n_tiles;
-    while (tiles_per_wg > 1 && units * 2 * gu_groups * ((n_tiles + tiles_per_wg - 1) / tiles_per_wg) < 1536)
+    while (tiles_per_wg > 1 &&
+           units * 2 * gu_groups * ((n_tiles + tiles_per_wg - 1) / tiles_per_wg) < policy::GATEUP_DECODE_MIN_WORKGROUPS)
         tiles_per_wg = (tiles_per_wg + 1) / 2;
     const int n_tchunks = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
     dim3 grid((unsigned)(e_dim * gu_groups * n_tchunks), 2);
@@ -899,7 +901,8 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     int dn_tiles_per_wg = n_tiles;
     // (600 measured best on the 26-layer stack at 32 tokens against 300, 1200 and 2400: the kernel is bound by the
     // instructions a workgroup issues, and more, shorter workgroups add their fixed part)
-    while (dn_tiles_per_wg > 1 && units * dn_groups * ((n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg) < 600)
+    while (dn_tiles_per_wg > 1 &&
+           units * dn_groups * ((n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg) < policy::DOWN_DECODE_MIN_WORKGROUPS)
         dn_tiles_per_wg = (dn_tiles_per_wg + 1) / 2;
     const size_t z_bytes = (size_t)MAX_A * (dn_tiles_per_wg * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4 + DN_SLABS_PER_WG * SLAB_ROWS * 8 + MAX_A * 8;
     const int dn_tchunks = (n_tiles + dn_tiles_per_wg - 1) / dn_tiles_per_wg;

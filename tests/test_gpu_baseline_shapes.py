@@ -253,3 +253,38 @@ def test_walking_gateup_popular_expert_and_offset_rows(cuda_device, dtype_name):
     out2 = hip.moe_forward_sets(hg, hu, tok, off, rw, gate, up, down, int(block.shared_u_down.shape[1]),
                                 int(block._packed_intermediate_size), 0)
     assert float((out2 - out).abs().max()) <= 2e-3 * float(out.abs().max())
+
+
+@pytest.mark.parametrize("inter", [256, 640, 1152])
+@pytest.mark.parametrize("n_experts", [48, 96, 160, 384])
+def test_sweep_across_launcher_thresholds(cuda_device, n_experts, inter):
+    """Parity on shapes NEXT to the ones the launchers' constants were measured on: layers of 48 / 96 / 160 / 384
+    experts (both sides of the 64-expert rule of the chunk grid and of the 256-expert rule of inline routing), 2 / 5 / 9
+    column tiles (both sides of the 8-tile rule), and per layer 1, 2, 3, 13, 15 and 17 assignments per expert on average
+    -- the active-expert / expert / chunk grid boundaries, the inline-routing boundary at two entries per expert and
+    the grouped-GEMM crossover at 14 -- from the router's output (one call) and through routing tables (two calls),
+    both against the C oracle.  Stops at the first failing case and names it."""
+    import torch
+
+    from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
+    from bitsmoe_amd.synth import LayerSpec, make_layer
+
+    spec = LayerSpec(f"sweep-{n_experts}-{inter}", "qwen3moe", n_experts, 2, 512, inter, (0.6, 0.25, 0.15), "normal", True, 0)
+    block = make_layer(spec, device=cuda_device, dtype=torch.bfloat16, seed=70 + n_experts)
+    block._ensure_runtime_cache(cuda_device)
+    gate, up, down = block._ensure_matsets()
+    rank_out, isz = int(block.shared_u_down.shape[1]), int(block._packed_intermediate_size)
+    for per_expert in (1, 2, 3, 13, 15, 17):
+        tokens = max(1, per_expert * n_experts // spec.top_k)
+        case = f"E={n_experts} I={inter} assignments/expert={per_expert} tokens={tokens}"
+        print(case, flush=True)
+        h_gate, h_up, selected, weights = _inputs(block, spec, tokens, 100 + per_expert, cuda_device)
+        tok, off, rw, two_calls = _run(block, h_gate, h_up, selected, weights)
+        ref = _oracle(block, h_gate, h_up, *(t.cpu().numpy() for t in (tok, off, rw)))
+        scale = float(np.abs(ref).max())
+        err = float(np.abs(two_calls.cpu().numpy() - ref).max()) / scale
+        assert err <= 1e-2, f"{case}: routing tables first, normalised error {err:.3e}"
+        one_call = hip.moe_forward_routed(h_gate, h_up, selected, weights, block._packed_global_to_local,
+                                          block._packed_local_to_global, gate, up, down, rank_out, isz, 0)
+        err = float(np.abs(one_call.cpu().numpy() - ref).max()) / scale
+        assert err <= 1e-2, f"{case}: from the router's output, normalised error {err:.3e}"
