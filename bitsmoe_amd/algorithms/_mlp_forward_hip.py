@@ -527,25 +527,57 @@ def pack_slabs(levels: torch.Tensor, scale: torch.Tensor, dim: int, bits: int) -
 
 
 def router_softmax_topk(router_logits: torch.Tensor, top_k: int, renormalize: bool = True,
-                        round_dtype: Optional[torch.dtype] = None) -> Tuple[torch.Tensor, torch.Tensor]:
-    """softmax (fp32) -> top-k -> optional renormalisation -> optional round trip through
-    `round_dtype`, in one kernel.  Returns (selected int64 [T, k], weights fp32 [T, k])."""
+                        round_dtype: Optional[torch.dtype] = None, weight_scale: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """softmax (fp32) -> top-k -> optional renormalisation -> * weight_scale -> optional round trip through
+    `round_dtype`, in one kernel.  The logits may be a column range of a wider row-major tensor (unit column
+    stride).  Returns (selected int64 [T, k], weights fp32 [T, k])."""
     _check(router_logits.dim() == 2, "router_logits must be [tokens, experts]")
     _check(router_logits.is_cuda, "router_logits must be CUDA tensor")
     _check(router_logits.dtype in (torch.float16, torch.bfloat16, torch.float32), "router_logits must be a float tensor")
     _check(round_dtype in (None, torch.float16, torch.bfloat16), "round_dtype must be None, float16 or bfloat16")
     dev = router_logits.device
-    logits = router_logits.contiguous()
+    logits = router_logits if router_logits.stride(1) == 1 else router_logits.contiguous()
     t, e = int(logits.shape[0]), int(logits.shape[1])
+    ld = int(logits.stride(0)) if t > 1 else e
     selected = torch.empty((t, int(top_k)), dtype=torch.int64, device=dev)
     weights = torch.empty((t, int(top_k)), dtype=torch.float32, device=dev)
     codes = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}
     with torch.cuda.device(dev):
-        _capi.check(_lib.bitsmoe_router_softmax_topk(
-            logits.data_ptr(), codes[logits.dtype], t, e, int(top_k), 1 if renormalize else 0,
+        _capi.check(_lib.bitsmoe_router_softmax_topk_strided(
+            logits.data_ptr(), codes[logits.dtype], ld, t, e, int(top_k), 1 if renormalize else 0, float(weight_scale),
             -1 if round_dtype is None else codes[round_dtype], selected.data_ptr(), 1, weights.data_ptr(),
             _stream_ptr(dev)))
     return selected, weights
+
+
+def block_finish(rank_accum: torch.Tensor, dtype: torch.dtype, shared_gate_out: Optional[torch.Tensor] = None,
+                 shared_up_out: Optional[torch.Tensor] = None, shared_gate_logit: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[T, rank_out + I_sh] in `dtype`: rank_accum cast, beside it silu(gate_out) * up_out (* sigmoid(gate_logit)) of an
+    always-on shared expert -- the operand of the block's single output GEMM.  gate_out / up_out [T, I_sh] may be
+    column ranges of one wider tensor (same row stride), gate_logit [T, 1] likewise."""
+    _check(rank_accum.dtype == torch.float32 and rank_accum.is_contiguous(), "rank_accum must be contiguous float32")
+    _check(dtype in (torch.float16, torch.bfloat16), "dtype must be float16 or bfloat16")
+    t, r = int(rank_accum.shape[0]), int(rank_accum.shape[1])
+    i_sh = 0 if shared_gate_out is None else int(shared_gate_out.shape[1])
+    dev = rank_accum.device
+    out = torch.empty((t, r + i_sh), dtype=dtype, device=dev)
+    ld_sh = ld_g = 0
+    if i_sh:
+        _check(shared_up_out is not None and shared_up_out.shape == shared_gate_out.shape and shared_gate_out.dtype == dtype
+               and shared_up_out.dtype == dtype and shared_gate_out.stride(1) == 1 and shared_up_out.stride(1) == 1,
+               "shared_gate_out / shared_up_out must be [T, I_sh] of the activation dtype with unit column stride")
+        ld_sh = int(shared_gate_out.stride(0)) if t > 1 else i_sh
+        _check(t <= 1 or int(shared_up_out.stride(0)) == ld_sh, "shared_gate_out / shared_up_out must share their row stride")
+        if shared_gate_logit is not None:
+            _check(shared_gate_logit.dtype == dtype and shared_gate_logit.shape[0] == t, "shared_gate_logit must be [T, 1]")
+            ld_g = int(shared_gate_logit.stride(0)) if t > 1 else 1
+    with torch.cuda.device(dev):
+        _capi.check(_lib.bitsmoe_block_finish(
+            rank_accum.data_ptr(), t, r, shared_gate_out.data_ptr() if i_sh else None,
+            shared_up_out.data_ptr() if i_sh else None, ld_sh, i_sh,
+            shared_gate_logit.data_ptr() if (i_sh and shared_gate_logit is not None) else None, ld_g,
+            _capi.DT_F16 if dtype == torch.float16 else _capi.DT_BF16, out.data_ptr(), r + i_sh, _stream_ptr(dev)))
+    return out
 
 
 # ----------------------------------------------------------------------------------------
@@ -558,8 +590,8 @@ _OPS.define("moe_packed_forward(Tensor h_gate, Tensor h_up, Tensor token_indices
             f"Tensor route_weights, {_MATRIX_ARGS}, int rank_out, int intermediate_size, int act_type) -> Tensor")
 _OPS.define("route(Tensor selected_experts, Tensor route_weights, Tensor global_to_local, int n_packed) "
             "-> (Tensor, Tensor, Tensor)")
-_OPS.define("router_softmax_topk(Tensor router_logits, int top_k, bool renormalize=True, ScalarType? round_dtype=None) "
-            "-> (Tensor, Tensor)")
+_OPS.define("router_softmax_topk(Tensor router_logits, int top_k, bool renormalize=True, ScalarType? round_dtype=None, "
+            "float weight_scale=1.0) -> (Tensor, Tensor)")
 # only an accelerator implementation exists: on other devices the dispatcher raises
 _OPS.impl("moe_packed_forward", moe_packed_forward, "CUDA")
 _OPS.impl("route", route, "CUDA")
@@ -580,7 +612,7 @@ def _route_fake(selected_experts, route_weights, global_to_local, n_packed):
 
 
 @torch.library.register_fake("bitsmoe::router_softmax_topk")
-def _router_fake(router_logits, top_k, renormalize=True, round_dtype=None):
+def _router_fake(router_logits, top_k, renormalize=True, round_dtype=None, weight_scale=1.0):
     t = router_logits.shape[0]
     return (router_logits.new_empty((t, int(top_k)), dtype=torch.int64),
             router_logits.new_empty((t, int(top_k)), dtype=torch.float32))

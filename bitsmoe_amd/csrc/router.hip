@@ -6,6 +6,8 @@
 // One wavefront per token; a lane holds the logits of experts lane, lane + 64, ...
 #include "common.h"
 
+#include <algorithm>
+
 namespace bitsmoe {
 
 constexpr int ROUTER_MAX_PER_LANE = 16;   // experts <= 1024
@@ -29,7 +31,8 @@ __device__ inline float wave_sum(float v) {
 
 // grid = ceil(T / 4), 256 threads (four tokens per workgroup)
 template <int DT>
-__global__ __launch_bounds__(256) void k_router_softmax_topk(const void* __restrict__ logits, int T, int E, int k,
+__global__ __launch_bounds__(256) void k_router_softmax_topk(const void* __restrict__ logits, int64_t ld, float wscale,
+                                                             int T, int E, int k,
                                                              int renorm, int round_dt, int32_t* __restrict__ sel32,
                                                              int64_t* __restrict__ sel64, float* __restrict__ weights) {
     const int lane = threadIdx.x & 63;
@@ -41,7 +44,7 @@ __global__ __launch_bounds__(256) void k_router_softmax_topk(const void* __restr
 #pragma unroll
     for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
         const int e = lane + 64 * i;
-        v[i] = (i < per && e < E) ? load_logit<DT>(logits, (int64_t)tkn * E + e) : -INFINITY;
+        v[i] = (i < per && e < E) ? load_logit<DT>(logits, (int64_t)tkn * ld + e) : -INFINITY;
         vmax = fmaxf(vmax, v[i]);
     }
 #pragma unroll
@@ -88,7 +91,7 @@ __global__ __launch_bounds__(256) void k_router_softmax_topk(const void* __restr
         }
     }
     if (lane < k) {
-        float w = renorm ? my_w / picked_sum : my_w;
+        float w = (renorm ? my_w / picked_sum : my_w) * wscale;
         if (round_dt == BITSMOE_DT_F16)
             w = __half2float(__float2half(w));
         else if (round_dt == BITSMOE_DT_BF16)
@@ -107,7 +110,8 @@ __global__ __launch_bounds__(256) void k_router_softmax_topk(const void* __restr
 // grid = ceil(T / 4), 256 threads (one wavefront per token).
 constexpr int ROUTER_RANK_PER_LANE = 4;
 template <int DT>
-__global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict__ logits, int T, int E, int k,
+__global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict__ logits, int64_t ld, float wscale, int T,
+                                                          int E, int k,
                                                           int renorm, int round_dt, int32_t* __restrict__ sel32,
                                                           int64_t* __restrict__ sel64, float* __restrict__ weights) {
     // sort key of a logit: the float mapped to an unsigned integer of the same order, above the
@@ -125,7 +129,7 @@ __global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict
 #pragma unroll
     for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) {
         const int e = lane + 64 * i;
-        v[i] = e < E ? load_logit<DT>(logits, (int64_t)tkn * E + e) : -INFINITY;
+        v[i] = e < E ? load_logit<DT>(logits, (int64_t)tkn * ld + e) : -INFINITY;
         vmax = fmaxf(vmax, v[i]);
         const uint32_t bits = __float_as_uint(v[i] + 0.0f);      // (-0 and +0 are one value)
         const uint32_t ordered = bits ^ ((bits >> 31) ? 0xFFFFFFFFu : 0x80000000u);
@@ -167,6 +171,7 @@ __global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict
         if (lane + 64 * i < E && rank[i] < k) {
             float w = pr[i] / denom;
             if (renorm) w /= picked_sum;
+            w *= wscale;
             if (round_dt == BITSMOE_DT_F16)
                 w = __half2float(__float2half(w));
             else if (round_dt == BITSMOE_DT_BF16)
@@ -183,15 +188,17 @@ __global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict
 
 using namespace bitsmoe;
 
-extern "C" int bitsmoe_router_softmax_topk(const void* logits, int32_t logits_dtype, int64_t n_tokens, int32_t n_experts,
-                                           int32_t top_k, int32_t renormalize, int32_t round_dtype, void* selected,
-                                           int32_t ids_are_i64, float* weights, void* stream) {
+extern "C" int bitsmoe_router_softmax_topk_strided(const void* logits, int32_t logits_dtype, int64_t ld_logits, int64_t n_tokens,
+                                                   int32_t n_experts, int32_t top_k, int32_t renormalize, float weight_scale,
+                                                   int32_t round_dtype, void* selected, int32_t ids_are_i64, float* weights,
+                                                   void* stream) {
     BITSMOE_REQUIRE(n_tokens >= 0 && n_tokens < ((int64_t)1 << 31), "token count out of range");
     BITSMOE_REQUIRE(n_experts >= 1 && n_experts <= 64 * ROUTER_MAX_PER_LANE, "n_experts must be in [1, %d]",
                     64 * ROUTER_MAX_PER_LANE);
     BITSMOE_REQUIRE(top_k >= 1 && top_k <= 64 && top_k <= n_experts, "top_k must be in [1, min(64, n_experts)]");
     BITSMOE_REQUIRE(logits_dtype >= 0 && logits_dtype <= 2, "logits_dtype must be 0 (fp16), 1 (bf16) or 2 (fp32)");
     BITSMOE_REQUIRE(round_dtype >= -1 && round_dtype <= 1, "round_dtype must be -1 (none), 0 (fp16) or 1 (bf16)");
+    BITSMOE_REQUIRE(ld_logits >= n_experts, "ld_logits must be at least n_experts");
     if (n_tokens == 0) return BITSMOE_OK;
     BITSMOE_REQUIRE(logits && selected && weights, "null pointer");
     hipStream_t st = (hipStream_t)stream;
@@ -200,8 +207,8 @@ extern "C" int bitsmoe_router_softmax_topk(const void* logits, int32_t logits_dt
     const dim3 grid((unsigned)((n_tokens + 3) / 4));
     const bool by_rank = n_experts <= 64 * ROUTER_RANK_PER_LANE;
 #define BITSMOE_ROUTER_LAUNCH(KERNEL)                                                                              \
-    hipLaunchKernelGGL(KERNEL, grid, dim3(256), 0, st, logits, (int)n_tokens, n_experts, top_k, renormalize, \
-                       round_dtype, s32, s64, weights)
+    hipLaunchKernelGGL(KERNEL, grid, dim3(256), 0, st, logits, ld_logits, weight_scale, (int)n_tokens, n_experts, top_k, \
+                       renormalize, round_dtype, s32, s64, weights)
     if (logits_dtype == 0) {
         if (by_rank) BITSMOE_ROUTER_LAUNCH(k_router_rank_topk<0>); else BITSMOE_ROUTER_LAUNCH(k_router_softmax_topk<0>);
     } else if (logits_dtype == 1) {
@@ -210,6 +217,103 @@ extern "C" int bitsmoe_router_softmax_topk(const void* logits, int32_t logits_dt
         if (by_rank) BITSMOE_ROUTER_LAUNCH(k_router_rank_topk<2>); else BITSMOE_ROUTER_LAUNCH(k_router_softmax_topk<2>);
     }
 #undef BITSMOE_ROUTER_LAUNCH
+    BITSMOE_HIP_TRY(hipGetLastError());
+    return BITSMOE_OK;
+}
+
+extern "C" int bitsmoe_router_softmax_topk(const void* logits, int32_t logits_dtype, int64_t n_tokens, int32_t n_experts,
+                                           int32_t top_k, int32_t renormalize, int32_t round_dtype, void* selected,
+                                           int32_t ids_are_i64, float* weights, void* stream) {
+    return bitsmoe_router_softmax_topk_strided(logits, logits_dtype, n_experts, n_tokens, n_experts, top_k, renormalize, 1.0f,
+                                               round_dtype, selected, ids_are_i64, weights, stream);
+}
+
+// ---- the block's closing elementwise pass ---------------------------------------------------------------------------
+// One row of the operand of the block's output GEMM, in the activation dtype:
+//     out[t, 0 .. R)        = rank_accum[t, :]                                   (fp32 -> 16 bit)
+//     out[t, R .. R + I_sh) = silu(a[t, c]) * b[t, c] * (g ? sigmoid(g[t]) : 1)   (the always-on shared expert's z)
+// so that the routed experts' output projection and the shared expert's down projection are ONE GEMM against
+// the stacked [U_down | W_down_shared] (bitsmoe/models/base_block.py:414, bitsmoe/models/qwen3next/bitsmoe_block.py:144-147,
+// bitsmoe/models/deepseekv2/bitsmoe_block.py:123-124 run them as separate modules and add).  Eight elements per thread.
+template <bool BF16>
+__global__ __launch_bounds__(256) void k_block_finish(const float* __restrict__ rank_accum, int64_t T, int R,
+                                                      const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
+                                                      int64_t ld_ab, int I_sh, const uint16_t* __restrict__ g, int64_t ld_g,
+                                                      uint16_t* __restrict__ out, int64_t ld_out) {
+    const int per_row = (R + I_sh) >> 3;
+    const int64_t total = T * per_row;
+    auto to_f32 = [](uint16_t v) {
+        if constexpr (BF16) return __uint_as_float((uint32_t)v << 16);
+        else return __half2float(__ushort_as_half(v));
+    };
+    auto to_16 = [](float v) -> uint16_t {
+        if constexpr (BF16) return __builtin_bit_cast(uint16_t, (__bf16)v);
+        else return __builtin_bit_cast(uint16_t, (_Float16)v);
+    };
+    typedef uint32_t v4 __attribute__((ext_vector_type(4)));
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t t = i / per_row;
+        const int c = (int)(i - t * per_row) * 8;
+        uint16_t o[8];
+        if (c < R) {
+            const f4 lo = *reinterpret_cast<const f4*>(rank_accum + t * R + c);
+            const f4 hi = *reinterpret_cast<const f4*>(rank_accum + t * R + c + 4);
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                o[x] = to_16(lo[x]);
+                o[4 + x] = to_16(hi[x]);
+            }
+        } else {
+            const int cs = c - R;
+            const v4 av = *reinterpret_cast<const v4*>(a + t * ld_ab + cs);
+            const v4 bv = *reinterpret_cast<const v4*>(b + t * ld_ab + cs);
+            float gate = 1.0f;
+            if (g) gate = 1.0f / (1.0f + __expf(-to_f32(g[t * ld_g])));
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const float a0 = to_f32((uint16_t)(av[x] & 0xFFFFu)), a1 = to_f32((uint16_t)(av[x] >> 16));
+                const float b0 = to_f32((uint16_t)(bv[x] & 0xFFFFu)), b1 = to_f32((uint16_t)(bv[x] >> 16));
+                // (rounded as the modules round: silu in the activation dtype, the product, the gate's scaling)
+                o[2 * x] = to_16(to_f32(to_16(to_f32(to_16(a0 / (1.0f + __expf(-a0)))) * b0)) * gate);
+                o[2 * x + 1] = to_16(to_f32(to_16(to_f32(to_16(a1 / (1.0f + __expf(-a1)))) * b1)) * gate);
+            }
+        }
+        v4 packed;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) packed[x] = (uint32_t)o[2 * x] | ((uint32_t)o[2 * x + 1] << 16);
+        *reinterpret_cast<v4*>(out + t * ld_out + c) = packed;
+    }
+}
+
+extern "C" int bitsmoe_block_finish(const float* rank_accum, int64_t n_tokens, int32_t rank_out, const void* shared_gate_out,
+                                    const void* shared_up_out, int64_t ld_shared, int32_t shared_intermediate,
+                                    const void* shared_gate_logit, int64_t ld_gate_logit, int32_t act_dtype, void* out,
+                                    int64_t ld_out, void* stream) {
+    BITSMOE_REQUIRE(n_tokens >= 0 && rank_out > 0 && shared_intermediate >= 0, "negative size");
+    BITSMOE_REQUIRE(rank_out % 8 == 0 && shared_intermediate % 8 == 0, "rank_out and shared_intermediate must be multiples of 8");
+    BITSMOE_REQUIRE(act_dtype == BITSMOE_DT_F16 || act_dtype == BITSMOE_DT_BF16, "act_dtype must be f16 (0) or bf16 (1)");
+    BITSMOE_REQUIRE(ld_out >= rank_out + shared_intermediate && ld_out % 8 == 0, "ld_out too small or not a multiple of 8");
+    if (n_tokens == 0) return BITSMOE_OK;
+    BITSMOE_REQUIRE(rank_accum && out, "null pointer");
+    BITSMOE_REQUIRE(((uintptr_t)rank_accum & 15) == 0 && ((uintptr_t)out & 15) == 0, "rank_accum and out must be 16-byte aligned");
+    if (shared_intermediate > 0) {
+        BITSMOE_REQUIRE(shared_gate_out && shared_up_out && ld_shared >= shared_intermediate && ld_shared % 8 == 0,
+                        "shared expert operands missing, or their row stride is not a multiple of 8");
+        BITSMOE_REQUIRE(((uintptr_t)shared_gate_out & 15) == 0 && ((uintptr_t)shared_up_out & 15) == 0,
+                        "shared expert operands must be 16-byte aligned");
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t total = n_tokens * ((rank_out + shared_intermediate) / 8);
+    const unsigned blocks = (unsigned)std::min<int64_t>((total + 255) / 256, 4096);
+    if (act_dtype == BITSMOE_DT_BF16)
+        hipLaunchKernelGGL(k_block_finish<true>, dim3(blocks), dim3(256), 0, st, rank_accum, n_tokens, rank_out,
+                           (const uint16_t*)shared_gate_out, (const uint16_t*)shared_up_out, ld_shared, shared_intermediate,
+                           (const uint16_t*)shared_gate_logit, ld_gate_logit, (uint16_t*)out, ld_out);
+    else
+        hipLaunchKernelGGL(k_block_finish<false>, dim3(blocks), dim3(256), 0, st, rank_accum, n_tokens, rank_out,
+                           (const uint16_t*)shared_gate_out, (const uint16_t*)shared_up_out, ld_shared, shared_intermediate,
+                           (const uint16_t*)shared_gate_logit, ld_gate_logit, (uint16_t*)out, ld_out);
     BITSMOE_HIP_TRY(hipGetLastError());
     return BITSMOE_OK;
 }

@@ -422,6 +422,140 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
                 "Packed routed experts require CUDA mlp_forward extension; python fallback is intentionally disabled.")
         return self._packed_forward_cuda(h_gate_proj, h_up_proj, token_indices, expert_offsets_t, route_flat, token_count)
 
+    # ---- the block as one GEMM in, the operator, one GEMM out ----------------------------------
+    # Everything that multiplies the block input by a weight matrix -- the two shared-basis projections
+    # (bitsmoe/models/qwen3moe/bitsmoe_block.py:63-64), the router's linear layer (:45), an always-on shared
+    # expert's gate and up projections and its sigmoid gate (bitsmoe/models/qwen3next/bitsmoe_block.py:144-147,
+    # bitsmoe/models/deepseekv2/bitsmoe_block.py:123-124) -- is ONE library GEMM against the row-stacked weights;
+    # the operator and the router kernel read their operands as column ranges of its output.  Everything that
+    # is projected back to hidden space -- rank_accum @ shared_u_down.T (bitsmoe/models/base_block.py:414) and the
+    # shared expert's down projection -- is ONE GEMM against the column-stacked weights, its operand written by
+    # one elementwise pass (bitsmoe_block_finish).  Beside the operator's own launches a block forward is then
+    # four launches instead of ten to twenty framework ops.
+    _FUSED_BLOCK = _os.environ.get("BITSMOE_FUSED_BLOCK", "1") != "0"
+
+    @staticmethod
+    def _plain_linear(mod, in_features: Optional[int] = None) -> bool:
+        return (isinstance(mod, nn.Linear) and mod.bias is None and isinstance(mod.weight, torch.Tensor)
+                and mod.weight.dim() == 2 and (in_features is None or int(mod.weight.shape[1]) == in_features))
+
+    def _fused_plan(self, dtype: torch.dtype, router: Optional[nn.Module], shared: Optional[nn.Module],
+                    shared_gate: Optional[nn.Module]):
+        """The stacked input / output weights and the column ranges of their parts, or None when a module is not
+        a bias-free linear layer of the expected shape.  Cached; rebuilt when a source tensor was rebound or written."""
+        hidden = int(self.shared_vh_gate_proj.shape[1])
+        sources = [self.shared_vh_gate_proj, self.shared_vh_up_proj, self.shared_u_down]
+        if router is not None:
+            if not self._plain_linear(router, hidden):
+                return None
+            sources.append(router.weight)
+        if shared is not None:
+            projs = [getattr(shared, n, None) for n in ("gate_proj", "up_proj", "down_proj")]
+            if not (self._plain_linear(projs[0], hidden) and self._plain_linear(projs[1], hidden) and self._plain_linear(projs[2])
+                    and projs[0].weight.shape == projs[1].weight.shape
+                    and tuple(projs[2].weight.shape) == (hidden, int(projs[0].weight.shape[0]))
+                    and int(projs[0].weight.shape[0]) % 8 == 0):
+                return None
+            sources += [p.weight for p in projs]
+            if shared_gate is not None:
+                if not (self._plain_linear(shared_gate, hidden) and int(shared_gate.weight.shape[0]) == 1):
+                    return None
+                sources.append(shared_gate.weight)
+        elif shared_gate is not None:
+            return None
+        if int(self.shared_u_down.shape[1]) % 8 or int(self.shared_vh_gate_proj.shape[0]) % 8 or int(self.shared_vh_up_proj.shape[0]) % 8:
+            return None
+        stamp = tuple((id(t), t.data_ptr(), -1 if t.is_inference() else t._version) for t in sources)
+        key = ("fused_plan", dtype, router is not None, shared is not None, shared_gate is not None)
+        cached = self._basis_cache.get(key)
+        if cached is not None and cached["stamp"] == stamp:
+            return cached
+        parts, ranges, col = [], {}, 0
+
+        def add(name, w):      # (every part starts on a multiple of 8 columns: 16-byte aligned rows of its range)
+            nonlocal col
+            w = w.detach().to(dtype)
+            pad = (-int(w.shape[0])) % 8
+            if pad:
+                w = torch.cat([w, w.new_zeros((pad, w.shape[1]))], dim=0)
+            parts.append(w)
+            ranges[name] = (col, col + int(w.shape[0]) - pad)
+            col += int(w.shape[0])
+
+        add("h_gate", self.shared_vh_gate_proj)
+        add("h_up", self.shared_vh_up_proj)
+        if router is not None:
+            add("logits", router.weight)
+        i_sh = 0
+        if shared is not None:
+            add("sh_gate", shared.gate_proj.weight)
+            add("sh_up", shared.up_proj.weight)
+            i_sh = int(shared.gate_proj.weight.shape[0])
+            if shared_gate is not None:
+                add("sh_logit", shared_gate.weight)
+        w_in = torch.cat(parts, dim=0).contiguous()
+        outs = [self.shared_u_down.detach().to(dtype)]
+        if shared is not None:
+            outs.append(shared.down_proj.weight.detach().to(dtype))
+        w_out = torch.cat(outs, dim=1).contiguous()      # [hidden, rank_out + I_sh]
+        cached = {"stamp": stamp, "w_in": w_in, "w_out": w_out, "ranges": ranges, "i_sh": i_sh}
+        self._basis_cache[key] = cached
+        return cached
+
+    def _fused_block_forward(self, hidden_states: torch.Tensor, *, router: Optional[nn.Module] = None, route_fn=None,
+                             renormalize: bool = True, round_weights: bool = True, weight_scale: float = 1.0,
+                             shared: Optional[nn.Module] = None, shared_gate: Optional[nn.Module] = None):
+        """hidden [T, H] -> (output [T, H], router logits [T, E] or None), or None when this block cannot take the
+        fused form (the caller then runs the module-by-module form).  `router`: the bias-free linear layer whose
+        logits go through softmax / top-k (renormalize, weight_scale, round trip through the activation dtype);
+        otherwise `route_fn(hidden) -> (selected [T, k], weights fp32 [T, k])`."""
+        if not (self._FUSED_BLOCK and hidden_states.is_cuda and _HAS_MLP_FORWARD_CUDA and self._packed_expert_count > 0
+                and self._packed_global_to_local is not None and hidden_states.dtype in (torch.float16, torch.bfloat16)
+                and not _dense_via_operator()):
+            return None
+        if self.shared_vh_gate_proj.numel() == 0 or self.shared_vh_up_proj.numel() == 0 or self.shared_u_down.numel() == 0:
+            return None
+        if router is not None and not (int(router.weight.shape[0]) <= 1024 and self.top_k <= 64):
+            return None
+        dtype = hidden_states.dtype
+        plan = self._fused_plan(dtype, router, shared, shared_gate)
+        if plan is None:
+            return None
+        token_count = int(hidden_states.shape[0])
+        big = hidden_states @ plan["w_in"].T
+        rng = plan["ranges"]
+        h_gate = big[:, rng["h_gate"][0]:rng["h_gate"][1]]
+        h_up = big[:, rng["h_up"][0]:rng["h_up"][1]]
+        logits = None
+        if router is not None:
+            logits = big[:, rng["logits"][0]:rng["logits"][1]]
+            selected, weights = mlp_forward_cuda.router_softmax_topk(logits, self.top_k, renormalize,
+                                                                     round_dtype=dtype if round_weights else None,
+                                                                     weight_scale=weight_scale)
+        else:
+            selected, weights = route_fn(hidden_states)
+            selected = selected.reshape(token_count, self.top_k)
+            weights = weights.reshape(token_count, self.top_k).to(torch.float32)
+        rank_out = int(self.shared_u_down.shape[1])
+        gate, up, down = self._ensure_matsets()
+        rank_accum = mlp_forward_cuda.moe_forward_routed(h_gate, h_up, selected, weights, self._packed_global_to_local,
+                                                         self._packed_local_to_global, gate, up, down, rank_out,
+                                                         int(self._packed_intermediate_size), self._act_type())
+        if shared is not None:
+            sh_logit = big[:, rng["sh_logit"][0]:rng["sh_logit"][1]] if shared_gate is not None else None
+            operand = mlp_forward_cuda.block_finish(rank_accum, dtype, big[:, rng["sh_gate"][0]:rng["sh_gate"][1]],
+                                                    big[:, rng["sh_up"][0]:rng["sh_up"][1]], sh_logit)
+        else:
+            operand = mlp_forward_cuda.block_finish(rank_accum, dtype)
+        out = operand @ plan["w_out"].T
+        if self._super_expert_items:
+            extra = torch.zeros_like(out)
+            self._run_super_experts(hidden_states, extra, selected.reshape(-1),
+                                    self._get_flat_token_ids(token_count, hidden_states.device),
+                                    weights.reshape(-1).to(dtype))
+            out = out + extra
+        return out, logits
+
     # ---- shared forward body --------------------------------------------------------------
     def _routed_forward(self, hidden_states: torch.Tensor, selected_experts: torch.Tensor,
                         routing_weights_fp32: torch.Tensor) -> torch.Tensor:

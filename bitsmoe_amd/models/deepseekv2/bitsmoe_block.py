@@ -31,12 +31,24 @@ class BitsMoE_DeepSeekSparseMoeBlock(BitsMoE_BaseSparseMoeBlock):
                 setattr(self, attr, int(getattr(source_block, attr)))
         self._init_bitsmoe_common_state(super_experts=super_experts, track_super_projected_weights=True)
 
+    def _gate_route(self, hidden_states: torch.Tensor):
+        topk_idx, topk_weight, _aux = self.gate(hidden_states)
+        return topk_idx.reshape(-1, topk_idx.shape[-1]), topk_weight.reshape(-1, topk_weight.shape[-1]).to(torch.float32)
+
     def forward(self, hidden_states: torch.Tensor):
         identity = hidden_states
         orig_shape = hidden_states.shape
+        flat = hidden_states.reshape(-1, orig_shape[-1])
+        self._ensure_runtime_cache(flat.device)
+        has_shared = getattr(self.config, "n_shared_experts", None) is not None and hasattr(self, "shared_experts")
+        # (the model's own gate module picks; the shared-basis projections, the shared experts and the output
+        # projection take the one-GEMM-in, one-GEMM-out form)
+        fused = self._fused_block_forward(flat, route_fn=lambda h2d: self._gate_route(h2d.reshape(orig_shape)),
+                                          shared=self.shared_experts if has_shared else None)
+        if fused is not None:
+            return fused[0].reshape(*orig_shape)
         topk_idx, topk_weight, _aux = self.gate(hidden_states)
         hidden_states = hidden_states.reshape(-1, orig_shape[-1])
-        self._ensure_runtime_cache(hidden_states.device)
         selected = topk_idx.reshape(-1, topk_idx.shape[-1])
         weights = topk_weight.reshape(-1, topk_weight.shape[-1]).to(torch.float32)
         y = self._routed_forward(hidden_states, selected, weights).reshape(*orig_shape)

@@ -47,7 +47,11 @@ class BitsMoE_Qwen3MoeSparseMoeBlock(BitsMoE_BaseSparseMoeBlock):
         batch_size, sequence_length, hidden_dim = hidden_states.shape
         hidden_states = hidden_states.reshape(-1, hidden_dim)
         self._ensure_runtime_cache(hidden_states.device)
-        router_logits, selected, weights = self._route(hidden_states)
-        final = self._routed_forward(hidden_states, selected, weights)
+        fused = self._fused_block_forward(hidden_states, router=self.gate, renormalize=self.norm_topk_prob)
+        if fused is not None:
+            final, router_logits = fused
+        else:
+            router_logits, selected, weights = self._route(hidden_states)
+            final = self._routed_forward(hidden_states, selected, weights)
         final = final.reshape(batch_size, sequence_length, hidden_dim)
         return final if self.host_expects_tensor else (final, router_logits)

@@ -25,6 +25,14 @@ class BitsMoE_Qwen3NextSparseMoeBlock(BitsMoE_Qwen3MoeSparseMoeBlock):
         batch_size, sequence_length, hidden_dim = hidden_states.shape
         hidden_states = hidden_states.reshape(-1, hidden_dim)
         self._ensure_runtime_cache(hidden_states.device)
+        has_shared = hasattr(self, "shared_expert") and hasattr(self, "shared_expert_gate")
+        fused = self._fused_block_forward(hidden_states, router=self.gate, renormalize=self.norm_topk_prob,
+                                          shared=self.shared_expert if has_shared else None,
+                                          shared_gate=self.shared_expert_gate if has_shared else None)
+        if fused is not None:
+            final, router_logits = fused
+            final = final.reshape(batch_size, sequence_length, hidden_dim)
+            return final if self.host_expects_tensor else (final, router_logits)
         router_logits, selected, weights = self._route(hidden_states)
         final = self._routed_forward(hidden_states, selected, weights)
         if hasattr(self, "shared_expert") and hasattr(self, "shared_expert_gate"):

@@ -143,6 +143,32 @@ int bitsmoe_router_softmax_topk(const void* logits, int32_t logits_dtype, int64_
                                 int32_t n_experts, int32_t top_k, int32_t renormalize,
                                 int32_t round_dtype, void* selected, int32_t ids_are_i64,
                                 float* weights, void* stream);
+/*
+ * The same front end for logits that are a column range of a wider row-major tensor (ld_logits elements from one
+ * token's row to the next: the router's logits as a slice of ONE projection GEMM that also yields the shared-basis
+ * projections), with the picked weights multiplied by weight_scale after the optional renormalisation -- the
+ * softmax -> greedy top-k -> * routed_scaling_factor form of the DeepSeek-V2 gate
+ * (bitsmoe/models/deepseekv2/configuration_deepseek.py:125-139, call site bitsmoe/models/deepseekv2/bitsmoe_block.py:72).
+ */
+int bitsmoe_router_softmax_topk_strided(const void* logits, int32_t logits_dtype, int64_t ld_logits, int64_t n_tokens,
+                                        int32_t n_experts, int32_t top_k, int32_t renormalize, float weight_scale,
+                                        int32_t round_dtype, void* selected, int32_t ids_are_i64, float* weights, void* stream);
+
+/*
+ * The block's closing elementwise pass: one row of the operand of the output GEMM in the activation dtype,
+ *   out[t, 0 .. rank_out)                      = rank_accum[t, :]  (fp32 -> 16 bit; bitsmoe/models/base_block.py:414 casts
+ *                                                 with a framework op)
+ *   out[t, rank_out .. + shared_intermediate)  = silu(gate_out[t, c]) * up_out[t, c] * (sigmoid(gate_logit[t]) or 1)
+ * so that the routed experts' output projection and the always-on shared expert's down projection
+ * (bitsmoe/models/qwen3next/bitsmoe_block.py:144-147, bitsmoe/models/deepseekv2/bitsmoe_block.py:123-124) are one GEMM
+ * against the stacked [shared_u_down | shared down_proj].  shared_intermediate may be 0 (then the pass is the cast
+ * alone and the shared pointers are ignored); shared_gate_logit may be NULL (no sigmoid gate).  Row strides in
+ * elements; rank_out, shared_intermediate, ld_shared and ld_out multiples of 8, pointers 16-byte aligned.
+ */
+int bitsmoe_block_finish(const float* rank_accum, int64_t n_tokens, int32_t rank_out, const void* shared_gate_out,
+                         const void* shared_up_out, int64_t ld_shared, int32_t shared_intermediate,
+                         const void* shared_gate_logit, int64_t ld_gate_logit, int32_t act_dtype, void* out, int64_t ld_out,
+                         void* stream);
 
 /*
  * The routed-expert forward.  Replaces moe_packed_forward

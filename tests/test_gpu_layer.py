@@ -160,11 +160,17 @@ def _block_reference(block, x):
     ("deepseekv2", {}),
 ])
 @pytest.mark.parametrize("tokens", [1, 24])
-def test_block_forward_matches_oracle(cuda_device, family, kw, tokens):
+@pytest.mark.parametrize("fused", [True, False])
+def test_block_forward_matches_oracle(cuda_device, family, kw, tokens, fused, monkeypatch):
+    """The block against the float64 restatement: in its one-GEMM-in / one-GEMM-out form (the shared-basis
+    projections, the router's linear layer and the shared expert's gate / up projections as one GEMM, the output
+    projection and the shared expert's down projection as another) and module by module."""
     import torch
 
+    from bitsmoe_amd.models.base_block import BitsMoE_BaseSparseMoeBlock
     from bitsmoe_amd.synth import make_layer
 
+    monkeypatch.setattr(BitsMoE_BaseSparseMoeBlock, "_FUSED_BLOCK", fused)
     spec = _small_spec(family, **kw)
     block = make_layer(spec, device=cuda_device, dtype=torch.bfloat16, seed=5, s_mode="rand")
     block.prepare_runtime_fastpath(warmup=True)
@@ -174,6 +180,8 @@ def test_block_forward_matches_oracle(cuda_device, family, kw, tokens):
         out = block(x)
     y = out[0] if isinstance(out, tuple) else out
     assert y.shape == x.shape and y.dtype == x.dtype
+    if fused:
+        assert any(isinstance(k, tuple) and k and k[0] == "fused_plan" for k in block._basis_cache)      # the fused form ran
     ref, idx = _block_reference(block, x.reshape(tokens, -1))
     err = helpers.norm_err(y.float().cpu().numpy().reshape(tokens, -1), ref)
     assert err <= 1e-2, f"{family}: normalised error {err:.3e}"
