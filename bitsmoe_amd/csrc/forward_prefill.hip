@@ -28,6 +28,25 @@
 #include "fast_helpers.h"
 #include "mtiles.h"
 
+// ---- optional in-kernel time stamps (timeline build: -DBITSMOE_TIMELINE) of k_gateup_mfma / k_down_mfma: thread 0 of a
+// workgroup writes the 100 MHz wall clock at: 0 entry, 1 tile record and tables at hand, 2 first pieces landed (before the
+// first step), 3 steps done, 6 exit (after the epilogue's stores were issued).
+#ifdef BITSMOE_TIMELINE
+namespace bitsmoe {
+constexpr int TLP_STAMPS = 8;
+constexpr int TLP_MAX_WG = 8192;
+__device__ unsigned long long g_tl_pf_gateup[TLP_MAX_WG * TLP_STAMPS];
+__device__ unsigned long long g_tl_pf_down[TLP_MAX_WG * TLP_STAMPS];
+}  // namespace bitsmoe
+#define BITSMOE_TLP(arr, i)                                                             \
+    do {                                                                                \
+        if (threadIdx.x == 0 && blockIdx.x < ::bitsmoe::TLP_MAX_WG)                     \
+            ::bitsmoe::arr[blockIdx.x * ::bitsmoe::TLP_STAMPS + (i)] = wall_clock64(); \
+    } while (0)
+#else
+#define BITSMOE_TLP(arr, i) do {} while (0)
+#endif
+
 namespace bitsmoe {
 
 // -(1.5 * 2^W) as a packed f16 pair: times the scale it is the constant that turns
@@ -616,6 +635,7 @@ __device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const 
         else
             wait_vmcnt<0>();
         barrier_no_drain();
+        BITSMOE_TLP(g_tl_pf_gateup, 2);
         // step s (s % 3 == U): slab s + 2 requested into the stage slab s - 1 used, slab s multiplied
         auto step = [&](auto u_c, int s) {
             constexpr int U = decltype(u_c)::value;
@@ -642,6 +662,7 @@ __device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const 
             if (s0 + 2 < nslabs) step(std::integral_constant<int, 2>{}, s0 + 2);
         }
     }
+    BITSMOE_TLP(g_tl_pf_gateup, 3);
     if (!active) return;
     // lane holds rows 16*mb + 4*kg + j, column 128*t + 64*wn + 16*nb + n
 #pragma unroll
@@ -684,6 +705,7 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     __shared__ __attribute__((aligned(16))) uint32_t sw0[DMA_WSTAGE], sw1[DMA_WSTAGE], sw2[DMA_WSTAGE];
     __shared__ __attribute__((aligned(16))) uint16_t ss0[DMA_SSTAGE], ss1[DMA_SSTAGE], ss2[DMA_SSTAGE];
     __shared__ int32_t pack_tab[DMA_MAX_SLABS], scale_tab[DMA_MAX_SLABS], rank_tab[DMA_MAX_SLABS * 8], bits_tab[DMA_MAX_SLABS];
+    BITSMOE_TLP(g_tl_pf_gateup, 0);
     const int n_tp = (n_tiles + 1) >> 1;
     // proj_sel < 0: both projections in this launch; 0 / 1: the gate / the up projection alone.  fuse (up alone, after
     // a gate launch): the epilogue stores z = silu(gate) * up over the gate sums instead of the up sums.
@@ -712,6 +734,7 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
     // with a quarter / half / three quarters of the accumulators, MFMAs and staging; complete
     // bodies, so that no accumulator lives across the choice
     const DmaStage st0 = {sa0, sw0, ss0}, st1 = {sa1, sw1, ss1}, st2 = {sa2, sw2, ss2};
+    BITSMOE_TLP(g_tl_pf_gateup, 1);
 #define BITSMOE_GU_BODY(W)                                                                                           \
     do {                                                                                                             \
         if (rows <= 32)                                                                                              \
@@ -749,6 +772,7 @@ __global__ __launch_bounds__(256, 2) void k_gateup_mfma(
         BITSMOE_GU_BODY(0);
 #undef BITSMOE_GU_BODY
 #undef BITSMOE_GU_BODY_MIXED
+    BITSMOE_TLP(g_tl_pf_gateup, 6);
 }
 
 // z = f16( silu(G) * U ), written over G; 8 elements per thread and iteration.
@@ -893,6 +917,7 @@ __device__ __forceinline__ void down_tile_loop(const uint32_t* __restrict__ payl
     request_z(st1, 1);
     wait_vmcnt<NJ>();                      // block 0 and piece 0 have landed
     barrier_no_drain();
+    BITSMOE_TLP(g_tl_pf_down, 2);
     // step h (h % 3 == U, h % 2 == HH): (first half of a tile) the tile's block taken into
     // registers; piece h + 2 requested into the stage piece h - 1 used, then (first half) the next
     // tile's block; piece h multiplied
@@ -955,6 +980,7 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
     __shared__ __attribute__((aligned(16))) uint16_t sz0[DMA_STAGE], sz1[DMA_STAGE], sz2[DMA_STAGE];
     __shared__ __attribute__((aligned(16))) uint32_t wbuf[4 * DN_WBUF];
     __shared__ __attribute__((aligned(16))) uint16_t sbuf[4 * DN_SBUF];
+    BITSMOE_TLP(g_tl_pf_down, 0);
     const int logical = xcd_logical(blockIdx.x, __builtin_amdgcn_readfirstlane(*n_mtiles), n_groups);
     if (logical < 0) return;
     const int mt_i = logical / n_groups, grp = logical - mt_i * n_groups;
@@ -978,6 +1004,7 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
     const int si = DN_SLABS_MFMA * grp + wave;
     FastSlab fs = FastSlab{0, 0, 0, 0};
     if (si < nslabs) fs = load_fast_slab(down_fs + (int64_t)e * max_slabs, si);
+    BITSMOE_TLP(g_tl_pf_down, 1);
 
     // tiles of at most 32 / 64 / 96 assignments run a body with a quarter / half / three quarters of
     // the accumulators and MFMAs: complete bodies, so that no accumulator lives across the choice
@@ -990,6 +1017,7 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
             for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0, 0, 0, 0};
         // wavefronts without a slab skip the MFMAs; all execute the same barriers
         down_tile_loop<NMB>(fe.payload, fe.scale, fs, z, I, n_tiles, a_begin, rows, sz0, sz1, sz2, wbuf, sbuf, tid, lane, acc);
+        BITSMOE_TLP(g_tl_pf_down, 3);
         if (fs.bits == 0) return;
 
         // lane holds assignments 16*mb + 4*kg + j, output rows 16*nb + n of the slab; the rows'
@@ -1018,6 +1046,7 @@ __global__ __launch_bounds__(256, 2) void k_down_mfma(const FastExpert* __restri
         run(std::integral_constant<int, 6>{});
     else
         run(std::integral_constant<int, 8>{});
+    BITSMOE_TLP(g_tl_pf_down, 6);
 }
 
 // ------------------------------------------------------------------------------- combine
@@ -1353,3 +1382,27 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
 }
 
 }  // namespace bitsmoe
+
+#ifdef BITSMOE_TIMELINE
+// which: 0 = k_gateup_mfma, 1 = k_down_mfma
+extern "C" int bitsmoe_timeline_read_prefill(int which, unsigned long long* host, int n_workgroups) {
+    using namespace bitsmoe;
+    if (!host || n_workgroups <= 0 || n_workgroups > TLP_MAX_WG || which < 0 || which > 1) return BITSMOE_E_INVALID;
+    BITSMOE_HIP_TRY(hipDeviceSynchronize());
+    const size_t bytes = sizeof(unsigned long long) * TLP_STAMPS * n_workgroups;
+    if (which == 0)
+        BITSMOE_HIP_TRY(hipMemcpyFromSymbol(host, HIP_SYMBOL(g_tl_pf_gateup), bytes));
+    else
+        BITSMOE_HIP_TRY(hipMemcpyFromSymbol(host, HIP_SYMBOL(g_tl_pf_down), bytes));
+    return BITSMOE_OK;
+}
+extern "C" int bitsmoe_timeline_clear_prefill(void) {
+    using namespace bitsmoe;
+    void* p = nullptr;
+    BITSMOE_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_tl_pf_gateup)));
+    BITSMOE_HIP_TRY(hipMemset(p, 0, sizeof(unsigned long long) * TLP_STAMPS * TLP_MAX_WG));
+    BITSMOE_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_tl_pf_down)));
+    BITSMOE_HIP_TRY(hipMemset(p, 0, sizeof(unsigned long long) * TLP_STAMPS * TLP_MAX_WG));
+    return BITSMOE_OK;
+}
+#endif

@@ -8,6 +8,7 @@ assignment chunk.  This script builds the synthetic layer of the named benchmark
 rotation of distinct layers (cold weights), reads the stamps of ONE forward and prints, in microseconds, when
 workgroups start and end relative to the kernel's first start and how long each phase lasts.
   --kernels two    (default) the gate/up kernel and the down kernel of the two-kernel decode forward
+  --kernels prefill  the grouped-GEMM kernels k_gateup_mfma / k_down_mfma (use with a prefill-sized --tokens)
   --kernels fused  the one-kernel forward (option decode_fused = 1): tables + routing scan | gate + up walk (per slab
                    group: operand staged | barrier | multiplied) | z + barrier | down + atomics
 """
@@ -32,7 +33,7 @@ def main() -> int:
     ap.add_argument("--workload", default="c2", help="layer shape of the benchmark set (c1, c2, c4, c5)")
     ap.add_argument("--tokens", type=int, default=64)
     ap.add_argument("--layers", type=int, default=4)
-    ap.add_argument("--kernels", default="two", choices=("two", "fused"))
+    ap.add_argument("--kernels", default="two", choices=("two", "fused", "prefill"))
     args = ap.parse_args()
 
     import torch
@@ -77,6 +78,36 @@ def main() -> int:
     torch.cuda.synchronize()
     block, sets, hg, hu, sel, w = states[0]
     us = lambda ticks: ticks / 100.0
+    if args.kernels == "prefill":
+        lib.bitsmoe_timeline_read_prefill.restype = ctypes.c_int32
+        lib.bitsmoe_timeline_read_prefill.argtypes = [ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32]
+        lib.bitsmoe_timeline_clear_prefill.restype = ctypes.c_int32
+        _capi.check(lib.bitsmoe_timeline_clear_prefill())
+        step(0)
+        torch.cuda.synchronize()
+        print(f"workload {args.workload} T={args.tokens}, grouped-GEMM kernels (the first 8192 workgroups of each launch)")
+        first_start = None
+        for which, kname in ((0, "k_gateup_mfma"), (1, "k_down_mfma")):
+            n = 8192
+            raw = (ctypes.c_uint64 * (8 * n))()
+            _capi.check(lib.bitsmoe_timeline_read_prefill(which, raw, n))
+            rows = [raw[8 * i:8 * i + 8] for i in range(n)]
+            started = [r for r in rows if r[0]]
+            worked = [r for r in started if r[6] and r[3] and r[2] and r[1]]
+            if not worked:
+                print(f"  {kname}: did not run")
+                continue
+            t0 = min(r[0] for r in started)
+            first_start = t0 if first_start is None else first_start
+            print(f"  {kname}: {len(started)} workgroups started, {len(worked)} had a tile; first start {us(t0 - first_start):.2f} us "
+                  f"after the first kernel's; span {us(max(r[6] or r[0] for r in started) - t0):.2f} us")
+            for label, vals in (("start", [us(r[0] - t0) for r in worked]), ("end", [us(r[6] - t0) for r in worked])):
+                print(f"    {label:>14}: p10 {_pct(vals, 0.1):7.2f}  p50 {_pct(vals, 0.5):7.2f}  p90 {_pct(vals, 0.9):7.2f}  max {max(vals):7.2f}")
+            for label, lo, hi in (("tables", 0, 1), ("first loads", 1, 2), ("steps", 2, 3), ("epilogue", 3, 6), ("lifetime", 0, 6)):
+                vals = [us(r[hi] - r[lo]) for r in worked]
+                print(f"    {label:>14}: mean {statistics.mean(vals):7.2f}  p10 {_pct(vals, 0.1):7.2f}  p50 {_pct(vals, 0.5):7.2f}  "
+                      f"p90 {_pct(vals, 0.9):7.2f}  max {max(vals):7.2f}")
+        return 0
     if args.kernels == "two":
         _capi.check(lib.bitsmoe_timeline_clear_decode())
         step(0)
