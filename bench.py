@@ -54,6 +54,10 @@ WORKLOADS = {
     "c3-t4096": ("c3", 4096, "mfma"),
     "c2-ckpt-t64": ("c2", 64, "hbm"),
     "c3-ckpt-t4096": ("c3", 4096, "mfma"),
+    # two of the 128 experts dense ("super" experts: 16-bit rows, run by the operator's side kernels)
+    "c2-super2-t64": ("c2", 64, "hbm"),
+    # intermediate size 1440: the last column tile holds 32 columns
+    "c2-i1440-t64": ("c2i", 64, "hbm"),
     "c1-t16": ("c1", 16, "hbm"),
     "c4-t256": ("c4", 256, "hbm"),
     "c5-stack-t32": ("c5", 32, "hbm"),
@@ -62,6 +66,7 @@ WORKLOADS = {
 WORKLOAD_DESC = {
     "c2": "Qwen3-30B-A3B-shaped MoE layer (128 experts, top-8, hidden 2048, intermediate 768, mixed 2/3/4-bit, group 128)",
     "c3": "Qwen3-30B-A3B-shaped MoE layer (128 experts, top-8, hidden 2048, intermediate 768, mixed 2/3/4-bit, group 128)",
+    "c2i": "Qwen3-30B-A3B-shaped MoE layer with intermediate 1440 (128 experts, top-8, hidden 2048, mixed 2/3/4-bit, group 128)",
     "c1": "DeepSeek-V2-Lite-shaped MoE layer (64 experts, top-6, hidden 2048, intermediate 1408, mixed 2/3/4-bit, group 128)",
     "c4": "Qwen3-Next-80B-A3B-shaped MoE layer (512 experts, top-10, one shared expert outside the operator, hidden 2048, "
           "intermediate 512, mixed 2/3/4-bit, group 128)",
@@ -77,8 +82,9 @@ def matrix_bytes(lists, e):
             + slab_meta[e].numel() * 4 + tile_meta[e].numel() * 4)
 
 
-def algorithmic_work(block, counts, tokens, n_assign):
-    """Algorithmic bytes (per kernel) and FLOPs of one forward for the ACTUAL active experts."""
+def algorithmic_work(block, counts, tokens, n_assign, super_counts=()):
+    """Algorithmic bytes (per kernel) and FLOPs of one forward for the ACTUAL active experts; `super_counts`:
+    assignments of the block's dense experts (f16 weights, hidden-sized activations)."""
     gate, up, down = (block._static_lists(p) for p in ("gate", "up", "down"))
     rank_g = int(block.shared_vh_gate_proj.shape[0])
     rank_u = int(block.shared_vh_up_proj.shape[0])
@@ -91,6 +97,14 @@ def algorithmic_work(block, counts, tokens, n_assign):
     b_down += 4 * tokens * rank_out + 8 * n_assign
     flops = sum(2 * counts[e] * isz * (gate[1][e].numel() + up[1][e].numel() + down[1][e].numel()) for e in active)
     fl_gateup = sum(2 * counts[e] * isz * (gate[1][e].numel() + up[1][e].numel()) for e in active)
+    for (_, layer), c in zip(block._super_expert_items, super_counts):
+        if c <= 0:
+            continue
+        wg, wd = layer.gate_proj.weight, layer.down_proj.weight
+        b_gateup += 2 * 2 * wg.numel() + 2 * tokens * int(wg.shape[1])
+        b_down += 2 * wd.numel() + 4 * tokens * int(wd.shape[0])
+        flops += 2 * c * 3 * wg.numel()
+        fl_gateup += 2 * c * 2 * wg.numel()
     return {"bytes_gateup": b_gateup, "bytes_down": b_down, "bytes_total": b_gateup + b_down,
             "flops": flops, "flops_gateup": fl_gateup, "flops_down": flops - fl_gateup, "active_experts": len(active)}
 
@@ -118,6 +132,12 @@ class _LayerState:
         self.g2l = block._packed_global_to_local
         self.l2g = block._packed_local_to_global
         self.n_packed = block._packed_expert_count
+        # dense ("super") experts among the routed ones: a second operator call on their own matrix sets
+        self.has_super = bool(block._super_expert_items)
+        if self.has_super:
+            self.super_out = torch.zeros((tokens, spec.hidden_size), dtype=torch.bfloat16, device=dev)
+            self.flat_selected = self.selected.reshape(-1)
+            self.flat_weights = self.weights.reshape(-1).to(torch.bfloat16)
 
 
 def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, layers_per_step=1, block_scope=True):
@@ -135,8 +155,12 @@ def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, l
     def layer_step(i, profile=None):
         st = layers[i % n_layers]
         gate, up, down = st.sets
-        return hip.moe_forward_routed(st.h_gate, st.h_up, st.selected, st.weights, st.g2l, st.l2g, gate, up, down,
-                                      st.rank_out, st.isz, 0, profile=profile)
+        out = hip.moe_forward_routed(st.h_gate, st.h_up, st.selected, st.weights, st.g2l, st.l2g, gate, up, down,
+                                     st.rank_out, st.isz, 0, profile=profile)
+        if st.has_super:      # (the block's own code: routing tables of the dense experts, operator, sum in hidden space)
+            st.super_out.zero_()
+            st.block._run_super_experts(st.x, st.super_out, st.flat_selected, None, st.flat_weights)
+        return out
 
     def layer_tables(i):      # (the routing tables, for the accounting and the CPU check only)
         st = layers[i % n_layers]
@@ -226,7 +250,9 @@ def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, l
         tok, off, rw = layer_tables(i)
         torch.cuda.synchronize(dev)
         counts = (off[1:] - off[:-1]).cpu().tolist()
-        works.append(algorithmic_work(layers[i].block, counts, tokens, int(tok.numel())))
+        sel_flat = layers[i].selected.reshape(-1)
+        super_counts = [int((sel_flat == idx).sum()) for idx, _ in layers[i].block._super_expert_items]
+        works.append(algorithmic_work(layers[i].block, counts, tokens, int(tok.numel()), super_counts))
         if i == 0:
             last = (tok, off, rw, out)
     work = {k: sum(w[k] for w in works) / n_layers for k in works[0]}
@@ -494,6 +520,7 @@ def main() -> int:
         _hip.set_option(name, int(value))
     use_graph = not args.no_graph
     built = {}       # spec key of the layer shape -> its distinct copies (c2 and c3 are one layer shape and seed)
+    build_seconds = {}
 
     def blocks_of(spec_key, layout="uniform"):
         shape_key = "c2" if spec_key == "c3" else spec_key
@@ -507,16 +534,17 @@ def main() -> int:
             # and factorising 78 matrices of 2048 x 2048 on the host would take longer than the benchmark)
             built[shape_key] = [make_layer(SPECS[shape_key.split("/")[0]], device=dev, dtype=torch.bfloat16, seed=42, layer_idx=i,
                                            basis_seed=(42 if spec.n_layers > 1 or layout != "uniform" else None),
-                                           layout=layout) for i in range(n)]
+                                           layout="uniform" if layout == "super2" else layout,
+                                           super_experts=(5, 77) if layout == "super2" else ()) for i in range(n)]
             torch.cuda.synchronize()
-            built[shape_key + "/build_s"] = time.perf_counter() - t0
+            build_seconds[id(built[shape_key])] = time.perf_counter() - t0
         return built[shape_key]
 
     def measure(name, steps, warmup):
         skey, toks, bnd = WORKLOADS[name]
         # "-ckpt-": the same shape with checkpoint-shaped matrices (three widths per matrix, ragged slabs,
         # dropped ranks) instead of one width per expert
-        blocks = blocks_of(skey, "checkpoint" if "-ckpt-" in name else "uniform")
+        blocks = blocks_of(skey, "checkpoint" if "-ckpt-" in name else "super2" if "-super2-" in name else "uniform")
         stack = SPECS[skey].n_layers > 1
         if stack:       # one step = one pass over the whole stack
             r, inp = run_workload(blocks, SPECS[skey], toks, max(2, steps // len(blocks)), max(1, warmup // len(blocks)),
@@ -568,7 +596,7 @@ def main() -> int:
                                f"{res['layers_in_rotation']} distinct layers in rotation "
                                f"({'cold' if res['layers_in_rotation'] > 1 else 'warm'} weights)",
                    "tokens": tokens, "mean_bits": sum(bits) / len(bits), "active_experts": res["active_experts"],
-                   "device": get_cuda_device_name(), "layer_build_s": round(built[shape_key + "/build_s"], 2),
+                   "device": get_cuda_device_name(), "layer_build_s": round(build_seconds[id(blocks)], 2),
                    "launch": res["launch"], "routing": res["routing"], "fused_kernel": bool(res.get("fused")),
                    "activation_dtype": "bf16",
                    "arithmetic": "bf16 activations in, f16 MFMA operands, fp32 accumulation"},

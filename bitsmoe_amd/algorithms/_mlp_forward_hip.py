@@ -96,6 +96,7 @@ class MatrixSet:
         self.regular = bool(info[4])
         self.fast_capable = bool(int(info[7]) & 1)   # the wave-native fast kernels can take this set
         self.role = -1                               # -1 until prepare() has re-laid the payload out
+        self.wide_slabs = 0                          # 64-row slabs of 6/8/16-bit rows in the prepared set's side table
 
     @property
     def handle(self) -> ctypes.c_void_p:
@@ -111,6 +112,9 @@ class MatrixSet:
         with torch.cuda.device(self.device):
             _capi.check(_lib.bitsmoe_matset_prepare(self._handle, int(role), _stream_ptr(self.device)))
         self.role = int(role)
+        info = (ctypes.c_int64 * 8)()
+        _capi.check(_lib.bitsmoe_matset_info(self._handle, info))
+        self.wide_slabs = int(info[7]) >> 8
         return True
 
     def is_current(self) -> bool:

@@ -50,7 +50,15 @@ def build_library(verbose: bool = True, jobs: int = 8, only: list[str] | None = 
     lib_path = CSRC / ("libbitsmoe_hip_timeline.so" if timeline else LIB_NAME)
     objdir.mkdir(exist_ok=True)
     srcs = sources()
-    stale = [s for s in srcs if only and s.name not in only and not (objdir / (s.stem + ".o")).exists()]
+    # with `only`: also every source whose object is missing or older than a header (the objects share struct layouts)
+    headers = [*CSRC.glob("*.h"), CSRC.parent.parent / "include" / "bitsmoe_hip.h"]
+    newest_header = max(h.stat().st_mtime for h in headers if h.exists())
+
+    def out_of_date(src: Path) -> bool:
+        obj = objdir / (src.stem + ".o")
+        return not obj.exists() or obj.stat().st_mtime < newest_header
+
+    stale = [s for s in srcs if only and s.name not in only and out_of_date(s)]
     todo = [s for s in srcs if not only or s.name in only or s in stale]
 
     def compile_one(src: Path) -> Path:

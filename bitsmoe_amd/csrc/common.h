@@ -96,6 +96,22 @@ int launch_forward_decode_fused(const bitsmoe_matset* gate, const bitsmoe_matset
                                 int64_t ldu, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int rank_out,
                                 int I, float* rank_accum, const DecodeRouted* routed, bitsmoe_profile* prof, hipStream_t st);
 
+// The side kernels for the wide rows of prepared sets (forward_wide.hip).  Gate/up: adds the wide rows' share to the
+// gate and up sums the fast kernel has written -- fp32 sums [A, I] by atomics (part 0 of the decode path's partial
+// results), or f16 sums (the grouped-GEMM path) by a plain read-add-write.  Down: reads z = silu(G) * U as f16
+// [A, I] (z_f16) or forms it from `n_part` fp32 partial sums, and adds the wide rows' outputs, scaled by the
+// routing weight, into rank_accum by atomics: after whatever writes or clears rank_accum.  Both need the routing
+// tables.  No-ops for sets without wide rows.
+bool has_wide_rows(const bitsmoe_matset* set);
+// every row of the three sets is wide (dense experts): the side kernels are the whole forward
+bool only_wide_rows(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down);
+int launch_wide_gateup(const bitsmoe_matset* gate, const bitsmoe_matset* up, const void* h_gate, const void* h_up,
+                       int act_dtype, int Rg, int Ru, int64_t ldg, int64_t ldu, const int32_t* tok, const int32_t* off,
+                       int64_t A, int I, void* G, void* U, bool sums_f16, hipStream_t st);
+int launch_wide_down(const bitsmoe_matset* down, const void* g_or_z, const float* u, bool z_f16, int n_part,
+                     int64_t part_stride, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int I,
+                     int rank_out, float* rank_accum, hipStream_t st);
+
 // How many partial results of the two fp32 intermediates the decode path's workspace holds (the gate/up kernel
 // may split its contraction over workgroups when there are few assignments).
 inline int decode_part_capacity(int64_t n_assign) { return n_assign <= 1024 ? 4 : n_assign <= 4096 ? 2 : 1; }
@@ -174,7 +190,7 @@ struct bitsmoe_matset {
     int32_t min_rank = 0;             // smallest logical rank
     bool regular = false;             // every matrix: 2/3/4-bit, k_slab % 16 == 0, full tiles
     bool regular64 = false;           // ... and every slab has exactly 64 rows, payload 16-byte aligned
-    bool fast_ok = false;             // every slab 2/3/4-bit over full 128-column tiles: bitsmoe_matset_prepare can take the set
+    bool fast_ok = false;             // every slab spans all column tiles: bitsmoe_matset_prepare can take the set
     int role = -1;                    // -1: not prepared; 0: gate/up layout; 1: down layout
     bool rank_chunked8 = false;       // slab i holds local rows 64*i.., and every aligned run of 8 local rows
                                       // maps to 8 consecutive logical ranks starting at a multiple of 8
@@ -201,6 +217,20 @@ struct bitsmoe_matset {
     std::vector<std::vector<int32_t>> rank_idx_host;
     bitsmoe::FastExpert* d_fast_experts = nullptr;   // [n_experts]
     bitsmoe::FastSlab* d_fast_slabs = nullptr;       // [n_experts][max_slabs]
+    // Rows of 6-, 8- and 16-bit slabs ("wide" rows) are no part of the prepared copy above: they sit in a side
+    // table of 64-row slabs of f16 weights (level * scale, or the stored half), laid out as the 16x16x32 MFMA's
+    // second operand, and the side kernels of forward_wide.hip add their share to what the fast kernels compute.
+    int64_t wide_slabs = 0;               // all experts
+    int64_t narrow_rows = 0;              // rows of 1/2/3/4-bit slabs, all experts (0: dense experts, wide rows only)
+    std::vector<int32_t> wide_first_host; // [n_experts + 1]: expert e owns wide slabs [wide_first[e], wide_first[e + 1])
+    int32_t n_wide_experts = 0;           // experts with at least one wide slab
+    int32_t* d_wide_tables = nullptr;     // one allocation: wide_first, wide_experts, rank' and source of every row, s'
+    const int32_t* d_wide_first = nullptr;
+    const int32_t* d_wide_experts = nullptr;
+    const int32_t* d_wide_rank = nullptr; // [wide_slabs * 64], -1 for padding rows
+    const int32_t* d_wide_src = nullptr;  // (source slab << 8) | row inside it, -1 for padding rows
+    const __half* d_wide_s = nullptr;
+    __half* d_wide = nullptr;             // [wide_slabs][n_tiles][8192]
     int device = -1;
     std::vector<bitsmoe_matrix_desc> descs;
     std::vector<std::vector<int32_t>> slab_meta_host;

@@ -51,8 +51,9 @@ extern "C" size_t bitsmoe_forward_workspace_bytes(int64_t n_tokens, int64_t n_as
     (void)n_experts;
     (void)rank_out;
     if (n_assign < 0 || intermediate_size < 0) return 0;
-    // two fp32 [A, I] intermediates (gate and up outputs), several partial results of them for small batches
-    const size_t inter = align_up((size_t)n_assign * (size_t)intermediate_size * sizeof(float), 256);
+    // two fp32 [A, I] intermediates (gate and up outputs), several partial results of them for small batches;
+    // the fast kernels keep whole 128-column tiles per row
+    const size_t inter = align_up((size_t)n_assign * align_up((size_t)intermediate_size, N_TILE) * sizeof(float), 256);
     return 2 * inter * (size_t)decode_part_capacity(n_assign) + 256;
 }
 
@@ -63,8 +64,7 @@ static int resolve_path(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
     const bool decode_ok = decode_path_supported(gate, up, down, intermediate_size);
     const bool mfma_ok = mfma_path_supported(gate, up, down, intermediate_size);
     if (path == BITSMOE_PATH_MFMA && !mfma_ok) {
-        set_error("MFMA path needs matrix sets prepared with bitsmoe_matset_prepare (gate/up role 0, down role 1), "
-                  "intermediate_size a multiple of 128 and 16-byte aligned scale / s / rank_idx buffers");
+        set_error("MFMA path needs matrix sets prepared with bitsmoe_matset_prepare (gate/up role 0, down role 1)");
         return BITSMOE_E_UNSUPPORTED;
     }
     if (path == BITSMOE_PATH_DECODE && !decode_ok) {
@@ -72,6 +72,8 @@ static int resolve_path(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
         return BITSMOE_E_UNSUPPORTED;
     }
     if (path != BITSMOE_PATH_AUTO) return path;
+    // dense experts (wide rows only): the decode launcher runs the side kernels alone, at any batch size
+    if (decode_ok && only_wide_rows(gate, up, down)) return BITSMOE_PATH_DECODE;
     // grouped GEMM from 14 assignments per expert on average (measured crossovers on layers of 64,
     // 128 and 512 experts: 12 to 16; the decode kernels re-stream the payload for every 16
     // assignments, the grouped GEMM pays for a longer launch chain)
@@ -87,7 +89,7 @@ extern "C" size_t bitsmoe_forward_workspace_bytes_sets(const bitsmoe_matset* gat
     if (!gate || !up || !down || n_assign < 0) return 0;
     const int I = gate->intermediate_size;
     const int chosen = resolve_path(gate, up, down, n_assign, I, path);
-    if (chosen == BITSMOE_PATH_MFMA) return mfma_workspace_bytes(gate, up, down, n_tokens, n_assign, I);
+    if (chosen == BITSMOE_PATH_MFMA) return mfma_workspace_bytes(gate, up, down, n_tokens, n_assign, gate->n_tiles * N_TILE);
     return bitsmoe_forward_workspace_bytes(n_tokens, n_assign, I, gate->n_experts, 0);
 }
 
@@ -182,16 +184,19 @@ static int forward_strided_impl(const bitsmoe_matset* gate, const bitsmoe_matset
     }
     BITSMOE_REQUIRE(((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
 
+    // The fast kernels work on whole 128-column tiles: their intermediates have `cols` columns per row, and the
+    // prepared weights of the columns past the matrices' last one are zeros.
+    const int cols = gate->n_tiles * N_TILE;
     if (chosen == BITSMOE_PATH_MFMA)
         return launch_forward_mfma(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
-                                   token_indices, expert_offsets, route_w, n_assign, rank_out, intermediate_size, rank_accum,
+                                   token_indices, expert_offsets, route_w, n_assign, rank_out, cols, rank_accum,
                                    workspace, front_done, profile, st);
-    const size_t inter = align_up((size_t)n_assign * (size_t)intermediate_size * sizeof(float), 256);
+    const size_t inter = align_up((size_t)n_assign * (size_t)cols * sizeof(float), 256);
     float* G = (float*)workspace;
     float* U = (float*)((char*)workspace + inter);
     if (chosen == BITSMOE_PATH_DECODE)
         return launch_forward_decode(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
-                                     token_indices, expert_offsets, route_w, n_assign, rank_out, intermediate_size,
+                                     token_indices, expert_offsets, route_w, n_assign, rank_out, cols,
                                      rank_accum, G, U, (int64_t)(inter / sizeof(float)), decode_part_capacity(n_assign), nullptr,
                                      profile, st);
     return launch_forward_generic(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
@@ -274,12 +279,13 @@ extern "C" int bitsmoe_moe_forward_routed(const bitsmoe_matset* gate, const bits
         resolve_path(gate, up, down, n_flat, intermediate_size, path) == BITSMOE_PATH_DECODE &&
         decode_inline_route_ok(gate, up, down, h_gate, h_up, rank_gate, rank_up, ld_gate, ld_up, n_tokens, top_k,
                                intermediate_size)) {
-        const size_t inter = align_up((size_t)n_flat * (size_t)intermediate_size * sizeof(float), 256);
+        const int cols = gate->n_tiles * N_TILE;
+        const size_t inter = align_up((size_t)n_flat * (size_t)cols * sizeof(float), 256);
         float* G = (float*)workspace;
         float* U = (float*)((char*)workspace + inter);
         const DecodeRouted routed = {selected, ids_are_i64, weights, top_k, local_to_global, global_to_local, n_global};
         return launch_forward_decode(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
-                                     nullptr, nullptr, nullptr, n_flat, rank_out, intermediate_size, rank_accum, G, U,
+                                     nullptr, nullptr, nullptr, n_flat, rank_out, cols, rank_accum, G, U,
                                      (int64_t)(inter / sizeof(float)), decode_part_capacity(n_flat), &routed, profile, st);
     }
     // Otherwise: routing tables at the end of the workspace, then the table form (which reports what is wrong
@@ -295,7 +301,7 @@ extern "C" int bitsmoe_moe_forward_routed(const bitsmoe_matset* gate, const bits
     RouteSideJobs jobs;
     const bool carry = options().route_jobs != 0 && shapes_ok && resolve_path(gate, up, down, n_flat, intermediate_size, path) == BITSMOE_PATH_MFMA &&
                        mfma_front_jobs(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
-                                       n_flat, intermediate_size, workspace, &jobs);
+                                       n_flat, gate->n_tiles * N_TILE, workspace, &jobs);
     int front_done = 0;
     const int rc = route_with_jobs(selected, ids_are_i64, weights, global_to_local, n_global, n_tokens, top_k, E, tok, off, rw,
                                    route_ws, bitsmoe_route_workspace_bytes(n_flat, E), carry ? &jobs : nullptr, &front_done, st);

@@ -702,8 +702,7 @@ static inline void record(bitsmoe_profile* p, int i, hipStream_t st) {
 bool decode_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I) {
     const int n_tiles = (I + N_TILE - 1) / N_TILE;
     const size_t z_bytes = (size_t)MAX_A * (n_tiles * N_TILE + 8) * 2 + MAX_A * ZSUM_STRIDE * 4 + DN_SLABS_PER_WG * SLAB_ROWS * 8 + MAX_A * 8;
-    return n_tiles <= ZSUM_STRIDE && gate->role == ROLE_GATE_UP && up->role == ROLE_GATE_UP && down->role == ROLE_DOWN && z_bytes <= 65536 &&
-           I % N_TILE == 0;
+    return n_tiles <= ZSUM_STRIDE && gate->role == ROLE_GATE_UP && up->role == ROLE_GATE_UP && down->role == ROLE_DOWN && z_bytes <= 65536;
 }
 
 // Can the decode kernels find their assignments among the routed ids themselves (no routing tables)?
@@ -711,6 +710,7 @@ bool decode_inline_route_ok(const bitsmoe_matset* gate, const bitsmoe_matset* up
                             const void* h_up, int Rg, int Ru, int64_t ldg, int64_t ldu, int64_t T, int top_k, int I) {
     const int64_t n_flat = T * top_k;
     if (options().route_inline == 0) return false;       // always build routing tables first (experiments)
+    if (has_wide_rows(gate) || has_wide_rows(up) || has_wide_rows(down)) return false;      // (their side kernels read the tables)
     if (!(decode_path_supported(gate, up, down, I) && walk_possible(gate, up, h_gate, h_up, Rg, Ru, ldg, ldu) &&
           options().decode_fused_z <= 0 && n_flat > 0 && n_flat <= ROUTE_INLINE_MAX_FLAT &&
           T <= ROUTE_INLINE_MAX_ROWS))
@@ -733,6 +733,26 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
                           const DecodeRouted* routed, bitsmoe_profile* prof, hipStream_t st) {
     const int E = gate->n_experts;
     const int n_tiles = gate->n_tiles;
+    // Dense experts (every row wide): the 2/3/4-bit kernels would run over padding only.  Clear the sums and the
+    // output, then the side kernels alone.
+    if (only_wide_rows(gate, up, down) && tok && off && rw) {
+        record(prof, 0, st);
+        const int64_t n1 = inter_floats + A * (int64_t)I, n2 = T * (int64_t)rank_out;
+        hipLaunchKernelGGL(k_fill_zero2, dim3((unsigned)std::min<int64_t>((std::max(n1, n2) + 255) / 256, 2048)), dim3(256), 0, st, G,
+                           n1, rank_accum, n2);
+        BITSMOE_HIP_TRY(hipGetLastError());
+        record(prof, 1, st);
+        int rc = launch_wide_gateup(gate, up, h_gate, h_up, act_dtype, Rg, Ru, ldg, ldu, tok, off, A, I, G, U, false, st);
+        if (rc != BITSMOE_OK) return rc;
+        record(prof, 2, st);
+        record(prof, 3, st);
+        rc = launch_wide_down(down, G, U, false, 1, 2 * inter_floats, tok, off, rw, A, I, rank_out, rank_accum, st);
+        if (rc != BITSMOE_OK) return rc;
+        record(prof, 4, st);
+        record(prof, 5, st);
+        if (prof) prof->recorded = true;
+        return BITSMOE_OK;
+    }
     // The whole chain in one kernel per (expert, tile) where the sets allow it (option decode_fused = 0 / 1: never /
     // wherever possible).
     if (options().decode_fused != 0 && options().decode_fused_z <= 0 &&
@@ -761,8 +781,9 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     // matrices of every expert share bit-width and slab count, and (expert, tile) pairs alone fill most of
     // the chip.  BITSMOE_DECODE_FUSED_Z=0 / 1 switches it off / on regardless of the size (experiments).
     const int fused_env = options().decode_fused_z;
+    const bool wide_gu = has_wide_rows(gate) || has_wide_rows(up);
     const bool fused_possible = walk && gate->all_affine && up->all_affine && gate->prep_max_slabs == up->prep_max_slabs &&
-                                gate->expert_bits == up->expert_bits;
+                                gate->expert_bits == up->expert_bits && !wide_gu;
     const bool fused_z = fused_possible && fused_env > 0;
     if (!walk) {
         // G and U are adjacent in the workspace: one range; rank_accum is the second
@@ -875,6 +896,11 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         with_mode(launch_gateup_mode, std::false_type{});
     }
     BITSMOE_HIP_TRY(hipGetLastError());
+    // rows of 6-, 8- and 16-bit slabs: their share of the gate and up sums, added to the first partial result
+    if (wide_gu) {
+        const int rc = launch_wide_gateup(gate, up, h_gate, h_up, act_dtype, Rg, Ru, ldg, ldu, tok, off, A, I, G, U, false, st);
+        if (rc != BITSMOE_OK) return rc;
+    }
     record(prof, 2, st);
     // z formed once by a small launch of its own instead of by every down workgroup: on the chunk grid (full
     // 16-assignment chunks: eight dependent round trips of two rows each in every one of the workgroups that share
@@ -945,6 +971,11 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     else
         with_mode(launch_down_mode, std::false_type{});
     BITSMOE_HIP_TRY(hipGetLastError());
+    if (has_wide_rows(down)) {      // (behind the gate/up kernel, which cleared rank_accum)
+        const int rc = launch_wide_down(down, down_g, down_u, split_z, split_z ? 1 : parts_in, part_stride, tok, off, rw, A, I,
+                                        rank_out, rank_accum, st);
+        if (rc != BITSMOE_OK) return rc;
+    }
     record(prof, 4, st);
     record(prof, 5, st);      // (the combine too)
     if (prof) prof->recorded = true;

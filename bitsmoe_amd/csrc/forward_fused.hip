@@ -609,7 +609,8 @@ bool decode_fused_possible(const bitsmoe_matset* gate, const bitsmoe_matset* up,
                            const void* h_gate, const void* h_up, int Rg, int Ru, int64_t ldg, int64_t ldu, int I) {
     return decode_path_supported(gate, up, down, I) && walk_possible(gate, up, h_gate, h_up, Rg, Ru, ldg, ldu) &&
            gate->uniform_experts && up->uniform_experts && down->uniform_experts &&
-           down->prep_max_slabs <= FUSED_MAX_DOWN_SLABS && I % N_TILE == 0;
+           down->prep_max_slabs <= FUSED_MAX_DOWN_SLABS &&
+           !has_wide_rows(gate) && !has_wide_rows(up) && !has_wide_rows(down);
 }
 
 // Measured on one MI355X under graph replay against the two-kernel form (cold weights): 64 tokens on the 128-expert

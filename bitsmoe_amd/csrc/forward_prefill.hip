@@ -1168,7 +1168,8 @@ static inline void record(bitsmoe_profile* p, int i, hipStream_t st) {
 }
 
 bool mfma_path_supported(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int I) {
-    return gate->role == ROLE_GATE_UP && up->role == ROLE_GATE_UP && down->role == ROLE_DOWN && I % N_TILE == 0 &&
+    (void)I;
+    return gate->role == ROLE_GATE_UP && up->role == ROLE_GATE_UP && down->role == ROLE_DOWN &&
            gate->vector_aligned && up->vector_aligned && down->vector_aligned;
 }
 
@@ -1337,7 +1338,8 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
         // memory, no SiLU pass).  Measured at 4096 tokens on the 128-expert layer: 241 us for the two launches against
         // 202 + 25 us -- two half-size grids end in two tails, and the epilogue waits for the gate sums -- so it is
         // off unless asked for.
-        const bool split = options().prefill_split > 0;
+        const bool wide_gu = has_wide_rows(gate) || has_wide_rows(up);
+        const bool split = options().prefill_split > 0 && !wide_gu;      // (the side kernel adds to the sums before SiLU)
         auto launch = [&](auto kernel, int proj_sel, int fuse) -> hipError_t {
             const int64_t wgs = (max_mtiles + 31) / 32 * 32 * (proj_sel < 0 ? 2 : 1) * n_tp;
             hipLaunchKernelGGL(kernel, dim3((unsigned)wgs), dim3(256), 0, st, gate->d_fast_experts, gate->d_fast_slabs,
@@ -1351,6 +1353,11 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
             record(prof, 2, st);
         } else {
             BITSMOE_HIP_TRY(direct ? launch(k_gateup_mfma<true>, -1, 0) : launch(k_gateup_mfma<false>, -1, 0));
+            if (wide_gu) {      // rows of 6-, 8- and 16-bit slabs: their share of the (f16) gate and up sums
+                const int rc = launch_wide_gateup(gate, up, h_gate, h_up, act_dtype, Rg, Ru, ldg_in, ldu_in, tok, off, A, I, z, Ubuf,
+                                                  true, st);
+                if (rc != BITSMOE_OK) return rc;
+            }
             record(prof, 2, st);
             const int64_t n8 = A * (int64_t)I / 8;
             hipLaunchKernelGGL(k_silu_mul_f16, dim3((unsigned)std::min<int64_t>((n8 + 255) / 256, 4096)), dim3(256), 0, st, z,
@@ -1375,6 +1382,10 @@ int launch_forward_mfma(const bitsmoe_matset* gate, const bitsmoe_matset* up, co
                                down->prep_max_slabs, y, ldy, token_start, counted ? token_count : nullptr, token_list, rw,
                                rank_out, rank_accum);
         BITSMOE_HIP_TRY(hipGetLastError());
+        if (has_wide_rows(down)) {      // (behind the combine, which writes every element of rank_accum)
+            const int rc = launch_wide_down(down, z, nullptr, true, 1, 0, tok, off, rw, A, I, rank_out, rank_accum, st);
+            if (rc != BITSMOE_OK) return rc;
+        }
     }
     record(prof, 5, st);
     if (prof) prof->recorded = true;

@@ -130,7 +130,7 @@ static int validate_matrix(const bitsmoe_matrix_desc& d, int e, int I,
         if (!(bits == 2 || bits == 3 || bits == 4) || (k_slab % K_STAGE) != 0 ||
             tile_end - tile_off != n_tiles_mat)
             *regular = false;
-        if (!(bits == 2 || bits == 3 || bits == 4) || tile_end - tile_off != n_tiles_mat) *fast_ok = false;
+        if (tile_end - tile_off != n_tiles_mat) *fast_ok = false;
         if (k_slab != K_SLAB) *regular64 = false;
         const int64_t words_tile = (int64_t)k_slab * MICROS * words_per_row(bits);
         for (int t = tile_off; t < tile_end; ++t) {
@@ -143,7 +143,8 @@ static int validate_matrix(const bitsmoe_matrix_desc& d, int e, int I,
                             "expert %d tile %d: scale range exceeds scale size %lld", e, t, (long long)d.scale_len);
             BITSMOE_REQUIRE(n_valid >= 1 && n_valid <= N_TILE, "expert %d tile %d: n_valid=%d outside [1,128]", e, t, n_valid);
             if (n_valid != N_TILE || (pack_off & 3) != 0) *regular = false;
-            if (n_valid != N_TILE) *fast_ok = false;
+            // (the last tile of a slab may be narrower: the matrix's own last columns)
+            if (n_valid != N_TILE && !(t == tile_end - 1 && n_valid == I - (n_tiles_mat - 1) * N_TILE)) *fast_ok = false;
         }
         rows_seen += k_slab;
     }
@@ -270,6 +271,8 @@ extern "C" void bitsmoe_matset_destroy(bitsmoe_matset* set) {
     if (set->d_prep_tasks) (void)hipFree(set->d_prep_tasks);
     if (set->d_fast_experts) (void)hipFree(set->d_fast_experts);
     if (set->d_fast_slabs) (void)hipFree(set->d_fast_slabs);
+    if (set->d_wide_tables) (void)hipFree(set->d_wide_tables);
+    if (set->d_wide) (void)hipFree(set->d_wide);
     delete set;
 }
 
@@ -282,7 +285,8 @@ extern "C" int bitsmoe_matset_info(const bitsmoe_matset* set, int64_t info[8]) {
     info[4] = set->regular ? 1 : 0;
     info[5] = set->max_slabs;
     info[6] = set->min_rank;
-    info[7] = (set->fast_ok ? 1 : 0) | (set->role >= 0 ? 2 : 0) | (set->role == 0 && set->all_affine && set->rank_chunked8 ? 4 : 0);
+    info[7] = (set->fast_ok ? 1 : 0) | (set->role >= 0 ? 2 : 0) | (set->role == 0 && set->all_affine && set->rank_chunked8 ? 4 : 0) |
+              (set->wide_slabs << 8);
     return BITSMOE_OK;
 }
 

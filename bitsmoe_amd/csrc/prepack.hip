@@ -1,6 +1,7 @@
 // One-time re-layout of a matrix set's payload into the wave64-native field layout
 // (wave_layout.h) and the dense dequantiser that reads it back (parity check of the layout).
 #include "wave_layout.h"
+#include "wide_layout.h"
 
 #include <algorithm>
 #include <cstring>
@@ -34,13 +35,15 @@ __device__ inline int source_level(const MatView& mv, const int32_t* __restrict_
     if (src < 0) return 0;
     const int s = src >> 8, r = src & 255;
     const int w = mv.slab_meta[s * 4 + 0], k_slab = mv.slab_meta[s * 4 + 1];
-    const uint32_t* __restrict__ blk = mv.payload + mv.tile_meta[(mv.slab_meta[s * 4 + 3] + t) * 3 + 0];
+    const int32_t* tm = mv.tile_meta + (mv.slab_meta[s * 4 + 3] + t) * 3;
+    if (col >= tm[2]) return 0;          // (columns past the matrix's last one: whatever the payload holds there)
+    const uint32_t* __restrict__ blk = mv.payload + tm[0];
     const int stage = r >> 4, rr = r & 15, micro = col >> 5, lane = col & 31;
     const int rows_cur = min(K_STAGE, k_slab - stage * K_STAGE);
     const uint32_t* words = blk + stage * (K_STAGE * MICROS * w) + micro * (rows_cur * w) + rr * w;
     int u = 0;
     for (int p = 0; p < w; ++p) u |= (int)((words[p] >> lane) & 1u) << p;
-    return u - level_offset(w);
+    return w == 1 ? 2 * u - 1 : u - level_offset(w);      // (1-bit codes are the levels -1 / +1)
 }
 
 // grid: (prepared slab tasks, tiles); every thread builds whole output words of one block.  Reads the
@@ -156,6 +159,53 @@ __global__ __launch_bounds__(64) void k_prepare_rows(const MatView* __restrict__
     if (t == 0) const_cast<__half*>(fe.s)[fs.rank_off + row] = __float2half(sv);
 }
 
+// The side table of wide rows (wide_layout.h) from the caller's layout.  grid (wide slabs, tiles).
+__global__ __launch_bounds__(256) void k_prepack_wide(const MatView* __restrict__ views, const int32_t* __restrict__ slab_expert,
+                                                      const int32_t* __restrict__ wide_src, int role, int n_tiles,
+                                                      __half* __restrict__ wide, __half* __restrict__ wide_s) {
+    const int ws = blockIdx.x, t = blockIdx.y;
+    const MatView mv = views[slab_expert[ws]];
+    __half* __restrict__ out = wide + ((int64_t)ws * n_tiles + t) * WIDE_BLOCK;
+    for (int idx = threadIdx.x; idx < WIDE_BLOCK; idx += blockDim.x) {
+        const int row = idx >> 7, col = idx & 127;
+        const int src = wide_src[ws * SLAB_ROWS + row];
+        float v = 0.0f;
+        if (src >= 0) {
+            const int s = src >> 8, r = src & 255;
+            const int bits = mv.slab_meta[s * 4 + 0], k_slab = mv.slab_meta[s * 4 + 1];
+            const int32_t* tm = mv.tile_meta + (mv.slab_meta[s * 4 + 3] + t) * 3;
+            if (col < tm[2]) {
+                const int w = words_per_row(bits);
+                const int stage = r >> 4, rr = r & 15, micro = col >> 5, lane = col & 31;
+                const int rows_cur = min(K_STAGE, k_slab - stage * K_STAGE);
+                v = decode_from_row_words(mv.payload + tm[0] + stage * (K_STAGE * MICROS * w) + micro * (rows_cur * w) + rr * w, bits, lane);
+                if (bits != 16) v *= __half2float(mv.scale[tm[1] + r]);
+            }
+        }
+        out[wide_index(role, row, col)] = __float2half(v);
+    }
+    if (t == 0 && threadIdx.x < SLAB_ROWS) {
+        const int src = wide_src[ws * SLAB_ROWS + threadIdx.x];
+        wide_s[ws * SLAB_ROWS + threadIdx.x] = src >= 0 ? mv.s[mv.slab_meta[(src >> 8) * 4 + 2] + (src & 255)] : __float2half(0.0f);
+    }
+}
+
+// Dense fp32 dequantisation of an expert's wide rows FROM THE SIDE TABLE (rows in the caller's local row order).
+// grid (wide slabs of the expert, tiles).
+__global__ __launch_bounds__(256) void k_dequant_wide(MatView mv, const __half* __restrict__ wide, const int32_t* __restrict__ wide_src,
+                                                      int ws0, int role, int n_tiles, int I, float* __restrict__ out) {
+    const int ws = ws0 + blockIdx.x, t = blockIdx.y;
+    const __half* __restrict__ blk = wide + ((int64_t)ws * n_tiles + t) * WIDE_BLOCK;
+    for (int idx = threadIdx.x; idx < WIDE_BLOCK; idx += blockDim.x) {
+        const int row = idx >> 7, col = idx & 127;
+        const int src = wide_src[ws * SLAB_ROWS + row];
+        const int c = t * N_TILE + col;
+        if (src < 0 || c >= I) continue;
+        const int local_row = mv.slab_meta[(src >> 8) * 4 + 2] + (src & 255);
+        out[(int64_t)local_row * I + c] = __half2float(blk[wide_index(role, row, col)]);
+    }
+}
+
 // Dense fp32 dequantisation FROM THE PREPARED COPY, written to mirror the decode of the hot kernels
 // (fields, not planes); rows in the caller's local row order, output identical to k_dequant_matrix.
 // grid (prepared slabs of the expert, tiles).
@@ -222,12 +272,15 @@ extern "C" int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* s
     if (rc != BITSMOE_OK) {
         // nothing of a failed attempt stays behind: the set remains usable by the generic kernels
         void** owned[] = {(void**)&set->d_prepared, (void**)&set->d_fast_experts, (void**)&set->d_fast_slabs,
-                          (void**)&set->d_scale_s, (void**)&set->d_prepared_rows, (void**)&set->d_prep_tasks};
+                          (void**)&set->d_scale_s, (void**)&set->d_prepared_rows, (void**)&set->d_prep_tasks,
+                          (void**)&set->d_wide_tables, (void**)&set->d_wide};
         for (void** p : owned) {
             if (*p) (void)hipFree(*p);
             *p = nullptr;
         }
         set->role = -1;
+        set->wide_slabs = 0;
+        set->n_wide_experts = 0;
     }
     return rc;
 }
@@ -236,22 +289,28 @@ static inline int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * 
 
 static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
     if (!set->fast_ok || set->total_slabs == 0) {
-        set_error("matrix set holds slabs of other widths than 2, 3 or 4 bits, or tiles of fewer than 128 columns: "
-                  "only the generic kernels can run it");
+        set_error("matrix set is empty or holds a slab that does not span all column tiles: only the generic kernels can run it");
         return BITSMOE_E_UNSUPPORTED;
     }
     const int E = set->n_experts, n_tiles = set->n_tiles;
     // The slabs of the prepared copy: the caller's local rows in their order, cut every 64 rows; gate/up
     // sets in whole groups of GU_SLABS slabs (what one workgroup of the walking kernel contracts over
     // between two barriers), a group stored at ONE width, the widest among its rows.
+    // Rows of 6-, 8- and 16-bit slabs are kept out of it: they go to the side table of wide rows (below).
     const int unit = role == ROLE_GATE_UP ? GU_SLABS : 1;
+    auto is_wide = [](int bits) { return bits > 4; };
     std::vector<int> n_ps(E);
+    std::vector<int32_t> wide_first(E + 1, 0);
     int pms = 0;
+    int64_t narrow_rows = 0;
     for (int e = 0; e < E; ++e) {
-        int64_t rows = 0;
-        for (int si = 0; si < set->descs[e].num_slabs; ++si) rows += set->slab_meta_host[e][si * 4 + 1];
+        int64_t rows = 0, rows_wide = 0;
+        for (int si = 0; si < set->descs[e].num_slabs; ++si)
+            (is_wide(set->slab_meta_host[e][si * 4 + 0]) ? rows_wide : rows) += set->slab_meta_host[e][si * 4 + 1];
         n_ps[e] = (int)round_up(std::max<int64_t>((rows + SLAB_ROWS - 1) / SLAB_ROWS, 1), unit);
         pms = std::max(pms, n_ps[e]);
+        narrow_rows += rows;
+        wide_first[e + 1] = wide_first[e] + (int32_t)((rows_wide + SLAB_ROWS - 1) / SLAB_ROWS);
     }
     set->prep_max_slabs = pms;
     std::vector<FastSlab> fslabs((size_t)E * pms, FastSlab{0, 0, 0, 0});
@@ -275,10 +334,11 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
         int64_t p = 0;
         for (int si = 0; si < set->descs[e].num_slabs; ++si) {
             const int bits = slab[si * 4 + 0], k_slab = slab[si * 4 + 1], rank_off = slab[si * 4 + 2];
+            if (is_wide(bits)) continue;
             for (int r = 0; r < k_slab; ++r, ++p) {
                 rr[p] = rk[rank_off + r];
                 rs[p] = (si << 8) | r;
-                width[p / SLAB_ROWS] = std::max(width[p / SLAB_ROWS], bits);
+                width[p / SLAB_ROWS] = std::max(width[p / SLAB_ROWS], std::max(bits, 2));      // (1-bit levels fit 2-bit fields)
             }
         }
         // Padding rows (zero scales) behind the last row.  When the real rows are the identity (row k holds
@@ -288,7 +348,7 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
         // eight that is all padding reads the ranks 0..7, the rest of a run that the last rows begin
         // continues that run, and any other padding row has rank -1 ("no such row" to every kernel).
         const int64_t rows_e = p, rows_p = (int64_t)n_ps[e] * SLAB_ROWS;
-        bool ident_e = true;
+        bool ident_e = rows_e > 0;      // (an expert without 2/3/4-bit rows: padding only, which reads the ranks 0..7)
         for (int64_t j = 0; j < rows_e && ident_e; ++j) ident_e = rr[j] == (int32_t)j;
         for (; p < rows_p; ++p) {
             const int64_t run0 = p & ~(int64_t)7;
@@ -403,6 +463,52 @@ static int prepare_impl(bitsmoe_matset* set, int32_t role, hipStream_t st) {
     hipLaunchKernelGGL(k_prepack, dim3((unsigned)tasks.size(), n_tiles), dim3(256), 0, st, set->d_views,
                        set->d_fast_experts, set->d_fast_slabs, pms, set->d_prep_tasks, ps_tab, role);
     BITSMOE_HIP_TRY(hipGetLastError());
+    // The side table of wide rows: an expert's rows of 6-, 8- and 16-bit slabs in their local order, 64 to a slab.
+    const int64_t n_ws = wide_first[E];
+    std::vector<int32_t> wide_tab;
+    if (n_ws > 0) {
+        std::vector<int32_t> wide_experts, slab_expert((size_t)n_ws);
+        std::vector<int32_t> wrank((size_t)n_ws * SLAB_ROWS, -1), wsrc((size_t)n_ws * SLAB_ROWS, -1);
+        for (int e = 0; e < E; ++e) {
+            if (wide_first[e + 1] > wide_first[e]) wide_experts.push_back(e);
+            for (int32_t j = wide_first[e]; j < wide_first[e + 1]; ++j) slab_expert[j] = e;
+            const auto& slab = set->slab_meta_host[e];
+            const auto& rk = set->rank_idx_host[e];
+            int64_t p = (int64_t)wide_first[e] * SLAB_ROWS;
+            for (int si = 0; si < set->descs[e].num_slabs; ++si) {
+                if (!is_wide(slab[si * 4 + 0])) continue;
+                for (int r = 0; r < slab[si * 4 + 1]; ++r, ++p) {
+                    wrank[p] = rk[slab[si * 4 + 2] + r];
+                    wsrc[p] = (si << 8) | r;
+                }
+            }
+        }
+        // one allocation: wide_first [E + 1], wide_experts, slab_expert, rank', source (int32 each), then s' (f16)
+        const size_t n_int = (size_t)(E + 1) + wide_experts.size() + slab_expert.size() + wrank.size() + wsrc.size();
+        const size_t int_bytes = (size_t)round_up((int64_t)n_int * 4, 256);
+        BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_wide_tables, int_bytes + (size_t)n_ws * SLAB_ROWS * 2));
+        BITSMOE_HIP_TRY(hipMalloc((void**)&set->d_wide, (size_t)n_ws * n_tiles * WIDE_BLOCK * 2));
+        wide_tab.reserve(n_int);
+        wide_tab.insert(wide_tab.end(), wide_first.begin(), wide_first.end());
+        wide_tab.insert(wide_tab.end(), wide_experts.begin(), wide_experts.end());
+        wide_tab.insert(wide_tab.end(), slab_expert.begin(), slab_expert.end());
+        wide_tab.insert(wide_tab.end(), wrank.begin(), wrank.end());
+        wide_tab.insert(wide_tab.end(), wsrc.begin(), wsrc.end());
+        BITSMOE_HIP_TRY(hipMemcpyAsync(set->d_wide_tables, wide_tab.data(), n_int * 4, hipMemcpyHostToDevice, st));
+        set->d_wide_first = set->d_wide_tables;
+        set->d_wide_experts = set->d_wide_first + (E + 1);
+        const int32_t* d_slab_expert = set->d_wide_experts + wide_experts.size();
+        set->d_wide_rank = d_slab_expert + slab_expert.size();
+        set->d_wide_src = set->d_wide_rank + wrank.size();
+        set->d_wide_s = (const __half*)((const char*)set->d_wide_tables + int_bytes);
+        set->n_wide_experts = (int32_t)wide_experts.size();
+        hipLaunchKernelGGL(k_prepack_wide, dim3((unsigned)n_ws, n_tiles), dim3(256), 0, st, set->d_views, d_slab_expert,
+                           set->d_wide_src, role, n_tiles, set->d_wide, const_cast<__half*>(set->d_wide_s));
+        BITSMOE_HIP_TRY(hipGetLastError());
+    }
+    set->wide_slabs = n_ws;
+    set->narrow_rows = narrow_rows;
+    set->wide_first_host = wide_first;
     BITSMOE_HIP_TRY(hipStreamSynchronize(st));      // (the host vectors above are read by the copies until here)
     set->fast_experts_host = fexp;
     set->prep_row_offsets = row_off;
@@ -435,5 +541,11 @@ extern "C" int bitsmoe_dequant_matrix_prepared(const bitsmoe_matset* set, int32_
                        set->d_fast_slabs + (int64_t)expert * set->prep_max_slabs, d_src, set->role, set->intermediate_size,
                        out_device);
     BITSMOE_HIP_TRY(hipGetLastError());
+    if (set->wide_slabs > 0 && set->wide_first_host[expert + 1] > set->wide_first_host[expert]) {
+        const int ws0 = set->wide_first_host[expert];
+        hipLaunchKernelGGL(k_dequant_wide, dim3(set->wide_first_host[expert + 1] - ws0, set->n_tiles), dim3(256), 0, st, mv,
+                           set->d_wide, set->d_wide_src, ws0, set->role, set->n_tiles, set->intermediate_size, out_device);
+        BITSMOE_HIP_TRY(hipGetLastError());
+    }
     return BITSMOE_OK;
 }

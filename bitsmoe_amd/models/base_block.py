@@ -33,10 +33,18 @@ _CHECK_VERSIONS = _os.environ.get("BITSMOE_BLOCK_CHECK_VERSIONS", "0") == "1"
 
 
 def _dense_via_operator() -> bool:
-    """BITSMOE_DENSE_VIA_OPERATOR=1: shared and super experts run as 16-bit packed experts of the operator."""
+    """BITSMOE_DENSE_VIA_OPERATOR=1: shared AND super experts run as 16-bit packed experts of the operator."""
     import os
 
     return os.environ.get("BITSMOE_DENSE_VIA_OPERATOR", "0") == "1"
+
+
+def _super_via_operator() -> bool:
+    """Dense "super" experts run as 16-bit packed experts of the operator, on the tokens that chose them (the
+    default); BITSMOE_SUPER_VIA_OPERATOR=0: as modules over all tokens, masked."""
+    import os
+
+    return _dense_via_operator() or os.environ.get("BITSMOE_SUPER_VIA_OPERATOR", "1") != "0"
 
 
 class BitsMoE_BaseSparseMoeBlock(nn.Module):
@@ -264,18 +272,18 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         """Dense "super" experts (reference: bitsmoe/models/base_block.py:291-307) without the reference's
         host synchronisation (`mask.any()` and boolean-mask indexing read the device per expert): the
         block stays capturable into a HIP graph when a layer has super experts.
-          * default: each super expert runs on ALL tokens and its output is scaled by the token's routing
-            weight for that expert -- zero where the token did not select it (library GEMMs; a handful of
-            experts in a few layers, so the extra rows cost little at decode sizes);
-          * BITSMOE_DENSE_VIA_OPERATOR=1: the super experts are packed as 16-bit matrices once and go through
-            the routed-expert operator like any packed expert (device-built routing tables, work
-            proportional to the tokens that selected them)."""
+          * default: the super experts are packed as 16-bit matrices once and go through the routed-expert
+            operator like any packed expert (device-built routing tables, work proportional to the tokens
+            that selected them: the operator's side kernels for 16-bit rows);
+          * BITSMOE_SUPER_VIA_OPERATOR=0 (and on the CPU): each super expert runs on ALL tokens and its output
+            is scaled by the token's routing weight for that expert -- zero where the token did not select it."""
         if not self._super_expert_items:
             return
         top_k = self.top_k
         sel = flat_selected_experts.reshape(-1, top_k)
         w = flat_route_weights_hidden.reshape(-1, top_k)
-        if _dense_via_operator():
+        if _super_via_operator() and hidden_states.is_cuda and _HAS_MLP_FORWARD_CUDA and \
+                hidden_states.dtype in (torch.float16, torch.bfloat16):
             g2l = self._super_global_to_local(hidden_states.device)
             tok, off, rw = mlp_forward_cuda.route(sel, w.to(torch.float32), g2l, len(self._super_expert_items))
             out = self._dense_operator_forward("super", [layer for _, layer in self._super_expert_items],

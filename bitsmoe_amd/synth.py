@@ -41,6 +41,8 @@ SPECS: Dict[str, LayerSpec] = {
     "c1": LayerSpec("c1", "deepseekv2", 64, 6, 2048, 1408, (0.6, 0.3, 0.1), "normal", False, 0, tokens=(16,)),
     # Qwen3-30B-A3B-shaped layer, decode
     "c2": LayerSpec("c2", "qwen3moe", 128, 8, 2048, 768, (0.8, 0.15, 0.05), "uniform", True, 0, tokens=(1, 8, 32, 64)),
+    # the same layer with an intermediate size that is no multiple of the 128-column tile (last tile: 32 columns)
+    "c2i": LayerSpec("c2i", "qwen3moe", 128, 8, 2048, 1440, (0.8, 0.15, 0.05), "uniform", True, 0, tokens=(64,)),
     # same layer, prefill
     "c3": LayerSpec("c3", "qwen3moe", 128, 8, 2048, 768, (0.8, 0.15, 0.05), "normal", True, 0, tokens=(4096,)),
     # Qwen3-Next-80B-A3B-shaped layer with a sigmoid-gated shared expert

@@ -187,19 +187,21 @@ def test_block_forward_matches_oracle(cuda_device, family, kw, tokens, fused, mo
     assert err <= 1e-2, f"{family}: normalised error {err:.3e}"
 
 
-@pytest.mark.parametrize("via_operator", [False, True])
+@pytest.mark.parametrize("dense", ["modules", "default", "operator"])
 @pytest.mark.parametrize("family,kw", [("qwen3moe", {}), ("qwen3next", {"shared_intermediate": 128}),
                                        ("deepseekv2", {"shared_intermediate": 256})])
-def test_block_with_super_and_shared_experts(cuda_device, family, kw, via_operator, monkeypatch):
+def test_block_with_super_and_shared_experts(cuda_device, family, kw, dense, monkeypatch):
     """A layer with two dense "super" experts among the routed ones (and the family's shared expert): the
-    block against the float64 restatement, with the dense experts as library GEMMs and as 16-bit packed
-    experts of the operator (BITSMOE_DENSE_VIA_OPERATOR=1); the forward does not synchronise with the
+    block against the float64 restatement, with the dense experts as library GEMMs ("modules":
+    BITSMOE_SUPER_VIA_OPERATOR=0), with the super experts as 16-bit packed experts of the operator (the default)
+    and with the shared expert there too (BITSMOE_DENSE_VIA_OPERATOR=1); the forward does not synchronise with the
     host, so it is captured into a HIP graph and every replay must equal the eager result."""
     import torch
 
     from bitsmoe_amd.synth import make_layer
 
-    monkeypatch.setenv("BITSMOE_DENSE_VIA_OPERATOR", "1" if via_operator else "0")
+    monkeypatch.setenv("BITSMOE_DENSE_VIA_OPERATOR", "1" if dense == "operator" else "0")
+    monkeypatch.setenv("BITSMOE_SUPER_VIA_OPERATOR", "0" if dense == "modules" else "1")
     spec = _small_spec(family, **kw)
     block = make_layer(spec, device=cuda_device, dtype=torch.bfloat16, seed=9, s_mode="rand", super_experts=(1, 6))
     block.prepare_runtime_fastpath(warmup=True)

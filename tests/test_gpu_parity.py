@@ -205,13 +205,18 @@ def test_prepared_layout_dequant_bit_exact(cuda_device, role, dim):
         assert np.array_equal(ms.dequant(e).cpu().numpy().view(np.uint32), ref.view(np.uint32))
 
 
-def test_irregular_sets_stay_on_generic_kernels(cuda_device):
+def test_every_packer_output_is_fast_capable(cuda_device):
+    """A last tile of fewer than 128 columns and slabs of any supported width: the prepared copy takes them all
+    (the wide widths in its side table)."""
     hip = _hip()
     rng = np.random.default_rng(1)
-    for mats in ([helpers.make_matrix(rng, 80, 160, [(2, (0, 80))])],            # a tail tile of 32 columns
-                 [helpers.make_matrix(rng, 128, 128, [(8, (0, 64)), (2, (64, 128))])]):      # an 8-bit slab
+    for mats, wide in (([helpers.make_matrix(rng, 80, 160, [(2, (0, 80))])], 0),            # a tail tile of 32 columns
+                       ([helpers.make_matrix(rng, 128, 128, [(8, (0, 64)), (2, (64, 128))])], 1),      # an 8-bit slab
+                       ([helpers.make_matrix(rng, 70, 96, [(1, (0, 70))])], 0)):              # 1-bit rows, one narrow tile
         ms = hip.MatrixSet(*helpers.to_device_lists(mats, cuda_device), intermediate_size=int(mats[0]["dim"]))
-        assert not ms.fast_capable and not ms.prepare(0)
+        assert ms.fast_capable and ms.prepare(0) and ms.wide_slabs == wide
+        ref = o.dequant_matrix(mats[0], int(mats[0]["dim"]))
+        assert np.allclose(ms.dequant_prepared(0).cpu().numpy(), ref, rtol=2.0 ** -11, atol=0.0)
 
 
 @pytest.mark.parametrize("role", [0, 1])
@@ -530,18 +535,20 @@ def test_forward_accepts_column_slices_of_one_projection(cuda_device, path_name,
     assert helpers.norm_err(out_v.cpu().numpy(), ref) <= 1e-2
 
 
-def test_forward_mfma_path_needs_prepared_sets(cuda_device):
+def test_forward_mfma_path_needs_prepared_sets(cuda_device, monkeypatch):
     import torch
 
-    from bitsmoe_amd.algorithms import _capi
+    from bitsmoe_amd.algorithms import _capi, _mlp_forward_hip
 
     hip = _hip()
-    gate, up, down = helpers.make_experts(5, 2, 80, 80, 128, choices=(8,), uniform_bits=True)   # 8-bit slabs: generic only
+    monkeypatch.setattr(_mlp_forward_hip, "_AUTO_PREPARE", False)      # (the sets stay as the caller built them)
+    gate, up, down = helpers.make_experts(5, 2, 80, 80, 128, choices=(4,), uniform_bits=True)
     sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=128) for m in (gate, up, down)]
     z = lambda *s, dt=torch.float16: torch.zeros(s, dtype=dt, device=cuda_device)
-    with pytest.raises(RuntimeError, match="MFMA path needs"):
-        hip.moe_forward_sets(z(4, 80), z(4, 80), z(4, dt=torch.int32), z(3, dt=torch.int32), z(4, dt=torch.float32),
-                             sets[0], sets[1], sets[2], 80, 128, 0, path=_capi.PATH_MFMA)
+    for path, what in ((_capi.PATH_MFMA, "MFMA path needs"), (_capi.PATH_DECODE, "decode path needs")):
+        with pytest.raises(RuntimeError, match=what):
+            hip.moe_forward_sets(z(4, 80), z(4, 80), z(4, dt=torch.int32), z(3, dt=torch.int32), z(4, dt=torch.float32),
+                                 sets[0], sets[1], sets[2], 80, 128, 0, path=path)
 
 
 def test_forward_rejects_a_rank_out_no_down_row_writes_into(cuda_device):
