@@ -134,10 +134,6 @@ class _LayerState:
         self.n_packed = block._packed_expert_count
         # dense ("super") experts among the routed ones: a second operator call on their own matrix sets
         self.has_super = bool(block._super_expert_items)
-        if self.has_super:
-            self.super_out = torch.zeros((tokens, spec.hidden_size), dtype=torch.bfloat16, device=dev)
-            self.flat_selected = self.selected.reshape(-1)
-            self.flat_weights = self.weights.reshape(-1).to(torch.bfloat16)
 
 
 def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, layers_per_step=1, block_scope=True):
@@ -155,11 +151,22 @@ def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, l
     def layer_step(i, profile=None):
         st = layers[i % n_layers]
         gate, up, down = st.sets
+        side = None
+        if st.has_super:
+            # the dense experts' matrix sets: a second call of the operator (output in hidden space), on a side stream
+            # beside the packed experts' call, as the block runs it
+            from bitsmoe_amd.models.base_block import _side_stream
+
+            cur = torch.cuda.current_stream(dev)
+            side = _side_stream(dev)
+            side.wait_stream(cur)
+            with torch.cuda.stream(side):
+                sup = st.block._super_operator_output(st.x, st.selected, st.weights)
         out = hip.moe_forward_routed(st.h_gate, st.h_up, st.selected, st.weights, st.g2l, st.l2g, gate, up, down,
                                      st.rank_out, st.isz, 0, profile=profile)
-        if st.has_super:      # (the block's own code: routing tables of the dense experts, operator, sum in hidden space)
-            st.super_out.zero_()
-            st.block._run_super_experts(st.x, st.super_out, st.flat_selected, None, st.flat_weights)
+        if side is not None:
+            cur.wait_stream(side)
+            sup.record_stream(cur)
         return out
 
     def layer_tables(i):      # (the routing tables, for the accounting and the CPU check only)

@@ -112,6 +112,14 @@ int launch_wide_down(const bitsmoe_matset* down, const void* g_or_z, const float
                      int64_t part_stride, const int32_t* tok, const int32_t* off, const float* rw, int64_t A, int I,
                      int rank_out, float* rank_accum, hipStream_t st);
 
+// Sets of dense experts only, a small batch, from the router's output: the side kernels find their assignments among the
+// routed ids themselves (no routing tables); launch_forward_wide_routed clears the sums, then two kernels.
+bool wide_routed_possible(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down, int64_t T, int top_k);
+int launch_forward_wide_routed(const bitsmoe_matset* gate, const bitsmoe_matset* up, const bitsmoe_matset* down,
+                               const void* h_gate, const void* h_up, int act_dtype, int64_t T, int Rg, int Ru, int64_t ldg,
+                               int64_t ldu, const DecodeRouted* routed, int64_t n_flat, int rank_out, int I, float* rank_accum,
+                               float* G, float* U, int64_t inter_floats, bitsmoe_profile* prof, hipStream_t st);
+
 // How many partial results of the two fp32 intermediates the decode path's workspace holds (the gate/up kernel
 // may split its contraction over workgroups when there are few assignments).
 inline int decode_part_capacity(int64_t n_assign) { return n_assign <= 1024 ? 4 : n_assign <= 4096 ? 2 : 1; }

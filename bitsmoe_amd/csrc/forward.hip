@@ -226,6 +226,7 @@ extern "C" int bitsmoe_forward_routed_is_inline(const bitsmoe_matset* gate, cons
     const int I = gate->intermediate_size;
     if (path != BITSMOE_PATH_AUTO && path != BITSMOE_PATH_DECODE) return 0;
     if (resolve_path(gate, up, down, n_tokens * top_k, I, path) != BITSMOE_PATH_DECODE) return 0;
+    if (wide_routed_possible(gate, up, down, n_tokens, top_k)) return 1;
     return decode_inline_route_ok(gate, up, down, h_gate, h_up, rank_gate, rank_up, ld_gate, ld_up, n_tokens, top_k, I) ? 1 : 0;
 }
 
@@ -275,6 +276,17 @@ extern "C" int bitsmoe_moe_forward_routed(const bitsmoe_matset* gate, const bits
                            up->max_rank_plus1 <= rank_up && up->min_rank >= 0 &&
                            (down->total_slabs == 0 || (down->min_rank < rank_out && down->max_rank_plus1 > 0)) &&
                            path >= BITSMOE_PATH_AUTO && path <= BITSMOE_PATH_MFMA;
+    if (shapes_ok && (path == BITSMOE_PATH_AUTO || path == BITSMOE_PATH_DECODE) &&
+        resolve_path(gate, up, down, n_flat, intermediate_size, path) == BITSMOE_PATH_DECODE &&
+        wide_routed_possible(gate, up, down, n_tokens, top_k)) {
+        // dense experts only: their side kernels scan the routed ids themselves
+        const int cols = gate->n_tiles * N_TILE;
+        const size_t inter = align_up((size_t)n_flat * (size_t)cols * sizeof(float), 256);
+        const DecodeRouted routed = {selected, ids_are_i64, weights, top_k, local_to_global, global_to_local, n_global};
+        return launch_forward_wide_routed(gate, up, down, h_gate, h_up, act_dtype, n_tokens, rank_gate, rank_up, ld_gate, ld_up,
+                                          &routed, n_flat, rank_out, cols, rank_accum, (float*)workspace,
+                                          (float*)((char*)workspace + inter), (int64_t)(inter / sizeof(float)), profile, st);
+    }
     if (shapes_ok && (path == BITSMOE_PATH_AUTO || path == BITSMOE_PATH_DECODE) &&
         resolve_path(gate, up, down, n_flat, intermediate_size, path) == BITSMOE_PATH_DECODE &&
         decode_inline_route_ok(gate, up, down, h_gate, h_up, rank_gate, rank_up, ld_gate, ld_up, n_tokens, top_k,

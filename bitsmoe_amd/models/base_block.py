@@ -30,6 +30,8 @@ _BUFFER_NAMES = ("payload", "rank_idx", "tile_meta", "slab_meta", "scale", "s")
 import os as _os
 
 _CHECK_VERSIONS = _os.environ.get("BITSMOE_BLOCK_CHECK_VERSIONS", "0") == "1"
+# BITSMOE_SUPER_SIDE_STREAM=0: the super experts' operator call on the caller's stream, after the packed experts'
+_SUPER_SIDE_STREAM = _os.environ.get("BITSMOE_SUPER_SIDE_STREAM", "1") != "0"
 
 
 def _dense_via_operator() -> bool:
@@ -45,6 +47,20 @@ def _super_via_operator() -> bool:
     import os
 
     return _dense_via_operator() or os.environ.get("BITSMOE_SUPER_VIA_OPERATOR", "1") != "0"
+
+
+_SIDE_STREAMS: Dict[int, "torch.cuda.Stream"] = {}
+
+
+def _side_stream(device: torch.device) -> "torch.cuda.Stream":
+    """One extra stream per device (default priority) for work that is independent of the packed experts'
+    operator call: the super experts' call runs there, between a fork and a join on the caller's stream."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    st = _SIDE_STREAMS.get(idx)
+    if st is None:
+        st = torch.cuda.Stream(device=device)
+        _SIDE_STREAMS[idx] = st
+    return st
 
 
 class BitsMoE_BaseSparseMoeBlock(nn.Module):
@@ -282,13 +298,9 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         top_k = self.top_k
         sel = flat_selected_experts.reshape(-1, top_k)
         w = flat_route_weights_hidden.reshape(-1, top_k)
-        if _super_via_operator() and hidden_states.is_cuda and _HAS_MLP_FORWARD_CUDA and \
-                hidden_states.dtype in (torch.float16, torch.bfloat16):
-            g2l = self._super_global_to_local(hidden_states.device)
-            tok, off, rw = mlp_forward_cuda.route(sel, w.to(torch.float32), g2l, len(self._super_expert_items))
-            out = self._dense_operator_forward("super", [layer for _, layer in self._super_expert_items],
-                                               hidden_states, tok, off, rw)
-            final_hidden_states.add_(out.to(hidden_states.dtype))
+        sup = self._super_operator_output(hidden_states, sel, w)
+        if sup is not None:
+            final_hidden_states.add_(sup)      # (fp32 added into the activation dtype: one kernel)
             return
         for expert_idx, layer in self._super_expert_items:
             picked = sel == expert_idx
@@ -299,6 +311,29 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
             final_hidden_states.add_(out.to(hidden_states.dtype))
 
     # ---- dense experts through the routed-expert operator ----------------------------------
+    def _super_operator_output(self, hidden_states: torch.Tensor, selected: torch.Tensor,
+                               weights: torch.Tensor) -> Optional[torch.Tensor]:
+        """The super experts' share of the output, fp32 [tokens, hidden], from the routed-expert operator: the
+        dense experts are 16-bit matrix sets of their own, called from the router's output like the packed
+        experts (ids of other experts are dropped by the id map; small batches run without routing tables).
+        selected / weights: [tokens, top_k]; the weights are used in fp32 (the reference rounds them to the
+        activation dtype first: bitsmoe/models/base_block.py:291-307).  None when the operator is not used."""
+        if not (self._super_expert_items and _super_via_operator() and hidden_states.is_cuda and _HAS_MLP_FORWARD_CUDA
+                and hidden_states.dtype in (torch.float16, torch.bfloat16)):
+            return None
+        dev = hidden_states.device
+        g2l = self._super_global_to_local(dev)
+        l2g = self._basis_cache.get(("super_l2g", str(dev)))
+        if l2g is None:
+            l2g = torch.tensor([idx for idx, _ in self._super_expert_items], dtype=torch.int32, device=dev)
+            self._basis_cache[("super_l2g", str(dev))] = l2g
+        (gate, up, down), inter = self._dense_sets_of("super", [layer for _, layer in self._super_expert_items], dev)
+        x = hidden_states.contiguous()
+        w32 = weights if weights.dtype == torch.float32 else weights.to(torch.float32)
+        hidden = int(x.shape[1])
+        return mlp_forward_cuda.moe_forward_routed(x, x, selected.reshape(-1, self.top_k), w32.reshape(-1, self.top_k).contiguous(),
+                                                   g2l, l2g, gate, up, down, hidden, inter, self._act_type())
+
     def _super_global_to_local(self, device: torch.device) -> torch.Tensor:
         cached = self._basis_cache.get(("super_g2l", str(device)))
         if cached is None:
@@ -314,20 +349,25 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         """Dense SwiGLU experts as packed 16-bit matrices through moe_forward_sets: fp32 [tokens, hidden].
         The packed copies are made once per block (a snapshot of the modules' weights; cleared with the
         runtime cache)."""
-        from bitsmoe_amd.models.dense import pack_dense_mlps
-
-        packed = self._dense_sets.get(key)
-        if packed is None:
-            gate_l, up_l, down_l, inter = pack_dense_mlps(modules, hidden_states.device)
-            sets = tuple(mlp_forward_cuda.MatrixSet(*lists, intermediate_size=inter, name=f"{key}_{p}")
-                         for lists, p in ((gate_l, "gate"), (up_l, "up"), (down_l, "down")))
-            packed = (sets, inter)
-            self._dense_sets[key] = packed
-        (gate, up, down), inter = packed
+        (gate, up, down), inter = self._dense_sets_of(key, modules, hidden_states.device)
         hidden = int(hidden_states.shape[1])
         x = hidden_states.contiguous()
         return mlp_forward_cuda.moe_forward_sets(x, x, token_indices, expert_offsets, route_flat, gate, up, down,
                                                  hidden, inter, self._act_type())
+
+    def _dense_sets_of(self, key: str, modules, device):
+        """((gate, up, down) matrix sets, intermediate size) of dense experts packed as 16-bit matrices: made once
+        per block (a snapshot of the modules' weights; cleared with the runtime cache)."""
+        from bitsmoe_amd.models.dense import pack_dense_mlps
+
+        packed = self._dense_sets.get(key)
+        if packed is None:
+            gate_l, up_l, down_l, inter = pack_dense_mlps(modules, device)
+            sets = tuple(mlp_forward_cuda.MatrixSet(*lists, intermediate_size=inter, name=f"{key}_{p}")
+                         for lists, p in ((gate_l, "gate"), (up_l, "up"), (down_l, "down")))
+            packed = (sets, inter)
+            self._dense_sets[key] = packed
+        return packed
 
     def _always_on_forward(self, key: str, module, hidden_states: torch.Tensor,
                            token_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -546,6 +586,14 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
             weights = weights.reshape(token_count, self.top_k).to(torch.float32)
         rank_out = int(self.shared_u_down.shape[1])
         gate, up, down = self._ensure_matsets()
+        # The super experts' operator call needs the router's output and the hidden states only: it runs on a side
+        # stream beside the packed experts' call (its small launches fill what the packed kernels leave idle).
+        sup, side = None, None
+        if self._super_expert_items and _SUPER_SIDE_STREAM and _super_via_operator():
+            side = _side_stream(hidden_states.device)
+            side.wait_stream(torch.cuda.current_stream(hidden_states.device))
+            with torch.cuda.stream(side):
+                sup = self._super_operator_output(hidden_states, selected, weights)
         rank_accum = mlp_forward_cuda.moe_forward_routed(h_gate, h_up, selected, weights, self._packed_global_to_local,
                                                          self._packed_local_to_global, gate, up, down, rank_out,
                                                          int(self._packed_intermediate_size), self._act_type())
@@ -557,11 +605,21 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
             operand = mlp_forward_cuda.block_finish(rank_accum, dtype)
         out = operand @ plan["w_out"].T
         if self._super_expert_items:
-            extra = torch.zeros_like(out)
-            self._run_super_experts(hidden_states, extra, selected.reshape(-1),
-                                    self._get_flat_token_ids(token_count, hidden_states.device),
-                                    weights.reshape(-1).to(dtype))
-            out = out + extra
+            if side is not None:
+                cur = torch.cuda.current_stream(hidden_states.device)
+                cur.wait_stream(side)
+                if sup is not None:
+                    sup.record_stream(cur)
+            else:
+                sup = self._super_operator_output(hidden_states, selected, weights)
+            if sup is not None:
+                out.add_(sup)
+            else:
+                extra = torch.zeros_like(out)
+                self._run_super_experts(hidden_states, extra, selected.reshape(-1),
+                                        self._get_flat_token_ids(token_count, hidden_states.device),
+                                        weights.reshape(-1).to(dtype))
+                out = out + extra
         return out, logits
 
     # ---- shared forward body --------------------------------------------------------------

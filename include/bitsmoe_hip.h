@@ -86,10 +86,16 @@ void bitsmoe_matset_destroy(bitsmoe_matset* set);
  * buffers are not modified; the library allocates the copy once and frees it in
  * bitsmoe_matset_destroy.  The copy is a SNAPSHOT: buffers overwritten afterwards need a new set.
  * role 0: gate / up (contraction over rows), role 1: down (contraction over columns).
+ * Every width the packer emits is taken (bitsmoe/quant/packer.py:566-589): rows of 1-, 2-, 3- and
+ * 4-bit slabs go into the field layout (1-bit levels as 2-bit fields); rows of 6-, 8- and 16-bit
+ * slabs go into a side table of f16 weights (level * scale rounded once, or the stored half) in MFMA
+ * operand order, which side kernels contract next to the field kernels.  A last column tile of
+ * fewer than 128 columns (bitsmoe/quant/packer.py:265-287) is stored as a whole tile whose excess
+ * columns are zero weights, whatever the caller's payload holds there.
  * Plays the part of the reference's one-time meta build
- * (bitsmoe/algorithms/cpp/mlp_forward.cu:2529-2697).  Returns BITSMOE_E_UNSUPPORTED for sets that
- * hold slabs of other widths than 2, 3 or 4 bits or tiles of fewer than 128 columns: those run
- * on the generic kernels only.  Synchronises `stream`.
+ * (bitsmoe/algorithms/cpp/mlp_forward.cu:2529-2697).  Returns BITSMOE_E_UNSUPPORTED for empty sets
+ * and for slabs that do not span all column tiles: those run on the generic kernels only.
+ * Synchronises `stream`.
  */
 int bitsmoe_matset_prepare(bitsmoe_matset* set, int32_t role, void* stream);
 /* Dense fp32 dequantisation read back FROM THE PREPARED LAYOUT (parity check of it). */
@@ -100,7 +106,8 @@ int bitsmoe_dequant_matrix_prepared(const bitsmoe_matset* set, int32_t expert, f
  * [4]=1 if every matrix has slabs of 16-row multiples, 2/3/4-bit, full tiles,
  * [5]=largest slab count, [6]=smallest logical rank, [7]=bit0: bitsmoe_matset_prepare can take the
  * set (fast kernels applicable), bit1: prepared, bit2: prepared for role 0 and every expert is one
- * run of equal-width slabs whose rows sit in aligned runs of eight ranks (the walking gate/up kernel) */
+ * run of equal-width slabs whose rows sit in aligned runs of eight ranks (the walking gate/up kernel),
+ * bits 8 and up: 64-row slabs in the prepared set's side table of 6/8/16-bit rows */
 int bitsmoe_matset_info(const bitsmoe_matset* set, int64_t info[8]);
 
 /*
