@@ -39,6 +39,7 @@ EXPORTED_SYMBOLS = (
     "bitsmoe_route",
     "bitsmoe_router_softmax_topk",
     "bitsmoe_router_softmax_topk_strided",
+    "bitsmoe_router_linear_topk",
     "bitsmoe_block_finish",
     "bitsmoe_forward_workspace_bytes",
     "bitsmoe_forward_workspace_bytes_sets",
@@ -121,6 +122,9 @@ def load() -> ctypes.CDLL:
     lib.bitsmoe_router_softmax_topk_strided.restype = c_int32
     lib.bitsmoe_router_softmax_topk_strided.argtypes = [c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_float,
                                                         c_int32, c_void_p, c_int32, c_void_p, c_void_p]
+    lib.bitsmoe_router_linear_topk.restype = c_int32
+    lib.bitsmoe_router_linear_topk.argtypes = [c_void_p, c_int32, c_int64, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32,
+                                               c_float, c_int32, c_void_p, c_int32, c_void_p, c_void_p]
     lib.bitsmoe_block_finish.restype = c_int32
     lib.bitsmoe_block_finish.argtypes = [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int64,
                                          c_int32, c_void_p, c_int64, c_void_p]

@@ -29,7 +29,7 @@ _AUTO_PREPARE = os.environ.get("BITSMOE_NO_PREPARE", "0") != "1"
 
 def set_option(name: str, value: int = -1) -> None:
     """One of the launchers' experiment switches for the whole process ("route_inline", "route_jobs",
-    "decode_fused_z", "decode_split_z", "decode_fused", "prefill_split"): 0 / 1, or -1 for the library's own choice.  The
+    "decode_fused_z", "decode_split_z", "decode_fused", "prefill_split", "router_wide"): 0 / 1, or -1 for the library's own choice.  The
     library reads the BITSMOE_* environment forms of these once, when it is loaded."""
     _capi.check(_lib.bitsmoe_set_option(name.encode(), int(value)))
 
@@ -551,6 +551,36 @@ def router_softmax_topk(router_logits: torch.Tensor, top_k: int, renormalize: bo
             logits.data_ptr(), codes[logits.dtype], ld, t, e, int(top_k), 1 if renormalize else 0, float(weight_scale),
             -1 if round_dtype is None else codes[round_dtype], selected.data_ptr(), 1, weights.data_ptr(),
             _stream_ptr(dev)))
+    return selected, weights
+
+
+def router_linear_topk_possible(hidden: torch.Tensor, weight: torch.Tensor, top_k: int) -> bool:
+    """Can router_linear_topk take these tensors?  (16-bit hidden states [T, K] with unit column stride and 16-byte
+    aligned rows, a contiguous weight [E, K] of the same dtype, K a multiple of 128, at most 256 experts.)"""
+    return (hidden.is_cuda and hidden.dim() == 2 and weight.dim() == 2 and hidden.dtype in (torch.float16, torch.bfloat16)
+            and weight.dtype == hidden.dtype and weight.is_contiguous() and hidden.stride(1) == 1
+            and int(hidden.shape[1]) == int(weight.shape[1]) and int(hidden.shape[1]) % 128 == 0
+            and (int(hidden.shape[0]) <= 1 or int(hidden.stride(0)) % 8 == 0) and hidden.data_ptr() % 16 == 0
+            and weight.data_ptr() % 16 == 0 and 1 <= int(top_k) <= min(64, int(weight.shape[0])) and int(weight.shape[0]) <= 256)
+
+
+def router_linear_topk(hidden: torch.Tensor, weight: torch.Tensor, top_k: int, renormalize: bool = True,
+                       round_dtype: Optional[torch.dtype] = None, weight_scale: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The router's linear layer with fp32 logits (hidden.float() @ weight.float().T: exact products of 16-bit values,
+    fp32 sums), softmax, top-k, optional renormalisation, * weight_scale, optional round trip through `round_dtype`:
+    ONE kernel, no logits in memory.  Returns (selected int64 [T, k], weights fp32 [T, k])."""
+    _check(router_linear_topk_possible(hidden, weight, top_k), "router_linear_topk: unsupported shapes, dtypes or alignment")
+    _check(round_dtype in (None, torch.float16, torch.bfloat16), "round_dtype must be None, float16 or bfloat16")
+    dev = hidden.device
+    t, k_dim, e = int(hidden.shape[0]), int(hidden.shape[1]), int(weight.shape[0])
+    selected = torch.empty((t, int(top_k)), dtype=torch.int64, device=dev)
+    weights = torch.empty((t, int(top_k)), dtype=torch.float32, device=dev)
+    codes = {torch.float16: 0, torch.bfloat16: 1}
+    with torch.cuda.device(dev):
+        _capi.check(_lib.bitsmoe_router_linear_topk(
+            hidden.data_ptr(), codes[hidden.dtype], int(hidden.stride(0)) if t > 1 else k_dim, weight.data_ptr(), t, k_dim, e,
+            int(top_k), 1 if renormalize else 0, float(weight_scale), -1 if round_dtype is None else codes[round_dtype],
+            selected.data_ptr(), 1, weights.data_ptr(), _stream_ptr(dev)))
     return selected, weights
 
 

@@ -267,6 +267,7 @@ struct Options {
     int decode_split_z = -1;    // 0 / 1: z by the down workgroups / by a launch of its own wherever possible
     int decode_fused = -1;      // 0 / 1: never / wherever possible the one-kernel decode forward
     int prefill_split = -1;     // 1: gate and up as two launches, SiLU in the second's epilogue (default: one launch and a SiLU pass)
+    int router_wide = -1;       // 0: the fused router kernel with four wavefronts per workgroup whatever the hidden size
 };
 Options& options();
 

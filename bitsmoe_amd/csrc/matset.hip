@@ -90,6 +90,7 @@ Options& options() {
         x.decode_split_z = env_switch("BITSMOE_DECODE_SPLIT_Z");
         x.decode_fused = env_switch("BITSMOE_DECODE_FUSED");
         x.prefill_split = env_switch("BITSMOE_PREFILL_SPLIT");
+        x.router_wide = env_switch("BITSMOE_ROUTER_WIDE");
         return x;
     }();
     return o;
@@ -102,7 +103,8 @@ extern "C" int bitsmoe_set_option(const char* name, int32_t value) {
     const std::string n(name);
     int* slot = n == "route_inline" ? &o.route_inline : n == "route_jobs" ? &o.route_jobs
                 : n == "decode_fused_z" ? &o.decode_fused_z : n == "decode_split_z" ? &o.decode_split_z
-                : n == "decode_fused" ? &o.decode_fused : n == "prefill_split" ? &o.prefill_split : nullptr;
+                : n == "decode_fused" ? &o.decode_fused : n == "prefill_split" ? &o.prefill_split
+                : n == "router_wide" ? &o.router_wide : nullptr;
     BITSMOE_REQUIRE(slot != nullptr, "unknown option '%s'", name);
     *slot = value < 0 ? -1 : (int)value;
     return BITSMOE_OK;

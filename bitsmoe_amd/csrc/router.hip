@@ -109,32 +109,29 @@ __global__ __launch_bounds__(256) void k_router_softmax_topk(const void* __restr
 // expert in the top-k list.  The logits of a token sit in LDS and are read as broadcasts.
 // grid = ceil(T / 4), 256 threads (one wavefront per token).
 constexpr int ROUTER_RANK_PER_LANE = 4;
-template <int DT>
-__global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict__ logits, int64_t ld, float wscale, int T,
-                                                          int E, int k,
-                                                          int renorm, int round_dt, int32_t* __restrict__ sel32,
-                                                          int64_t* __restrict__ sel64, float* __restrict__ weights) {
+template <int NW>      // wavefronts per workgroup
+struct RankTopkLds {
     // sort key of a logit: the float mapped to an unsigned integer of the same order, above the
     // complemented expert index, so that one 64-bit comparison is "precedes in the top-k order"
-    __shared__ __attribute__((aligned(16))) uint64_t keys[4][64 * ROUTER_RANK_PER_LANE];
-    __shared__ float picked[4][64];
-    const int lane = threadIdx.x & 63;
-    const int wv = threadIdx.x >> 6;
-    const int tkn = blockIdx.x * 4 + wv;
-    if (tkn >= T) return;            // (no workgroup barrier below: a wavefront only reads what it wrote)
+    uint64_t keys[NW][64 * ROUTER_RANK_PER_LANE];
+    float picked[NW][64];
+};
+// One token by one wavefront (`wv` of its workgroup): v[i] is the logit of expert lane + 64 i (-inf past E).
+template <int NW>
+__device__ inline void rank_topk_token(float (&v)[ROUTER_RANK_PER_LANE], RankTopkLds<NW>& lds, int wv, int lane, int tkn, float wscale,
+                                       int E, int k, int renorm, int round_dt, int32_t* __restrict__ sel32,
+                                       int64_t* __restrict__ sel64, float* __restrict__ weights) {
     const int e2 = (E + 1) & ~1;
-    float v[ROUTER_RANK_PER_LANE];
     uint64_t mine[ROUTER_RANK_PER_LANE];
     float vmax = -INFINITY;
 #pragma unroll
     for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) {
         const int e = lane + 64 * i;
-        v[i] = e < E ? load_logit<DT>(logits, (int64_t)tkn * ld + e) : -INFINITY;
         vmax = fmaxf(vmax, v[i]);
         const uint32_t bits = __float_as_uint(v[i] + 0.0f);      // (-0 and +0 are one value)
         const uint32_t ordered = bits ^ ((bits >> 31) ? 0xFFFFFFFFu : 0x80000000u);
         mine[i] = e < E ? ((uint64_t)ordered << 32) | (uint32_t)(0xFFFFFFFFu - (uint32_t)e) : 0ull;   // padding sorts last
-        keys[wv][e] = mine[i];
+        lds.keys[wv][e] = mine[i];
     }
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, d));
@@ -154,18 +151,18 @@ __global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict
     int rank[ROUTER_RANK_PER_LANE] = {0, 0, 0, 0};
 #pragma unroll 4
     for (int o = 0; o < e2; o += 2) {
-        const uint64_t q0 = keys[wv][o], q1 = keys[wv][o + 1];
+        const uint64_t q0 = lds.keys[wv][o], q1 = lds.keys[wv][o + 1];
 #pragma unroll
         for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) rank[i] += (int)(q0 > mine[i]) + (int)(q1 > mine[i]);
     }
 #pragma unroll
     for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i)
-        if (lane + 64 * i < E && rank[i] < k) picked[wv][rank[i]] = pr[i] / denom;
+        if (lane + 64 * i < E && rank[i] < k) lds.picked[wv][rank[i]] = pr[i] / denom;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     float picked_sum = 0.0f;
-    for (int j = 0; j < k; ++j) picked_sum += picked[wv][j];
+    for (int j = 0; j < k; ++j) picked_sum += lds.picked[wv][j];
 #pragma unroll
     for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) {
         if (lane + 64 * i < E && rank[i] < k) {
@@ -181,6 +178,147 @@ __global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict
             if (sel64) sel64[o] = lane + 64 * i;
             weights[o] = w;
         }
+    }
+    // (the next token of this wavefront overwrites keys / picked: its reads above are done first)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict__ logits, int64_t ld, float wscale, int T,
+                                                          int E, int k,
+                                                          int renorm, int round_dt, int32_t* __restrict__ sel32,
+                                                          int64_t* __restrict__ sel64, float* __restrict__ weights) {
+    __shared__ __attribute__((aligned(16))) RankTopkLds<4> lds;
+    const int lane = threadIdx.x & 63;
+    const int wv = threadIdx.x >> 6;
+    const int tkn = blockIdx.x * 4 + wv;
+    if (tkn >= T) return;            // (no workgroup barrier below: a wavefront only reads what it wrote)
+    float v[ROUTER_RANK_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) {
+        const int e = lane + 64 * i;
+        v[i] = e < E ? load_logit<DT>(logits, (int64_t)tkn * ld + e) : -INFINITY;
+    }
+    rank_topk_token(v, lds, wv, lane, tkn, wscale, E, k, renorm, round_dt, sel32, sel64, weights);
+}
+
+// The router's linear layer and the top-k in ONE kernel, for gates that compute their logits in fp32 from 16-bit
+// hidden states and a 16-bit weight (DeepSeek-V2's gate: bitsmoe/models/deepseekv2/configuration_deepseek.py:125-139
+// names its form; the reference calls the model's own gate module, bitsmoe/models/deepseekv2/bitsmoe_block.py:74):
+// the products of 16-bit values are exact in fp32, so MFMA sums in fp32 are the module's logits up to summation
+// order.  A workgroup of NW wavefronts takes 16 tokens: wavefront w contracts over the w-th part of the hidden size
+// for all experts (NB 16-expert blocks; sixteen wavefronts: all its operands of a 2048-wide layer are ONE batch of
+// loads), the partial sums meet in LDS (a tree in a fixed order: the same logits whenever the inputs are the same), then
+// the wavefronts rank the tokens, 16 / NW each.
+// x [T, K] and weight [E, K] are read as MFMA operands straight from memory (16 bytes per lane).
+template <bool BF16, int NB, int NW>
+__global__ __launch_bounds__(NW * 64) void k_router_linear_topk(const uint16_t* __restrict__ x, int64_t ld_x,
+                                                                const uint16_t* __restrict__ weight, int T, int K, int E, int k,
+                                                                float wscale, int renorm, int round_dt,
+                                                                int32_t* __restrict__ sel32, int64_t* __restrict__ sel64,
+                                                                float* __restrict__ weights) {
+    constexpr int U = NB <= 4 ? 4 : NB <= 8 ? 2 : 1;      // k-steps whose operands are requested together
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+    typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+    constexpr int LD = NB * 16 + 1;
+    // DIRECT: every wavefront's partial sums fit the LDS side by side and the ranking wavefront adds them up itself (one
+    // barrier); otherwise a tree over half as many slots (slot 0 ends as the total).  Both add in a fixed order.
+    constexpr bool DIRECT = NW * 16 * LD * 4 + sizeof(RankTopkLds<NW>) <= 160 * 1024;
+    __shared__ float part[(DIRECT ? NW : NW / 2) * 16 * LD];
+    __shared__ __attribute__((aligned(16))) RankTopkLds<NW> lds;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int t0 = blockIdx.x * 16;
+    const int row = t0 + (lane & 15);
+    const int kq = K / NW;                       // contraction range of this wavefront (a multiple of 32)
+    const int kbase = wv * kq + (lane >> 4) * 8;
+    f32x4 acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    const uint16_t* __restrict__ xp = x + (int64_t)min(row, T - 1) * ld_x + kbase;
+    for (int s0 = 0; s0 < kq; s0 += 32 * U) {
+        u32x4 a[U], b[U][NB];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int ks = min(s0 + 32 * u, kq - 32);      // (a short last group repeats its final step: masked below)
+            a[u] = *reinterpret_cast<const u32x4*>(xp + ks);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const int e = min(nb * 16 + (lane & 15), E - 1);
+                b[u][nb] = *reinterpret_cast<const u32x4*>(weight + (int64_t)e * K + kbase + ks);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);      // (every request of the group is out before its first MFMA)
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            // (no branch between the steps: a step past the end contributes zeros)
+            const bool live = s0 + 32 * u < kq;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) a[u][c] = live ? a[u][c] : 0u;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                if constexpr (BF16)
+                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[u]), __builtin_bit_cast(bf16x8, b[u][nb]),
+                                                                      acc[nb], 0, 0, 0);
+                else
+                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a[u]), __builtin_bit_cast(f16x8, b[u][nb]),
+                                                                     acc[nb], 0, 0, 0);
+            }
+        }
+    }
+    // lane holds tokens 4 (lane / 16) + j, expert 16 nb + lane % 16
+    auto slot_of = [&](int w, int nb, int j) -> float& { return part[(w * 16 + 4 * (lane >> 4) + j) * LD + nb * 16 + (lane & 15)]; };
+    if constexpr (DIRECT) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) slot_of(wv, nb, j) = acc[nb][j];
+    }
+    for (int half = DIRECT ? 0 : NW / 2; half >= 1; half >>= 1) {      // wavefronts [half, 2 half) hand their sums to [0, half)
+        if (wv >= half && wv < 2 * half) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) slot_of(wv - half, nb, j) = acc[nb][j];
+        }
+        __syncthreads();
+        if (wv < half) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[nb][j] += slot_of(wv, nb, j);
+        }
+        __syncthreads();
+    }
+    if (!DIRECT && wv == 0) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) slot_of(0, nb, j) = acc[nb][j];
+    }
+    __syncthreads();
+    constexpr int PER = 16 / NW > 0 ? 16 / NW : 1;
+    for (int i = 0; i < PER; ++i) {
+        const int tl = wv * PER + i, tkn = t0 + tl;
+        if (tl >= 16 || tkn >= T) break;       // (wave-uniform; no workgroup barrier below)
+        float v[ROUTER_RANK_PER_LANE];
+#pragma unroll
+        for (int q = 0; q < ROUTER_RANK_PER_LANE; ++q) {
+            const int e = lane + 64 * q;
+            float sum = -INFINITY;
+            if (e < E && e < NB * 16) {
+                sum = part[tl * LD + e];
+                if constexpr (DIRECT) {
+#pragma unroll
+                    for (int w = 1; w < NW; ++w) sum += part[(w * 16 + tl) * LD + e];
+                }
+            }
+            v[q] = sum;
+        }
+        rank_topk_token(v, lds, wv, lane, tkn, wscale, E, k, renorm, round_dt, sel32, sel64, weights);
     }
 }
 
@@ -226,6 +364,51 @@ extern "C" int bitsmoe_router_softmax_topk(const void* logits, int32_t logits_dt
                                            int32_t ids_are_i64, float* weights, void* stream) {
     return bitsmoe_router_softmax_topk_strided(logits, logits_dtype, n_experts, n_tokens, n_experts, top_k, renormalize, 1.0f,
                                                round_dtype, selected, ids_are_i64, weights, stream);
+}
+
+extern "C" int bitsmoe_router_linear_topk(const void* hidden, int32_t dtype, int64_t ld_hidden, const void* weight,
+                                          int64_t n_tokens, int32_t hidden_size, int32_t n_experts, int32_t top_k,
+                                          int32_t renormalize, float weight_scale, int32_t round_dtype, void* selected,
+                                          int32_t ids_are_i64, float* weights, void* stream) {
+    BITSMOE_REQUIRE(n_tokens >= 0 && n_tokens < ((int64_t)1 << 31), "token count out of range");
+    BITSMOE_REQUIRE(dtype == BITSMOE_DT_F16 || dtype == BITSMOE_DT_BF16, "dtype must be f16 (0) or bf16 (1)");
+    BITSMOE_REQUIRE(n_experts >= 1 && n_experts <= 64 * ROUTER_RANK_PER_LANE, "n_experts must be in [1, %d]", 64 * ROUTER_RANK_PER_LANE);
+    BITSMOE_REQUIRE(top_k >= 1 && top_k <= 64 && top_k <= n_experts, "top_k must be in [1, min(64, n_experts)]");
+    BITSMOE_REQUIRE(hidden_size >= 128 && hidden_size % 128 == 0, "hidden_size must be a positive multiple of 128");
+    // (option router_wide = 0: four wavefronts per workgroup whatever the hidden size; experiments)
+    const bool wide_wg = hidden_size % 512 == 0 && options().router_wide != 0;      // sixteen wavefronts, a sixteenth of the contraction each
+    BITSMOE_REQUIRE(ld_hidden >= hidden_size && ld_hidden % 8 == 0, "ld_hidden must be at least hidden_size and a multiple of 8");
+    BITSMOE_REQUIRE(round_dtype >= -1 && round_dtype <= 1, "round_dtype must be -1 (none), 0 (fp16) or 1 (bf16)");
+    if (n_tokens == 0) return BITSMOE_OK;
+    BITSMOE_REQUIRE(hidden && weight && selected && weights, "null pointer");
+    BITSMOE_REQUIRE((((uintptr_t)hidden | (uintptr_t)weight) & 15) == 0, "hidden and weight must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    int32_t* s32 = ids_are_i64 ? nullptr : (int32_t*)selected;
+    int64_t* s64 = ids_are_i64 ? (int64_t*)selected : nullptr;
+    const dim3 grid((unsigned)((n_tokens + 15) / 16));
+    const bool bf16 = dtype == BITSMOE_DT_BF16;
+#define BITSMOE_ROUTER_LINEAR(B, NB, NWIDE)                                                                                  \
+    do {                                                                                                                     \
+        if (wide_wg)                                                                                                         \
+            hipLaunchKernelGGL((k_router_linear_topk<B, NB, NWIDE>), grid, dim3(NWIDE * 64), 0, st, (const uint16_t*)hidden, \
+                               ld_hidden, (const uint16_t*)weight, (int)n_tokens, hidden_size, n_experts, top_k,             \
+                               weight_scale, renormalize, round_dtype, s32, s64, weights);                                   \
+        else                                                                                                                 \
+            hipLaunchKernelGGL((k_router_linear_topk<B, NB, 4>), grid, dim3(256), 0, st, (const uint16_t*)hidden, ld_hidden,  \
+                               (const uint16_t*)weight, (int)n_tokens, hidden_size, n_experts, top_k, weight_scale,          \
+                               renormalize, round_dtype, s32, s64, weights);                                                 \
+    } while (0)
+    // (more than 128 experts: eight wavefronts, the partial sums of sixteen would not fit the LDS)
+    if (n_experts <= 64) {
+        if (bf16) BITSMOE_ROUTER_LINEAR(true, 4, 16); else BITSMOE_ROUTER_LINEAR(false, 4, 16);
+    } else if (n_experts <= 128) {
+        if (bf16) BITSMOE_ROUTER_LINEAR(true, 8, 16); else BITSMOE_ROUTER_LINEAR(false, 8, 16);
+    } else {
+        if (bf16) BITSMOE_ROUTER_LINEAR(true, 16, 8); else BITSMOE_ROUTER_LINEAR(false, 16, 8);
+    }
+#undef BITSMOE_ROUTER_LINEAR
+    BITSMOE_HIP_TRY(hipGetLastError());
+    return BITSMOE_OK;
 }
 
 // ---- the block's closing elementwise pass ---------------------------------------------------------------------------

@@ -9,6 +9,7 @@ from typing import List, Optional
 import torch
 import torch.nn as nn
 
+from bitsmoe_amd.algorithms import _HAS_MLP_FORWARD_CUDA, mlp_forward_cuda
 from bitsmoe_amd.models.base_block import BitsMoE_BaseSparseMoeBlock
 
 
@@ -32,6 +33,20 @@ class BitsMoE_DeepSeekSparseMoeBlock(BitsMoE_BaseSparseMoeBlock):
         self._init_bitsmoe_common_state(super_experts=super_experts, track_super_projected_weights=True)
 
     def _gate_route(self, hidden_states: torch.Tensor):
+        gate = self.gate
+        # A gate of the plain form -- fp32 logits, softmax, greedy top-k, then renormalisation or the scaling factor
+        # (the defaults of bitsmoe/models/deepseekv2/configuration_deepseek.py:125-139; "gready" is that file's
+        # spelling) -- in evaluation mode: linear layer, softmax and top-k as ONE kernel.  Any other gate: the module.
+        if (not getattr(gate, "training", False) and getattr(gate, "scoring_func", "softmax") == "softmax"
+                and getattr(gate, "topk_method", "greedy") in ("greedy", "gready") and hasattr(gate, "top_k")
+                and hasattr(gate, "norm_topk_prob") and hasattr(gate, "routed_scaling_factor")
+                and isinstance(getattr(gate, "weight", None), torch.Tensor) and hidden_states.is_cuda and _HAS_MLP_FORWARD_CUDA):
+            x = hidden_states.reshape(-1, hidden_states.shape[-1])
+            top_k = int(gate.top_k)
+            if mlp_forward_cuda.router_linear_topk_possible(x, gate.weight, top_k):
+                renorm = top_k > 1 and bool(gate.norm_topk_prob)
+                return mlp_forward_cuda.router_linear_topk(x, gate.weight.detach(), top_k, renorm, round_dtype=None,
+                                                           weight_scale=1.0 if renorm else float(gate.routed_scaling_factor))
         topk_idx, topk_weight, _aux = self.gate(hidden_states)
         return topk_idx.reshape(-1, topk_idx.shape[-1]), topk_weight.reshape(-1, topk_weight.shape[-1]).to(torch.float32)
 

@@ -52,6 +52,13 @@ class SoftmaxGreedyGate(nn.Module):
         if x.is_cuda and self.weight.shape[0] <= 1024 and self.top_k <= 64:
             from bitsmoe_amd.algorithms import _HAS_MLP_FORWARD_CUDA, mlp_forward_cuda
 
+            scale = 1.0 if renorm else self.routed_scaling_factor
+            if _HAS_MLP_FORWARD_CUDA and mlp_forward_cuda.router_linear_topk_possible(x, self.weight, self.top_k):
+                # fp32 logits (exact products of the 16-bit values, fp32 sums), softmax, greedy top-k and the
+                # renormalisation or scaling in ONE kernel
+                idx, weight = mlp_forward_cuda.router_linear_topk(x, self.weight.detach(), self.top_k, renorm, round_dtype=None,
+                                                                  weight_scale=scale)
+                return idx, weight, None
             if _HAS_MLP_FORWARD_CUDA:
                 # fp32 logits as the module computes them (one cast, one GEMM against the cached fp32 weight), then
                 # softmax / greedy top-k / renormalisation or scaling in one kernel instead of four framework ops

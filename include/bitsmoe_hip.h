@@ -160,6 +160,19 @@ int bitsmoe_router_softmax_topk(const void* logits, int32_t logits_dtype, int64_
 int bitsmoe_router_softmax_topk_strided(const void* logits, int32_t logits_dtype, int64_t ld_logits, int64_t n_tokens,
                                         int32_t n_experts, int32_t top_k, int32_t renormalize, float weight_scale,
                                         int32_t round_dtype, void* selected, int32_t ids_are_i64, float* weights, void* stream);
+/*
+ * The router's linear layer and the front end above in ONE kernel, for gates that compute fp32 logits from 16-bit
+ * hidden states and a 16-bit weight (the DeepSeek-V2 gate casts both to fp32 and multiplies; the reference calls
+ * the model's own gate module: bitsmoe/models/deepseekv2/bitsmoe_block.py:72-74).  Products of two 16-bit values
+ * are exact in fp32, so the MFMA sums equal the module's logits up to summation order; no logits reach memory.
+ *   hidden  device f16 / bf16 [T, hidden_size], ld_hidden elements between rows (a multiple of 8), 16-byte aligned
+ *   weight  device, the same dtype, [n_experts, hidden_size] contiguous; hidden_size a multiple of 128,
+ *           n_experts <= 256
+ */
+int bitsmoe_router_linear_topk(const void* hidden, int32_t dtype, int64_t ld_hidden, const void* weight,
+                               int64_t n_tokens, int32_t hidden_size, int32_t n_experts, int32_t top_k,
+                               int32_t renormalize, float weight_scale, int32_t round_dtype, void* selected,
+                               int32_t ids_are_i64, float* weights, void* stream);
 
 /*
  * The block's closing elementwise pass: one row of the operand of the output GEMM in the activation dtype,

@@ -642,3 +642,36 @@ def test_router_kernel_matches_oracle(cuda_device, tokens, n_experts, top_k, ren
     sel2, w2 = hip.router_softmax_topk(t.to(cuda_device), top_k, renorm, round_dtype=torch.bfloat16)
     assert torch.equal(sel2, sel)
     assert np.allclose(w2.cpu().numpy(), helpers.bf16_round(w_ref), rtol=2 ** -7, atol=0)
+
+
+@pytest.mark.parametrize("tokens,hidden,n_experts,top_k,renorm,scale", [
+    (1, 2048, 64, 6, False, 16.0), (32, 2048, 64, 6, False, 1.0), (70, 1536, 160, 6, True, 1.0), (16, 640, 256, 8, True, 1.0),
+    (5, 128, 8, 2, False, 2.5), (257, 2048, 66, 6, False, 1.0)])
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+def test_router_linear_kernel_matches_oracle(cuda_device, tokens, hidden, n_experts, top_k, renorm, scale, dtype_name):
+    """The gate's linear layer, softmax and top-k in one kernel: logits are fp32 sums of exact products of the
+    16-bit values, so the picks are the oracle's on float64 logits of the same values and the weights agree to
+    fp32 rounding of the sums."""
+    import torch
+
+    hip = _hip()
+    rng = np.random.default_rng(tokens * 13 + n_experts)
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    x = torch.from_numpy(rng.normal(size=(tokens, hidden)).astype(np.float32)).to(dt)
+    w = torch.from_numpy((rng.normal(size=(n_experts, hidden)) * 0.05).astype(np.float32)).to(dt)
+    logits = (x.double().numpy() @ w.double().numpy().T).astype(np.float32)
+    idx_ref, w_ref = o.router_qwen(logits, top_k, renorm)
+    assert hip.router_linear_topk_possible(x.to(cuda_device), w.to(cuda_device), top_k)
+    sel, wt = hip.router_linear_topk(x.to(cuda_device), w.to(cuda_device), top_k, renorm, weight_scale=scale)
+    assert sel.dtype == torch.int64 and np.array_equal(sel.cpu().numpy(), idx_ref)
+    assert np.allclose(wt.cpu().numpy(), w_ref * scale, rtol=2e-5, atol=1e-9)
+    # the two-step form (fp32 logits in memory, then the softmax / top-k kernel) picks the same
+    sel2, wt2 = hip.router_softmax_topk(torch.from_numpy(logits).to(cuda_device), top_k, renorm, weight_scale=scale)
+    assert torch.equal(sel2, sel) and torch.allclose(wt2, wt, rtol=2e-5, atol=1e-9)
+    # rows of a wider tensor
+    wide = torch.zeros((tokens, hidden + 64), dtype=dt, device=cuda_device)
+    wide[:, 32:32 + hidden] = x.to(cuda_device)
+    view = wide[:, 32:32 + hidden]
+    if hip.router_linear_topk_possible(view, w.to(cuda_device), top_k):
+        sel3, wt3 = hip.router_linear_topk(view, w.to(cuda_device), top_k, renorm, weight_scale=scale)
+        assert torch.equal(sel3, sel) and torch.equal(wt3, wt)

@@ -148,3 +148,47 @@ def test_wide_rows_only_in_some_experts_and_some_projections(cuda_device):
     for path_name in ("decode", "mfma"):
         sets, err = _case(cuda_device, 400, e, t, k, rank, rank, dim, "f16", _paths()[path_name], make)
         assert [s.wide_slabs for s in sets] == [1, 0, 2]
+
+
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+@pytest.mark.parametrize("tokens,top_k,inline", [(1, 8, True), (5, 4, True), (64, 8, True), (128, 8, True), (200, 6, False),
+                                                 (40, 1, False)])
+@pytest.mark.parametrize("identity", [True, False])
+def test_dense_experts_from_the_router_output(cuda_device, tokens, top_k, inline, identity, dtype_name):
+    """Two dense experts among 16 router ids (the others belong to no expert of these sets, as for a block's super
+    experts): from the router's output, small batches run without routing tables -- the side kernels scan the
+    routed ids themselves -- and must equal the table form and the oracle.  identity=False: the rows read the
+    activations in a scrambled order (no 16-byte activation loads)."""
+    import torch
+
+    hip = _hip()
+    rng = np.random.default_rng(500 + tokens + top_k)
+    n_global, ids, rank, dim = 16, (3, 11), 256, 384
+    gate, up, down = [], [], []
+    for _ in ids:
+        for lst in (gate, up, down):
+            lst.append(helpers.make_matrix(rng, rank, dim, [(16, (0, rank))], s_mode="ones" if identity else "rand", std=0.05))
+    if not identity:
+        for m in gate + up:
+            m["rank_idx"] = rng.permutation(rank).astype(np.int32)[m["rank_idx"]]
+    g2l = np.full(n_global, -1, np.int32)
+    g2l[list(ids)] = np.arange(len(ids), dtype=np.int32)
+    l2g = np.asarray(ids, np.int32)
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    h = torch.from_numpy(rng.normal(size=(tokens, rank)).astype(np.float32)).to(dt)
+    idx, w = o.router_qwen(rng.normal(size=(tokens, n_global)).astype(np.float32), top_k)
+    tok, off, rw = o.build_routing(idx, w, g2l, len(ids))
+    ref = o.moe_forward(h.float().numpy(), h.float().numpy(), tok, off, rw, gate, up, down, rank, dim)
+    sets = [hip.MatrixSet(*helpers.to_device_lists(m, cuda_device), intermediate_size=dim) for m in (gate, up, down)]
+    assert sets[0].prepare(0) and sets[1].prepare(0) and sets[2].prepare(1)
+    hd = h.to(cuda_device)
+    assert hip.routed_is_inline(hd, hd, top_k, *sets) == inline
+    sel = torch.from_numpy(idx.astype(np.int64)).to(cuda_device)
+    wt = torch.from_numpy(w).to(cuda_device)
+    g2l_t, l2g_t = torch.from_numpy(g2l).to(cuda_device), torch.from_numpy(l2g).to(cuda_device)
+    for _ in range(2):      # (the second call finds the intermediates as the first left them)
+        got = hip.moe_forward_routed(hd, hd, sel, wt, g2l_t, l2g_t, *sets, rank, dim, 0)
+        assert helpers.norm_err(got.cpu().numpy(), ref) <= 3e-3
+    tok_d, off_d, rw_d = hip.route(sel, wt, g2l_t, len(ids))
+    tables = hip.moe_forward_sets(hd, hd, tok_d, off_d, rw_d, *sets, rank, dim, 0)
+    assert float((got - tables).abs().max()) <= 1e-5 * max(float(tables.abs().max()), 1e-6)

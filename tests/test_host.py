@@ -231,7 +231,7 @@ def test_bench_last_line_is_compact():
 def test_set_option_names():
     from bitsmoe_amd.algorithms import mlp_forward_cuda as hip
 
-    for name in ("route_inline", "route_jobs", "decode_fused_z", "decode_split_z", "decode_fused", "prefill_split"):
+    for name in ("route_inline", "route_jobs", "decode_fused_z", "decode_split_z", "decode_fused", "prefill_split", "router_wide"):
         hip.set_option(name, 1)
         hip.set_option(name, -1)
     with pytest.raises(RuntimeError, match="unknown option"):
