@@ -20,7 +20,7 @@ beside them as `warm`.  `c5-stack-*` runs the stack configuration of the benchma
 shaped stack, one step = one pass over all 26 layers (per-layer figures reported).
 
 The LAST stdout line is one compact JSON record (< 4 KB); the full record with every field of every workload
-is written to gpurun_out/bench_full.json (--full-json PATH; --print-full also prints it as an earlier line).
+is written to bench_out/bench_full.json (--full-json PATH; --print-full also prints it as an earlier line).
 `value` is tokens/s of the primary workload (default: the
 Qwen3-30B-A3B-shaped layer at decode, 64 tokens); `extras` holds the other decode batch
 sizes, the 4096-token prefill, the other layer shapes of the benchmark set (c1, c4), checkpoint-shaped experts and the
@@ -496,7 +496,7 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only (no HIP graph replay)")
     ap.add_argument("--full-json", default=None,
-                    help="where the full record is written (default gpurun_out/bench_full.json)")
+                    help="where the full record is written (default bench_out/bench_full.json)")
     ap.add_argument("--print-full", action="store_true", help="also print the full record as an earlier stdout line")
     ap.add_argument("--no-warm", action="store_true", help="skip the one-layer (warm) replay of the same workload")
     ap.add_argument("--no-block", action="store_true", help="skip the block-scope timing")
@@ -615,7 +615,7 @@ def main() -> int:
     }
     # The full record (every workload with all its fields) goes to a file and to an EARLIER stdout line; the
     # LAST line is the compact one, small enough for any harness that keeps only the tail of stdout.
-    full_path = args.full_json or os.path.join(ROOT, "gpurun_out", "bench_full.json")
+    full_path = args.full_json or os.path.join(ROOT, "bench_out", "bench_full.json")
     try:
         os.makedirs(os.path.dirname(full_path), exist_ok=True)
         with open(full_path, "w") as f:
