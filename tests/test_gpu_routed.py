@@ -34,7 +34,7 @@ def _case(cuda_device, seed, n_global, n_super, tokens, top_k, rank, dim, i64, d
         gate, up, down = helpers.make_experts(seed, e, rank, rank, dim, choices=(2, 3, 4), uniform_bits=True)
     elif experts == "mixed":
         gate, up, down = helpers.make_experts(seed, e, rank, rank, dim, choices=(2, 3, 4), slab_multiple=64)
-    else:       # slabs of other widths: the generic kernels, routing tables
+    else:       # 8-bit slabs too: their rows run the side kernels next to the field kernels, behind routing tables
         gate, up, down = helpers.make_experts(seed, e, rank, rank, dim, choices=(2, 8), slab_multiple=64)
     if scramble_ranks:       # rows of gate / up read arbitrary columns of h instead of runs of eight
         for m in gate + up:
@@ -56,7 +56,9 @@ def _case(cuda_device, seed, n_global, n_super, tokens, top_k, rank, dim, i64, d
     two_calls = hip.moe_forward_sets(h_gate.to(cuda_device), h_up.to(cuda_device), tok_d, off_d, rw_d, *sets, rank, dim, 0,
                                      **kwargs)
     scale = float(two_calls.abs().max())
-    assert float((got - two_calls).abs().max()) <= 1e-5 * scale        # same sums, fp32 atomics in another order
+    # same sums, fp32 atomics in another order; where 6/8/16-bit rows add to the gate and up sums by atomics, an
+    # element of z may round to the neighbouring f16 value under another order of the adds
+    assert float((got - two_calls).abs().max()) <= (1e-5 if experts in ("uniform", "mixed") else 1e-3) * scale
     err = helpers.norm_err(got.cpu().numpy(), ref)
     assert err <= 3e-3, f"normalised error {err:.3e}"
     inline = hip.routed_is_inline(h_gate.to(cuda_device), h_up.to(cuda_device), top_k, *sets, **kwargs)
@@ -123,8 +125,8 @@ def test_grouped_gemm_from_router_output_with_scattered_ranks(cuda_device, dtype
 
 @pytest.mark.parametrize("experts", ["mixed", "generic"])
 def test_forward_from_router_output_other_layouts(cuda_device, experts):
-    """Experts of mixed widths (the walking kernel's mixed form, rank 512: whole groups) and sets the fast
-    kernels cannot take (8-bit slabs: routing tables, generic kernels)."""
+    """Experts of mixed widths (the walking kernel's mixed form, rank 512: whole groups) and sets with 8-bit slabs
+    (their rows run the side kernels, which read routing tables: no routing inside the kernels)."""
     _, inline = _case(cuda_device, 77, 12, 1, 11, 2, 512, 256, True, "bf16", experts=experts)
     assert inline == (experts == "mixed")
 

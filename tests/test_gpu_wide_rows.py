@@ -191,4 +191,5 @@ def test_dense_experts_from_the_router_output(cuda_device, tokens, top_k, inline
         assert helpers.norm_err(got.cpu().numpy(), ref) <= 3e-3
     tok_d, off_d, rw_d = hip.route(sel, wt, g2l_t, len(ids))
     tables = hip.moe_forward_sets(hd, hd, tok_d, off_d, rw_d, *sets, rank, dim, 0)
-    assert float((got - tables).abs().max()) <= 1e-5 * max(float(tables.abs().max()), 1e-6)
+    # (the same sums, added by atomics in another order: an element of z may round to the neighbouring f16 value)
+    assert float((got - tables).abs().max()) <= 1e-3 * max(float(tables.abs().max()), 1e-6)
