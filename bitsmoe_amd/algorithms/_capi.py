@@ -41,6 +41,7 @@ EXPORTED_SYMBOLS = (
     "bitsmoe_router_softmax_topk_strided",
     "bitsmoe_router_linear_topk",
     "bitsmoe_block_finish",
+    "bitsmoe_skinny_linear",
     "bitsmoe_forward_workspace_bytes",
     "bitsmoe_forward_workspace_bytes_sets",
     "bitsmoe_moe_forward",
@@ -125,6 +126,8 @@ def load() -> ctypes.CDLL:
     lib.bitsmoe_router_linear_topk.restype = c_int32
     lib.bitsmoe_router_linear_topk.argtypes = [c_void_p, c_int32, c_int64, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32,
                                                c_float, c_int32, c_void_p, c_int32, c_void_p, c_void_p]
+    lib.bitsmoe_skinny_linear.restype = c_int32
+    lib.bitsmoe_skinny_linear.argtypes = [c_void_p, c_int32, c_int64, c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int64, c_void_p]
     lib.bitsmoe_block_finish.restype = c_int32
     lib.bitsmoe_block_finish.argtypes = [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int64,
                                          c_int32, c_void_p, c_int64, c_void_p]

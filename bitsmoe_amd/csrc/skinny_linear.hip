@@ -1,0 +1,155 @@
+// A bias-free linear layer for a FEW rows: out[T, N] = x[T, K] * W[N, K]^T with T <= 64, 16-bit x / W / out, fp32 sums.
+// The two GEMMs around the routed-expert operator (the row-stacked shared-basis / router / shared-expert projections
+// in, the column-stacked output projections out: bitsmoe/models/qwen3moe/bitsmoe_block.py:63-64,
+// bitsmoe/models/base_block.py:414) are this shape at decode sizes: tens of MB of weights against a handful of tokens,
+// i.e. a stream of W at HBM speed, which general GEMM kernels tiled for square problems reach a fraction of.
+// W stays in the framework's [out_features, in_features] layout: a lane's 16 bytes of a weight row are eight
+// consecutive contraction indices, which is what the 16x16x32 MFMA takes as its second operand.
+// A workgroup owns 16 * NBW output columns; its four wavefronts contract a quarter of K each, two batches of four
+// k-steps in flight (every load of a batch is out before the previous batch's MFMAs run), and add up in LDS.
+#include "common.h"
+
+#include <algorithm>
+
+namespace bitsmoe {
+
+typedef float sk_f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t sk_u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 sk_f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 sk_bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int SK_U = 4;      // k-steps per batch of loads
+
+template <bool BF16, int NMB, int NBW>
+__global__ __launch_bounds__(256) void k_skinny_linear(const uint16_t* __restrict__ x, int64_t ld_x, const uint16_t* __restrict__ w,
+                                                       int T, int K, int N, uint16_t* __restrict__ out, int64_t ld_out) {
+    __shared__ float part[4][NMB * 16][NBW * 16 + 1];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int n0 = blockIdx.x * (NBW * 16);
+    const int kq = K >> 2;                       // contraction range of this wavefront (a multiple of 32)
+    const int kbase = wv * kq + (lane >> 4) * 8;
+    const uint16_t* xp[NMB];
+    const uint16_t* wp[NBW];
+#pragma unroll
+    for (int mb = 0; mb < NMB; ++mb) xp[mb] = x + (int64_t)min(mb * 16 + (lane & 15), T - 1) * ld_x + kbase;
+#pragma unroll
+    for (int nb = 0; nb < NBW; ++nb) wp[nb] = w + (int64_t)min(n0 + nb * 16 + (lane & 15), N - 1) * K + kbase;
+    sk_f32x4 acc[NMB][NBW];
+#pragma unroll
+    for (int mb = 0; mb < NMB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NBW; ++nb) acc[mb][nb] = sk_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    sk_u32x4 a[2][SK_U][NMB], b[2][SK_U][NBW];
+    auto request = [&](auto buf_c, int s0) {
+        constexpr int B = decltype(buf_c)::value;
+#pragma unroll
+        for (int u = 0; u < SK_U; ++u) {
+            const int ks = min(s0 + 32 * u, kq - 32);      // (a short last batch repeats its final step: masked below)
+#pragma unroll
+            for (int nb = 0; nb < NBW; ++nb) b[B][u][nb] = *reinterpret_cast<const sk_u32x4*>(wp[nb] + ks);
+#pragma unroll
+            for (int mb = 0; mb < NMB; ++mb) a[B][u][mb] = *reinterpret_cast<const sk_u32x4*>(xp[mb] + ks);
+        }
+    };
+    auto multiply = [&](auto buf_c, int s0) {
+        constexpr int B = decltype(buf_c)::value;
+#pragma unroll
+        for (int u = 0; u < SK_U; ++u) {
+            const bool live = s0 + 32 * u < kq;      // (no branch between the steps: a step past the end contributes zeros)
+#pragma unroll
+            for (int nb = 0; nb < NBW; ++nb) {
+                sk_u32x4 bv = b[B][u][nb];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) bv[c] = live ? bv[c] : 0u;
+#pragma unroll
+                for (int mb = 0; mb < NMB; ++mb) {
+                    if constexpr (BF16)
+                        acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sk_bf16x8, a[B][u][mb]),
+                                                                              __builtin_bit_cast(sk_bf16x8, bv), acc[mb][nb], 0, 0, 0);
+                    else
+                        acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(sk_f16x8, a[B][u][mb]),
+                                                                             __builtin_bit_cast(sk_f16x8, bv), acc[mb][nb], 0, 0, 0);
+                }
+            }
+        }
+    };
+    using B0 = std::integral_constant<int, 0>;
+    using B1 = std::integral_constant<int, 1>;
+    constexpr int STEP = 32 * SK_U;
+    request(B0{}, 0);
+    for (int s0 = 0; s0 < kq; s0 += 2 * STEP) {
+        if (s0 + STEP < kq) request(B1{}, s0 + STEP);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(B0{}, s0);
+        if (s0 + STEP < kq) {
+            if (s0 + 2 * STEP < kq) request(B0{}, s0 + 2 * STEP);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(B1{}, s0 + STEP);
+        }
+    }
+    // lane holds rows 16 mb + 4 (lane / 16) + j, column 16 nb + lane % 16
+#pragma unroll
+    for (int mb = 0; mb < NMB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NBW; ++nb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) part[wv][mb * 16 + 4 * (lane >> 4) + j][nb * 16 + (lane & 15)] = acc[mb][nb][j];
+    __syncthreads();
+    // the four partial sums in a fixed order, two neighbouring columns per thread
+    constexpr int PAIRS = NMB * 16 * NBW * 8;
+    for (int i = threadIdx.x; i < PAIRS; i += 256) {
+        const int row = i / (NBW * 8), c = (i - row * (NBW * 8)) * 2;
+        if (row >= T || n0 + c >= N) continue;
+        float v0 = part[0][row][c] + part[1][row][c] + part[2][row][c] + part[3][row][c];
+        float v1 = part[0][row][c + 1] + part[1][row][c + 1] + part[2][row][c + 1] + part[3][row][c + 1];
+        uint32_t packed;
+        if constexpr (BF16)
+            packed = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)v0) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)v1) << 16);
+        else
+            packed = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)v0) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)v1) << 16);
+        *reinterpret_cast<uint32_t*>(out + (int64_t)row * ld_out + n0 + c) = packed;
+    }
+}
+
+}  // namespace bitsmoe
+
+using namespace bitsmoe;
+
+extern "C" int bitsmoe_skinny_linear(const void* x, int32_t dtype, int64_t ld_x, const void* weight, int64_t n_rows,
+                                     int32_t in_features, int32_t out_features, void* out, int64_t ld_out, void* stream) {
+    BITSMOE_REQUIRE(dtype == BITSMOE_DT_F16 || dtype == BITSMOE_DT_BF16, "dtype must be f16 (0) or bf16 (1)");
+    BITSMOE_REQUIRE(n_rows >= 0 && n_rows <= 64, "n_rows must be in [0, 64]");
+    BITSMOE_REQUIRE(in_features >= 128 && in_features % 128 == 0, "in_features must be a positive multiple of 128");
+    BITSMOE_REQUIRE(out_features >= 2 && out_features % 2 == 0, "out_features must be even");
+    BITSMOE_REQUIRE(ld_x >= in_features && ld_x % 8 == 0, "ld_x must be at least in_features and a multiple of 8");
+    BITSMOE_REQUIRE(ld_out >= out_features && ld_out % 2 == 0, "ld_out must be at least out_features and even");
+    if (n_rows == 0) return BITSMOE_OK;
+    BITSMOE_REQUIRE(x && weight && out, "null pointer");
+    BITSMOE_REQUIRE((((uintptr_t)x | (uintptr_t)weight) & 15) == 0 && ((uintptr_t)out & 3) == 0,
+                    "x and weight must be 16-byte aligned, out 4-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const bool bf16 = dtype == BITSMOE_DT_BF16;
+    // two 16-column blocks per wavefront once that still leaves a workgroup per CU and more (half the re-reads of x)
+    const bool two = out_features >= 32 * 512;
+    const int nmb = (int)((n_rows + 15) / 16);
+    const unsigned grid = (unsigned)((out_features + (two ? 32 : 16) - 1) / (two ? 32 : 16));
+#define BITSMOE_SKINNY(B, NMB, NBW)                                                                                     \
+    hipLaunchKernelGGL((k_skinny_linear<B, NMB, NBW>), dim3(grid), dim3(256), 0, st, (const uint16_t*)x, ld_x,           \
+                       (const uint16_t*)weight, (int)n_rows, in_features, out_features, (uint16_t*)out, ld_out)
+#define BITSMOE_SKINNY_M(B, NBW)                                      \
+    do {                                                              \
+        if (nmb == 1) BITSMOE_SKINNY(B, 1, NBW);                      \
+        else if (nmb == 2) BITSMOE_SKINNY(B, 2, NBW);                 \
+        else if (nmb == 3) BITSMOE_SKINNY(B, 3, NBW);                 \
+        else BITSMOE_SKINNY(B, 4, NBW);                               \
+    } while (0)
+    if (bf16) {
+        if (two) BITSMOE_SKINNY_M(true, 2); else BITSMOE_SKINNY_M(true, 1);
+    } else {
+        if (two) BITSMOE_SKINNY_M(false, 2); else BITSMOE_SKINNY_M(false, 1);
+    }
+#undef BITSMOE_SKINNY_M
+#undef BITSMOE_SKINNY
+    BITSMOE_HIP_TRY(hipGetLastError());
+    return BITSMOE_OK;
+}

@@ -175,6 +175,17 @@ int bitsmoe_router_linear_topk(const void* hidden, int32_t dtype, int64_t ld_hid
                                int32_t ids_are_i64, float* weights, void* stream);
 
 /*
+ * A bias-free linear layer for at most 64 rows: out[T, N] = x[T, K] * W[N, K]^T, 16-bit x / W / out of one dtype, fp32
+ * sums in a fixed order.  The two GEMMs around the operator -- shared-basis, router and shared-expert projections in
+ * (bitsmoe/models/qwen3moe/bitsmoe_block.py:63-64 and the routers' linear layers), output projections out
+ * (bitsmoe/models/base_block.py:414) -- have this shape at decode sizes: tens of MB of weights against a handful of
+ * tokens.  W in the framework's [out_features, in_features] layout, contiguous; in_features a multiple of 128,
+ * out_features even; x rows ld_x elements apart (a multiple of 8), x and W 16-byte aligned.
+ */
+int bitsmoe_skinny_linear(const void* x, int32_t dtype, int64_t ld_x, const void* weight, int64_t n_rows,
+                          int32_t in_features, int32_t out_features, void* out, int64_t ld_out, void* stream);
+
+/*
  * The block's closing elementwise pass: one row of the operand of the output GEMM in the activation dtype,
  *   out[t, 0 .. rank_out)                      = rank_accum[t, :]  (fp32 -> 16 bit; bitsmoe/models/base_block.py:414 casts
  *                                                 with a framework op)

@@ -159,7 +159,7 @@ def _block_reference(block, x):
     ("deepseekv2", {"shared_intermediate": 256}),
     ("deepseekv2", {}),
 ])
-@pytest.mark.parametrize("tokens", [1, 24])
+@pytest.mark.parametrize("tokens", [1, 9, 24])
 @pytest.mark.parametrize("fused", [True, False])
 def test_block_forward_matches_oracle(cuda_device, family, kw, tokens, fused, monkeypatch):
     """The block against the float64 restatement: in its one-GEMM-in / one-GEMM-out form (the shared-basis

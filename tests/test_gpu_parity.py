@@ -675,3 +675,31 @@ def test_router_linear_kernel_matches_oracle(cuda_device, tokens, hidden, n_expe
     if hip.router_linear_topk_possible(view, w.to(cuda_device), top_k):
         sel3, wt3 = hip.router_linear_topk(view, w.to(cuda_device), top_k, renorm, weight_scale=scale)
         assert torch.equal(sel3, sel) and torch.equal(wt3, wt)
+
+
+@pytest.mark.parametrize("rows,k,n", [(1, 2048, 4224), (32, 2048, 9728), (64, 2048, 2048), (33, 4864, 2048), (7, 128, 2),
+                                      (48, 640, 1000), (16, 1536, 16384)])
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+def test_skinny_linear_matches_float64(cuda_device, rows, k, n, dtype_name):
+    """out = x @ W.T for a few rows: equal to the float64 product of the same 16-bit values up to fp32 summation and one
+    rounding to the 16-bit output; the same bits on every call; rows of a wider tensor as input."""
+    import torch
+
+    hip = _hip()
+    rng = np.random.default_rng(rows * 31 + n)
+    dt = torch.float16 if dtype_name == "f16" else torch.bfloat16
+    x = torch.from_numpy(rng.normal(size=(rows, k)).astype(np.float32)).to(dt)
+    w = torch.from_numpy((rng.normal(size=(n, k)) * 0.05).astype(np.float32)).to(dt)
+    ref = x.double().numpy() @ w.double().numpy().T
+    xd, wd = x.to(cuda_device), w.to(cuda_device)
+    assert hip.skinny_linear_possible(xd, wd)
+    out = hip.skinny_linear(xd, wd)
+    assert out.dtype == dt and tuple(out.shape) == (rows, n)
+    eps = 2.0 ** -8 if dtype_name == "bf16" else 2.0 ** -11
+    err = np.abs(out.double().cpu().numpy() - ref)
+    assert float((err / (np.abs(ref) * eps + 1e-4 * np.abs(ref).max())).max()) <= 1.0
+    assert torch.equal(hip.skinny_linear(xd, wd), out)
+    wide = torch.zeros((rows, k + 64), dtype=dt, device=cuda_device)
+    wide[:, 16:16 + k] = xd
+    if hip.skinny_linear_possible(wide[:, 16:16 + k], wd):
+        assert torch.equal(hip.skinny_linear(wide[:, 16:16 + k], wd), out)
