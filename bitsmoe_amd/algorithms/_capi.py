@@ -127,7 +127,8 @@ def load() -> ctypes.CDLL:
     lib.bitsmoe_router_linear_topk.argtypes = [c_void_p, c_int32, c_int64, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32,
                                                c_float, c_int32, c_void_p, c_int32, c_void_p, c_void_p]
     lib.bitsmoe_skinny_linear.restype = c_int32
-    lib.bitsmoe_skinny_linear.argtypes = [c_void_p, c_int32, c_int64, c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int64, c_void_p]
+    lib.bitsmoe_skinny_linear.argtypes = [c_void_p, c_int32, c_int32, c_int64, c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int64,
+                                          c_void_p]
     lib.bitsmoe_block_finish.restype = c_int32
     lib.bitsmoe_block_finish.argtypes = [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int64,
                                          c_int32, c_void_p, c_int64, c_void_p]

@@ -588,26 +588,32 @@ SKINNY_LINEAR_MAX_ROWS = 64
 
 
 def skinny_linear_possible(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Can skinny_linear take these tensors?  (at most 64 rows of 16-bit x [T, K] with unit column stride and 16-byte
-    aligned rows, a contiguous weight [N, K] of the same dtype, K a multiple of 128, N even.)"""
-    return (x.is_cuda and x.dim() == 2 and weight.dim() == 2 and x.dtype in (torch.float16, torch.bfloat16)
-            and weight.dtype == x.dtype and weight.is_contiguous() and x.stride(1) == 1
-            and 1 <= int(x.shape[0]) <= SKINNY_LINEAR_MAX_ROWS and int(x.shape[1]) == int(weight.shape[1])
-            and int(x.shape[1]) % 128 == 0 and int(weight.shape[0]) % 2 == 0
-            and (int(x.shape[0]) <= 1 or int(x.stride(0)) % 8 == 0) and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+    """Can skinny_linear take these tensors?  (at most 64 rows of x [T, K] in the weight's 16-bit dtype -- or at most 16
+    rows of fp32, rounded to that dtype inside the kernel -- with unit column stride and 16-byte aligned rows, a
+    contiguous weight [N, K], K a multiple of 128, N even.)"""
+    if not (x.is_cuda and x.dim() == 2 and weight.dim() == 2 and weight.dtype in (torch.float16, torch.bfloat16)
+            and weight.is_contiguous() and x.stride(1) == 1 and int(x.shape[1]) == int(weight.shape[1])
+            and int(x.shape[1]) % 128 == 0 and int(weight.shape[0]) % 2 == 0 and x.data_ptr() % 16 == 0
+            and weight.data_ptr() % 16 == 0):
+        return False
+    rows = int(x.shape[0])
+    if x.dtype == torch.float32:
+        return 1 <= rows <= 16 and (rows <= 1 or int(x.stride(0)) % 4 == 0)
+    return x.dtype == weight.dtype and 1 <= rows <= SKINNY_LINEAR_MAX_ROWS and (rows <= 1 or int(x.stride(0)) % 8 == 0)
 
 
 def skinny_linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """x @ weight.T for a few rows (a bias-free linear layer at decode sizes): the weight is streamed once at HBM speed,
-    fp32 sums in a fixed order, result in x's dtype."""
+    fp32 sums in a fixed order, result in the weight's dtype.  fp32 x (at most 16 rows) is rounded to that dtype first,
+    inside the kernel: x.to(weight.dtype) @ weight.T without the cast's own pass."""
     _check(skinny_linear_possible(x, weight), "skinny_linear: unsupported shapes, dtypes or alignment")
     dev = x.device
     t, k, n = int(x.shape[0]), int(x.shape[1]), int(weight.shape[0])
-    out = torch.empty((t, n), dtype=x.dtype, device=dev)
+    out = torch.empty((t, n), dtype=weight.dtype, device=dev)
     with torch.cuda.device(dev):
-        _capi.check(_lib.bitsmoe_skinny_linear(x.data_ptr(), _capi.DT_F16 if x.dtype == torch.float16 else _capi.DT_BF16,
-                                               int(x.stride(0)) if t > 1 else k, weight.data_ptr(), t, k, n, out.data_ptr(), n,
-                                               _stream_ptr(dev)))
+        _capi.check(_lib.bitsmoe_skinny_linear(x.data_ptr(), _capi.DT_F16 if weight.dtype == torch.float16 else _capi.DT_BF16,
+                                               1 if x.dtype == torch.float32 else 0, int(x.stride(0)) if t > 1 else k,
+                                               weight.data_ptr(), t, k, n, out.data_ptr(), n, _stream_ptr(dev)))
     return out
 
 

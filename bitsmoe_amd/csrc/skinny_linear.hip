@@ -20,9 +20,14 @@ typedef __bf16 sk_bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int SK_U = 4;      // k-steps per batch of loads
 
-template <bool BF16, int NMB, int NBW>
-__global__ __launch_bounds__(256) void k_skinny_linear(const uint16_t* __restrict__ x, int64_t ld_x, const uint16_t* __restrict__ w,
+// XF32: x is fp32 and is rounded to the 16-bit type on its way into the MFMA (the cast of the operator's fp32 output in
+// front of the output projection, bitsmoe/models/base_block.py:414, without a pass of its own); one 16-row block only.
+template <bool BF16, int NMB, int NBW, bool XF32 = false>
+__global__ __launch_bounds__(256) void k_skinny_linear(const void* __restrict__ x_any, int64_t ld_x, const uint16_t* __restrict__ w,
                                                        int T, int K, int N, uint16_t* __restrict__ out, int64_t ld_out) {
+    static_assert(!XF32 || NMB == 1, "fp32 rows: one block of 16 rows");
+    const uint16_t* __restrict__ x = reinterpret_cast<const uint16_t*>(x_any);
+    const float* __restrict__ xf = reinterpret_cast<const float*>(x_any);
     __shared__ float part[4][NMB * 16][NBW * 16 + 1];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int n0 = blockIdx.x * (NBW * 16);
@@ -30,6 +35,7 @@ __global__ __launch_bounds__(256) void k_skinny_linear(const uint16_t* __restric
     const int kbase = wv * kq + (lane >> 4) * 8;
     const uint16_t* xp[NMB];
     const uint16_t* wp[NBW];
+    const float* xfp = xf + (int64_t)min(lane & 15, T - 1) * ld_x + kbase;
 #pragma unroll
     for (int mb = 0; mb < NMB; ++mb) xp[mb] = x + (int64_t)min(mb * 16 + (lane & 15), T - 1) * ld_x + kbase;
 #pragma unroll
@@ -40,6 +46,7 @@ __global__ __launch_bounds__(256) void k_skinny_linear(const uint16_t* __restric
 #pragma unroll
         for (int nb = 0; nb < NBW; ++nb) acc[mb][nb] = sk_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     sk_u32x4 a[2][SK_U][NMB], b[2][SK_U][NBW];
+    sk_f32x4 af[2][SK_U][XF32 ? 2 : 1];      // (fp32 rows as loaded: eight values per lane and k-step)
     auto request = [&](auto buf_c, int s0) {
         constexpr int B = decltype(buf_c)::value;
 #pragma unroll
@@ -47,15 +54,33 @@ __global__ __launch_bounds__(256) void k_skinny_linear(const uint16_t* __restric
             const int ks = min(s0 + 32 * u, kq - 32);      // (a short last batch repeats its final step: masked below)
 #pragma unroll
             for (int nb = 0; nb < NBW; ++nb) b[B][u][nb] = *reinterpret_cast<const sk_u32x4*>(wp[nb] + ks);
+            if constexpr (XF32) {
+                af[B][u][0] = *reinterpret_cast<const sk_f32x4*>(xfp + ks);
+                af[B][u][1] = *reinterpret_cast<const sk_f32x4*>(xfp + ks + 4);
+            } else {
 #pragma unroll
-            for (int mb = 0; mb < NMB; ++mb) a[B][u][mb] = *reinterpret_cast<const sk_u32x4*>(xp[mb] + ks);
+                for (int mb = 0; mb < NMB; ++mb) a[B][u][mb] = *reinterpret_cast<const sk_u32x4*>(xp[mb] + ks);
+            }
         }
+    };
+    auto round16 = [](float v) -> uint32_t {
+        if constexpr (BF16)
+            return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)v);
+        else
+            return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)v);
     };
     auto multiply = [&](auto buf_c, int s0) {
         constexpr int B = decltype(buf_c)::value;
 #pragma unroll
         for (int u = 0; u < SK_U; ++u) {
             const bool live = s0 + 32 * u < kq;      // (no branch between the steps: a step past the end contributes zeros)
+            if constexpr (XF32) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const sk_f32x4 v = af[B][u][c >> 1];
+                    a[B][u][0][c] = round16(v[2 * (c & 1)]) | (round16(v[2 * (c & 1) + 1]) << 16);
+                }
+            }
 #pragma unroll
             for (int nb = 0; nb < NBW; ++nb) {
                 sk_u32x4 bv = b[B][u][nb];
@@ -115,13 +140,15 @@ __global__ __launch_bounds__(256) void k_skinny_linear(const uint16_t* __restric
 
 using namespace bitsmoe;
 
-extern "C" int bitsmoe_skinny_linear(const void* x, int32_t dtype, int64_t ld_x, const void* weight, int64_t n_rows,
-                                     int32_t in_features, int32_t out_features, void* out, int64_t ld_out, void* stream) {
+extern "C" int bitsmoe_skinny_linear(const void* x, int32_t dtype, int32_t x_is_f32, int64_t ld_x, const void* weight,
+                                     int64_t n_rows, int32_t in_features, int32_t out_features, void* out, int64_t ld_out,
+                                     void* stream) {
     BITSMOE_REQUIRE(dtype == BITSMOE_DT_F16 || dtype == BITSMOE_DT_BF16, "dtype must be f16 (0) or bf16 (1)");
-    BITSMOE_REQUIRE(n_rows >= 0 && n_rows <= 64, "n_rows must be in [0, 64]");
+    BITSMOE_REQUIRE(n_rows >= 0 && n_rows <= (x_is_f32 ? 16 : 64), "n_rows must be in [0, 64] (fp32 rows: [0, 16])");
     BITSMOE_REQUIRE(in_features >= 128 && in_features % 128 == 0, "in_features must be a positive multiple of 128");
     BITSMOE_REQUIRE(out_features >= 2 && out_features % 2 == 0, "out_features must be even");
-    BITSMOE_REQUIRE(ld_x >= in_features && ld_x % 8 == 0, "ld_x must be at least in_features and a multiple of 8");
+    BITSMOE_REQUIRE(ld_x >= in_features && ld_x % (x_is_f32 ? 4 : 8) == 0,
+                    "ld_x must be at least in_features and a multiple of 8 (fp32 rows: of 4)");
     BITSMOE_REQUIRE(ld_out >= out_features && ld_out % 2 == 0, "ld_out must be at least out_features and even");
     if (n_rows == 0) return BITSMOE_OK;
     BITSMOE_REQUIRE(x && weight && out, "null pointer");
@@ -134,7 +161,7 @@ extern "C" int bitsmoe_skinny_linear(const void* x, int32_t dtype, int64_t ld_x,
     const int nmb = (int)((n_rows + 15) / 16);
     const unsigned grid = (unsigned)((out_features + (two ? 32 : 16) - 1) / (two ? 32 : 16));
 #define BITSMOE_SKINNY(B, NMB, NBW)                                                                                     \
-    hipLaunchKernelGGL((k_skinny_linear<B, NMB, NBW>), dim3(grid), dim3(256), 0, st, (const uint16_t*)x, ld_x,           \
+    hipLaunchKernelGGL((k_skinny_linear<B, NMB, NBW>), dim3(grid), dim3(256), 0, st, x, ld_x,           \
                        (const uint16_t*)weight, (int)n_rows, in_features, out_features, (uint16_t*)out, ld_out)
 #define BITSMOE_SKINNY_M(B, NBW)                                      \
     do {                                                              \
@@ -143,7 +170,14 @@ extern "C" int bitsmoe_skinny_linear(const void* x, int32_t dtype, int64_t ld_x,
         else if (nmb == 3) BITSMOE_SKINNY(B, 3, NBW);                 \
         else BITSMOE_SKINNY(B, 4, NBW);                               \
     } while (0)
-    if (bf16) {
+    if (x_is_f32) {
+        if (bf16)
+            hipLaunchKernelGGL((k_skinny_linear<true, 1, 1, true>), dim3((unsigned)((out_features + 15) / 16)), dim3(256), 0, st, x,
+                               ld_x, (const uint16_t*)weight, (int)n_rows, in_features, out_features, (uint16_t*)out, ld_out);
+        else
+            hipLaunchKernelGGL((k_skinny_linear<false, 1, 1, true>), dim3((unsigned)((out_features + 15) / 16)), dim3(256), 0, st, x,
+                               ld_x, (const uint16_t*)weight, (int)n_rows, in_features, out_features, (uint16_t*)out, ld_out);
+    } else if (bf16) {
         if (two) BITSMOE_SKINNY_M(true, 2); else BITSMOE_SKINNY_M(true, 1);
     } else {
         if (two) BITSMOE_SKINNY_M(false, 2); else BITSMOE_SKINNY_M(false, 1);

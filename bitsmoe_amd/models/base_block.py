@@ -616,6 +616,8 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
             sh_logit = big[:, rng["sh_logit"][0]:rng["sh_logit"][1]] if shared_gate is not None else None
             operand = mlp_forward_cuda.block_finish(rank_accum, dtype, big[:, rng["sh_gate"][0]:rng["sh_gate"][1]],
                                                     big[:, rng["sh_up"][0]:rng["sh_up"][1]], sh_logit)
+        elif 0 < token_count <= min(_SKINNY_ROWS, 16) and mlp_forward_cuda.skinny_linear_possible(rank_accum, plan["w_out"]):
+            operand = rank_accum      # (fp32: the few-rows kernel rounds it to the activation dtype on its way in)
         else:
             operand = mlp_forward_cuda.block_finish(rank_accum, dtype)
         out = _block_linear(operand, plan["w_out"])

@@ -181,9 +181,13 @@ int bitsmoe_router_linear_topk(const void* hidden, int32_t dtype, int64_t ld_hid
  * (bitsmoe/models/base_block.py:414) -- have this shape at decode sizes: tens of MB of weights against a handful of
  * tokens.  W in the framework's [out_features, in_features] layout, contiguous; in_features a multiple of 128,
  * out_features even; x rows ld_x elements apart (a multiple of 8), x and W 16-byte aligned.
+ * x_is_f32 = 1: x is fp32 (at most 16 rows, ld_x a multiple of 4) and is rounded to `dtype` on its way into the MFMA:
+ * the cast of the operator's fp32 rank_accum in front of the output projection (bitsmoe/models/base_block.py:414)
+ * without a pass of its own.
  */
-int bitsmoe_skinny_linear(const void* x, int32_t dtype, int64_t ld_x, const void* weight, int64_t n_rows,
-                          int32_t in_features, int32_t out_features, void* out, int64_t ld_out, void* stream);
+int bitsmoe_skinny_linear(const void* x, int32_t dtype, int32_t x_is_f32, int64_t ld_x, const void* weight,
+                          int64_t n_rows, int32_t in_features, int32_t out_features, void* out, int64_t ld_out,
+                          void* stream);
 
 /*
  * The block's closing elementwise pass: one row of the operand of the output GEMM in the activation dtype,

@@ -703,3 +703,8 @@ def test_skinny_linear_matches_float64(cuda_device, rows, k, n, dtype_name):
     wide[:, 16:16 + k] = xd
     if hip.skinny_linear_possible(wide[:, 16:16 + k], wd):
         assert torch.equal(hip.skinny_linear(wide[:, 16:16 + k], wd), out)
+    # fp32 rows (at most 16) are rounded to the weight's dtype inside the kernel: the same bits as casting first
+    xf = torch.from_numpy(rng.normal(size=(rows, k)).astype(np.float32)).to(cuda_device)
+    assert hip.skinny_linear_possible(xf, wd) == (rows <= 16)
+    if rows <= 16:
+        assert torch.equal(hip.skinny_linear(xf, wd), hip.skinny_linear(xf.to(dt), wd))
