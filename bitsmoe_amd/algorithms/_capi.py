@@ -42,6 +42,8 @@ EXPORTED_SYMBOLS = (
     "bitsmoe_router_linear_topk",
     "bitsmoe_block_finish",
     "bitsmoe_skinny_linear",
+    "bitsmoe_prepared_linear_weight_elements",
+    "bitsmoe_prepare_linear_weight",
     "bitsmoe_forward_workspace_bytes",
     "bitsmoe_forward_workspace_bytes_sets",
     "bitsmoe_moe_forward",
@@ -124,11 +126,15 @@ def load() -> ctypes.CDLL:
     lib.bitsmoe_router_softmax_topk_strided.argtypes = [c_void_p, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_float,
                                                         c_int32, c_void_p, c_int32, c_void_p, c_void_p]
     lib.bitsmoe_router_linear_topk.restype = c_int32
-    lib.bitsmoe_router_linear_topk.argtypes = [c_void_p, c_int32, c_int64, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32,
-                                               c_float, c_int32, c_void_p, c_int32, c_void_p, c_void_p]
+    lib.bitsmoe_router_linear_topk.argtypes = [c_void_p, c_int32, c_int64, c_void_p, c_int32, c_int64, c_int32, c_int32, c_int32,
+                                               c_int32, c_float, c_int32, c_void_p, c_int32, c_void_p, c_void_p]
     lib.bitsmoe_skinny_linear.restype = c_int32
-    lib.bitsmoe_skinny_linear.argtypes = [c_void_p, c_int32, c_int32, c_int64, c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int64,
-                                          c_void_p]
+    lib.bitsmoe_skinny_linear.argtypes = [c_void_p, c_int32, c_int32, c_int64, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p,
+                                          c_int64, c_void_p]
+    lib.bitsmoe_prepared_linear_weight_elements.restype = c_int64
+    lib.bitsmoe_prepared_linear_weight_elements.argtypes = [c_int32, c_int32]
+    lib.bitsmoe_prepare_linear_weight.restype = c_int32
+    lib.bitsmoe_prepare_linear_weight.argtypes = [c_void_p, c_int32, c_int32, c_void_p, c_void_p]
     lib.bitsmoe_block_finish.restype = c_int32
     lib.bitsmoe_block_finish.argtypes = [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_int64,
                                          c_int32, c_void_p, c_int64, c_void_p]

@@ -554,66 +554,119 @@ def router_softmax_topk(router_logits: torch.Tensor, top_k: int, renormalize: bo
     return selected, weights
 
 
-def router_linear_topk_possible(hidden: torch.Tensor, weight: torch.Tensor, top_k: int) -> bool:
+def router_linear_topk_possible(hidden: torch.Tensor, weight, top_k: int) -> bool:
     """Can router_linear_topk take these tensors?  (16-bit hidden states [T, K] with unit column stride and 16-byte
-    aligned rows, a contiguous weight [E, K] of the same dtype, K a multiple of 128, at most 256 experts.)"""
-    return (hidden.is_cuda and hidden.dim() == 2 and weight.dim() == 2 and hidden.dtype in (torch.float16, torch.bfloat16)
-            and weight.dtype == hidden.dtype and weight.is_contiguous() and hidden.stride(1) == 1
-            and int(hidden.shape[1]) == int(weight.shape[1]) and int(hidden.shape[1]) % 128 == 0
+    aligned rows, a contiguous weight [E, K] of the same dtype -- or a PreparedLinearWeight of it --, K a multiple of
+    128, at most 256 experts.)"""
+    if isinstance(weight, PreparedLinearWeight):
+        w_dtype, e, k = weight.dtype, weight.out_features, weight.in_features
+    else:
+        if not (weight.dim() == 2 and weight.is_contiguous() and weight.data_ptr() % 16 == 0):
+            return False
+        w_dtype, e, k = weight.dtype, int(weight.shape[0]), int(weight.shape[1])
+    return (hidden.is_cuda and hidden.dim() == 2 and hidden.dtype in (torch.float16, torch.bfloat16) and w_dtype == hidden.dtype
+            and hidden.stride(1) == 1 and int(hidden.shape[1]) == k and k % 128 == 0
             and (int(hidden.shape[0]) <= 1 or int(hidden.stride(0)) % 8 == 0) and hidden.data_ptr() % 16 == 0
-            and weight.data_ptr() % 16 == 0 and 1 <= int(top_k) <= min(64, int(weight.shape[0])) and int(weight.shape[0]) <= 256)
+            and 1 <= int(top_k) <= min(64, e) and e <= 256)
 
 
-def router_linear_topk(hidden: torch.Tensor, weight: torch.Tensor, top_k: int, renormalize: bool = True,
+def router_linear_topk(hidden: torch.Tensor, weight, top_k: int, renormalize: bool = True,
                        round_dtype: Optional[torch.dtype] = None, weight_scale: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
     """The router's linear layer with fp32 logits (hidden.float() @ weight.float().T: exact products of 16-bit values,
     fp32 sums), softmax, top-k, optional renormalisation, * weight_scale, optional round trip through `round_dtype`:
-    ONE kernel, no logits in memory.  Returns (selected int64 [T, k], weights fp32 [T, k])."""
+    ONE kernel, no logits in memory.  `weight`: a tensor [E, K] or a PreparedLinearWeight of it (the same sums in the same
+    order from consecutive memory).  Returns (selected int64 [T, k], weights fp32 [T, k])."""
     _check(router_linear_topk_possible(hidden, weight, top_k), "router_linear_topk: unsupported shapes, dtypes or alignment")
     _check(round_dtype in (None, torch.float16, torch.bfloat16), "round_dtype must be None, float16 or bfloat16")
     dev = hidden.device
-    t, k_dim, e = int(hidden.shape[0]), int(hidden.shape[1]), int(weight.shape[0])
+    prepared = isinstance(weight, PreparedLinearWeight)
+    t, k_dim = int(hidden.shape[0]), int(hidden.shape[1])
+    e = weight.out_features if prepared else int(weight.shape[0])
     selected = torch.empty((t, int(top_k)), dtype=torch.int64, device=dev)
     weights = torch.empty((t, int(top_k)), dtype=torch.float32, device=dev)
     codes = {torch.float16: 0, torch.bfloat16: 1}
     with torch.cuda.device(dev):
         _capi.check(_lib.bitsmoe_router_linear_topk(
-            hidden.data_ptr(), codes[hidden.dtype], int(hidden.stride(0)) if t > 1 else k_dim, weight.data_ptr(), t, k_dim, e,
+            hidden.data_ptr(), codes[hidden.dtype], int(hidden.stride(0)) if t > 1 else k_dim,
+            weight.data.data_ptr() if prepared else weight.data_ptr(), 1 if prepared else 0, t, k_dim, e,
             int(top_k), 1 if renormalize else 0, float(weight_scale), -1 if round_dtype is None else codes[round_dtype],
             selected.data_ptr(), 1, weights.data_ptr(), _stream_ptr(dev)))
     return selected, weights
 
 
+def prepared_linear_weight_of(owner, weight: torch.Tensor) -> "PreparedLinearWeight":
+    """The PreparedLinearWeight of `weight`, cached on `owner` (any object) and remade when the tensor is rebound or
+    written in place (address and version counter)."""
+    stamp = (weight.data_ptr(), -1 if weight.is_inference() else weight._version, tuple(weight.shape), weight.dtype)
+    cached = getattr(owner, "_bitsmoe_prepared_weight", None)
+    if cached is None or cached[0] != stamp:
+        cached = (stamp, PreparedLinearWeight(weight.detach()))
+        try:
+            object.__setattr__(owner, "_bitsmoe_prepared_weight", cached)
+        except (AttributeError, TypeError):
+            pass
+    return cached[1]
+
+
 SKINNY_LINEAR_MAX_ROWS = 64
 
 
-def skinny_linear_possible(x: torch.Tensor, weight: torch.Tensor) -> bool:
+class PreparedLinearWeight:
+    """A weight [N, K] re-laid out once into the order the few-rows kernel's MFMAs take it (every load of a wavefront
+    is then 1 KB of consecutive memory).  A snapshot of the weight's values."""
+
+    def __init__(self, weight: torch.Tensor):
+        _check(weight.is_cuda and weight.dim() == 2 and weight.dtype in (torch.float16, torch.bfloat16) and weight.is_contiguous()
+               and int(weight.shape[1]) % 128 == 0 and int(weight.shape[0]) >= 1 and weight.data_ptr() % 16 == 0,
+               "PreparedLinearWeight: a contiguous 16-bit CUDA weight [N, K] with K a multiple of 128")
+        self.out_features, self.in_features = int(weight.shape[0]), int(weight.shape[1])
+        self.dtype, self.device = weight.dtype, weight.device
+        n = int(_lib.bitsmoe_prepared_linear_weight_elements(self.in_features, self.out_features))
+        self.data = torch.empty((n,), dtype=weight.dtype, device=weight.device)
+        with torch.cuda.device(weight.device):
+            _capi.check(_lib.bitsmoe_prepare_linear_weight(weight.data_ptr(), self.in_features, self.out_features,
+                                                           self.data.data_ptr(), _stream_ptr(weight.device)))
+
+
+def skinny_linear_possible(x: torch.Tensor, weight) -> bool:
     """Can skinny_linear take these tensors?  (at most 64 rows of x [T, K] in the weight's 16-bit dtype -- or at most 16
     rows of fp32, rounded to that dtype inside the kernel -- with unit column stride and 16-byte aligned rows, a
-    contiguous weight [N, K], K a multiple of 128, N even.)"""
-    if not (x.is_cuda and x.dim() == 2 and weight.dim() == 2 and weight.dtype in (torch.float16, torch.bfloat16)
-            and weight.is_contiguous() and x.stride(1) == 1 and int(x.shape[1]) == int(weight.shape[1])
-            and int(x.shape[1]) % 128 == 0 and int(weight.shape[0]) % 2 == 0 and x.data_ptr() % 16 == 0
-            and weight.data_ptr() % 16 == 0):
+    contiguous weight [N, K], K a multiple of 128, N even; a PreparedLinearWeight: at most 16 rows.)"""
+    prepared = isinstance(weight, PreparedLinearWeight)
+    if prepared:
+        w_dtype, n, k = weight.dtype, weight.out_features, weight.in_features
+        if n % 2 != 0:
+            return False
+    else:
+        if not (weight.dim() == 2 and weight.dtype in (torch.float16, torch.bfloat16) and weight.is_contiguous()
+                and weight.data_ptr() % 16 == 0 and int(weight.shape[0]) % 2 == 0):
+            return False
+        w_dtype, n, k = weight.dtype, int(weight.shape[0]), int(weight.shape[1])
+    if not (x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and int(x.shape[1]) == k and k % 128 == 0 and x.data_ptr() % 16 == 0):
         return False
     rows = int(x.shape[0])
     if x.dtype == torch.float32:
         return 1 <= rows <= 16 and (rows <= 1 or int(x.stride(0)) % 4 == 0)
-    return x.dtype == weight.dtype and 1 <= rows <= SKINNY_LINEAR_MAX_ROWS and (rows <= 1 or int(x.stride(0)) % 8 == 0)
+    return x.dtype == w_dtype and 1 <= rows <= SKINNY_LINEAR_MAX_ROWS and (rows <= 1 or int(x.stride(0)) % 8 == 0)
 
 
-def skinny_linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+def skinny_linear(x: torch.Tensor, weight) -> torch.Tensor:
     """x @ weight.T for a few rows (a bias-free linear layer at decode sizes): the weight is streamed once at HBM speed,
     fp32 sums in a fixed order, result in the weight's dtype.  fp32 x (at most 16 rows) is rounded to that dtype first,
-    inside the kernel: x.to(weight.dtype) @ weight.T without the cast's own pass."""
+    inside the kernel: x.to(weight.dtype) @ weight.T without the cast's own pass.  `weight`: a tensor [N, K] or a
+    PreparedLinearWeight."""
     _check(skinny_linear_possible(x, weight), "skinny_linear: unsupported shapes, dtypes or alignment")
     dev = x.device
-    t, k, n = int(x.shape[0]), int(x.shape[1]), int(weight.shape[0])
-    out = torch.empty((t, n), dtype=weight.dtype, device=dev)
+    prepared = isinstance(weight, PreparedLinearWeight)
+    w_dtype = weight.dtype
+    t, k = int(x.shape[0]), int(x.shape[1])
+    n = weight.out_features if prepared else int(weight.shape[0])
+    out = torch.empty((t, n), dtype=w_dtype, device=dev)
+    w_ptr = weight.data.data_ptr() if prepared else weight.data_ptr()
     with torch.cuda.device(dev):
-        _capi.check(_lib.bitsmoe_skinny_linear(x.data_ptr(), _capi.DT_F16 if weight.dtype == torch.float16 else _capi.DT_BF16,
-                                               1 if x.dtype == torch.float32 else 0, int(x.stride(0)) if t > 1 else k,
-                                               weight.data_ptr(), t, k, n, out.data_ptr(), n, _stream_ptr(dev)))
+        _capi.check(_lib.bitsmoe_skinny_linear(x.data_ptr(), _capi.DT_F16 if w_dtype == torch.float16 else _capi.DT_BF16,
+                                               1 if x.dtype == torch.float32 else 0, int(x.stride(0)) if t > 1 else k, w_ptr,
+                                               1 if prepared else 0, t, k, n, out.data_ptr(), n, _stream_ptr(dev)))
     return out
 
 

@@ -213,7 +213,9 @@ __global__ __launch_bounds__(256) void k_router_rank_topk(const void* __restrict
 // loads), the partial sums meet in LDS (a tree in a fixed order: the same logits whenever the inputs are the same), then
 // the wavefronts rank the tokens, 16 / NW each.
 // x [T, K] and weight [E, K] are read as MFMA operands straight from memory (16 bytes per lane).
-template <bool BF16, int NB, int NW>
+// PREP: the weight in MFMA operand order ([16-expert block][k-step of 32][lane][8 values]: bitsmoe_prepare_linear_weight):
+// a wavefront's load is 1 KB of consecutive memory.
+template <bool BF16, int NB, int NW, bool PREP>
 __global__ __launch_bounds__(NW * 64) void k_router_linear_topk(const uint16_t* __restrict__ x, int64_t ld_x,
                                                                 const uint16_t* __restrict__ weight, int T, int K, int E, int k,
                                                                 float wscale, int renorm, int round_dt,
@@ -247,8 +249,13 @@ __global__ __launch_bounds__(NW * 64) void k_router_linear_topk(const uint16_t* 
             a[u] = *reinterpret_cast<const u32x4*>(xp + ks);
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
-                const int e = min(nb * 16 + (lane & 15), E - 1);
-                b[u][nb] = *reinterpret_cast<const u32x4*>(weight + (int64_t)e * K + kbase + ks);
+                if constexpr (PREP) {
+                    const int blk = min(nb, (E - 1) >> 4);      // (blocks past the last expert repeat it: masked below)
+                    b[u][nb] = *reinterpret_cast<const u32x4*>(weight + (((int64_t)blk * (K >> 5) + ((wv * kq + ks) >> 5)) * 64 + lane) * 8);
+                } else {
+                    const int e = min(nb * 16 + (lane & 15), E - 1);
+                    b[u][nb] = *reinterpret_cast<const u32x4*>(weight + (int64_t)e * K + kbase + ks);
+                }
             }
         }
         __builtin_amdgcn_sched_barrier(0);      // (every request of the group is out before its first MFMA)
@@ -367,7 +374,7 @@ extern "C" int bitsmoe_router_softmax_topk(const void* logits, int32_t logits_dt
 }
 
 extern "C" int bitsmoe_router_linear_topk(const void* hidden, int32_t dtype, int64_t ld_hidden, const void* weight,
-                                          int64_t n_tokens, int32_t hidden_size, int32_t n_experts, int32_t top_k,
+                                          int32_t weight_is_prepared, int64_t n_tokens, int32_t hidden_size, int32_t n_experts, int32_t top_k,
                                           int32_t renormalize, float weight_scale, int32_t round_dtype, void* selected,
                                           int32_t ids_are_i64, float* weights, void* stream) {
     BITSMOE_REQUIRE(n_tokens >= 0 && n_tokens < ((int64_t)1 << 31), "token count out of range");
@@ -387,16 +394,21 @@ extern "C" int bitsmoe_router_linear_topk(const void* hidden, int32_t dtype, int
     int64_t* s64 = ids_are_i64 ? (int64_t*)selected : nullptr;
     const dim3 grid((unsigned)((n_tokens + 15) / 16));
     const bool bf16 = dtype == BITSMOE_DT_BF16;
-#define BITSMOE_ROUTER_LINEAR(B, NB, NWIDE)                                                                                  \
+#define BITSMOE_ROUTER_LINEAR_P(B, NB, NWIDE, PR)                                                                             \
     do {                                                                                                                     \
         if (wide_wg)                                                                                                         \
-            hipLaunchKernelGGL((k_router_linear_topk<B, NB, NWIDE>), grid, dim3(NWIDE * 64), 0, st, (const uint16_t*)hidden, \
+            hipLaunchKernelGGL((k_router_linear_topk<B, NB, NWIDE, PR>), grid, dim3(NWIDE * 64), 0, st,                      \
+                               (const uint16_t*)hidden, ld_hidden, (const uint16_t*)weight, (int)n_tokens, hidden_size,      \
+                               n_experts, top_k, weight_scale, renormalize, round_dtype, s32, s64, weights);                 \
+        else                                                                                                                 \
+            hipLaunchKernelGGL((k_router_linear_topk<B, NB, 4, PR>), grid, dim3(256), 0, st, (const uint16_t*)hidden,        \
                                ld_hidden, (const uint16_t*)weight, (int)n_tokens, hidden_size, n_experts, top_k,             \
                                weight_scale, renormalize, round_dtype, s32, s64, weights);                                   \
-        else                                                                                                                 \
-            hipLaunchKernelGGL((k_router_linear_topk<B, NB, 4>), grid, dim3(256), 0, st, (const uint16_t*)hidden, ld_hidden,  \
-                               (const uint16_t*)weight, (int)n_tokens, hidden_size, n_experts, top_k, weight_scale,          \
-                               renormalize, round_dtype, s32, s64, weights);                                                 \
+    } while (0)
+#define BITSMOE_ROUTER_LINEAR(B, NB, NWIDE)                                                      \
+    do {                                                                                         \
+        if (weight_is_prepared) BITSMOE_ROUTER_LINEAR_P(B, NB, NWIDE, true);                     \
+        else BITSMOE_ROUTER_LINEAR_P(B, NB, NWIDE, false);                                       \
     } while (0)
     // (more than 128 experts: eight wavefronts, the partial sums of sixteen would not fit the LDS)
     if (n_experts <= 64) {
@@ -407,6 +419,7 @@ extern "C" int bitsmoe_router_linear_topk(const void* hidden, int32_t dtype, int
         if (bf16) BITSMOE_ROUTER_LINEAR(true, 16, 8); else BITSMOE_ROUTER_LINEAR(false, 16, 8);
     }
 #undef BITSMOE_ROUTER_LINEAR
+#undef BITSMOE_ROUTER_LINEAR_P
     BITSMOE_HIP_TRY(hipGetLastError());
     return BITSMOE_OK;
 }

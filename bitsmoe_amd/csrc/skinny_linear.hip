@@ -22,7 +22,10 @@ constexpr int SK_U = 4;      // k-steps per batch of loads
 
 // XF32: x is fp32 and is rounded to the 16-bit type on its way into the MFMA (the cast of the operator's fp32 output in
 // front of the output projection, bitsmoe/models/base_block.py:414, without a pass of its own); one 16-row block only.
-template <bool BF16, int NMB, int NBW, bool XF32 = false>
+// PREP: W was re-laid out once (bitsmoe_prepare_linear_weight) into the order the MFMA takes it: [16-column block]
+// [k-step of 32][lane][8 values], so that a wavefront's load is 1 KB of consecutive memory instead of sixteen 64-byte
+// pieces of sixteen rows.
+template <bool BF16, int NMB, int NBW, bool XF32 = false, bool PREP = false>
 __global__ __launch_bounds__(256) void k_skinny_linear(const void* __restrict__ x_any, int64_t ld_x, const uint16_t* __restrict__ w,
                                                        int T, int K, int N, uint16_t* __restrict__ out, int64_t ld_out) {
     static_assert(!XF32 || NMB == 1, "fp32 rows: one block of 16 rows");
@@ -39,7 +42,12 @@ __global__ __launch_bounds__(256) void k_skinny_linear(const void* __restrict__ 
 #pragma unroll
     for (int mb = 0; mb < NMB; ++mb) xp[mb] = x + (int64_t)min(mb * 16 + (lane & 15), T - 1) * ld_x + kbase;
 #pragma unroll
-    for (int nb = 0; nb < NBW; ++nb) wp[nb] = w + (int64_t)min(n0 + nb * 16 + (lane & 15), N - 1) * K + kbase;
+    for (int nb = 0; nb < NBW; ++nb) {
+        if constexpr (PREP)      // (N is a multiple of 16 * NBW there; step ks of this wavefront: + (ks / 32) * 512 elements)
+            wp[nb] = w + ((int64_t)(blockIdx.x * NBW + nb) * (K >> 5) + wv * (kq >> 5)) * 512 + lane * 8;
+        else
+            wp[nb] = w + (int64_t)min(n0 + nb * 16 + (lane & 15), N - 1) * K + kbase;
+    }
     sk_f32x4 acc[NMB][NBW];
 #pragma unroll
     for (int mb = 0; mb < NMB; ++mb)
@@ -53,7 +61,8 @@ __global__ __launch_bounds__(256) void k_skinny_linear(const void* __restrict__ 
         for (int u = 0; u < SK_U; ++u) {
             const int ks = min(s0 + 32 * u, kq - 32);      // (a short last batch repeats its final step: masked below)
 #pragma unroll
-            for (int nb = 0; nb < NBW; ++nb) b[B][u][nb] = *reinterpret_cast<const sk_u32x4*>(wp[nb] + ks);
+            for (int nb = 0; nb < NBW; ++nb)
+                b[B][u][nb] = *reinterpret_cast<const sk_u32x4*>(wp[nb] + (PREP ? ks * 16 : ks));
             if constexpr (XF32) {
                 af[B][u][0] = *reinterpret_cast<const sk_f32x4*>(xfp + ks);
                 af[B][u][1] = *reinterpret_cast<const sk_f32x4*>(xfp + ks + 4);
@@ -136,13 +145,47 @@ __global__ __launch_bounds__(256) void k_skinny_linear(const void* __restrict__ 
     }
 }
 
+// W [N, K] -> [ceil(N / 16)][K / 32][64 lanes][8]: lane = 16 * (k % 32 / 8) + n % 16 holds W[n][32 ks + 8 (lane / 16) .. + 7];
+// rows past N are zeros.  One thread per 16-byte piece.
+__global__ __launch_bounds__(256) void k_prepare_linear_weight(const uint16_t* __restrict__ w, int N, int K, uint16_t* __restrict__ out,
+                                                               int64_t pieces) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= pieces) return;
+    const int lane = (int)(i & 63);
+    const int64_t blk = i >> 6;
+    const int ksteps = K >> 5;
+    const int ks = (int)(blk % ksteps), nb = (int)(blk / ksteps);
+    const int n = nb * 16 + (lane & 15), k = ks * 32 + (lane >> 4) * 8;
+    sk_u32x4 v = {0u, 0u, 0u, 0u};
+    if (n < N) v = *reinterpret_cast<const sk_u32x4*>(w + (int64_t)n * K + k);
+    *reinterpret_cast<sk_u32x4*>(out + i * 8) = v;
+}
+
 }  // namespace bitsmoe
 
 using namespace bitsmoe;
 
+extern "C" int64_t bitsmoe_prepared_linear_weight_elements(int32_t in_features, int32_t out_features) {
+    if (in_features <= 0 || out_features <= 0) return 0;
+    return (int64_t)((out_features + 15) / 16) * 16 * in_features;
+}
+
+extern "C" int bitsmoe_prepare_linear_weight(const void* weight, int32_t in_features, int32_t out_features, void* prepared,
+                                             void* stream) {
+    BITSMOE_REQUIRE(in_features >= 128 && in_features % 128 == 0, "in_features must be a positive multiple of 128");
+    BITSMOE_REQUIRE(out_features >= 1, "out_features must be positive");
+    BITSMOE_REQUIRE(weight && prepared, "null pointer");
+    BITSMOE_REQUIRE((((uintptr_t)weight | (uintptr_t)prepared) & 15) == 0, "weight and prepared must be 16-byte aligned");
+    const int64_t pieces = bitsmoe_prepared_linear_weight_elements(in_features, out_features) / 8;
+    hipLaunchKernelGGL(k_prepare_linear_weight, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint16_t*)weight, out_features, in_features, (uint16_t*)prepared, pieces);
+    BITSMOE_HIP_TRY(hipGetLastError());
+    return BITSMOE_OK;
+}
+
 extern "C" int bitsmoe_skinny_linear(const void* x, int32_t dtype, int32_t x_is_f32, int64_t ld_x, const void* weight,
-                                     int64_t n_rows, int32_t in_features, int32_t out_features, void* out, int64_t ld_out,
-                                     void* stream) {
+                                     int32_t weight_is_prepared, int64_t n_rows, int32_t in_features, int32_t out_features,
+                                     void* out, int64_t ld_out, void* stream) {
     BITSMOE_REQUIRE(dtype == BITSMOE_DT_F16 || dtype == BITSMOE_DT_BF16, "dtype must be f16 (0) or bf16 (1)");
     BITSMOE_REQUIRE(n_rows >= 0 && n_rows <= (x_is_f32 ? 16 : 64), "n_rows must be in [0, 64] (fp32 rows: [0, 16])");
     BITSMOE_REQUIRE(in_features >= 128 && in_features % 128 == 0, "in_features must be a positive multiple of 128");
@@ -170,13 +213,26 @@ extern "C" int bitsmoe_skinny_linear(const void* x, int32_t dtype, int32_t x_is_
         else if (nmb == 3) BITSMOE_SKINNY(B, 3, NBW);                 \
         else BITSMOE_SKINNY(B, 4, NBW);                               \
     } while (0)
-    if (x_is_f32) {
-        if (bf16)
-            hipLaunchKernelGGL((k_skinny_linear<true, 1, 1, true>), dim3((unsigned)((out_features + 15) / 16)), dim3(256), 0, st, x,
-                               ld_x, (const uint16_t*)weight, (int)n_rows, in_features, out_features, (uint16_t*)out, ld_out);
-        else
-            hipLaunchKernelGGL((k_skinny_linear<false, 1, 1, true>), dim3((unsigned)((out_features + 15) / 16)), dim3(256), 0, st, x,
-                               ld_x, (const uint16_t*)weight, (int)n_rows, in_features, out_features, (uint16_t*)out, ld_out);
+    if (x_is_f32 || weight_is_prepared) {
+        // (the forms the block uses at a few tokens: one column block per wavefront)
+        BITSMOE_REQUIRE(!x_is_f32 || n_rows <= 16, "fp32 rows: at most 16 rows");
+        const dim3 g1((unsigned)((out_features + 15) / 16));
+        const int nmb1 = (int)((n_rows + 15) / 16);
+#define BITSMOE_SKINNY_1(B, NMB, XF, PR)                                                                                   \
+        hipLaunchKernelGGL((k_skinny_linear<B, NMB, 1, XF, PR>), g1, dim3(256), 0, st, x, ld_x, (const uint16_t*)weight,   \
+                           (int)n_rows, in_features, out_features, (uint16_t*)out, ld_out)
+#define BITSMOE_SKINNY_P(B)                                                                  \
+        do {                                                                                 \
+            if (x_is_f32 && weight_is_prepared) BITSMOE_SKINNY_1(B, 1, true, true);          \
+            else if (x_is_f32) BITSMOE_SKINNY_1(B, 1, true, false);                          \
+            else if (nmb1 == 1) BITSMOE_SKINNY_1(B, 1, false, true);                         \
+            else if (nmb1 == 2) BITSMOE_SKINNY_1(B, 2, false, true);                         \
+            else if (nmb1 == 3) BITSMOE_SKINNY_1(B, 3, false, true);                         \
+            else BITSMOE_SKINNY_1(B, 4, false, true);                                        \
+        } while (0)
+        if (bf16) BITSMOE_SKINNY_P(true); else BITSMOE_SKINNY_P(false);
+#undef BITSMOE_SKINNY_P
+#undef BITSMOE_SKINNY_1
     } else if (bf16) {
         if (two) BITSMOE_SKINNY_M(true, 2); else BITSMOE_SKINNY_M(true, 1);
     } else {

@@ -49,18 +49,39 @@ def _super_via_operator() -> bool:
     return _dense_via_operator() or os.environ.get("BITSMOE_SUPER_VIA_OPERATOR", "1") != "0"
 
 
-# Rows up to which the block's two stacked GEMMs run the library's own few-rows kernel instead of the framework's GEMM.
-# Whole block under graph replay, cold weights, 128-expert layer of hidden size 2048: 1 token 34.1 vs 40.2 us, 8 tokens
-# 55.3 vs 64.5, 16 tokens 70.7 vs 77.4, 32 tokens 82.8 vs 83.6, 64 tokens 100.8 vs 90.8; the 64-expert layer with two
-# shared experts (9728 stacked output features) at 32 tokens 118.6 vs 109.1: every workgroup of the kernel reads all rows
-# of x, which costs more than it saves from 32 rows on.  BITSMOE_BLOCK_SKINNY_ROWS overrides, 0 switches it off.
-_SKINNY_ROWS = int(_os.environ.get("BITSMOE_BLOCK_SKINNY_ROWS", "16"))
+# Rows up to which the block's two stacked GEMMs run the library's own few-rows kernel (against a copy of the stacked
+# weights in MFMA operand order) instead of the framework's GEMM.  Whole block under graph replay, cold weights,
+# 128-expert layer of hidden size 2048 (4224 stacked input features): 1 token 30.4 vs 40.6 us, 8 tokens 51.8 vs 65.5,
+# 16 tokens 67.1 vs 77.3, 24 tokens 76.9 vs 83.2, 32 tokens 79.2 vs 83.3, 48 tokens 88.9 vs 87.4, 64 tokens 97.4 vs 91.0.
+# Every workgroup of the kernel reads all rows of x, so from 17 rows on it is used only while there is about one workgroup
+# per CU and the contraction is short: the 64-expert layer with two shared experts (9728 stacked input features, 4864
+# output-side contraction) at 32 tokens ran 111.3 vs 108.2 us with the kernel for both GEMMs, 108.5 with it for the output
+# GEMM alone.  BITSMOE_BLOCK_SKINNY_ROWS overrides the row limit, 0 switches the kernel off.
+_SKINNY_ROWS = int(_os.environ.get("BITSMOE_BLOCK_SKINNY_ROWS", "32"))
+_SKINNY_WIDE_FEATURES = 5120      # output features up to which 17 to 32 rows still take the few-rows kernel
+_SKINNY_LONG_CONTRACTION = 4096   # ... and input features
+# BITSMOE_BLOCK_SKINNY_PREPARED=0: the few-rows kernel reads the stacked weights in the framework's layout (no extra copy)
+_SKINNY_PREPARED = _os.environ.get("BITSMOE_BLOCK_SKINNY_PREPARED", "1") != "0"
 
 
-def _block_linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """x [T, K] @ weight [N, K].T in x's dtype."""
-    if 0 < int(x.shape[0]) <= _SKINNY_ROWS and _HAS_MLP_FORWARD_CUDA and mlp_forward_cuda.skinny_linear_possible(x, weight):
-        return mlp_forward_cuda.skinny_linear(x, weight)
+def _block_linear(x: torch.Tensor, plan: dict, key: str) -> torch.Tensor:
+    """x [T, K] @ plan[key] [N, K].T in the weight's dtype.  At a few rows: the library's few-rows kernel against a copy of
+    the weight in MFMA operand order (made on first use, kept with the plan: one more copy of the stacked weights)."""
+    weight = plan[key]
+    rows = int(x.shape[0])
+    # (from 17 rows on only while there is about one workgroup per CU: every workgroup reads all rows of x)
+    few = 0 < rows <= _SKINNY_ROWS and (rows <= 16 or (int(weight.shape[0]) <= _SKINNY_WIDE_FEATURES
+                                                       and int(weight.shape[1]) <= _SKINNY_LONG_CONTRACTION))
+    if few and _HAS_MLP_FORWARD_CUDA:
+        if _SKINNY_PREPARED:
+            prepared = plan.get(key + "_prepared")
+            if prepared is None and mlp_forward_cuda.skinny_linear_possible(x, weight):
+                prepared = mlp_forward_cuda.PreparedLinearWeight(weight)
+                plan[key + "_prepared"] = prepared
+            if prepared is not None and mlp_forward_cuda.skinny_linear_possible(x, prepared):
+                return mlp_forward_cuda.skinny_linear(x, prepared)
+        if mlp_forward_cuda.skinny_linear_possible(x, weight):
+            return mlp_forward_cuda.skinny_linear(x, weight)
     return x @ weight.T
 
 
@@ -585,7 +606,7 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
         if plan is None:
             return None
         token_count = int(hidden_states.shape[0])
-        big = _block_linear(hidden_states, plan["w_in"])
+        big = _block_linear(hidden_states, plan, "w_in")
         rng = plan["ranges"]
         h_gate = big[:, rng["h_gate"][0]:rng["h_gate"][1]]
         h_up = big[:, rng["h_up"][0]:rng["h_up"][1]]
@@ -620,7 +641,7 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
             operand = rank_accum      # (fp32: the few-rows kernel rounds it to the activation dtype on its way in)
         else:
             operand = mlp_forward_cuda.block_finish(rank_accum, dtype)
-        out = _block_linear(operand, plan["w_out"])
+        out = _block_linear(operand, plan, "w_out")
         if self._super_expert_items:
             if side is not None:
                 cur = torch.cuda.current_stream(hidden_states.device)

@@ -45,7 +45,8 @@ class BitsMoE_DeepSeekSparseMoeBlock(BitsMoE_BaseSparseMoeBlock):
             top_k = int(gate.top_k)
             if mlp_forward_cuda.router_linear_topk_possible(x, gate.weight, top_k):
                 renorm = top_k > 1 and bool(gate.norm_topk_prob)
-                return mlp_forward_cuda.router_linear_topk(x, gate.weight.detach(), top_k, renorm, round_dtype=None,
+                return mlp_forward_cuda.router_linear_topk(x, mlp_forward_cuda.prepared_linear_weight_of(gate, gate.weight), top_k,
+                                                           renorm, round_dtype=None,
                                                            weight_scale=1.0 if renorm else float(gate.routed_scaling_factor))
         topk_idx, topk_weight, _aux = self.gate(hidden_states)
         return topk_idx.reshape(-1, topk_idx.shape[-1]), topk_weight.reshape(-1, topk_weight.shape[-1]).to(torch.float32)

@@ -56,8 +56,8 @@ class SoftmaxGreedyGate(nn.Module):
             if _HAS_MLP_FORWARD_CUDA and mlp_forward_cuda.router_linear_topk_possible(x, self.weight, self.top_k):
                 # fp32 logits (exact products of the 16-bit values, fp32 sums), softmax, greedy top-k and the
                 # renormalisation or scaling in ONE kernel
-                idx, weight = mlp_forward_cuda.router_linear_topk(x, self.weight.detach(), self.top_k, renorm, round_dtype=None,
-                                                                  weight_scale=scale)
+                idx, weight = mlp_forward_cuda.router_linear_topk(x, mlp_forward_cuda.prepared_linear_weight_of(self, self.weight),
+                                                                  self.top_k, renorm, round_dtype=None, weight_scale=scale)
                 return idx, weight, None
             if _HAS_MLP_FORWARD_CUDA:
                 # fp32 logits as the module computes them (one cast, one GEMM against the cached fp32 weight), then

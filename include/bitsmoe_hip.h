@@ -167,10 +167,10 @@ int bitsmoe_router_softmax_topk_strided(const void* logits, int32_t logits_dtype
  * are exact in fp32, so the MFMA sums equal the module's logits up to summation order; no logits reach memory.
  *   hidden  device f16 / bf16 [T, hidden_size], ld_hidden elements between rows (a multiple of 8), 16-byte aligned
  *   weight  device, the same dtype, [n_experts, hidden_size] contiguous; hidden_size a multiple of 128,
- *           n_experts <= 256
+ *           n_experts <= 256; weight_is_prepared = 1: the copy bitsmoe_prepare_linear_weight made of it
  */
 int bitsmoe_router_linear_topk(const void* hidden, int32_t dtype, int64_t ld_hidden, const void* weight,
-                               int64_t n_tokens, int32_t hidden_size, int32_t n_experts, int32_t top_k,
+                               int32_t weight_is_prepared, int64_t n_tokens, int32_t hidden_size, int32_t n_experts, int32_t top_k,
                                int32_t renormalize, float weight_scale, int32_t round_dtype, void* selected,
                                int32_t ids_are_i64, float* weights, void* stream);
 
@@ -184,10 +184,16 @@ int bitsmoe_router_linear_topk(const void* hidden, int32_t dtype, int64_t ld_hid
  * x_is_f32 = 1: x is fp32 (at most 16 rows, ld_x a multiple of 4) and is rounded to `dtype` on its way into the MFMA:
  * the cast of the operator's fp32 rank_accum in front of the output projection (bitsmoe/models/base_block.py:414)
  * without a pass of its own.
+ * weight_is_prepared = 1 (at most 16 rows): `weight` is the copy bitsmoe_prepare_linear_weight made of W, in the order the
+ * MFMA takes it ([16-column block][k-step of 32][lane][8 values]; bitsmoe_prepared_linear_weight_elements 16-bit elements):
+ * every load of a wavefront is 1 KB of consecutive memory.
  */
 int bitsmoe_skinny_linear(const void* x, int32_t dtype, int32_t x_is_f32, int64_t ld_x, const void* weight,
-                          int64_t n_rows, int32_t in_features, int32_t out_features, void* out, int64_t ld_out,
-                          void* stream);
+                          int32_t weight_is_prepared, int64_t n_rows, int32_t in_features, int32_t out_features,
+                          void* out, int64_t ld_out, void* stream);
+int64_t bitsmoe_prepared_linear_weight_elements(int32_t in_features, int32_t out_features);
+int bitsmoe_prepare_linear_weight(const void* weight, int32_t in_features, int32_t out_features, void* prepared,
+                                  void* stream);
 
 /*
  * The block's closing elementwise pass: one row of the operand of the output GEMM in the activation dtype,

@@ -665,6 +665,10 @@ def test_router_linear_kernel_matches_oracle(cuda_device, tokens, hidden, n_expe
     sel, wt = hip.router_linear_topk(x.to(cuda_device), w.to(cuda_device), top_k, renorm, weight_scale=scale)
     assert sel.dtype == torch.int64 and np.array_equal(sel.cpu().numpy(), idx_ref)
     assert np.allclose(wt.cpu().numpy(), w_ref * scale, rtol=2e-5, atol=1e-9)
+    # the weight re-laid out once in MFMA operand order: the same sums in the same order
+    selp, wtp = hip.router_linear_topk(x.to(cuda_device), hip.PreparedLinearWeight(w.to(cuda_device)), top_k, renorm,
+                                       weight_scale=scale)
+    assert torch.equal(selp, sel) and torch.equal(wtp, wt)
     # the two-step form (fp32 logits in memory, then the softmax / top-k kernel) picks the same
     sel2, wt2 = hip.router_softmax_topk(torch.from_numpy(logits).to(cuda_device), top_k, renorm, weight_scale=scale)
     assert torch.equal(sel2, sel) and torch.allclose(wt2, wt, rtol=2e-5, atol=1e-9)
@@ -703,8 +707,13 @@ def test_skinny_linear_matches_float64(cuda_device, rows, k, n, dtype_name):
     wide[:, 16:16 + k] = xd
     if hip.skinny_linear_possible(wide[:, 16:16 + k], wd):
         assert torch.equal(hip.skinny_linear(wide[:, 16:16 + k], wd), out)
+    # the weight re-laid out once in MFMA operand order: the same sums in the same order
+    pw = hip.PreparedLinearWeight(wd)
+    assert hip.skinny_linear_possible(xd, pw)
+    assert torch.equal(hip.skinny_linear(xd, pw), out)
     # fp32 rows (at most 16) are rounded to the weight's dtype inside the kernel: the same bits as casting first
     xf = torch.from_numpy(rng.normal(size=(rows, k)).astype(np.float32)).to(cuda_device)
     assert hip.skinny_linear_possible(xf, wd) == (rows <= 16)
     if rows <= 16:
         assert torch.equal(hip.skinny_linear(xf, wd), hip.skinny_linear(xf.to(dt), wd))
+        assert torch.equal(hip.skinny_linear(xf, hip.PreparedLinearWeight(wd)), hip.skinny_linear(xf.to(dt), wd))
