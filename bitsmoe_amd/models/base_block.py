@@ -56,10 +56,13 @@ def _super_via_operator() -> bool:
 # Every workgroup of the kernel reads all rows of x, so from 17 rows on it is used only while there is about one workgroup
 # per CU and the contraction is short: the 64-expert layer with two shared experts (9728 stacked input features, 4864
 # output-side contraction) at 32 tokens ran 111.3 vs 108.2 us with the kernel for both GEMMs, 108.5 with it for the output
-# GEMM alone.  BITSMOE_BLOCK_SKINNY_ROWS overrides the row limit, 0 switches the kernel off.
-_SKINNY_ROWS = int(_os.environ.get("BITSMOE_BLOCK_SKINNY_ROWS", "32"))
+# GEMM alone.  From 33 to 64 rows only the narrow output GEMM (2048 features) takes it: 40 tokens 85.0 vs 87.5 (both GEMMs:
+# 87.2), 48 tokens 87.0 vs 88.7 (90.4), 64 tokens 92.2 vs 93.1 (99.1).  BITSMOE_BLOCK_SKINNY_ROWS caps the rows, 0 switches
+# the kernel off.
+_SKINNY_ROWS = int(_os.environ.get("BITSMOE_BLOCK_SKINNY_ROWS", "64"))
 _SKINNY_WIDE_FEATURES = 5120      # output features up to which 17 to 32 rows still take the few-rows kernel
-_SKINNY_LONG_CONTRACTION = 4096   # ... and input features
+_SKINNY_NARROW_FEATURES = 2048    # ... and 33 to 64 rows
+_SKINNY_LONG_CONTRACTION = 4096   # input features up to which more than 16 rows take it
 # BITSMOE_BLOCK_SKINNY_PREPARED=0: the few-rows kernel reads the stacked weights in the framework's layout (no extra copy)
 _SKINNY_PREPARED = _os.environ.get("BITSMOE_BLOCK_SKINNY_PREPARED", "1") != "0"
 
@@ -70,8 +73,10 @@ def _block_linear(x: torch.Tensor, plan: dict, key: str) -> torch.Tensor:
     weight = plan[key]
     rows = int(x.shape[0])
     # (from 17 rows on only while there is about one workgroup per CU: every workgroup reads all rows of x)
-    few = 0 < rows <= _SKINNY_ROWS and (rows <= 16 or (int(weight.shape[0]) <= _SKINNY_WIDE_FEATURES
-                                                       and int(weight.shape[1]) <= _SKINNY_LONG_CONTRACTION))
+    n_out, n_in = int(weight.shape[0]), int(weight.shape[1])
+    few = 0 < rows <= _SKINNY_ROWS and (
+        rows <= 16 or (n_in <= _SKINNY_LONG_CONTRACTION
+                       and n_out <= (_SKINNY_WIDE_FEATURES if rows <= 32 else _SKINNY_NARROW_FEATURES)))
     if few and _HAS_MLP_FORWARD_CUDA:
         if _SKINNY_PREPARED:
             prepared = plan.get(key + "_prepared")
