@@ -130,7 +130,7 @@ def load() -> ctypes.CDLL:
                                                c_int32, c_float, c_int32, c_void_p, c_int32, c_void_p, c_void_p]
     lib.bitsmoe_skinny_linear.restype = c_int32
     lib.bitsmoe_skinny_linear.argtypes = [c_void_p, c_int32, c_int32, c_int64, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p,
-                                          c_int64, c_void_p]
+                                          c_int64, c_void_p, c_int64, c_void_p]
     lib.bitsmoe_prepared_linear_weight_elements.restype = c_int64
     lib.bitsmoe_prepared_linear_weight_elements.argtypes = [c_int32, c_int32]
     lib.bitsmoe_prepare_linear_weight.restype = c_int32

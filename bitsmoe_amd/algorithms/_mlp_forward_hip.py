@@ -650,11 +650,11 @@ def skinny_linear_possible(x: torch.Tensor, weight) -> bool:
     return x.dtype == w_dtype and 1 <= rows <= SKINNY_LINEAR_MAX_ROWS and (rows <= 1 or int(x.stride(0)) % 8 == 0)
 
 
-def skinny_linear(x: torch.Tensor, weight) -> torch.Tensor:
+def skinny_linear(x: torch.Tensor, weight, addend: Optional[torch.Tensor] = None) -> torch.Tensor:
     """x @ weight.T for a few rows (a bias-free linear layer at decode sizes): the weight is streamed once at HBM speed,
     fp32 sums in a fixed order, result in the weight's dtype.  fp32 x (at most 16 rows) is rounded to that dtype first,
     inside the kernel: x.to(weight.dtype) @ weight.T without the cast's own pass.  `weight`: a tensor [N, K] or a
-    PreparedLinearWeight."""
+    PreparedLinearWeight.  `addend`: fp32 [T, N] added to the sums before the result is rounded."""
     _check(skinny_linear_possible(x, weight), "skinny_linear: unsupported shapes, dtypes or alignment")
     dev = x.device
     prepared = isinstance(weight, PreparedLinearWeight)
@@ -663,10 +663,15 @@ def skinny_linear(x: torch.Tensor, weight) -> torch.Tensor:
     n = weight.out_features if prepared else int(weight.shape[0])
     out = torch.empty((t, n), dtype=w_dtype, device=dev)
     w_ptr = weight.data.data_ptr() if prepared else weight.data_ptr()
+    if addend is not None:
+        _check(addend.dtype == torch.float32 and tuple(addend.shape) == (t, n) and addend.stride(1) == 1 and addend.device == dev,
+               "skinny_linear: addend must be float32 [T, N] with unit column stride on x's device")
     with torch.cuda.device(dev):
         _capi.check(_lib.bitsmoe_skinny_linear(x.data_ptr(), _capi.DT_F16 if w_dtype == torch.float16 else _capi.DT_BF16,
                                                1 if x.dtype == torch.float32 else 0, int(x.stride(0)) if t > 1 else k, w_ptr,
-                                               1 if prepared else 0, t, k, n, out.data_ptr(), n, _stream_ptr(dev)))
+                                               1 if prepared else 0, t, k, n, out.data_ptr(), n,
+                                               None if addend is None else addend.data_ptr(),
+                                               0 if addend is None else (int(addend.stride(0)) if t > 1 else n), _stream_ptr(dev)))
     return out
 
 

@@ -27,7 +27,8 @@ constexpr int SK_U = 4;      // k-steps per batch of loads
 // pieces of sixteen rows.
 template <bool BF16, int NMB, int NBW, bool XF32 = false, bool PREP = false>
 __global__ __launch_bounds__(256) void k_skinny_linear(const void* __restrict__ x_any, int64_t ld_x, const uint16_t* __restrict__ w,
-                                                       int T, int K, int N, uint16_t* __restrict__ out, int64_t ld_out) {
+                                                       int T, int K, int N, uint16_t* __restrict__ out, int64_t ld_out,
+                                                       const float* __restrict__ addend, int64_t ld_add) {
     static_assert(!XF32 || NMB == 1, "fp32 rows: one block of 16 rows");
     const uint16_t* __restrict__ x = reinterpret_cast<const uint16_t*>(x_any);
     const float* __restrict__ xf = reinterpret_cast<const float*>(x_any);
@@ -136,6 +137,10 @@ __global__ __launch_bounds__(256) void k_skinny_linear(const void* __restrict__ 
         if (row >= T || n0 + c >= N) continue;
         float v0 = part[0][row][c] + part[1][row][c] + part[2][row][c] + part[3][row][c];
         float v1 = part[0][row][c + 1] + part[1][row][c + 1] + part[2][row][c + 1] + part[3][row][c + 1];
+        if (addend) {      // (fp32 [T, N] added to the sums before the one rounding of the result)
+            v0 += addend[(int64_t)row * ld_add + n0 + c];
+            v1 += addend[(int64_t)row * ld_add + n0 + c + 1];
+        }
         uint32_t packed;
         if constexpr (BF16)
             packed = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)v0) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)v1) << 16);
@@ -185,7 +190,7 @@ extern "C" int bitsmoe_prepare_linear_weight(const void* weight, int32_t in_feat
 
 extern "C" int bitsmoe_skinny_linear(const void* x, int32_t dtype, int32_t x_is_f32, int64_t ld_x, const void* weight,
                                      int32_t weight_is_prepared, int64_t n_rows, int32_t in_features, int32_t out_features,
-                                     void* out, int64_t ld_out, void* stream) {
+                                     void* out, int64_t ld_out, const float* addend, int64_t ld_addend, void* stream) {
     BITSMOE_REQUIRE(dtype == BITSMOE_DT_F16 || dtype == BITSMOE_DT_BF16, "dtype must be f16 (0) or bf16 (1)");
     BITSMOE_REQUIRE(n_rows >= 0 && n_rows <= (x_is_f32 ? 16 : 64), "n_rows must be in [0, 64] (fp32 rows: [0, 16])");
     BITSMOE_REQUIRE(in_features >= 128 && in_features % 128 == 0, "in_features must be a positive multiple of 128");
@@ -193,6 +198,7 @@ extern "C" int bitsmoe_skinny_linear(const void* x, int32_t dtype, int32_t x_is_
     BITSMOE_REQUIRE(ld_x >= in_features && ld_x % (x_is_f32 ? 4 : 8) == 0,
                     "ld_x must be at least in_features and a multiple of 8 (fp32 rows: of 4)");
     BITSMOE_REQUIRE(ld_out >= out_features && ld_out % 2 == 0, "ld_out must be at least out_features and even");
+    BITSMOE_REQUIRE(addend == nullptr || ld_addend >= out_features, "ld_addend must be at least out_features");
     if (n_rows == 0) return BITSMOE_OK;
     BITSMOE_REQUIRE(x && weight && out, "null pointer");
     BITSMOE_REQUIRE((((uintptr_t)x | (uintptr_t)weight) & 15) == 0 && ((uintptr_t)out & 3) == 0,
@@ -205,7 +211,7 @@ extern "C" int bitsmoe_skinny_linear(const void* x, int32_t dtype, int32_t x_is_
     const unsigned grid = (unsigned)((out_features + (two ? 32 : 16) - 1) / (two ? 32 : 16));
 #define BITSMOE_SKINNY(B, NMB, NBW)                                                                                     \
     hipLaunchKernelGGL((k_skinny_linear<B, NMB, NBW>), dim3(grid), dim3(256), 0, st, x, ld_x,           \
-                       (const uint16_t*)weight, (int)n_rows, in_features, out_features, (uint16_t*)out, ld_out)
+                       (const uint16_t*)weight, (int)n_rows, in_features, out_features, (uint16_t*)out, ld_out, (const float*)addend, ld_addend)
 #define BITSMOE_SKINNY_M(B, NBW)                                      \
     do {                                                              \
         if (nmb == 1) BITSMOE_SKINNY(B, 1, NBW);                      \
@@ -220,7 +226,7 @@ extern "C" int bitsmoe_skinny_linear(const void* x, int32_t dtype, int32_t x_is_
         const int nmb1 = (int)((n_rows + 15) / 16);
 #define BITSMOE_SKINNY_1(B, NMB, XF, PR)                                                                                   \
         hipLaunchKernelGGL((k_skinny_linear<B, NMB, 1, XF, PR>), g1, dim3(256), 0, st, x, ld_x, (const uint16_t*)weight,   \
-                           (int)n_rows, in_features, out_features, (uint16_t*)out, ld_out)
+                           (int)n_rows, in_features, out_features, (uint16_t*)out, ld_out, (const float*)addend, ld_addend)
 #define BITSMOE_SKINNY_P(B)                                                                  \
         do {                                                                                 \
             if (x_is_f32 && weight_is_prepared) BITSMOE_SKINNY_1(B, 1, true, true);          \

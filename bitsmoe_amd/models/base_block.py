@@ -67,9 +67,10 @@ _SKINNY_LONG_CONTRACTION = 4096   # input features up to which more than 16 rows
 _SKINNY_PREPARED = _os.environ.get("BITSMOE_BLOCK_SKINNY_PREPARED", "1") != "0"
 
 
-def _block_linear(x: torch.Tensor, plan: dict, key: str) -> torch.Tensor:
-    """x [T, K] @ plan[key] [N, K].T in the weight's dtype.  At a few rows: the library's few-rows kernel against a copy of
-    the weight in MFMA operand order (made on first use, kept with the plan: one more copy of the stacked weights)."""
+def _block_linear(x: torch.Tensor, plan: dict, key: str, addend: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [T, K] @ plan[key] [N, K].T (+ addend, fp32 [T, N]) in the weight's dtype.  At a few rows: the library's few-rows
+    kernel against a copy of the weight in MFMA operand order (made on first use, kept with the plan: one more copy of the
+    stacked weights), the addend taken in before the result is rounded."""
     weight = plan[key]
     rows = int(x.shape[0])
     # (from 17 rows on only while there is about one workgroup per CU: every workgroup reads all rows of x)
@@ -84,10 +85,11 @@ def _block_linear(x: torch.Tensor, plan: dict, key: str) -> torch.Tensor:
                 prepared = mlp_forward_cuda.PreparedLinearWeight(weight)
                 plan[key + "_prepared"] = prepared
             if prepared is not None and mlp_forward_cuda.skinny_linear_possible(x, prepared):
-                return mlp_forward_cuda.skinny_linear(x, prepared)
+                return mlp_forward_cuda.skinny_linear(x, prepared, addend)
         if mlp_forward_cuda.skinny_linear_possible(x, weight):
-            return mlp_forward_cuda.skinny_linear(x, weight)
-    return x @ weight.T
+            return mlp_forward_cuda.skinny_linear(x, weight, addend)
+    out = x @ weight.T
+    return out if addend is None else out.add_(addend)
 
 
 _SIDE_STREAMS: Dict[int, "torch.cuda.Stream"] = {}
@@ -646,8 +648,9 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
             operand = rank_accum      # (fp32: the few-rows kernel rounds it to the activation dtype on its way in)
         else:
             operand = mlp_forward_cuda.block_finish(rank_accum, dtype)
-        out = _block_linear(operand, plan, "w_out")
         if self._super_expert_items:
+            # (the super experts' share is ready long before the packed experts' call ends: joined here, it goes into the
+            # output GEMM's epilogue where the few-rows kernel runs, else it is added behind the GEMM)
             if side is not None:
                 cur = torch.cuda.current_stream(hidden_states.device)
                 cur.wait_stream(side)
@@ -655,14 +658,13 @@ class BitsMoE_BaseSparseMoeBlock(nn.Module):
                     sup.record_stream(cur)
             else:
                 sup = self._super_operator_output(hidden_states, selected, weights)
-            if sup is not None:
-                out.add_(sup)
-            else:
-                extra = torch.zeros_like(out)
-                self._run_super_experts(hidden_states, extra, selected.reshape(-1),
-                                        self._get_flat_token_ids(token_count, hidden_states.device),
-                                        weights.reshape(-1).to(dtype))
-                out = out + extra
+        out = _block_linear(operand, plan, "w_out", addend=sup)
+        if self._super_expert_items and sup is None:
+            extra = torch.zeros_like(out)
+            self._run_super_experts(hidden_states, extra, selected.reshape(-1),
+                                    self._get_flat_token_ids(token_count, hidden_states.device),
+                                    weights.reshape(-1).to(dtype))
+            out = out + extra
         return out, logits
 
     # ---- shared forward body --------------------------------------------------------------

@@ -187,10 +187,13 @@ int bitsmoe_router_linear_topk(const void* hidden, int32_t dtype, int64_t ld_hid
  * weight_is_prepared = 1 (at most 16 rows): `weight` is the copy bitsmoe_prepare_linear_weight made of W, in the order the
  * MFMA takes it ([16-column block][k-step of 32][lane][8 values]; bitsmoe_prepared_linear_weight_elements 16-bit elements):
  * every load of a wavefront is 1 KB of consecutive memory.
+ * addend (may be null): fp32 [n_rows, out_features], rows ld_addend elements apart, added to the sums before the one
+ * rounding of the result -- the dense experts' share of the block output, which the reference adds in a pass of its own
+ * (bitsmoe/models/base_block.py:291-307).
  */
 int bitsmoe_skinny_linear(const void* x, int32_t dtype, int32_t x_is_f32, int64_t ld_x, const void* weight,
                           int32_t weight_is_prepared, int64_t n_rows, int32_t in_features, int32_t out_features,
-                          void* out, int64_t ld_out, void* stream);
+                          void* out, int64_t ld_out, const float* addend, int64_t ld_addend, void* stream);
 int64_t bitsmoe_prepared_linear_weight_elements(int32_t in_features, int32_t out_features);
 int bitsmoe_prepare_linear_weight(const void* weight, int32_t in_features, int32_t out_features, void* prepared,
                                   void* stream);

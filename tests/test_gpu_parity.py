@@ -707,6 +707,11 @@ def test_skinny_linear_matches_float64(cuda_device, rows, k, n, dtype_name):
     wide[:, 16:16 + k] = xd
     if hip.skinny_linear_possible(wide[:, 16:16 + k], wd):
         assert torch.equal(hip.skinny_linear(wide[:, 16:16 + k], wd), out)
+    # an fp32 addend goes into the sums before the one rounding
+    add = torch.from_numpy(rng.normal(size=(rows, n)).astype(np.float32)).to(cuda_device)
+    with_add = hip.skinny_linear(xd, wd, add)
+    err = np.abs(with_add.double().cpu().numpy() - (ref + add.double().cpu().numpy()))
+    assert float((err / (np.abs(ref + add.double().cpu().numpy()) * eps + 1e-4 * np.abs(ref).max())).max()) <= 1.0
     # the weight re-laid out once in MFMA operand order: the same sums in the same order
     pw = hip.PreparedLinearWeight(wd)
     assert hip.skinny_linear_possible(xd, pw)
