@@ -280,7 +280,9 @@ __device__ __forceinline__ u32x4 scaled_f16x8(u32x4 raw, u32x4 sc) {
 // guarantees that no wavefront still reads either when the item begins (a workgroup barrier).
 // KEEP: the tile's sums are not stored; `keep[nbl]` receives them (the lane's rows a = 4*kg + j of column
 // 32*pair + 16*nbl + n), for a caller that goes on with them in registers.
-template <bool BF16, bool IDENT, int W, bool SPLIT, class AS, bool KEEP = false>
+// MANY: the activations of the wavefront's third and fourth assignment (chunks of more than eight assignments) are
+// requested ahead like those of the first two, instead of when they are staged (a memory round trip each, every group).
+template <bool BF16, bool IDENT, int W, bool SPLIT, class AS, bool KEEP = false, bool MANY = false>
 __device__ __forceinline__ void gateup_walk_item(gptr<uint32_t> payload, gptr<__half> scale_s, gptr<int32_t> rank_idx,
                                                  const FastSlab first, const uint16_t* __restrict__ h, int64_t ld,
                                                  const AS& as, int a0, int n_a, int T,
@@ -349,6 +351,11 @@ __device__ __forceinline__ void gateup_walk_item(gptr<uint32_t> payload, gptr<__
     // the number of loads in flight does not depend on the path and the waits can be counted)
     raw0 = act_at(0, rank_cur);
     raw1 = act_at(1, rank_cur);
+    [[maybe_unused]] u32x4 raw2 = {0, 0, 0, 0}, raw3 = {0, 0, 0, 0};
+    if constexpr (MANY) {
+        raw2 = act_at(2, rank_cur);
+        raw3 = act_at(3, rank_cur);
+    }
     // The payload of the first group is requested only now: loads return in order, so anything
     // requested behind it would be held back until it has arrived from HBM, and the first
     // operand could not be staged in the meantime.
@@ -368,12 +375,21 @@ __device__ __forceinline__ void gateup_walk_item(gptr<uint32_t> payload, gptr<__
         hs = hs_all + (g & 1) * (MAX_A * GU_STRIDE);
         if (pair < n_a) stage(I0{}, raw0, sc_cur);
         if (pair + 4 < n_a) stage(I1{}, raw1, sc_cur);
-        if (pair + 8 < n_a) stage(I2{}, act_at(2, rank_cur), sc_cur);      // (rare: fetched here, not ahead)
-        if (pair + 12 < n_a) stage(I3{}, act_at(3, rank_cur), sc_cur);
+        if constexpr (MANY) {
+            if (pair + 8 < n_a) stage(I2{}, raw2, sc_cur);
+            if (pair + 12 < n_a) stage(I3{}, raw3, sc_cur);
+        } else {
+            if (pair + 8 < n_a) stage(I2{}, act_at(2, rank_cur), sc_cur);      // (fetched here, not ahead)
+            if (pair + 12 < n_a) stage(I3{}, act_at(3, rank_cur), sc_cur);
+        }
         __syncthreads();   // the operand is complete
         if constexpr (more) {
             raw0 = act_at(0, rank_nxt);
             raw1 = act_at(1, rank_nxt);
+            if constexpr (MANY) {
+                raw2 = act_at(2, rank_nxt);
+                raw3 = act_at(3, rank_nxt);
+            }
         }
         // (inside the one-kernel forward the scheduler otherwise sinks these two requests behind the payload
         // requests below -- loads return in order, the next operand would wait for the next group's payload)

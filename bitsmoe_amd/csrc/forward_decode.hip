@@ -453,9 +453,14 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
                                                        g_begin, g_end, out, hs_all, cterm_lds, tid);
         } else {
             auto run = [&](auto w_c) {
-                gateup_walk_item<BF16, IDENT, decltype(w_c)::value, false>(payload, scale_s, rank_idx, first, h, ld, as, a0,
-                                                                           n_a, T, I, n_tiles, t, g_begin, g_end, out, hs_all,
-                                                                           cterm_lds, tid);
+                if (n_a > 8)      // (the chunk's wavefronts stage three or four assignments each)
+                    gateup_walk_item<BF16, IDENT, decltype(w_c)::value, false, decltype(as), false, true>(
+                        payload, scale_s, rank_idx, first, h, ld, as, a0, n_a, T, I, n_tiles, t, g_begin, g_end, out, hs_all,
+                        cterm_lds, tid);
+                else
+                    gateup_walk_item<BF16, IDENT, decltype(w_c)::value, false>(payload, scale_s, rank_idx, first, h, ld, as, a0,
+                                                                               n_a, T, I, n_tiles, t, g_begin, g_end, out, hs_all,
+                                                                               cterm_lds, tid);
             };
             if (first.bits == 2)
                 run(std::integral_constant<int, 2>{});

@@ -117,15 +117,16 @@ struct RankTopkLds {
     float picked[NW][64];
 };
 // One token by one wavefront (`wv` of its workgroup): v[i] is the logit of expert lane + 64 i (-inf past E).
-template <int NW>
-__device__ inline void rank_topk_token(float (&v)[ROUTER_RANK_PER_LANE], RankTopkLds<NW>& lds, int wv, int lane, int tkn, float wscale,
-                                       int E, int k, int renorm, int round_dt, int32_t* __restrict__ sel32,
-                                       int64_t* __restrict__ sel64, float* __restrict__ weights) {
+// LIVE: logits per lane that can exist (E <= 64 LIVE); the counting loop, which is most of the work, runs over those only.
+template <int LIVE, int NW>
+__device__ inline void rank_topk_live(float (&v)[ROUTER_RANK_PER_LANE], RankTopkLds<NW>& lds, int wv, int lane, int tkn, float wscale,
+                                      int E, int k, int renorm, int round_dt, int32_t* __restrict__ sel32,
+                                      int64_t* __restrict__ sel64, float* __restrict__ weights) {
     const int e2 = (E + 1) & ~1;
-    uint64_t mine[ROUTER_RANK_PER_LANE];
+    uint64_t mine[LIVE];
     float vmax = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) {
+    for (int i = 0; i < LIVE; ++i) {
         const int e = lane + 64 * i;
         vmax = fmaxf(vmax, v[i]);
         const uint32_t bits = __float_as_uint(v[i] + 0.0f);      // (-0 and +0 are one value)
@@ -135,10 +136,10 @@ __device__ inline void rank_topk_token(float (&v)[ROUTER_RANK_PER_LANE], RankTop
     }
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, d));
-    float pr[ROUTER_RANK_PER_LANE];
+    float pr[LIVE];
     float part = 0.0f;
 #pragma unroll
-    for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) {
+    for (int i = 0; i < LIVE; ++i) {
         pr[i] = (v[i] == -INFINITY) ? 0.0f : expf(v[i] - vmax);
         part += pr[i];
     }
@@ -148,15 +149,15 @@ __device__ inline void rank_topk_token(float (&v)[ROUTER_RANK_PER_LANE], RankTop
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    int rank[ROUTER_RANK_PER_LANE] = {0, 0, 0, 0};
+    int rank[LIVE] = {};
 #pragma unroll 4
     for (int o = 0; o < e2; o += 2) {
         const uint64_t q0 = lds.keys[wv][o], q1 = lds.keys[wv][o + 1];
 #pragma unroll
-        for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) rank[i] += (int)(q0 > mine[i]) + (int)(q1 > mine[i]);
+        for (int i = 0; i < LIVE; ++i) rank[i] += (int)(q0 > mine[i]) + (int)(q1 > mine[i]);
     }
 #pragma unroll
-    for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i)
+    for (int i = 0; i < LIVE; ++i)
         if (lane + 64 * i < E && rank[i] < k) lds.picked[wv][rank[i]] = pr[i] / denom;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -164,7 +165,7 @@ __device__ inline void rank_topk_token(float (&v)[ROUTER_RANK_PER_LANE], RankTop
     float picked_sum = 0.0f;
     for (int j = 0; j < k; ++j) picked_sum += lds.picked[wv][j];
 #pragma unroll
-    for (int i = 0; i < ROUTER_RANK_PER_LANE; ++i) {
+    for (int i = 0; i < LIVE; ++i) {
         if (lane + 64 * i < E && rank[i] < k) {
             float w = pr[i] / denom;
             if (renorm) w /= picked_sum;
@@ -183,6 +184,18 @@ __device__ inline void rank_topk_token(float (&v)[ROUTER_RANK_PER_LANE], RankTop
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int NW>
+__device__ inline void rank_topk_token(float (&v)[ROUTER_RANK_PER_LANE], RankTopkLds<NW>& lds, int wv, int lane, int tkn, float wscale,
+                                       int E, int k, int renorm, int round_dt, int32_t* __restrict__ sel32,
+                                       int64_t* __restrict__ sel64, float* __restrict__ weights) {
+    if (E <= 64)
+        rank_topk_live<1>(v, lds, wv, lane, tkn, wscale, E, k, renorm, round_dt, sel32, sel64, weights);
+    else if (E <= 128)
+        rank_topk_live<2>(v, lds, wv, lane, tkn, wscale, E, k, renorm, round_dt, sel32, sel64, weights);
+    else
+        rank_topk_live<ROUTER_RANK_PER_LANE>(v, lds, wv, lane, tkn, wscale, E, k, renorm, round_dt, sel32, sel64, weights);
 }
 
 template <int DT>
