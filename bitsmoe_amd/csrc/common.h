@@ -58,8 +58,13 @@ struct FastSlab {              // tile t of the slab: payload word pack_off + t*
 
 // Kernel argument (by value): the expert a grid coordinate stands for.
 constexpr int EXPERT_ORDER_MAX = 512;
-struct ExpertOrder {
-    uint16_t e[EXPERT_ORDER_MAX];
+struct ExpertOrder {      // (two 16-bit entries per word: a wave-uniform index then reads it with ONE scalar load of the
+    uint32_t w[EXPERT_ORDER_MAX / 2];      // kernel-argument segment; a 16-bit array element costs a vector load and its wait)
+    __host__ __device__ __forceinline__ int at(int i) const { return (int)((w[i >> 1] >> ((i & 1) * 16)) & 0xFFFFu); }
+    __host__ inline void set(int i, uint16_t v) {
+        const int sh = (i & 1) * 16;
+        w[i >> 1] = (w[i >> 1] & ~(0xFFFFu << sh)) | ((uint32_t)v << sh);
+    }
 };
 
 struct SlabTask {              // one (expert, slab) unit of the down projection

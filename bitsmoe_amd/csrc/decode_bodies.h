@@ -128,21 +128,33 @@ __device__ __forceinline__ int routed_id(const void* __restrict__ selected, int 
 // ids 32 or 64 bits wide), in entry order -- the order the routing kernel's stable sort gives
 // (bitsmoe/models/base_block.py:258-289) -- written to `r`; returns their number (wave-uniform).  All 256
 // threads call it; it contains two workgroup barriers.  Ids that belong to no packed expert match nothing.
-__device__ inline int inline_route(const void* __restrict__ selected, int ids_are_i64, int n_flat, int top_k, int gid,
-                                   InlineRouteLds& r, int tid) {
-    const int lane = tid & 63, wave = tid >> 6;
+// In two halves, so that a caller can put the requests for its other tables between the request for the ids and their
+// first use (one round trip for all of them): inline_route_request, then inline_route_finish.
+struct RouteIds {
+    int ids[4];      // entries 4 tid .. 4 tid + 3 (the last entry again past the end)
+};
+__device__ __forceinline__ RouteIds inline_route_request(const void* __restrict__ selected, int ids_are_i64, int n_flat, int tid) {
+    RouteIds q;
     const int base = 4 * tid;
-    int ids[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const int i = min(base + k, n_flat - 1);
-        ids[k] = ids_are_i64 ? (int)reinterpret_cast<const int64_t*>(selected)[i] : reinterpret_cast<const int32_t*>(selected)[i];
+        q.ids[k] = ids_are_i64 ? (int)reinterpret_cast<const int64_t*>(selected)[i] : reinterpret_cast<const int32_t*>(selected)[i];
     }
+    return q;
+}
+// (the ids are in registers from here on, whatever the compiler would have liked to do with their loads)
+__device__ __forceinline__ void hold_route_ids(RouteIds& q) {
+    asm volatile("" : "+v"(q.ids[0]), "+v"(q.ids[1]), "+v"(q.ids[2]), "+v"(q.ids[3]));
+}
+__device__ inline int inline_route_finish(const RouteIds& q, int n_flat, int top_k, int gid, InlineRouteLds& r, int tid) {
+    const int lane = tid & 63, wave = tid >> 6;
+    const int base = 4 * tid;
     int count = 0;
     bool hit[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        hit[k] = base + k < n_flat && ids[k] == gid;
+        hit[k] = base + k < n_flat && q.ids[k] == gid;
         count += hit[k] ? 1 : 0;
     }
     const int incl = wave_inclusive_scan(count);
@@ -166,6 +178,11 @@ __device__ inline int inline_route(const void* __restrict__ selected, int ids_ar
     }
     __syncthreads();
     return __builtin_amdgcn_readfirstlane(min(total, ROUTE_INLINE_MAX_ROWS));
+}
+__device__ inline int inline_route(const void* __restrict__ selected, int ids_are_i64, int n_flat, int top_k, int gid,
+                                   InlineRouteLds& r, int tid) {
+    const RouteIds q = inline_route_request(selected, ids_are_i64, n_flat, tid);
+    return inline_route_finish(q, n_flat, top_k, gid, r, tid);
 }
 
 constexpr int GRID_EXPERTS = 0;   // the expert coordinate of the grid is the expert

@@ -41,9 +41,9 @@ inline bool walk_possible(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
 
 // The expert a grid coordinate stands for: by decreasing payload size, or the identity.
 inline ExpertOrder expert_order_of(const bitsmoe_matset* set) {
-    ExpertOrder o;
+    ExpertOrder o{};
     for (int i = 0; i < EXPERT_ORDER_MAX; ++i)
-        o.e[i] = set->has_cost_order && i < set->n_experts ? set->cost_order[i] : (uint16_t)i;
+        o.set(i, set->has_cost_order && i < set->n_experts ? set->cost_order[i] : (uint16_t)i);
     return o;
 }
 

@@ -33,6 +33,21 @@ __device__ inline FastSlab load_fast_slab(const FastSlab* __restrict__ tab, int 
                     __builtin_amdgcn_readfirstlane(v[2]), __builtin_amdgcn_readfirstlane(v[3])};
 }
 
+// The fields of an expert's record held in scalar registers from HERE on.  They are first used behind the routing scan's
+// workgroup barriers; loads from tables the kernel only reads may be moved, and left alone the compiler moves them down
+// to those uses, where each is one more dependent round trip in front of the first payload request.  Called after
+// everything else the start-up needs has been requested.
+__device__ __forceinline__ void hold_fast_expert(FastExpert& fe) {
+    uint64_t p0 = (uint64_t)fe.payload, p1 = (uint64_t)fe.scale, p2 = (uint64_t)fe.s, p3 = (uint64_t)fe.rank_idx,
+             p4 = (uint64_t)fe.scale_s;
+    asm volatile("" : "+s"(p0), "+s"(p1), "+s"(p2), "+s"(p3), "+s"(p4), "+s"(fe.num_slabs), "+s"(fe.uniform_bits));
+    fe.payload = (const uint32_t*)p0;
+    fe.scale = (const __half*)p1;
+    fe.s = (const __half*)p2;
+    fe.rank_idx = (const int32_t*)p3;
+    fe.scale_s = (const __half*)p4;
+}
+
 // The words of one wavefront's column-block pair for one (slab, tile) block: 2-bit {nb0, nb1};
 // 4-bit {nb0 j0, nb0 j1, nb1 j0, nb1 j1}; 3-bit {low nb0, low nb1, high nb0, high nb1}.
 // `blk` is wave-uniform, `unit` = pair*64 + lane and `hi_unit` are 32-bit lane offsets.

@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_decode(
     int e = bid / (n_tchunks * n_groups);
     int chunk = -1;
     if constexpr (MODE == GRID_EXPERTS) {      // expensive experts first (the identity when there is no order)
-        if (E <= EXPERT_ORDER_MAX) e = mt ? up_order.e[e] : gate_order.e[e];
+        if (E <= EXPERT_ORDER_MAX) e = mt ? up_order.at(e) : gate_order.at(e);
     } else if constexpr (MODE == GRID_ACTIVE) {
         e = nth_active_expert(expert_offsets, E, A, e, tid & 63);
         if (e < 0) return;
@@ -341,6 +341,13 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     static_assert(!ROUTED || MODE != GRID_CHUNKS, "inline routing serves whole experts");
     BITSMOE_TL(g_tl_walk, 0);
     const int tid = threadIdx.x;
+    // (the routed ids do not depend on the workgroup's expert: requested before anything else, they arrive while the
+    // expert's tables are looked up; all of it is waited for together, in front of the scan)
+    [[maybe_unused]] RouteIds rid;
+    if constexpr (ROUTED && MODE == GRID_EXPERTS) rid = inline_route_request(selected, ids_are_i64, n_flat, tid);
+    // (the arguments the start-up goes through, in scalar registers now: one batch of loads from the argument segment
+    // and one wait, where the compiler would fetch each in front of its first use, one dependent wait after the other)
+    asm volatile("" ::"s"(gate_max_slabs), "s"(up_max_slabs), "s"(E), "s"(n_tiles), "s"(n_unsplit), "s"(split), "s"(top_k));
     {   // this workgroup's share of the accumulator (before any exit)
         const int64_t total = (int64_t)gridDim.x * 256;
         for (int64_t i = (int64_t)blockIdx.x * 256 + tid; i < zero_n; i += total) zero_out[i] = 0.0f;
@@ -358,7 +365,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     int e = bid / n_tiles;
     int chunk = -1;
     if constexpr (MODE == GRID_EXPERTS) {      // expensive experts first (the identity when there is no order)
-        if (E <= EXPERT_ORDER_MAX) e = mt ? up_order.e[e] : gate_order.e[e];
+        if (E <= EXPERT_ORDER_MAX) e = mt ? up_order.at(e) : gate_order.at(e);
     } else if constexpr (MODE == GRID_ACTIVE && !ROUTED) {
         e = nth_active_expert(expert_offsets, E, A, e, tid & 63);
         if (e < 0) return;
@@ -394,8 +401,10 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     const FastExpert* __restrict__ fe_tab = mt ? up_fe : gate_fe;
     const FastSlab* __restrict__ fs_tab = mt ? up_fs : gate_fs;
     const int max_slabs = mt ? up_max_slabs : gate_max_slabs;
-    const FastExpert fe = fe_tab[e];
+    FastExpert fe = fe_tab[e];
     const FastSlab first = load_fast_slab(fs_tab, e * max_slabs);
+    hold_fast_expert(fe);
+    const int fe_num_slabs = fe.num_slabs;
     // the widths and payload offsets of the expert's slab groups (read by the mixed-width walk only, but
     // requested here, together with the expert's record)
     __shared__ int2 grp_tab[MIXED ? WALK_MAX_GROUPS : 1];
@@ -405,12 +414,19 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
             grp_tab[tid] = int2{gs.bits, gs.pack_off};
         }
     }
-    if constexpr (ROUTED && MODE == GRID_EXPERTS) a_end = inline_route(selected, ids_are_i64, n_flat, top_k, gid, route_lds, tid);
+    if constexpr (ROUTED && MODE == GRID_EXPERTS) {
+        hold_route_ids(rid);
+        a_end = inline_route_finish(rid, n_flat, top_k, gid, route_lds, tid);
+    }
     if (a_end <= a_begin || first.bits == 0) return;
     BITSMOE_TL(g_tl_walk, 1);
-    const int n_groups = fe.num_slabs / GU_SLABS;
-    // this workgroup's share of the slab groups, and the partial result it writes
-    const int g_begin = (int)((int64_t)part * n_groups / parts), g_end = (int)((int64_t)(part + 1) * n_groups / parts);
+    const int n_groups = fe_num_slabs / GU_SLABS;
+    // this workgroup's share of the slab groups, and the partial result it writes (no division for a whole item)
+    int g_begin = 0, g_end = n_groups;
+    if (parts > 1) {
+        g_begin = part * n_groups / parts;
+        g_end = (part + 1) * n_groups / parts;
+    }
 
     gptr<uint32_t> payload = as_global(fe.payload);
     gptr<__half> scale_s = as_global(fe.scale_s);
@@ -493,7 +509,7 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk_z(
     int e = bid / n_tiles;
     int chunk = -1;
     if constexpr (MODE == GRID_EXPERTS) {      // expensive experts first (the identity when there is no order)
-        if (E <= EXPERT_ORDER_MAX) e = order.e[e];
+        if (E <= EXPERT_ORDER_MAX) e = order.at(e);
     } else if constexpr (MODE == GRID_ACTIVE) {
         e = nth_active_expert(expert_offsets, E, A, e, tid & 63);
         if (e < 0) return;
@@ -600,6 +616,12 @@ __global__ __launch_bounds__(256, ZR > ZROWS ? 3 : 4) void k_down_decode(
     const float* __restrict__ sel_weights, const int32_t* __restrict__ global_to_local, int n_global) {
     static_assert(!ROUTED || (MODE != GRID_CHUNKS && !ZREADY), "inline routing serves whole experts");
     BITSMOE_TL(g_tl_down, 0);
+    // (the routed ids do not depend on the workgroup's expert: requested before anything else)
+    [[maybe_unused]] RouteIds rid;
+    if constexpr (ROUTED && MODE == GRID_EXPERTS) rid = inline_route_request(selected, ids_are_i64, n_flat, threadIdx.x);
+    // (the arguments the start-up goes through, in scalar registers now: one batch of loads from the argument segment)
+    asm volatile("" ::"s"(max_slabs), "s"(E), "s"(n_tiles), "s"(n_groups), "s"(n_tchunks), "s"(tiles_per_wg), "s"(n_work),
+                 "s"(top_k));
     // Workgroup b runs on XCD b % 8, and every XCD has its own L2: the workgroups of one expert coordinate
     // (which all read the same G / U rows) are given ids of one residue class, so that they share one L2;
     // on the active-expert and the chunk grid coordinate c goes to XCD c % 8, so that the coordinates that have
@@ -651,10 +673,14 @@ __global__ __launch_bounds__(256, ZR > ZROWS ? 3 : 4) void k_down_decode(
             a_end = min(a_end, a_begin + MAX_A);
         }
     }
-    const FastExpert fe = down_fe[e];
+    FastExpert fe = down_fe[e];
     FastSlab fs = FastSlab{0, 0, 0, 0};
     if (si < max_slabs) fs = load_fast_slab(down_fs, e * max_slabs + si);
-    if constexpr (ROUTED && MODE == GRID_EXPERTS) a_end = inline_route(selected, ids_are_i64, n_flat, top_k, gid, route_lds, tid);
+    hold_fast_expert(fe);
+    if constexpr (ROUTED && MODE == GRID_EXPERTS) {
+        hold_route_ids(rid);
+        a_end = inline_route_finish(rid, n_flat, top_k, gid, route_lds, tid);
+    }
     if (a_end <= a_begin || grp * DN_SLABS_PER_WG >= fe.num_slabs) return;
     BITSMOE_TL(g_tl_down, 1);
     auto assignments = [&]() {
@@ -811,8 +837,8 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
     dim3 grid((unsigned)(e_dim * gu_groups * n_tchunks), 2);
     // the expert a grid coordinate stands for: by decreasing payload size, or the identity
     auto order_of = [&](const bitsmoe_matset* set) {
-        ExpertOrder o;
-        for (int i = 0; i < EXPERT_ORDER_MAX; ++i) o.e[i] = set->has_cost_order && i < E ? set->cost_order[i] : (uint16_t)i;
+        ExpertOrder o{};
+        for (int i = 0; i < EXPERT_ORDER_MAX; ++i) o.set(i, set->has_cost_order && i < E ? set->cost_order[i] : (uint16_t)i);
         return o;
     };
     const ExpertOrder gate_order = order_of(gate), up_order = order_of(up);

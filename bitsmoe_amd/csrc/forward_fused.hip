@@ -436,7 +436,7 @@ __global__ __launch_bounds__(256, 3) void k_decode_fused(
     int e = bid / n_tiles;
     int chunk = -1;
     if constexpr (MODE == GRID_EXPERTS) {      // expensive experts first (the identity when there is no order)
-        if (E <= EXPERT_ORDER_MAX) e = order.e[e];
+        if (E <= EXPERT_ORDER_MAX) e = order.at(e);
     } else if constexpr (MODE == GRID_ACTIVE && !ROUTED) {
         e = nth_active_expert(expert_offsets, E, A, e, tid & 63);
         if (e < 0) return;
