@@ -840,7 +840,9 @@ __device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4
 // Otherwise G and U are the first of `n_part` partial results, part_stride floats apart, that are added up.
 // ZR: assignment rows whose G / U loads are in flight together while z is built (one memory round trip per ZR
 // rows: the pass is latency-bound; more rows need more registers).
-template <int W, bool ZREADY, int ZR, class AS>
+// ZBY: z is built a row per wavefront (see there); a variant of its own, chosen by the launcher for batches of several
+// assignments per expert -- in one kernel with the column-wise form either is slowed down by the other's registers.
+template <int W, bool ZREADY, int ZR, bool ZBY, class AS>
 __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> scale, gptr<__half> svec, gptr<int32_t> rank_idx,
                                  const FastSlab fs, const float* __restrict__ G, const float* __restrict__ U, int n_part,
                                  int64_t part_stride, const AS& as,
@@ -919,6 +921,62 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
             if (tid < n_a * nt) {
                 const int a = tid / nt, i = tid - a * nt;
                 zsum[a * ZSUM_STRIDE + tb + i] = U[(int64_t)(a0 + a) * (((I + N_TILE - 1) / N_TILE)) + tb + i];
+            }
+        } else if constexpr (ZBY) {
+            // z[a][c] = silu(G) * U as 16-bit operands for the rows a < n_a (other rows feed output rows that are never
+            // stored).  A wavefront takes whole rows -- w, w + 4, ... -- and a lane four neighbouring columns of each 256
+            // of the row, ZP such pieces of G and of U requested together: the rows of a chunk are ceil(n_a / 4) memory
+            // round trips, where four columns per thread over all rows, two at a time, were ceil(n_a / 2).
+            constexpr int ZP = ZR > ZROWS ? 6 : 3;
+            const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+            const int c_begin = tb * N_TILE, c_end = min((tb + nt) * N_TILE, I);
+            for (int a = wv; a < n_a; a += 4) {
+                const int64_t row_off = (int64_t)as.row(a0 + a) * I;
+                for (int p0 = c_begin; p0 < c_end; p0 += 256 * ZP) {
+                    f32x4 gv[ZP], uv[ZP];
+#pragma unroll
+                    for (int p = 0; p < ZP; ++p) {
+                        const int c = min(p0 + 256 * p + 4 * lane, c_end - 4);      // (a piece past the end repeats the last)
+                        gv[p] = *reinterpret_cast<const f32x4*>(G + row_off + c);
+                        uv[p] = *reinterpret_cast<const f32x4*>(U + row_off + c);
+                    }
+                    for (int q = 1; q < n_part; ++q) {
+#pragma unroll
+                        for (int p = 0; p < ZP; ++p) {
+                            const int c = min(p0 + 256 * p + 4 * lane, c_end - 4);
+                            gv[p] += *reinterpret_cast<const f32x4*>(G + row_off + c + q * part_stride);
+                            uv[p] += *reinterpret_cast<const f32x4*>(U + row_off + c + q * part_stride);
+                        }
+                    }
+#pragma unroll
+                    for (int p = 0; p < ZP; ++p) {
+                        const int c = p0 + 256 * p + 4 * lane;
+                        if (p0 + 256 * p >= c_end) break;      // (wave-uniform)
+                        const bool live = c < c_end;
+                        uint16_t zb[4];
+                        float part = 0.0f;      // sum of the four operands as rounded
+#pragma unroll
+                        for (int x = 0; x < 4; ++x) {
+                            zb[x] = to_operand<false>(silu_f32(gv[p][x]) * uv[p][x]);
+                            part += __half2float(__ushort_as_half(zb[x]));
+                        }
+                        part = live ? part : 0.0f;
+                        if (live) {
+                            u32x2 packed;
+                            packed[0] = (uint32_t)zb[0] | ((uint32_t)zb[1] << 16);
+                            packed[1] = (uint32_t)zb[2] | ((uint32_t)zb[3] << 16);
+                            *reinterpret_cast<u32x2*>(z + a * z_stride + c - c_begin) = packed;
+                        }
+                        // the 32 lanes of a half wavefront hold one tile's 128 columns: their sum arrives in lanes 31 and 63
+                        part = dpp_add_f32<0x111>(part);
+                        part = dpp_add_f32<0x112>(part);
+                        part = dpp_add_f32<0x114>(part);
+                        part = dpp_add_f32<0x118>(part);
+                        part = dpp_add_f32<0x142, 0xa>(part);
+                        const int c_tile = p0 + 256 * p + 4 * (lane & 32);      // first column of this half's tile
+                        if ((lane & 31) == 31 && c_tile < c_end) zsum[a * ZSUM_STRIDE + c_tile / N_TILE] = part;
+                    }
+                }
             }
         } else
         // z[a][c] = silu(G) * U as 16-bit operands for the rows a < n_a (other rows feed

@@ -605,7 +605,7 @@ __global__ __launch_bounds__(256) void k_decode_silu(const float* __restrict__ G
 // from `sel_weights` in entry order.
 // ZR: rows of G / U in flight while z is built; more than the usual two only where z is so large that three
 // workgroups fit a CU, which leaves each of them more registers (launch bounds follow).
-template <int MODE, bool ZREADY, bool ROUTED, int ZR>
+template <int MODE, bool ZREADY, bool ROUTED, int ZR, bool ZBY = false>
 __global__ __launch_bounds__(256, ZR > ZROWS ? 3 : 4) void k_down_decode(
     const FastExpert* __restrict__ down_fe, const FastSlab* __restrict__ down_fs, int max_slabs,
     const float* __restrict__ G, const float* __restrict__ U, int n_part, int64_t part_stride,
@@ -705,16 +705,16 @@ __global__ __launch_bounds__(256, ZR > ZROWS ? 3 : 4) void k_down_decode(
     // the four wavefronts may run four different instantiations; every one of them executes
     // the same two workgroup barriers per assignment chunk
     if (fs.bits == 2)
-        down_wave<2, ZREADY, ZR>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
+        down_wave<2, ZREADY, ZR, ZBY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else if (fs.bits == 3)
-        down_wave<3, ZREADY, ZR>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
+        down_wave<3, ZREADY, ZR, ZBY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else if (fs.bits == 4)
-        down_wave<4, ZREADY, ZR>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
+        down_wave<4, ZREADY, ZR, ZBY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     else
-        down_wave<0, ZREADY, ZR>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
+        down_wave<0, ZREADY, ZR, ZBY>(payload, scale, svec, rank_idx, fs, G, U, n_part, part_stride, as, a_begin, a_end, T, I, tb, nt,
                            rank_out, rank_accum, z, z_stride, zsum, rows, assigns, tid, lane);
     BITSMOE_TL(g_tl_down, 6);
 }
@@ -991,6 +991,14 @@ int launch_forward_decode(const bitsmoe_matset* gate, const bitsmoe_matset* up, 
         if constexpr (!Z) {
             if (wide) {
                 launch_down(k_down_decode<M, Z, false, ZROWS_WIDE>);
+                return;
+            }
+        }
+        // z a row per wavefront: from five assignments per expert on average (512-expert layer, 256 tokens, top-10: the
+        // kernel 5 % faster; 128 experts with four per expert: no difference; with one or two: slower)
+        if constexpr (!Z && M != GRID_CHUNKS) {
+            if (A >= policy::DOWN_Z_BY_ROWS_MIN_PER_EXPERT * (int64_t)E) {
+                launch_down(k_down_decode<M, Z, false, ZROWS, true>);
                 return;
             }
         }

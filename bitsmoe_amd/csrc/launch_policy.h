@@ -42,6 +42,11 @@ constexpr int GATEUP_DECODE_MIN_WORKGROUPS = 1536;
 // stack at 32 tokens against 300, 1200 and 2400: the kernel is bound by the instructions a workgroup issues; more,
 // shorter workgroups add their fixed part).
 constexpr int DOWN_DECODE_MIN_WORKGROUPS = 600;
+// k_down_decode builds z a row per wavefront (ceil(n_a / 4) memory round trips per chunk instead of ceil(n_a / 2)) from
+// this many assignments per expert on average, on the grids that go by routing tables: 512 experts, 256 tokens, top-10
+// (five per expert) 55.2 -> 52.4 us; 128 experts with four per expert: no difference; with one or two per expert the
+// column-wise form is faster (all threads share a row).
+constexpr int DOWN_Z_BY_ROWS_MIN_PER_EXPERT = 5;
 
 }  // namespace policy
 }  // namespace bitsmoe
