@@ -781,7 +781,7 @@ __device__ __forceinline__ void gateup_walk_z_item(const WalkMatrix& mg, const W
 #pragma unroll
         for (int nbl = 0; nbl < 2; ++nbl) {
             const int c = t * N_TILE + 32 * pair + 16 * nbl + n;
-            const uint16_t zb = to_operand<false>(silu_f32(acc_g[nbl][j] - cg) * (acc[nbl][j] - cu));
+            const uint16_t zb = z_operand(acc_g[nbl][j] - cg, acc[nbl][j] - cu);
             if (a < n_a && c < I) Z[(int64_t)(a0 + a) * I + c] = zb;
             zpart[j] += __half2float(__ushort_as_half(zb));
         }
@@ -957,7 +957,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                         float part = 0.0f;      // sum of the four operands as rounded
 #pragma unroll
                         for (int x = 0; x < 4; ++x) {
-                            zb[x] = to_operand<false>(silu_f32(gv[p][x]) * uv[p][x]);
+                            zb[x] = z_operand(gv[p][x], uv[p][x]);
                             part += __half2float(__ushort_as_half(zb[x]));
                         }
                         part = live ? part : 0.0f;
@@ -1009,7 +1009,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
                         float part = 0.0f;      // sum of the four operands as rounded
 #pragma unroll
                         for (int x = 0; x < 4; ++x) {
-                            zb[x] = to_operand<false>(silu_f32(gv[j][x]) * uv[j][x]);
+                            zb[x] = z_operand(gv[j][x], uv[j][x]);
                             part += __half2float(__ushort_as_half(zb[x]));
                         }
                         u32x2 packed;

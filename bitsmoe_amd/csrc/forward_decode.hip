@@ -379,31 +379,41 @@ __global__ __launch_bounds__(256, 4) void k_gateup_walk(
     int a_begin = 0, a_end = 0;
     int gid = -1;
     __shared__ std::conditional_t<ROUTED, InlineRouteLds, int> route_lds;
-    if constexpr (ROUTED && MODE == GRID_ACTIVE) {
-        // `e` is an entry index: serve the expert it names if this is the expert's first entry
-        const int slot = e;
-        if (slot >= n_flat) return;
-        gid = routed_id(selected, ids_are_i64, slot);
-        a_end = inline_route(selected, ids_are_i64, n_flat, top_k, gid, route_lds, tid);
-        if (a_end == 0 || route_lds.ent[0] != slot || gid < 0 || gid >= n_global) return;
-        e = global_to_local[gid];
-        if (e < 0 || e >= E) return;
-    } else if constexpr (ROUTED) {
-        gid = local_to_global[e];
-    } else {
-        a_begin = max(expert_offsets[e], 0);
-        a_end = min(expert_offsets[e + 1], A);
-        if (chunk >= 0) {
-            a_begin += MAX_A * chunk;
-            a_end = min(a_end, a_begin + MAX_A);
-        }
-    }
     const FastExpert* __restrict__ fe_tab = mt ? up_fe : gate_fe;
     const FastSlab* __restrict__ fs_tab = mt ? up_fs : gate_fs;
     const int max_slabs = mt ? up_max_slabs : gate_max_slabs;
-    FastExpert fe = fe_tab[e];
-    const FastSlab first = load_fast_slab(fs_tab, e * max_slabs);
-    hold_fast_expert(fe);
+    FastExpert fe;
+    FastSlab first;
+    if constexpr (ROUTED && MODE == GRID_ACTIVE) {
+        // `e` is an entry index: serve the expert it names if this is the expert's first entry.  The local id of that
+        // expert and its record are asked for as soon as the entry's id is here; the scan of all ids runs meanwhile.
+        const int slot = e;
+        if (slot >= n_flat) return;
+        const RouteIds all = inline_route_request(selected, ids_are_i64, n_flat, tid);
+        gid = __builtin_amdgcn_readfirstlane(routed_id(selected, ids_are_i64, slot));
+        if (gid < 0 || gid >= n_global) return;
+        e = __builtin_amdgcn_readfirstlane(global_to_local[gid]);
+        if (e < 0 || e >= E) return;
+        fe = fe_tab[e];
+        first = load_fast_slab(fs_tab, e * max_slabs);
+        a_end = inline_route_finish(all, n_flat, top_k, gid, route_lds, tid);
+        hold_fast_expert(fe);
+        if (a_end == 0 || route_lds.ent[0] != slot) return;
+    } else {
+        if constexpr (ROUTED) {
+            gid = local_to_global[e];
+        } else {
+            a_begin = max(expert_offsets[e], 0);
+            a_end = min(expert_offsets[e + 1], A);
+            if (chunk >= 0) {
+                a_begin += MAX_A * chunk;
+                a_end = min(a_end, a_begin + MAX_A);
+            }
+        }
+        fe = fe_tab[e];
+        first = load_fast_slab(fs_tab, e * max_slabs);
+        hold_fast_expert(fe);
+    }
     const int fe_num_slabs = fe.num_slabs;
     // the widths and payload offsets of the expert's slab groups (read by the mixed-width walk only, but
     // requested here, together with the expert's record)
@@ -581,7 +591,7 @@ __global__ __launch_bounds__(256) void k_decode_silu(const float* __restrict__ G
     float part = 0.0f;      // sum of the four operands as rounded
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
-        zb[x] = in ? to_operand<false>(silu_f32(gv[x]) * uv[x]) : (uint16_t)0;
+        zb[x] = in ? z_operand(gv[x], uv[x]) : (uint16_t)0;
         part += __half2float(__ushort_as_half(zb[x]));
     }
     if (in) {
@@ -654,29 +664,38 @@ __global__ __launch_bounds__(256, ZR > ZROWS ? 3 : 4) void k_down_decode(
 
     int a_begin = 0, a_end = 0, gid = -1;
     __shared__ std::conditional_t<ROUTED, InlineRouteLds, int> route_lds;
+    FastExpert fe;
+    FastSlab fs = FastSlab{0, 0, 0, 0};
     if constexpr (ROUTED && MODE == GRID_ACTIVE) {
-        // `e` is an entry index: serve the expert it names if this is the expert's first entry
+        // `e` is an entry index: serve the expert it names if this is the expert's first entry (its local id and record
+        // are asked for as soon as the entry's id is here; the scan of all ids runs meanwhile)
         const int slot = e;
         if (slot >= n_flat) return;
-        gid = routed_id(selected, ids_are_i64, slot);
-        a_end = inline_route(selected, ids_are_i64, n_flat, top_k, gid, route_lds, tid);
-        if (a_end == 0 || route_lds.ent[0] != slot || gid < 0 || gid >= n_global) return;
-        e = global_to_local[gid];
+        const RouteIds all = inline_route_request(selected, ids_are_i64, n_flat, tid);
+        gid = __builtin_amdgcn_readfirstlane(routed_id(selected, ids_are_i64, slot));
+        if (gid < 0 || gid >= n_global) return;
+        e = __builtin_amdgcn_readfirstlane(global_to_local[gid]);
         if (e < 0 || e >= E) return;
-    } else if constexpr (ROUTED) {
-        gid = local_to_global[e];
+        fe = down_fe[e];
+        if (si < max_slabs) fs = load_fast_slab(down_fs, e * max_slabs + si);
+        a_end = inline_route_finish(all, n_flat, top_k, gid, route_lds, tid);
+        hold_fast_expert(fe);
+        if (a_end == 0 || route_lds.ent[0] != slot) return;
     } else {
-        a_begin = max(expert_offsets[e], 0);
-        a_end = min(expert_offsets[e + 1], A);
-        if (chunk >= 0) {      // this workgroup's chunk only
-            a_begin += MAX_A * chunk;
-            a_end = min(a_end, a_begin + MAX_A);
+        if constexpr (ROUTED) {
+            gid = local_to_global[e];
+        } else {
+            a_begin = max(expert_offsets[e], 0);
+            a_end = min(expert_offsets[e + 1], A);
+            if (chunk >= 0) {      // this workgroup's chunk only
+                a_begin += MAX_A * chunk;
+                a_end = min(a_end, a_begin + MAX_A);
+            }
         }
+        fe = down_fe[e];
+        if (si < max_slabs) fs = load_fast_slab(down_fs, e * max_slabs + si);
+        hold_fast_expert(fe);
     }
-    FastExpert fe = down_fe[e];
-    FastSlab fs = FastSlab{0, 0, 0, 0};
-    if (si < max_slabs) fs = load_fast_slab(down_fs, e * max_slabs + si);
-    hold_fast_expert(fe);
     if constexpr (ROUTED && MODE == GRID_EXPERTS) {
         hold_route_ids(rid);
         a_end = inline_route_finish(rid, n_flat, top_k, gid, route_lds, tid);

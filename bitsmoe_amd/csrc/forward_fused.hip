@@ -176,7 +176,7 @@ __device__ __forceinline__ void fused_z_down(DownRing<WD>& ring, int n_pre, cons
         float v = 0.0f;
 #pragma unroll
         for (int nbl = 0; nbl < 2; ++nbl) {
-            uint16_t zb = to_operand<false>(silu_f32(g[nbl][j]) * u[nbl][j]);
+            uint16_t zb = z_operand(g[nbl][j], u[nbl][j]);
             if (a >= n_a) zb = 0;      // (rows without an assignment hold whatever LDS held)
             z_lds[a * FZ_STRIDE + 32 * wave + 16 * nbl + n] = zb;
             v += __half2float(__ushort_as_half(zb));

@@ -486,7 +486,7 @@ __device__ __forceinline__ void gateup_tile_body(const FastExpert fe, const Fast
 #pragma unroll
                 for (int nb = 0; nb < 4; ++nb) {
                     const float g = __half2float(__ushort_as_half(gbits[nb]));
-                    dst[16 * nb] = __builtin_bit_cast(uint16_t, (_Float16)(silu_f32(g) * acc[mb][nb][j]));
+                    dst[16 * nb] = z_operand(g, acc[mb][nb][j]);
                 }
                 continue;
             }
@@ -681,7 +681,7 @@ __device__ __forceinline__ void gateup_tile_body_dma(const FastExpert fe, const 
 #pragma unroll
                 for (int nb = 0; nb < 4; ++nb) {
                     const float g = __half2float(__ushort_as_half(gbits[nb]));
-                    dst[16 * nb] = __builtin_bit_cast(uint16_t, (_Float16)(silu_f32(g) * acc[mb][nb][j]));
+                    dst[16 * nb] = z_operand(g, acc[mb][nb][j]);
                 }
                 continue;
             }
@@ -787,8 +787,8 @@ __global__ __launch_bounds__(256) void k_silu_mul_f16(uint16_t* __restrict__ G, 
             const float g1 = __half2float(__ushort_as_half((uint16_t)(g[k] >> 16)));
             const float u0 = __half2float(__ushort_as_half((uint16_t)(u[k] & 0xFFFFu)));
             const float u1 = __half2float(__ushort_as_half((uint16_t)(u[k] >> 16)));
-            const uint32_t lo = __builtin_bit_cast(uint16_t, (_Float16)(silu_f32(g0) * u0));
-            const uint32_t hi = __builtin_bit_cast(uint16_t, (_Float16)(silu_f32(g1) * u1));
+            const uint32_t lo = z_operand(g0, u0);
+            const uint32_t hi = z_operand(g1, u1);
             o[k] = lo | (hi << 16);
         }
         *reinterpret_cast<u32x4*>(G + i * 8) = o;

@@ -301,10 +301,10 @@ __global__ __launch_bounds__(256) void k_wide_down(WideSet down, int max_slabs, 
                                 gv += *reinterpret_cast<const f32x4*>(gp + p * part_stride + c * 8 + hv * 4);
                                 uv += *reinterpret_cast<const f32x4*>(up + p * part_stride + c * 8 + hv * 4);
                             }
-                            zp[q][c][2 * hv] = (uint32_t)to_operand<false>(silu_f32(gv[0]) * uv[0]) |
-                                               ((uint32_t)to_operand<false>(silu_f32(gv[1]) * uv[1]) << 16);
-                            zp[q][c][2 * hv + 1] = (uint32_t)to_operand<false>(silu_f32(gv[2]) * uv[2]) |
-                                                   ((uint32_t)to_operand<false>(silu_f32(gv[3]) * uv[3]) << 16);
+                            zp[q][c][2 * hv] = (uint32_t)z_operand(gv[0], uv[0]) |
+                                               ((uint32_t)z_operand(gv[1], uv[1]) << 16);
+                            zp[q][c][2 * hv + 1] = (uint32_t)z_operand(gv[2], uv[2]) |
+                                                   ((uint32_t)z_operand(gv[3], uv[3]) << 16);
                         }
                 }
             }

@@ -297,4 +297,17 @@ __device__ inline uint16_t to_operand(float v) {
     }
 }
 
+// z = silu(g) * u as a 16-bit MFMA operand: the product rounded to fp32, THEN to 16 bits -- the two steps of the
+// reference's __float2half(silu(g) * u) (the tensor-core down kernel's operand, bitsmoe/algorithms/cpp/mlp_forward.cu).
+// Left to itself the compiler folds product and conversion into one instruction with a single rounding wherever it sees
+// both side by side (and a two-step conversion elsewhere in the same kernel), so that an element of z differed by one
+// f16 unit now and then, and not alike from one variant of a kernel to the next.  The empty statement keeps the fp32
+// product a value of its own.
+template <bool BF16 = false>
+__device__ __forceinline__ uint16_t z_operand(float g, float u) {
+    float p = silu_f32(g) * u;
+    asm("" : "+v"(p));
+    return to_operand<BF16>(p);
+}
+
 }  // namespace bitsmoe
