@@ -43,6 +43,8 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E peak, GB/s
+GRAPH_LAYER_STEPS = 32         # layer-steps one HIP graph of a decode-size workload holds (rounds over the distinct layers)
+GRAPH_ROUNDS_MAX_TOKENS = 256  # ... larger batches: one round (every captured call keeps a workspace of its own)
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA peak, TFLOP/s
 
 WORKLOADS = {
@@ -202,8 +204,11 @@ def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, l
                     layer_step(i)
             torch.cuda.current_stream(dev).wait_stream(side)
             torch.cuda.synchronize(dev)
+            # (a decode-size batch: several rounds over the layers in ONE graph -- a serving step replays the MoE layers
+            # of a whole model as one graph, and a graph of eight kernels would charge its launch to four layer-steps)
+            rounds = max(1, GRAPH_LAYER_STEPS // n_layers) if tokens <= GRAPH_ROUNDS_MAX_TOKENS else 1
             with torch.cuda.graph(graph):
-                g_outs = [layer_step(i) for i in range(n_layers)]
+                g_outs = [layer_step(i) for i in range(n_layers * rounds)]
             # every replay must reproduce the eager result (fp32 atomics: summation order may differ)
             for _ in range(3):
                 graph.replay()
@@ -213,15 +218,16 @@ def run_workload(blocks, spec, tokens, steps, warmup, seed=42, use_graph=True, l
                     torch.cuda.synchronize(dev)
                     if not torch.allclose(g_outs[i], ref_out, rtol=1e-4, atol=1e-5 * float(ref_out.abs().max())):
                         raise RuntimeError("graph replay differs from the eager result")
-            replays = max(1, (n_layer_steps + n_layers - 1) // n_layers)
-            for _ in range(max(1, (warmup * layers_per_step) // n_layers)):
+            per_replay = n_layers * rounds
+            replays = max(1, (n_layer_steps + per_replay - 1) // per_replay)
+            for _ in range(max(1, (warmup * layers_per_step) // per_replay)):
                 graph.replay()
             torch.cuda.synchronize(dev)
             t0 = time.perf_counter()
             for _ in range(replays):
                 graph.replay()
             torch.cuda.synchronize(dev)
-            replay = (time.perf_counter() - t0) * n_layer_steps / (replays * n_layers)     # for the same number of layer-steps
+            replay = (time.perf_counter() - t0) * n_layer_steps / (replays * per_replay)     # for the same number of layer-steps
             if replay < eager:       # large steps hide the launch cost anyway and replay has its own
                 elapsed, launch = replay, "hipgraph"
             graph_ms = replay / steps * 1e3
@@ -321,9 +327,10 @@ def run_block_scope(layers, tokens, steps, layers_per_step, use_graph):
         try:       # the block forward has no host synchronisation either: capture and replay it
             bgraph = torch.cuda.CUDAGraph()
             first = lambda y: y[0] if isinstance(y, tuple) else y
+            rounds = max(1, GRAPH_LAYER_STEPS // n_layers) if tokens <= GRAPH_ROUNDS_MAX_TOKENS else 1
             with torch.no_grad():
                 with torch.cuda.graph(bgraph):
-                    ybs = [first(layers[i].block(xs[i])) for i in range(n_layers)]
+                    ybs = [first(layers[i % n_layers].block(xs[i % n_layers])) for i in range(n_layers * rounds)]
                 for _ in range(3):
                     bgraph.replay()
                     torch.cuda.synchronize(dev)
@@ -331,12 +338,13 @@ def run_block_scope(layers, tokens, steps, layers_per_step, use_graph):
                     torch.cuda.synchronize(dev)
                     if not torch.allclose(ybs[-1].float(), ye.float(), rtol=2e-2, atol=2e-2 * float(ye.float().abs().max())):
                         raise RuntimeError("block graph replay differs from the eager result")
-                replays = max(1, (n_layer_steps + n_layers - 1) // n_layers)
+                per_replay = n_layers * rounds
+                replays = max(1, (n_layer_steps + per_replay - 1) // per_replay)
                 t0 = time.perf_counter()
                 for _ in range(replays):
                     bgraph.replay()
                 torch.cuda.synchronize(dev)
-            replay_s = (time.perf_counter() - t0) * layers_per_step / (replays * n_layers)
+            replay_s = (time.perf_counter() - t0) * layers_per_step / (replays * per_replay)
             out["hipgraph_ms_per_step"] = replay_s * 1e3
             if replay_s < block_s:
                 out.update(ms_per_step=replay_s * 1e3, tokens_per_s=tokens / replay_s, launch="hipgraph")
