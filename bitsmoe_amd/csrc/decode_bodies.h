@@ -828,10 +828,14 @@ __device__ __forceinline__ void down_block(const Block16& b, const u32x4 (&az)[4
 
 // Everything one wavefront of the down kernel does after the metadata has arrived, compiled
 // per bit-width of the wavefront's slab (W == 0: no slab, the wavefront only helps to build z).
-// The payload of the first two tiles is requested BEFORE z is built, so that the weights
-// are in flight while G and U are read and SiLU is evaluated; afterwards the tiles stream
-// through three register buffers, two tiles ahead of the one being computed (4-bit slabs, 16
-// registers per tile: two buffers, one tile ahead).  The register budget is 128, so that all four
+// The payload of the first tile is requested BEFORE z is built, so that weights are in flight
+// while G and U are read and SiLU is evaluated -- of ONE tile: loads return in the order they
+// were asked for, so the rows of G and U wait behind whatever payload was requested first, and
+// every workgroup of the launch is at this point at the same time (two tiles ahead of z: the down
+// kernel 5 to 7 % slower on 128 experts at 8 and 64 tokens and on 64 experts at 16 tokens, 3 % on
+// 512 experts at 256 tokens; none: 2 to 6 % slower).  The second tile is requested when z is
+// done; afterwards the tiles stream through two register buffers, one tile ahead of the one
+// being computed.  The register budget is 128, so that all four
 // workgroups of a CU -- on the 64-token benchmark layer the whole grid -- are resident at once:
 // what only the epilogue needs (rank and multiplier of the rows, token and weight of the
 // assignments) waits in LDS, and z is built two assignment rows at a time.
@@ -858,8 +862,8 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
         const int n_a = min(MAX_A, a_end - a0);
         int chunk_zero = 0;
         asm volatile("" : "+s"(chunk_zero));   // keeps this chunk's address arithmetic inside the loop
-        Block16 buf[3];
-        float sc[3][4];
+        Block16 buf[2];
+        float sc[2][4];
         f32x4 acc[4];
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) acc[nb] = f32x4{0, 0, 0, 0};
@@ -889,8 +893,7 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
         int row_rank = -1;
         float row_s = 0.0f;
         if constexpr (W != 0) {
-            issue(I0{}, 0);
-            if (nt > 1) issue(I1{}, 1);
+            issue(I0{}, 0);      // (ONE tile ahead of z: see above)
             row_rank = rank_idx[fs.rank_off + lane];
             row_s = gload_half(svec + fs.rank_off + lane);
         }
@@ -1032,27 +1035,18 @@ __device__ __forceinline__ void down_wave(gptr<uint32_t> payload, gptr<__half> s
         if (lane < MAX_A) assigns[lane] = int2{tok_lane, __float_as_int(rw_lane)};
         __syncthreads();
         if (a0 == a_begin) BITSMOE_TL_DOWN_STAMP(2);
-        if constexpr (W == 4) {
-            // (16 payload registers per tile: two buffers, one tile ahead)
+        if constexpr (W != 0) {
+            if (nt > 1) issue(I1{}, 1);
+        }
+        if constexpr (W != 0) {
+            // two buffers, one tile ahead of the one being computed (two ahead through three buffers: 3 to 5 % slower at 8
+            // to 256 tokens on 64, 128 and 512 experts, 1 % faster at 64 tokens on 128)
             for (int i = 0; i < nt; i += 2) {
                 compute(I0{}, i);
                 if (i + 1 < nt) {
                     if (i + 2 < nt) issue(I0{}, i + 2);
                     compute(I1{}, i + 1);
                     if (i + 3 < nt) issue(I1{}, i + 3);
-                }
-            }
-        } else if constexpr (W != 0) {
-            for (int i = 0; i < nt; i += 3) {
-                if (i + 2 < nt) issue(I2{}, i + 2);
-                compute(I0{}, i);
-                if (i + 1 < nt) {
-                    if (i + 3 < nt) issue(I0{}, i + 3);
-                    compute(I1{}, i + 1);
-                }
-                if (i + 2 < nt) {
-                    if (i + 4 < nt) issue(I1{}, i + 4);
-                    compute(I2{}, i + 2);
                 }
             }
         }
