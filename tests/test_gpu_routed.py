@@ -134,6 +134,30 @@ def test_forward_from_router_output_other_layouts(cuda_device, experts):
     assert inline == (experts == "mixed")
 
 
+def _random_shape(seed):
+    """One shape drawn from the seed: router ids 3..130 (some of them not packed), 1..257 tokens, top-k up to 8, intermediate
+    sizes of one to three tiles, ids of either width, either activation dtype, experts of one or of mixed widths."""
+    rng = np.random.default_rng(seed)
+    n_global = int(rng.choice([3, 8, 17, 40, 64, 130]))
+    n_super = int(rng.integers(0, min(3, n_global - 2)))
+    top_k = int(rng.integers(1, min(8, n_global - n_super) + 1))
+    tokens = int(rng.choice([1, 2, 3, 5, 8, 13, 31, 64, 100, 128, 200, 256, 257]))
+    tokens = min(tokens, max(1, 2048 // top_k))
+    dim = int(rng.choice([128, 256, 384]))
+    return (n_global, n_super, tokens, top_k, dim, bool(rng.integers(0, 2)), "f16" if rng.integers(0, 2) else "bf16",
+            str(rng.choice(["uniform", "mixed"])))
+
+
+@pytest.mark.parametrize("seed", range(9100, 9124))
+def test_forward_from_router_output_random_shapes(cuda_device, seed):
+    """Shapes nobody picked by hand (every grid form and both sides of their thresholds get hit over the seeds): the
+    one-call forward against the two-call form and against the oracle."""
+    n_global, n_super, tokens, top_k, dim, i64, dtype_name, experts = _random_shape(seed)
+    print(f"seed={seed} ids={n_global} not_packed={n_super} tokens={tokens} top_k={top_k} I={dim} i64={i64} {dtype_name} {experts}",
+          flush=True)
+    _case(cuda_device, seed, n_global, n_super, tokens, top_k, 512, dim, i64, dtype_name, experts=experts)
+
+
 def test_forward_from_router_output_under_graph_replay(cuda_device):
     """The one-call forward neither allocates nor synchronises: captured into a HIP graph, every replay -- with
     eager work and synchronisations in between -- reproduces the eager result."""
